@@ -1,0 +1,258 @@
+/* dnnrt.h -- C ABI of the gfx950 (MI355X) runtime that Occamy's DNN dialect
+ * lowers to.
+ *
+ * Every entry point below stands where one row of the reference's runtime API
+ * table stands (src/Conversion/DNNToLLVM/DNNAPISpecs.inc); the row and the
+ * wrapper it replaces are cited on each declaration.  Calling convention is
+ * the reference's: plain C, arguments by value, every tensor passed as its raw
+ * device pointer plus a HOST array of int64 dims (dense, row-major, no
+ * strides), scalar attributes as i64 / i32 / float.  Compute functions return
+ * the output device pointer (NULL on error, dnnrtLastError() says why);
+ * memory functions return 0 on success and non-zero on error (the reference
+ * printf()s and exit(-1)s instead, src/Tools/dnn-wrapper/cuda/wrapDNNMalloc.cpp:11-16).
+ *
+ * Differences from the reference table, all deliberate:
+ *   - a dnnrtHandle_t replaces cudnnHandle_t and is the first argument of
+ *     EVERY compute call (the reference passes a handle to the 7 cuDNN-backed
+ *     calls only).  The handle carries the stream kernels are launched on.
+ *   - every compute call takes a trailing `int32_t dtype` (DNNRT_F32 /
+ *     DNNRT_F16).  The reference is float-only.
+ *   - dnnrtConvBiasActiv takes `group` (the reference drops it,
+ *     src/Transform/DNN/opFusing/fuseConvBiasRelu.cpp:107-114).
+ *   - dnnrtMemOffset does not clear the slot (the reference memsets it,
+ *     src/Tools/dnn-wrapper/cuda/wrapDNNMemOffset.cpp:27); every kernel here
+ *     fully overwrites its output.
+ *   - one dnnrtTranspose replaces the per-rank Transpose{2,3,4,6}D symbols.
+ *   - new: dnnrtSync, dnnrtSetStream, dnnrtSetTensorFormat, dnnrtLayerNorm,
+ *     dnnrtGelu, dnnrtHostAlloc/Free, dnnrtLastError.
+ *
+ * The library is not re-entrant per handle; calls on one handle must come
+ * from one host thread at a time (the reference keeps its handles in
+ * file-scope globals, src/Conversion/DNNToLLVM/Ops/cudnn/ConvForward.cpp:15).
+ */
+#ifndef DNNRT_H
+#define DNNRT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dnnrtContext *dnnrtHandle_t; /* replaces cudnnHandle_t */
+typedef void *dnnrtStream_t;                /* a hipStream_t */
+
+enum { DNNRT_F32 = 0, DNNRT_F16 = 1, DNNRT_I64 = 2 };
+
+/* Physical layout of rank-4 activation tensors.  Dims are always passed in
+ * logical N,C,H,W order; the format says how they lie in memory.
+ * DNNRT_NCHW_TO_NHWC is honoured by the convolution calls only: X is read as
+ * NCHW, Y is written as NHWC (used for the first convolution of an fp16
+ * channels-last program, whose input arrives from the host as NCHW). */
+enum { DNNRT_NCHW = 0, DNNRT_NHWC = 1, DNNRT_NCHW_TO_NHWC = 2 };
+
+/* activation modes: cudnnActivationMode_t values the reference emits
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNActiveFunc.cpp:8-91;
+ *  fusedOp/CUDNNConvBiasReluFunc.cpp:65-68). */
+enum { DNNRT_ACT_SIGMOID = 0, DNNRT_ACT_RELU = 1, DNNRT_ACT_TANH = 2,
+       DNNRT_ACT_IDENTITY = 5 };
+
+/* tensor-op modes: cudnnOpTensorOp_t values the reference emits
+ * (src/Conversion/DNNToLLVM/Ops/cudnn/Add.cpp:148, Mul.cpp:144, Sqrt.cpp:112). */
+enum { DNNRT_OP_ADD = 0, DNNRT_OP_MUL = 1, DNNRT_OP_SQRT = 4 };
+
+/* reduce mode: only AVG (5) is ever emitted
+ * (src/Conversion/ONNXToDNN/Ops/cudnn/ReduceMeanV13.cpp:37). */
+enum { DNNRT_REDUCE_AVG = 5 };
+
+/* memcpy kinds (src/Dialect/DNN/DNN.td:61-83). */
+enum { DNNRT_H2D = 1, DNNRT_D2H = 2, DNNRT_D2D = 3 };
+
+/* ---- handle / stream ------------------------------------------------- */
+
+/* DNNAPISpecs.inc:92 "cudnnCreate" (emitted at function entry,
+ * src/Conversion/DNNToLLVM/DNNToLLVMCommon.cpp:172-177). */
+int32_t dnnrtCreate(dnnrtHandle_t *handle);
+/* DNNAPISpecs.inc:93 "cudnnDestroy". */
+int32_t dnnrtDestroy(dnnrtHandle_t handle);
+/* DNNAPISpecs.inc:94 "cudaStreamCreate" (DNNToLLVMCommon.cpp:208-213). */
+int32_t dnnrtStreamCreate(dnnrtStream_t *stream);
+/* DNNAPISpecs.inc:95 "cudaStreamDestroy". */
+int32_t dnnrtStreamDestroy(dnnrtStream_t stream);
+/* New.  Kernels of `handle` are launched on `stream` from now on (the
+ * reference launches kernels on the NULL stream and copies on its one stream). */
+int32_t dnnrtSetStream(dnnrtHandle_t handle, dnnrtStream_t stream);
+/* New.  Physical layout of rank-4 activations for subsequent calls. */
+int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format);
+/* New.  Blocks until all work on the handle's stream is done; the reference
+ * returns to the host without waiting for its device-to-host copies
+ * (src/Tools/dnn-wrapper/cuda/wrapDNNMemcpy.cpp:32). */
+int32_t dnnrtSync(dnnrtHandle_t handle);
+/* New.  Text of the calling thread's last error ("" if none). */
+const char *dnnrtLastError(void);
+/* New.  0 when built for the GPU, 1 for a host-only build of the same ABI. */
+int32_t dnnrtIsHostBackend(void);
+
+/* ---- memory ---------------------------------------------------------- */
+
+/* DNNAPISpecs.inc:49 "wrapDNNMemPoolInit"
+ * (src/Tools/dnn-wrapper/cuda/wrapDNNMemPoolInit.cpp:19-29). */
+int32_t dnnrtMemPoolInit(void **pool, int64_t bytes);
+/* DNNAPISpecs.inc:47 "wrapDNNMemOffset" (wrapDNNMemOffset.cpp:19-34). */
+int32_t dnnrtMemOffset(void **ptr, void *base, int64_t offset, int64_t bytes);
+/* DNNAPISpecs.inc:45 "wrapDNNMemcpy" (wrapDNNMemcpy.cpp:17-61). */
+int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind,
+                    dnnrtStream_t stream);
+/* DNNAPISpecs.inc:40 "wrapDNNMalloc" (wrapDNNMalloc.cpp). */
+int32_t dnnrtMalloc(void **ptr, int64_t bytes);
+/* DNNAPISpecs.inc:19 "wrapDNNDealloc" (wrapDNNDealloc.cpp). */
+int32_t dnnrtDealloc(void *ptr);
+/* New.  Pinned host staging memory for constants and results. */
+int32_t dnnrtHostAlloc(void **ptr, int64_t bytes);
+int32_t dnnrtHostFree(void *ptr);
+
+/* ---- convolution ----------------------------------------------------- */
+
+/* DNNAPISpecs.inc:108 "DNNConvFunc"
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNConvFunc.cpp:9-105).
+ * Y = conv2d(X[N,C,H,W], W[K,C/group,R,S]); cross-correlation, dilation 1,
+ * pads = {pad_h, pad_w} (symmetric), strides = {stride_h, stride_w}.
+ * `workspace`, `workspaceBytes` and `algo` are accepted and ignored. */
+void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                const void *W, const int64_t *dimW, void *workspace,
+                int64_t workspaceBytes, int64_t algo, int64_t group,
+                const int64_t *pads, const int64_t *strides, void *Y,
+                int32_t dtype);
+/* DNNAPISpecs.inc:121 "DNNConvBiasActivFunc"
+ * (src/Tools/dnn-wrapper/cudnn/fusedOp/CUDNNConvBiasReluFunc.cpp:8-140).
+ * Y = act(conv(X, W) + B), B holds K values (dimB is {1,K,1,1}),
+ * activMode DNNRT_ACT_RELU or DNNRT_ACT_IDENTITY. */
+void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X,
+                         const int64_t *dimX, const void *W,
+                         const int64_t *dimW, const void *B,
+                         const int64_t *dimB, void *workspace,
+                         int64_t workspaceBytes, int64_t algo, int64_t group,
+                         const int64_t *pads, const int64_t *strides,
+                         int64_t activMode, void *Y, int32_t dtype);
+
+/* ---- elementwise / broadcast ----------------------------------------- */
+
+/* DNNAPISpecs.inc:97 "DNNActiveFunc"
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNActiveFunc.cpp:8-91); dimX has 4 entries. */
+void *dnnrtActive(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                  int32_t mode, void *Y, int32_t dtype);
+/* DNNAPISpecs.inc:99 "DNNTensorOpFunc"
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNTensorOpFunc.cpp:8-149).
+ * O = op(A, coefB * B); B is broadcast along every dim where dimB[i] == 1;
+ * dimA == dimO; the three ranks are equal.  SQRT ignores B. */
+void *dnnrtTensorOp(dnnrtHandle_t handle, int64_t op, const void *A,
+                    const int64_t *dimA, int32_t rankA, const void *B,
+                    const int64_t *dimB, int32_t rankB, void *O,
+                    const int64_t *dimO, int32_t rankO, float coefB,
+                    int32_t dtype);
+/* DNNAPISpecs.inc:13 "CUDAClipFunc" (cuda/CUDAClipFunc.cu:5-28). */
+void *dnnrtClip(dnnrtHandle_t handle, const void *X, void *Y,
+                const int64_t *dimY, float lo, float hi, int64_t rank,
+                int32_t dtype);
+/* DNNAPISpecs.inc:30 "CUDAErfFunc" (cuda/CUDAErfFunc.cu:4-27). */
+void *dnnrtErf(dnnrtHandle_t handle, const void *X, void *Y,
+               const int64_t *dim, int64_t rank, int32_t dtype);
+/* DNNAPISpecs.inc:50 "CUDANegativeFunc" (cuda/CUDANegativeFunc.cu:4-28). */
+void *dnnrtNegative(dnnrtHandle_t handle, const void *X, void *Y,
+                    const int64_t *dim, int64_t rank, int32_t dtype);
+/* DNNAPISpecs.inc:60 "CUDAReciprocalFunc" (cuda/CUDAReciprocalFunc.cu:4-28). */
+void *dnnrtReciprocal(dnnrtHandle_t handle, const void *X, void *Y,
+                      const int64_t *dim, int64_t rank, int32_t dtype);
+/* DNNAPISpecs.inc:56 "CUDAPowFunc" (cuda/CUDAPowFunc.cu:4-32): the exponent
+ * is read from a one-element DEVICE tensor. */
+void *dnnrtPow(dnnrtHandle_t handle, const void *X, const void *exponent,
+               void *Y, const int64_t *dimY, int64_t rank, int32_t dtype);
+/* DNNAPISpecs.inc:11 "CUDACastI64toFloatFunc" (cuda/CUDACastI64toFloatFunc.cu:4-26).
+ * Returns Y (the reference returns its input pointer). */
+void *dnnrtCastI64toFloat(dnnrtHandle_t handle, const int64_t *X, void *Y,
+                          const int64_t *dimY, int64_t rank, int32_t dtype);
+/* New (no row in the reference table; the reference lowers GELU to
+ * Div, Erf, Add, Mul, Mul): Y = 0.5 x (1 + erf(x / sqrt 2)). */
+void *dnnrtGelu(dnnrtHandle_t handle, const void *X, void *Y,
+                const int64_t *dim, int64_t rank, int32_t dtype);
+
+/* ---- reductions / normalisation -------------------------------------- */
+
+/* DNNAPISpecs.inc:116 "DNNReduceFunc"
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNReduceFunc.cpp:8-142): reduces every dim
+ * where dimY[i] == 1 and dimX[i] != 1; dimY keeps the rank of dimX. */
+void *dnnrtReduce(dnnrtHandle_t handle, int32_t rank, const void *X,
+                  const int64_t *dimX, void *Y, const int64_t *dimY,
+                  int32_t mode, int32_t dtype);
+/* DNNAPISpecs.inc:64 "CUDASoftmaxFunc" (cuda/CUDASoftmaxFunc.cu:7-128);
+ * softmax along `axis` (negative axes count from the back). */
+void *dnnrtSoftmax(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                   void *Y, const int64_t *dimY, int64_t axis, int64_t rank,
+                   int32_t dtype);
+/* New (the reference lowers LayerNorm to 9 primitive calls):
+ * Y = (X - mean) / sqrt(var + eps) * gamma + beta over the last dim. */
+void *dnnrtLayerNorm(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                     int64_t rank, const void *gamma, const void *beta,
+                     float eps, void *Y, int32_t dtype);
+
+/* ---- pooling --------------------------------------------------------- */
+
+/* DNNAPISpecs.inc:113 "DNNMaxPoolFunc"
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNMaxPoolFunc.cpp:8-78): kernel[2],
+ * pads[4] = {h_begin, w_begin, h_end, w_end} of which [0] and [1] are used
+ * symmetrically, strides[2]; padding never wins the max. */
+void *dnnrtMaxPool(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                   void *Y, const int64_t *dimY, const int64_t *kernel,
+                   const int64_t *pads, const int64_t *strides, int32_t dtype);
+/* DNNAPISpecs.inc:105 "DNNAveragePoolFunc"
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNAveragePoolFunc.cpp:8-78); padding is
+ * counted in the divisor as the reference does (:44). */
+void *dnnrtAveragePool(dnnrtHandle_t handle, const void *X,
+                       const int64_t *dimX, void *Y, const int64_t *dimY,
+                       const int64_t *kernel, const int64_t *pads,
+                       const int64_t *strides, int32_t dtype);
+
+/* ---- matrix products ------------------------------------------------- */
+
+/* DNNAPISpecs.inc:4 "CUBLASMatmul2dFunc"
+ * (src/Tools/dnn-wrapper/cublas/CUBLASMatmul2dFunc.cu:9-153):
+ * Out = alpha op(A) op(B) + beta C, row-major; C may be NULL when beta == 0. */
+void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A,
+                    const int64_t *dimA, const void *B, const int64_t *dimB,
+                    const void *C, const int64_t *dimC, void *Out,
+                    const int64_t *dimOut, float alpha, float beta,
+                    int64_t transA, int64_t transB, int32_t dtype);
+/* DNNAPISpecs.inc:41 "CUDAMatmulNdFunc" (cuda/CUDAMatmulNdFunc.cu:14-173):
+ * numpy.matmul for ranks 2..4; an operand of lower rank is broadcast over the
+ * leading (batch) dims of the other. */
+void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
+                    int32_t rankA, const void *B, const int64_t *dimB,
+                    int32_t rankB, void *Y, const int64_t *dimY, int32_t rankY,
+                    int32_t dtype);
+
+/* ---- data movement --------------------------------------------------- */
+
+/* DNNAPISpecs.inc:36 "CUDAFlattenFunc" (cuda/CUDAFlattenFunc.cpp): copy. */
+void *dnnrtFlatten(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                   void *Y, const int64_t *dimY, int32_t axis, int64_t rank,
+                   int32_t dtype);
+/* DNNAPISpecs.inc:62 "CUDAReshapeFunc" (cuda/CUDAReshapeFunc.cpp): copy. */
+void *dnnrtReshape(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                   int64_t rankX, void *Y, int32_t dtype);
+/* DNNAPISpecs.inc:72-87 "CUDATranspose{2,3,4,6}D{Float,Int64}Func"
+ * (cuda/CUDATranspose4DFloatFunc.cu): Y = numpy.transpose(X, perm), rank <= 6;
+ * dtype DNNRT_I64 selects the Int64 variants. */
+void *dnnrtTranspose(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                     void *Y, const int64_t *dimY, const int64_t *perm,
+                     int64_t rank, int32_t dtype);
+/* DNNAPISpecs.inc:25 "CUDAGatherFloatFunc" (cuda/CUDAGatherFloatFunc.cu:7-82):
+ * numpy.take(X, indices, axis); negative indices count from the back. */
+void *dnnrtGather(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                  int64_t rankX, void *Y, const int64_t *dimY, int64_t rankY,
+                  const int64_t *indices, const int64_t *dimIndices,
+                  int64_t rankIndices, int64_t axis, int32_t dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DNNRT_H */

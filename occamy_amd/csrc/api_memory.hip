@@ -1,0 +1,141 @@
+// Handle, stream and memory entry points of the runtime
+// (reference: src/Tools/dnn-wrapper/cuda/wrapDNN*.cpp and the
+// cudnnCreate/cudaStreamCreate rows of DNNAPISpecs.inc:92-95).
+#include "common.h"
+
+#include <stdarg.h>
+#include <string.h>
+
+namespace dnnrt {
+static thread_local char g_err[512] = "";
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+}
+}  // namespace dnnrt
+
+using dnnrt::set_error;
+
+#define HIP_RET(call, what)                                                    \
+  do {                                                                         \
+    hipError_t e_ = (call);                                                    \
+    if (e_ != hipSuccess) {                                                    \
+      set_error("%s: %s", what, hipGetErrorString(e_));                        \
+      return (int32_t)e_;                                                      \
+    }                                                                          \
+  } while (0)
+
+extern "C" {
+
+const char *dnnrtLastError(void) { return dnnrt::g_err; }
+int32_t dnnrtIsHostBackend(void) { return 0; }
+
+int32_t dnnrtCreate(dnnrtHandle_t *handle) {
+  if (!handle) { set_error("dnnrtCreate: null handle pointer"); return 1; }
+  int dev = 0;
+  HIP_RET(hipGetDevice(&dev), "dnnrtCreate: hipGetDevice");
+  hipDeviceProp_t prop;
+  HIP_RET(hipGetDeviceProperties(&prop, dev), "dnnrtCreate: hipGetDeviceProperties");
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error("dnnrtCreate: this library holds gfx950 code only, device is %s", prop.gcnArchName);
+    return 1;
+  }
+  dnnrtContext *c = new dnnrtContext();
+  c->stream = nullptr;
+  c->format = DNNRT_NCHW;
+  c->device = dev;
+  c->num_cu = prop.multiProcessorCount;
+  *handle = c;
+  return 0;
+}
+
+int32_t dnnrtDestroy(dnnrtHandle_t handle) {
+  delete handle;
+  return 0;
+}
+
+int32_t dnnrtStreamCreate(dnnrtStream_t *stream) {
+  hipStream_t s;
+  HIP_RET(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "dnnrtStreamCreate");
+  *stream = s;
+  return 0;
+}
+
+int32_t dnnrtStreamDestroy(dnnrtStream_t stream) {
+  HIP_RET(hipStreamDestroy((hipStream_t)stream), "dnnrtStreamDestroy");
+  return 0;
+}
+
+int32_t dnnrtSetStream(dnnrtHandle_t handle, dnnrtStream_t stream) {
+  if (!handle) { set_error("dnnrtSetStream: null handle"); return 1; }
+  handle->stream = (hipStream_t)stream;
+  return 0;
+}
+
+int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format) {
+  if (!handle) { set_error("dnnrtSetTensorFormat: null handle"); return 1; }
+  if (format != DNNRT_NCHW && format != DNNRT_NHWC && format != DNNRT_NCHW_TO_NHWC) {
+    set_error("dnnrtSetTensorFormat: unknown format %d", format);
+    return 1;
+  }
+  handle->format = format;
+  return 0;
+}
+
+int32_t dnnrtSync(dnnrtHandle_t handle) {
+  if (!handle) { set_error("dnnrtSync: null handle"); return 1; }
+  HIP_RET(hipStreamSynchronize(handle->stream), "dnnrtSync");
+  return 0;
+}
+
+int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
+  if (!pool || bytes < 0) { set_error("dnnrtMemPoolInit: bad arguments"); return 1; }
+  HIP_RET(hipMalloc(pool, (size_t)(bytes > 0 ? bytes : 1)), "dnnrtMemPoolInit: hipMalloc");
+  return 0;
+}
+
+int32_t dnnrtMemOffset(void **ptr, void *base, int64_t offset, int64_t bytes) {
+  (void)bytes;
+  if (!ptr || !base || offset < 0) { set_error("dnnrtMemOffset: bad arguments"); return 1; }
+  *ptr = static_cast<char *>(base) + offset;
+  return 0;
+}
+
+int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind, dnnrtStream_t stream) {
+  hipMemcpyKind k;
+  switch (kind) {
+    case DNNRT_H2D: k = hipMemcpyHostToDevice; break;
+    case DNNRT_D2H: k = hipMemcpyDeviceToHost; break;
+    case DNNRT_D2D: k = hipMemcpyDeviceToDevice; break;
+    default: set_error("dnnrtMemcpy: kind %d", kind); return 1;
+  }
+  if (bytes <= 0) return 0;
+  HIP_RET(hipMemcpyAsync(dst, src, (size_t)bytes, k, (hipStream_t)stream), "dnnrtMemcpy");
+  return 0;
+}
+
+int32_t dnnrtMalloc(void **ptr, int64_t bytes) {
+  if (!ptr || bytes < 0) { set_error("dnnrtMalloc: bad arguments"); return 1; }
+  HIP_RET(hipMalloc(ptr, (size_t)(bytes > 0 ? bytes : 1)), "dnnrtMalloc: hipMalloc");
+  return 0;
+}
+
+int32_t dnnrtDealloc(void *ptr) {
+  HIP_RET(hipFree(ptr), "dnnrtDealloc");
+  return 0;
+}
+
+int32_t dnnrtHostAlloc(void **ptr, int64_t bytes) {
+  if (!ptr || bytes < 0) { set_error("dnnrtHostAlloc: bad arguments"); return 1; }
+  HIP_RET(hipHostMalloc(ptr, (size_t)(bytes > 0 ? bytes : 1), hipHostMallocDefault), "dnnrtHostAlloc");
+  return 0;
+}
+
+int32_t dnnrtHostFree(void *ptr) {
+  HIP_RET(hipHostFree(ptr), "dnnrtHostFree");
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,46 @@
+// Shared declarations of the gfx950 runtime library: the handle, error
+// reporting and small host helpers.  Everything here is internal; the public
+// surface is include/dnnrt.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/dnnrt.h"
+
+struct dnnrtContext {
+  hipStream_t stream;  // kernels of this handle are launched here
+  int format;          // DNNRT_NCHW / DNNRT_NHWC / DNNRT_NCHW_TO_NHWC
+  int device;
+  int num_cu;
+};
+
+namespace dnnrt {
+
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+// Compute entry points return NULL on error.
+#define DNNRT_FAIL(...)                                                        \
+  do {                                                                         \
+    ::dnnrt::set_error(__VA_ARGS__);                                           \
+    return nullptr;                                                            \
+  } while (0)
+
+#define DNNRT_CHECK_LAUNCH(what)                                               \
+  do {                                                                         \
+    hipError_t e_ = hipGetLastError();                                         \
+    if (e_ != hipSuccess) DNNRT_FAIL("%s: launch failed: %s", what, hipGetErrorString(e_)); \
+  } while (0)
+
+inline int64_t numel(const int64_t *d, int64_t rank) {
+  int64_t n = 1;
+  for (int64_t i = 0; i < rank; i++) n *= d[i];
+  return n;
+}
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool float_dtype(int32_t dt) { return dt == DNNRT_F32 || dt == DNNRT_F16; }
+
+}  // namespace dnnrt

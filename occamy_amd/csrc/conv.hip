@@ -1,0 +1,175 @@
+// Convolution entry points: dnnrtConv / dnnrtConvBiasActiv
+// (reference: src/Tools/dnn-wrapper/cudnn/CUDNNConvFunc.cpp:9-105 and
+//  cudnn/fusedOp/CUDNNConvBiasReluFunc.cpp:8-140).
+//
+// Dispatch: depthwise (one input channel per group) goes to a memory-bound
+// direct kernel; everything else is implicit GEMM on MFMA (igemm_f32.hip for
+// fp32 NCHW, conv_f16.hip for fp16).
+#include "common.h"
+#include "igemm_f32.h"
+#include "conv_f16.h"
+
+namespace dnnrt {
+
+// ---- depthwise, fp32, NCHW ------------------------------------------------
+// One thread per output element, q fastest so that a wavefront reads
+// contiguous input rows.  The R*S filter taps of a channel are wave-uniform
+// most of the time and come from the scalar/L1 path.
+template <int R, int S>
+__global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
+    const float *__restrict__ X, const float *__restrict__ Wt, const float *__restrict__ bias,
+    float *__restrict__ Y, int C, int H, int W, int K, int Kg, int P, int Q, int ph, int pw,
+    int sh, int sw, int rr, int ss, int act, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int q = (int)(i % Q);
+  int64_t t = i / Q;
+  const int p = (int)(t % P);
+  t /= P;
+  const int k = (int)(t % K);
+  const int n = (int)(t / K);
+  const int c = k / Kg;
+  const int Rr = R ? R : rr, Ss = S ? S : ss;
+  const float *x = X + ((int64_t)n * C + c) * H * W;
+  const float *w = Wt + (int64_t)k * Rr * Ss;
+  const int ih0 = p * sh - ph, iw0 = q * sw - pw;
+  float acc = 0.f;
+#pragma unroll
+  for (int r = 0; r < Rr; r++) {
+    const int ih = ih0 + r;
+    if ((unsigned)ih >= (unsigned)H) continue;
+#pragma unroll
+    for (int s = 0; s < Ss; s++) {
+      const int iw = iw0 + s;
+      if ((unsigned)iw < (unsigned)W) acc = fmaf(x[(int64_t)ih * W + iw], w[r * Ss + s], acc);
+    }
+  }
+  if (bias) acc += bias[k];
+  if (act == DNNRT_ACT_RELU) acc = acc < 0.f ? 0.f : acc;
+  Y[i] = acc;
+}
+
+struct ConvShape {
+  int N, C, H, W, K, Cg, R, S, P, Q, ph, pw, sh, sw, group;
+};
+
+static bool parse_conv(const char *who, const int64_t *dX, const int64_t *dW, int64_t group,
+                       const int64_t *pads, const int64_t *strides, ConvShape &s) {
+  if (!dX || !dW || !pads || !strides) { set_error("%s: null dims", who); return false; }
+  for (int i = 0; i < 4; i++)
+    if (dX[i] <= 0 || dW[i] <= 0 || dX[i] > INT32_MAX || dW[i] > INT32_MAX) {
+      set_error("%s: dims must be positive 32-bit values", who);
+      return false;
+    }
+  if (group < 1 || dW[0] % group || dX[1] != dW[1] * group) {
+    set_error("%s: C=%ld, W holds C/group=%ld, group=%ld, K=%ld do not agree", who, (long)dX[1],
+              (long)dW[1], (long)group, (long)dW[0]);
+    return false;
+  }
+  if (pads[0] < 0 || pads[1] < 0 || strides[0] < 1 || strides[1] < 1) {
+    set_error("%s: bad pads/strides", who);
+    return false;
+  }
+  s.N = (int)dX[0]; s.C = (int)dX[1]; s.H = (int)dX[2]; s.W = (int)dX[3];
+  s.K = (int)dW[0]; s.Cg = (int)dW[1]; s.R = (int)dW[2]; s.S = (int)dW[3];
+  s.ph = (int)pads[0]; s.pw = (int)pads[1]; s.sh = (int)strides[0]; s.sw = (int)strides[1];
+  s.group = (int)group;
+  const int64_t P = (s.H + 2 * (int64_t)s.ph - s.R) / s.sh + 1, Q = (s.W + 2 * (int64_t)s.pw - s.S) / s.sw + 1;
+  if (s.H + 2 * s.ph < s.R || s.W + 2 * s.pw < s.S || P < 1 || Q < 1) { set_error("%s: empty output", who); return false; }
+  s.P = (int)P; s.Q = (int)Q;
+  if ((int64_t)s.N * P * Q > INT32_MAX || (int64_t)s.Cg * s.R * s.S > INT32_MAX ||
+      (int64_t)s.C * s.H * s.W > INT32_MAX) {
+    set_error("%s: problem too large for 32-bit tile indices", who);
+    return false;
+  }
+  return true;
+}
+
+static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const float *X,
+                           const float *Wt, const float *bias, int act, float *Y) {
+  if (s.Cg == 1 && s.group > 1) {  // depthwise
+    const int64_t total = (int64_t)s.N * s.K * s.P * s.Q;
+    const int Kg = s.K / s.group;
+    dim3 grid((unsigned)ceil_div(total, 256)), block(256);
+    if (ceil_div(total, 256) > INT32_MAX) DNNRT_FAIL("conv: depthwise output too large");
+    if (s.R == 3 && s.S == 3)
+      hipLaunchKernelGGL((dwconv_f32_nchw_kernel<3, 3>), grid, block, 0, ctx->stream, X, Wt, bias, Y,
+                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, total);
+    else
+      hipLaunchKernelGGL((dwconv_f32_nchw_kernel<0, 0>), grid, block, 0, ctx->stream, X, Wt, bias, Y,
+                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, total);
+    DNNRT_CHECK_LAUNCH("conv(depthwise)");
+    return Y;
+  }
+  IgemmArgs a{};
+  const int Kg = s.K / s.group;
+  a.A = Wt; a.X = X; a.Y = Y; a.bias = bias; a.Cin = nullptr;
+  a.alpha = 1.f; a.beta = 0.f; a.act = act;
+  a.M = Kg; a.Kdim = s.Cg * s.R * s.S; a.Ncols = s.N * s.P * s.Q;
+  a.H = s.H; a.W = s.W; a.R = s.R; a.S = s.S; a.P = s.P; a.Q = s.Q;
+  a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw;
+  a.x_img_stride = (int64_t)s.C * s.H * s.W;
+  a.y_img_stride = (int64_t)s.K * s.P * s.Q;
+  a.y_row_stride = (int64_t)s.P * s.Q;
+  a.Z = s.group;
+  a.a_z_stride = (int64_t)Kg * a.Kdim;
+  a.x_z_stride = (int64_t)s.Cg * s.H * s.W;
+  a.y_z_stride = (int64_t)Kg * s.P * s.Q;
+  a.bias_z_stride = Kg;
+  a.b_kcontig = false; a.a_mcontig = false;
+  a.a_vec4 = (a.Kdim % 4 == 0) && aligned16(Wt);
+  a.b_vec4 = false;
+  if (!launch_igemm_f32(ctx, a)) return nullptr;
+  return Y;
+}
+
+static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX,
+                           const void *W, const int64_t *dW, const void *B, int64_t group,
+                           const int64_t *pads, const int64_t *strides, int act, void *Y,
+                           int32_t dtype) {
+  if (!h) DNNRT_FAIL("%s: null handle", who);
+  if (!X || !W || !Y) DNNRT_FAIL("%s: null tensor", who);
+  ConvShape s;
+  if (!parse_conv(who, dX, dW, group, pads, strides, s)) return nullptr;
+  if (dtype == DNNRT_F32) {
+    if (h->format != DNNRT_NCHW) DNNRT_FAIL("%s: fp32 tensors are NCHW only", who);
+    return conv_f32_nchw(h, s, (const float *)X, (const float *)W, (const float *)B, act, (float *)Y);
+  }
+  if (dtype == DNNRT_F16) {
+    ConvF16Args a{};
+    a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Y = (__half *)Y;
+    a.N = s.N; a.C = s.C; a.H = s.H; a.W = s.W; a.K = s.K; a.Cg = s.Cg; a.R = s.R; a.S = s.S;
+    a.P = s.P; a.Q = s.Q; a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw; a.group = s.group;
+    a.act = act; a.format = h->format;
+    if (!launch_conv_f16(h, a)) return nullptr;
+    return Y;
+  }
+  DNNRT_FAIL("%s: dtype %d", who, dtype);
+}
+
+}  // namespace dnnrt
+
+extern "C" {
+
+void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
+                const int64_t *dimW, void *workspace, int64_t workspaceBytes, int64_t algo,
+                int64_t group, const int64_t *pads, const int64_t *strides, void *Y, int32_t dtype) {
+  (void)workspace; (void)workspaceBytes; (void)algo;
+  return dnnrt::conv_dispatch("dnnrtConv", handle, X, dimX, W, dimW, nullptr, group, pads, strides,
+                              DNNRT_ACT_IDENTITY, Y, dtype);
+}
+
+void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
+                         const int64_t *dimW, const void *B, const int64_t *dimB, void *workspace,
+                         int64_t workspaceBytes, int64_t algo, int64_t group, const int64_t *pads,
+                         const int64_t *strides, int64_t activMode, void *Y, int32_t dtype) {
+  (void)workspace; (void)workspaceBytes; (void)algo;
+  if (activMode != DNNRT_ACT_RELU && activMode != DNNRT_ACT_IDENTITY)
+    DNNRT_FAIL("dnnrtConvBiasActiv: activMode %ld (1 = ReLU, 5 = identity)", (long)activMode);
+  if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
+    DNNRT_FAIL("dnnrtConvBiasActiv: bias must hold K values");
+  return dnnrt::conv_dispatch("dnnrtConvBiasActiv", handle, X, dimX, W, dimW, B, group, pads,
+                              strides, (int)activMode, Y, dtype);
+}
+
+}  // extern "C"

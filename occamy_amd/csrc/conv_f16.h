@@ -1,0 +1,17 @@
+// fp16 convolution (fp32 accumulate) on gfx950 MFMA.
+#pragma once
+#include "common.h"
+
+namespace dnnrt {
+
+struct ConvF16Args {
+  const __half *X, *Wt, *bias;
+  __half *Y;
+  int N, C, H, W, K, Cg, R, S, P, Q, ph, pw, sh, sw, group;
+  int act;     // DNNRT_ACT_RELU / DNNRT_ACT_IDENTITY
+  int format;  // physical layout of X and Y (DNNRT_NCHW / NHWC / NCHW_TO_NHWC)
+};
+
+bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a);
+
+}  // namespace dnnrt

@@ -1,0 +1,41 @@
+// fp32 implicit-GEMM on gfx950 MFMA: one kernel family serves dense
+// convolution (NCHW), 2-D GEMM and batched matmul.
+//
+//   D[m, col] = act(alpha * sum_k A[m, k] * B[k, col] + bias[m] + beta * Cin[m, col])
+//
+// A is the weight / left matrix, B the im2col view of the input / right
+// matrix.  Columns are output pixels (n, p, q) flattened; for a plain matrix
+// product the "image" is 1 x Ncols.
+#pragma once
+#include "common.h"
+
+namespace dnnrt {
+
+struct IgemmArgs {
+  const float *A;     // [M][Kdim] (k contiguous), or [Kdim][M] when a_mcontig
+  const float *X;     // conv input / right matrix
+  float *Y;
+  const float *bias;  // per row m, may be null
+  const float *Cin;   // same indexing as Y, scaled by beta, may be null
+  float alpha, beta;
+  int act;            // DNNRT_ACT_RELU or DNNRT_ACT_IDENTITY
+  int M, Kdim, Ncols;
+  // geometry of B: column -> (img, p, q); k -> (c, r, s)
+  int H, W, R, S, P, Q, ph, pw, sh, sw;
+  int64_t x_img_stride;   // elements between images of X (C*H*W)
+  int64_t y_img_stride;   // elements between images of Y (K*P*Q)
+  int64_t y_row_stride;   // elements between rows m of Y (P*Q, or ldc)
+  // blockIdx.z: group of a grouped convolution or batch of a batched matmul
+  int Z;
+  int64_t a_z_stride, x_z_stride, y_z_stride, bias_z_stride;
+  bool b_kcontig;     // B stored [Ncols][Kdim] (k contiguous): GEMM with transB
+  bool a_mcontig;     // A stored [Kdim][M]: GEMM with transA
+  bool a_vec4;        // A rows may be read as aligned float4
+  bool b_vec4;        // (b_kcontig) B rows may be read as aligned float4
+};
+
+// Launches the kernel on `stream`; returns false (with the error text set) if
+// the shape cannot be handled.
+bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a);
+
+}  // namespace dnnrt

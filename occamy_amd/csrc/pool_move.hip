@@ -1,0 +1,230 @@
+// Pooling and pure data-movement entry points (all HBM-bound).
+// Reference wrappers replaced (under src/Tools/dnn-wrapper/):
+//   cudnn/CUDNNMaxPoolFunc.cpp, cudnn/CUDNNAveragePoolFunc.cpp,
+//   cuda/CUDAFlattenFunc.cpp, CUDAReshapeFunc.cpp,
+//   CUDATranspose{2,3,4,6}D{Float,Int64}Func.cu, CUDAGatherFloatFunc.cu.
+#include "common.h"
+
+namespace dnnrt {
+
+__device__ __forceinline__ float pl_ld(const float *p) { return *p; }
+__device__ __forceinline__ float pl_ld(const __half *p) { return __half2float(*p); }
+__device__ __forceinline__ void pl_st(float *p, float v) { *p = v; }
+__device__ __forceinline__ void pl_st(__half *p, float v) { *p = __float2half_rn(v); }
+
+// One thread per output element.  Element strides of the input / output are
+// passed in, so the same kernel serves NCHW (w fastest) and NHWC (c fastest);
+// the thread index runs over the output in its memory order.
+struct PoolGeom {
+  int N, C, H, W, P, Q, R, S, ph, pw, sh, sw;
+  int nhwc;
+};
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(256) void pool_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                   PoolGeom g, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  int n, c, p, q;
+  int64_t t = i;
+  if (g.nhwc) {
+    c = (int)(t % g.C); t /= g.C; q = (int)(t % g.Q); t /= g.Q; p = (int)(t % g.P); n = (int)(t / g.P);
+  } else {
+    q = (int)(t % g.Q); t /= g.Q; p = (int)(t % g.P); t /= g.P; c = (int)(t % g.C); n = (int)(t / g.C);
+  }
+  const int64_t sx_w = g.nhwc ? g.C : 1, sx_h = sx_w * g.W;
+  const T *xb = g.nhwc ? x + (int64_t)n * g.H * g.W * g.C + c : x + ((int64_t)n * g.C + c) * g.H * g.W;
+  const int ih0 = p * g.sh - g.ph, iw0 = q * g.sw - g.pw;
+  float m = -INFINITY, s = 0.f;
+  bool nan = false;
+  for (int r = 0; r < g.R; r++) {
+    const int ih = ih0 + r;
+    if ((unsigned)ih >= (unsigned)g.H) continue;
+    for (int ss = 0; ss < g.S; ss++) {
+      const int iw = iw0 + ss;
+      if ((unsigned)iw >= (unsigned)g.W) continue;
+      const float v = pl_ld(xb + ih * sx_h + iw * sx_w);
+      nan = nan || (v != v);
+      m = v > m ? v : m;
+      s += v;
+    }
+  }
+  const float out = IS_MAX ? (nan ? __builtin_nanf("") : m) : s / (float)(g.R * g.S);
+  pl_st(y + i, out);
+}
+
+static void *pool_entry(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
+                        const int64_t *dY, const int64_t *kr, const int64_t *pads, const int64_t *st,
+                        bool is_max, int32_t dtype) {
+  if (!h) DNNRT_FAIL("%s: null handle", who);
+  if (!X || !Y || !dX || !dY || !kr || !pads || !st) DNNRT_FAIL("%s: null argument", who);
+  for (int i = 0; i < 4; i++)
+    if (dX[i] <= 0 || dY[i] <= 0 || dX[i] > INT32_MAX) DNNRT_FAIL("%s: bad dims", who);
+  if (dY[0] != dX[0] || dY[1] != dX[1]) DNNRT_FAIL("%s: N and C of X and Y differ", who);
+  if (kr[0] < 1 || kr[1] < 1 || st[0] < 1 || st[1] < 1 || pads[0] < 0 || pads[1] < 0)
+    DNNRT_FAIL("%s: bad kernel/strides/pads", who);
+  PoolGeom g;
+  g.N = (int)dX[0]; g.C = (int)dX[1]; g.H = (int)dX[2]; g.W = (int)dX[3];
+  g.P = (int)dY[2]; g.Q = (int)dY[3]; g.R = (int)kr[0]; g.S = (int)kr[1];
+  g.ph = (int)pads[0]; g.pw = (int)pads[1]; g.sh = (int)st[0]; g.sw = (int)st[1];
+  g.nhwc = h->format != DNNRT_NCHW;
+  // every window must touch the input, or max would be -inf / avg 0 silently
+  if ((int64_t)(g.P - 1) * g.sh - g.ph >= g.H || (int64_t)(g.Q - 1) * g.sw - g.pw >= g.W ||
+      g.ph >= g.R || g.pw >= g.S)
+    DNNRT_FAIL("%s: a pooling window lies outside the input", who);
+  const int64_t total = numel(dY, 4), blocks = ceil_div(total, 256);
+  if (blocks > INT32_MAX) DNNRT_FAIL("%s: tensor too large", who);
+#define POOL_LAUNCH(T, MX)                                                                       \
+  hipLaunchKernelGGL((pool_kernel<T, MX>), dim3((unsigned)blocks), dim3(256), 0, h->stream,      \
+                     (const T *)X, (T *)Y, g, total)
+  if (dtype == DNNRT_F32) { if (is_max) POOL_LAUNCH(float, true); else POOL_LAUNCH(float, false); }
+  else if (dtype == DNNRT_F16) { if (is_max) POOL_LAUNCH(__half, true); else POOL_LAUNCH(__half, false); }
+  else DNNRT_FAIL("%s: dtype %d", who, dtype);
+#undef POOL_LAUNCH
+  DNNRT_CHECK_LAUNCH(who);
+  return Y;
+}
+
+struct PermGeom {
+  int64_t dy[6];  // output dims
+  int64_t sx[6];  // input stride of the dim each output dim comes from
+};
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                        PermGeom g, int rank, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  int64_t rem = i, ix = 0;
+  for (int d = rank - 1; d >= 0; d--) {
+    const int64_t q = rem / g.dy[d];
+    ix += (rem - q * g.dy[d]) * g.sx[d];
+    rem = q;
+  }
+  y[i] = x[ix];
+}
+
+// Y[o, j, in] = X[o, idx[j], in]; out-of-range indices produce zeros.
+template <typename T>
+__global__ __launch_bounds__(256) void gather_kernel(const T *__restrict__ x, const int64_t *__restrict__ idx,
+                                                     T *__restrict__ y, int64_t ni, int64_t L,
+                                                     int64_t inner, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t in = i % inner, t = i / inner, j = t % ni, o = t / ni;
+  int64_t k = idx[j];
+  if (k < 0) k += L;
+  T v = T(0);
+  if (k >= 0 && k < L) v = x[(o * L + k) * inner + in];
+  y[i] = v;
+}
+
+static int64_t esize(int32_t dtype) {
+  return dtype == DNNRT_F32 ? 4 : dtype == DNNRT_F16 ? 2 : dtype == DNNRT_I64 ? 8 : 0;
+}
+
+static void *copy_entry(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rank,
+                        void *Y, int32_t dtype) {
+  if (!h) DNNRT_FAIL("%s: null handle", who);
+  if (!X || !Y || !dX) DNNRT_FAIL("%s: null argument", who);
+  const int64_t es = esize(dtype);
+  if (!es) DNNRT_FAIL("%s: dtype %d", who, dtype);
+  if (h->format != DNNRT_NCHW && rank == 4 && dX[1] > 1 && dX[2] * dX[3] > 1)
+    DNNRT_FAIL("%s: a channels-last tensor with spatial extent cannot be re-viewed by a copy", who);
+  const int64_t bytes = numel(dX, rank) * es;
+  if (bytes > 0 && X != Y) {
+    hipError_t e = hipMemcpyAsync(Y, X, (size_t)bytes, hipMemcpyDeviceToDevice, h->stream);
+    if (e != hipSuccess) DNNRT_FAIL("%s: %s", who, hipGetErrorString(e));
+  }
+  return Y;
+}
+
+}  // namespace dnnrt
+
+using namespace dnnrt;
+
+extern "C" {
+
+void *dnnrtMaxPool(dnnrtHandle_t handle, const void *X, const int64_t *dimX, void *Y, const int64_t *dimY,
+                   const int64_t *kernel, const int64_t *pads, const int64_t *strides, int32_t dtype) {
+  return pool_entry("dnnrtMaxPool", handle, X, dimX, Y, dimY, kernel, pads, strides, true, dtype);
+}
+void *dnnrtAveragePool(dnnrtHandle_t handle, const void *X, const int64_t *dimX, void *Y,
+                       const int64_t *dimY, const int64_t *kernel, const int64_t *pads,
+                       const int64_t *strides, int32_t dtype) {
+  return pool_entry("dnnrtAveragePool", handle, X, dimX, Y, dimY, kernel, pads, strides, false, dtype);
+}
+
+void *dnnrtFlatten(dnnrtHandle_t handle, const void *X, const int64_t *dimX, void *Y, const int64_t *dimY,
+                   int32_t axis, int64_t rank, int32_t dtype) {
+  (void)dimY; (void)axis;
+  return copy_entry("dnnrtFlatten", handle, X, dimX, rank, Y, dtype);
+}
+void *dnnrtReshape(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
+                   int32_t dtype) {
+  return copy_entry("dnnrtReshape", handle, X, dimX, rankX, Y, dtype);
+}
+
+void *dnnrtTranspose(dnnrtHandle_t handle, const void *X, const int64_t *dimX, void *Y,
+                     const int64_t *dimY, const int64_t *perm, int64_t rank, int32_t dtype) {
+  if (!handle) DNNRT_FAIL("dnnrtTranspose: null handle");
+  if (!X || !Y || !dimX || !dimY || !perm) DNNRT_FAIL("dnnrtTranspose: null argument");
+  if (rank < 1 || rank > 6) DNNRT_FAIL("dnnrtTranspose: rank %ld (1..6)", (long)rank);
+  if (handle->format != DNNRT_NCHW && rank == 4) DNNRT_FAIL("dnnrtTranspose: channels-last tensors are not supported");
+  int64_t sx[6], s = 1;
+  bool seen[6] = {false, false, false, false, false, false};
+  for (int i = (int)rank - 1; i >= 0; i--) { sx[i] = s; s *= dimX[i]; }
+  PermGeom g;
+  for (int i = 0; i < rank; i++) {
+    if (perm[i] < 0 || perm[i] >= rank || seen[perm[i]]) DNNRT_FAIL("dnnrtTranspose: perm is not a permutation");
+    seen[perm[i]] = true;
+    if (dimY[i] != dimX[perm[i]] || dimY[i] <= 0) DNNRT_FAIL("dnnrtTranspose: dimY[%d] != dimX[perm[%d]]", i, i);
+    g.dy[i] = dimY[i];
+    g.sx[i] = sx[perm[i]];
+  }
+  const int64_t total = s, blocks = ceil_div(total, 256);
+  if (blocks > INT32_MAX) DNNRT_FAIL("dnnrtTranspose: tensor too large");
+  if (dtype == DNNRT_F32)
+    hipLaunchKernelGGL((transpose_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
+                       (const float *)X, (float *)Y, g, (int)rank, total);
+  else if (dtype == DNNRT_F16)
+    hipLaunchKernelGGL((transpose_kernel<uint16_t>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
+                       (const uint16_t *)X, (uint16_t *)Y, g, (int)rank, total);
+  else if (dtype == DNNRT_I64)
+    hipLaunchKernelGGL((transpose_kernel<int64_t>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
+                       (const int64_t *)X, (int64_t *)Y, g, (int)rank, total);
+  else DNNRT_FAIL("dnnrtTranspose: dtype %d", dtype);
+  DNNRT_CHECK_LAUNCH("dnnrtTranspose");
+  return Y;
+}
+
+void *dnnrtGather(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
+                  const int64_t *dimY, int64_t rankY, const int64_t *indices, const int64_t *dimIndices,
+                  int64_t rankIndices, int64_t axis, int32_t dtype) {
+  (void)dimY; (void)rankY;
+  if (!handle) DNNRT_FAIL("dnnrtGather: null handle");
+  if (!X || !Y || !dimX || !indices || (rankIndices > 0 && !dimIndices)) DNNRT_FAIL("dnnrtGather: null argument");
+  if (rankX < 1 || rankX > 8) DNNRT_FAIL("dnnrtGather: rank %ld", (long)rankX);
+  if (axis < 0) axis += rankX;
+  if (axis < 0 || axis >= rankX) DNNRT_FAIL("dnnrtGather: axis out of range");
+  int64_t outer = 1, inner = 1;
+  const int64_t ni = numel(dimIndices, rankIndices), L = dimX[axis];
+  for (int64_t i = 0; i < axis; i++) outer *= dimX[i];
+  for (int64_t i = axis + 1; i < rankX; i++) inner *= dimX[i];
+  const int64_t total = outer * ni * inner;
+  if (total == 0) return Y;
+  const int64_t blocks = ceil_div(total, 256);
+  if (blocks > INT32_MAX) DNNRT_FAIL("dnnrtGather: tensor too large");
+  if (dtype == DNNRT_F32)
+    hipLaunchKernelGGL((gather_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
+                       (const float *)X, indices, (float *)Y, ni, L, inner, total);
+  else if (dtype == DNNRT_F16)
+    hipLaunchKernelGGL((gather_kernel<uint16_t>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
+                       (const uint16_t *)X, indices, (uint16_t *)Y, ni, L, inner, total);
+  else if (dtype == DNNRT_I64)
+    hipLaunchKernelGGL((gather_kernel<int64_t>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
+                       (const int64_t *)X, indices, (int64_t *)Y, ni, L, inner, total);
+  else DNNRT_FAIL("dnnrtGather: dtype %d", dtype);
+  DNNRT_CHECK_LAUNCH("dnnrtGather");
+  return Y;
+}
+
+}  // extern "C"

@@ -1,0 +1,688 @@
+/* dnnrt_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT.
+ *
+ * A CPU restatement, in plain C, of what each call of the reference's runtime
+ * wrapper library (src/Tools/dnn-wrapper/ in the reference tree) computes,
+ * exported under the same C ABI as the GPU library (include/dnnrt.h) so that
+ * one DNN program can be executed against either.  Only tests, the smoke
+ * check and the CPU-baseline leg of the benchmark may load this file's shared
+ * object; nothing in the product package links or opens it.
+ *
+ * The reference's arithmetic for these calls lives in closed-source cuDNN
+ * 8.9.0 / cuBLASLt (CUDA 11.8) and in its own CUDA kernels; neither can be
+ * built or run here, and the reference's tests hold no golden vectors for
+ * them.  Each function below therefore states the published definition of the
+ * operator at the reference's call site (cited), and is pinned by the tests
+ * against closed forms, brute force on tiny shapes and an independent library
+ * (torch CPU) -- see tests/test_oracle_ops.py.  Nothing here was checked
+ * against reference OUTPUT: parity with the reference's numbers is unpinned.
+ *
+ * Arithmetic: tensors are fp32 or fp16 in memory; fp16 tensors are widened to
+ * fp32 on load and rounded to nearest-even on store.  Reductions (convolution,
+ * matrix products, means, softmax sums) accumulate in double and round once,
+ * so the oracle sits closer to the exact value than any fp32 summation order.
+ * Layout is dense NCHW / row-major, as in the reference
+ * (src/Tools/dnn-wrapper/cudnn/CUDNNConvFunc.cpp:48-60).
+ */
+#include "../include/dnnrt.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static __thread char g_err[256];
+static int g_threads = 0; /* 0 = OpenMP default */
+
+#define FAIL(...)                                                              \
+  do {                                                                         \
+    snprintf(g_err, sizeof g_err, __VA_ARGS__);                                \
+    return NULL;                                                               \
+  } while (0)
+
+const char *dnnrtLastError(void) { return g_err; }
+int32_t dnnrtIsHostBackend(void) { return 1; }
+
+/* Oracle-only: number of OpenMP threads used by the heavy loops. */
+int32_t dnnrtOracleSetThreads(int32_t n) {
+  g_threads = n;
+#ifdef _OPENMP
+  if (n > 0) omp_set_num_threads(n);
+#endif
+  return 0;
+}
+int32_t dnnrtOracleGetThreads(void) {
+#ifdef _OPENMP
+  return g_threads > 0 ? g_threads : omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* ---- fp16 <-> fp32 (IEEE binary16, round to nearest even) -------------- */
+
+static float h2f(uint16_t h) {
+  uint32_t s = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1fu,
+           m = h & 0x3ffu, u;
+  if (e == 0) {
+    if (m == 0) u = s;
+    else {
+      int sh = 0;
+      while (!(m & 0x400u)) { m <<= 1; sh++; }
+      u = s | ((uint32_t)(113 - sh) << 23) | ((m & 0x3ffu) << 13);
+    }
+  } else if (e == 31) u = s | 0x7f800000u | (m << 13);
+  else u = s | ((e + 112) << 23) | (m << 13);
+  float f; memcpy(&f, &u, 4); return f;
+}
+static uint16_t f2h(float f) {
+  uint32_t u; memcpy(&u, &f, 4);
+  uint32_t s = (u >> 16) & 0x8000u; int32_t e = (int32_t)((u >> 23) & 0xff);
+  uint32_t m = u & 0x7fffffu;
+  if (e == 255) return (uint16_t)(s | 0x7c00u | (m ? 0x200u | (m >> 13) : 0));
+  e -= 112;
+  if (e >= 31) return (uint16_t)(s | 0x7c00u);
+  if (e <= 0) {
+    if (e < -10) return (uint16_t)s;
+    m |= 0x800000u;
+    uint32_t shift = (uint32_t)(14 - e), r = m >> shift,
+             rem = m & ((1u << shift) - 1), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (r & 1))) r++;
+    return (uint16_t)(s | r);
+  }
+  uint32_t r = ((uint32_t)e << 10) | (m >> 13), rem = m & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (r & 1))) r++;
+  return (uint16_t)(s | r);
+}
+
+static int64_t numel(const int64_t *d, int64_t rank) {
+  int64_t n = 1;
+  for (int64_t i = 0; i < rank; i++) n *= d[i];
+  return n;
+}
+/* widen a tensor to a fresh float buffer (fp32: plain copy of the pointer) */
+static const float *widen(const void *p, int64_t n, int32_t dtype, float **tmp) {
+  *tmp = NULL;
+  if (dtype == DNNRT_F32) return (const float *)p;
+  float *t = (float *)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
+  const uint16_t *h = (const uint16_t *)p;
+  for (int64_t i = 0; i < n; i++) t[i] = h2f(h[i]);
+  *tmp = t;
+  return t;
+}
+static float *outbuf(void *p, int64_t n, int32_t dtype, float **tmp) {
+  *tmp = NULL;
+  if (dtype == DNNRT_F32) return (float *)p;
+  *tmp = (float *)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1));
+  return *tmp;
+}
+static void narrow(void *p, float *tmp, int64_t n, int32_t dtype) {
+  if (dtype == DNNRT_F32 || !tmp) return;
+  uint16_t *h = (uint16_t *)p;
+  for (int64_t i = 0; i < n; i++) h[i] = f2h(tmp[i]);
+  free(tmp);
+}
+static int bad_dtype(int32_t dtype) { return dtype != DNNRT_F32 && dtype != DNNRT_F16; }
+
+/* ---- handle / stream / memory: host stand-ins -------------------------- */
+
+struct dnnrtContext { int format; };
+
+int32_t dnnrtCreate(dnnrtHandle_t *h) {
+  *h = (dnnrtHandle_t)calloc(1, sizeof(struct dnnrtContext));
+  return *h ? 0 : 1;
+}
+int32_t dnnrtDestroy(dnnrtHandle_t h) { free(h); return 0; }
+int32_t dnnrtStreamCreate(dnnrtStream_t *s) { *s = NULL; return 0; }
+int32_t dnnrtStreamDestroy(dnnrtStream_t s) { (void)s; return 0; }
+int32_t dnnrtSetStream(dnnrtHandle_t h, dnnrtStream_t s) { (void)h; (void)s; return 0; }
+int32_t dnnrtSetTensorFormat(dnnrtHandle_t h, int32_t format) {
+  if (format != DNNRT_NCHW) {
+    snprintf(g_err, sizeof g_err, "oracle: only NCHW is implemented");
+    return 1;
+  }
+  h->format = format;
+  return 0;
+}
+int32_t dnnrtSync(dnnrtHandle_t h) { (void)h; return 0; }
+
+/* wrapDNNMemPoolInit.cpp:19-29 / wrapDNNMalloc.cpp: one allocation. */
+int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
+  *pool = malloc((size_t)(bytes > 0 ? bytes : 1));
+  return *pool ? 0 : 1;
+}
+int32_t dnnrtMalloc(void **p, int64_t bytes) { return dnnrtMemPoolInit(p, bytes); }
+int32_t dnnrtDealloc(void *p) { free(p); return 0; }
+int32_t dnnrtHostAlloc(void **p, int64_t bytes) { return dnnrtMemPoolInit(p, bytes); }
+int32_t dnnrtHostFree(void *p) { free(p); return 0; }
+/* wrapDNNMemOffset.cpp:26: *p = base + offset. */
+int32_t dnnrtMemOffset(void **p, void *base, int64_t off, int64_t bytes) {
+  (void)bytes;
+  *p = (char *)base + off;
+  return 0;
+}
+/* wrapDNNMemcpy.cpp:17-61. */
+int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind, dnnrtStream_t s) {
+  (void)kind; (void)s;
+  if (bytes > 0) memmove(dst, src, (size_t)bytes);
+  return 0;
+}
+
+/* ---- convolution -------------------------------------------------------
+ * CUDNNConvFunc.cpp:9-105 calls cudnnConvolutionForward with
+ * CUDNN_CROSS_CORRELATION, dilation 1, alpha 1, beta 0, `group` groups; the
+ * published definition is
+ *   Y[n,k,p,q] = sum_{c,r,s} X[n, g*Cg + c, p*sh - ph + r, q*sw - pw + s]
+ *                            * W[k, c, r, s],        g = k / (K/group)
+ * with out-of-range taps contributing 0.  CUDNNConvBiasReluFunc.cpp:8-140
+ * adds B[k] and applies ReLU (mode 1) or identity (mode 5). */
+static float act_apply(float v, int64_t mode) {
+  switch (mode) {
+  case DNNRT_ACT_RELU: return v < 0.0f ? 0.0f : v; /* NaN passes through */
+  case DNNRT_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+  case DNNRT_ACT_TANH: return tanhf(v);
+  default: return v;
+  }
+}
+
+static void conv_core(const float *X, const int64_t *dX, const float *Wt,
+                      const int64_t *dW, const float *B, int64_t group,
+                      const int64_t *pads, const int64_t *strides, int64_t act,
+                      float *Y) {
+  const int64_t N = dX[0], C = dX[1], H = dX[2], Wd = dX[3];
+  const int64_t K = dW[0], Cg = dW[1], R = dW[2], S = dW[3];
+  const int64_t ph = pads[0], pw = pads[1], sh = strides[0], sw = strides[1];
+  const int64_t P = (H + 2 * ph - R) / sh + 1, Q = (Wd + 2 * pw - S) / sw + 1;
+  const int64_t Kg = K / group;
+  (void)C;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+  for (int64_t n = 0; n < N; n++)
+    for (int64_t k = 0; k < K; k++) {
+      double *acc = (double *)calloc((size_t)(P * Q), sizeof(double));
+      const int64_t g = k / Kg;
+      for (int64_t c = 0; c < Cg; c++) {
+        const float *xc = X + ((n * dX[1] + g * Cg + c) * H) * Wd;
+        for (int64_t r = 0; r < R; r++)
+          for (int64_t s = 0; s < S; s++) {
+            const double w = Wt[((k * Cg + c) * R + r) * S + s];
+            for (int64_t p = 0; p < P; p++) {
+              const int64_t ih = p * sh - ph + r;
+              if (ih < 0 || ih >= H) continue;
+              /* q range with 0 <= q*sw - pw + s < W */
+              int64_t q0 = 0, q1 = Q;
+              while (q0 < Q && q0 * sw - pw + s < 0) q0++;
+              while (q1 > q0 && (q1 - 1) * sw - pw + s >= Wd) q1--;
+              const float *xr = xc + ih * Wd - pw + s;
+              double *ar = acc + p * Q;
+              for (int64_t q = q0; q < q1; q++) ar[q] += w * (double)xr[q * sw];
+            }
+          }
+      }
+      float *y = Y + (n * K + k) * P * Q;
+      const double b = B ? (double)B[k] : 0.0;
+      for (int64_t i = 0; i < P * Q; i++) y[i] = act_apply((float)(acc[i] + b), act);
+      free(acc);
+    }
+}
+
+static void *conv_entry(const void *X, const int64_t *dX, const void *W,
+                        const int64_t *dW, const void *B, int64_t group,
+                        const int64_t *pads, const int64_t *strides,
+                        int64_t act, void *Y, int32_t dtype) {
+  if (bad_dtype(dtype)) FAIL("conv: bad dtype %d", dtype);
+  if (group < 1 || dX[1] != dW[1] * group || dW[0] % group)
+    FAIL("conv: C=%ld, W has C/g=%ld, group=%ld, K=%ld do not agree",
+         (long)dX[1], (long)dW[1], (long)group, (long)dW[0]);
+  const int64_t P = (dX[2] + 2 * pads[0] - dW[2]) / strides[0] + 1,
+                Q = (dX[3] + 2 * pads[1] - dW[3]) / strides[1] + 1;
+  if (P < 1 || Q < 1) FAIL("conv: empty output");
+  float *tx, *tw, *tb = NULL, *ty;
+  const float *x = widen(X, numel(dX, 4), dtype, &tx);
+  const float *w = widen(W, numel(dW, 4), dtype, &tw);
+  const float *b = B ? widen(B, dW[0], dtype, &tb) : NULL;
+  const int64_t ny = dX[0] * dW[0] * P * Q;
+  float *y = outbuf(Y, ny, dtype, &ty);
+  conv_core(x, dX, w, dW, b, group, pads, strides, act, y);
+  narrow(Y, ty, ny, dtype);
+  free(tx); free(tw); free(tb);
+  return Y;
+}
+
+void *dnnrtConv(dnnrtHandle_t h, const void *X, const int64_t *dX, const void *W,
+                const int64_t *dW, void *ws, int64_t wsBytes, int64_t algo,
+                int64_t group, const int64_t *pads, const int64_t *strides,
+                void *Y, int32_t dtype) {
+  (void)h; (void)ws; (void)wsBytes; (void)algo;
+  return conv_entry(X, dX, W, dW, NULL, group, pads, strides, DNNRT_ACT_IDENTITY, Y, dtype);
+}
+void *dnnrtConvBiasActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
+                         const void *W, const int64_t *dW, const void *B,
+                         const int64_t *dB, void *ws, int64_t wsBytes,
+                         int64_t algo, int64_t group, const int64_t *pads,
+                         const int64_t *strides, int64_t act, void *Y,
+                         int32_t dtype) {
+  (void)h; (void)ws; (void)wsBytes; (void)algo;
+  if (act != DNNRT_ACT_RELU && act != DNNRT_ACT_IDENTITY)
+    FAIL("convBiasActiv: activMode %ld", (long)act);
+  if (numel(dB, 4) != dW[0]) FAIL("convBiasActiv: bias must hold K values");
+  return conv_entry(X, dX, W, dW, B, group, pads, strides, act, Y, dtype);
+}
+
+/* ---- elementwise -------------------------------------------------------- */
+
+/* CUDNNActiveFunc.cpp:8-91: cudnnActivationForward, alpha 1 beta 0. */
+void *dnnrtActive(dnnrtHandle_t h, const void *X, const int64_t *dX, int32_t mode,
+                  void *Y, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("active: bad dtype");
+  if (mode != DNNRT_ACT_RELU && mode != DNNRT_ACT_SIGMOID && mode != DNNRT_ACT_TANH)
+    FAIL("active: mode %d", mode);
+  const int64_t n = numel(dX, 4);
+  float *tx, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t i = 0; i < n; i++) y[i] = act_apply(x[i], mode);
+  narrow(Y, ty, n, dtype); free(tx);
+  return Y;
+}
+
+/* CUDNNTensorOpFunc.cpp:8-149: cudnnOpTensor, C = op(1*A, coefB*B) + 0*C,
+ * B broadcast where its dim is 1. */
+void *dnnrtTensorOp(dnnrtHandle_t h, int64_t op, const void *A, const int64_t *dA,
+                    int32_t rA, const void *B, const int64_t *dB, int32_t rB,
+                    void *O, const int64_t *dO, int32_t rO, float coefB,
+                    int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("tensorOp: bad dtype");
+  if (op != DNNRT_OP_ADD && op != DNNRT_OP_MUL && op != DNNRT_OP_SQRT)
+    FAIL("tensorOp: op %ld", (long)op);
+  if (rA != rO || (op != DNNRT_OP_SQRT && rB != rA) || rA < 1 || rA > 8)
+    FAIL("tensorOp: ranks %d %d %d", rA, rB, rO);
+  for (int i = 0; i < rA; i++) {
+    if (dA[i] != dO[i]) FAIL("tensorOp: dimA != dimO");
+    if (op != DNNRT_OP_SQRT && dB[i] != dA[i] && dB[i] != 1)
+      FAIL("tensorOp: dimB[%d]=%ld cannot broadcast to %ld", i, (long)dB[i], (long)dA[i]);
+  }
+  const int64_t n = numel(dA, rA);
+  float *ta, *tb = NULL, *to;
+  const float *a = widen(A, n, dtype, &ta);
+  float *o = outbuf(O, n, dtype, &to);
+  if (op == DNNRT_OP_SQRT) {
+    for (int64_t i = 0; i < n; i++) o[i] = sqrtf(a[i]);
+  } else {
+    const float *b = widen(B, numel(dB, rB), dtype, &tb);
+    int64_t sB[8], s = 1;
+    for (int i = rA - 1; i >= 0; i--) { sB[i] = dB[i] == 1 ? 0 : s; s *= dB[i]; }
+    for (int64_t i = 0; i < n; i++) {
+      int64_t rem = i, ib = 0;
+      for (int d = rA - 1; d >= 0; d--) { ib += (rem % dA[d]) * sB[d]; rem /= dA[d]; }
+      const float bv = coefB * b[ib];
+      o[i] = op == DNNRT_OP_ADD ? a[i] + bv : a[i] * bv;
+    }
+  }
+  narrow(O, to, n, dtype); free(ta); free(tb);
+  return O;
+}
+
+#define UNARY(NAME, EXPR)                                                      \
+  void *NAME(dnnrtHandle_t h, const void *X, void *Y, const int64_t *d,        \
+             int64_t rank, int32_t dtype) {                                    \
+    (void)h;                                                                   \
+    if (bad_dtype(dtype)) FAIL(#NAME ": bad dtype");                           \
+    const int64_t n = numel(d, rank);                                          \
+    float *tx, *ty;                                                            \
+    const float *x = widen(X, n, dtype, &tx);                                  \
+    float *y = outbuf(Y, n, dtype, &ty);                                       \
+    for (int64_t i = 0; i < n; i++) { const float v = x[i]; y[i] = (EXPR); }   \
+    narrow(Y, ty, n, dtype); free(tx);                                         \
+    return Y;                                                                  \
+  }
+/* CUDAErfFunc.cu:4-27, CUDANegativeFunc.cu:4-28, CUDAReciprocalFunc.cu:4-28 */
+UNARY(dnnrtErf, erff(v))
+UNARY(dnnrtNegative, -v)
+UNARY(dnnrtReciprocal, 1.0f / v)
+/* GELU(erf), the chain the reference lowers to: Div(sqrt 2), Erf, Add 1,
+ * Mul x, Mul 0.5 -- evaluated in double, rounded once. */
+UNARY(dnnrtGelu, (float)(0.5 * (double)v * (1.0 + erf((double)v / sqrt(2.0)))))
+
+/* CUDAClipFunc.cu:5-28: min(max(x, lo), hi). */
+void *dnnrtClip(dnnrtHandle_t h, const void *X, void *Y, const int64_t *d, float lo,
+                float hi, int64_t rank, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("clip: bad dtype");
+  const int64_t n = numel(d, rank);
+  float *tx, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t i = 0; i < n; i++) {
+    float v = x[i];
+    v = v < lo ? lo : v;
+    v = v > hi ? hi : v;
+    y[i] = v;
+  }
+  narrow(Y, ty, n, dtype); free(tx);
+  return Y;
+}
+
+/* CUDAPowFunc.cu:4-32: exponent from a 1-element tensor; exponent 2 is x*x. */
+void *dnnrtPow(dnnrtHandle_t h, const void *X, const void *E, void *Y,
+               const int64_t *d, int64_t rank, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("pow: bad dtype");
+  const int64_t n = numel(d, rank);
+  float *tx, *te, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  const float *e = widen(E, 1, dtype, &te);
+  float *y = outbuf(Y, n, dtype, &ty);
+  if (e[0] == 2.0f) for (int64_t i = 0; i < n; i++) y[i] = x[i] * x[i];
+  else for (int64_t i = 0; i < n; i++) y[i] = powf(x[i], e[0]);
+  narrow(Y, ty, n, dtype); free(tx); free(te);
+  return Y;
+}
+
+/* CUDACastI64toFloatFunc.cu:4-26. */
+void *dnnrtCastI64toFloat(dnnrtHandle_t h, const int64_t *X, void *Y,
+                          const int64_t *d, int64_t rank, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("cast: bad dtype");
+  const int64_t n = numel(d, rank);
+  float *ty;
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t i = 0; i < n; i++) y[i] = (float)X[i];
+  narrow(Y, ty, n, dtype);
+  return Y;
+}
+
+/* ---- reductions ---------------------------------------------------------
+ * CUDNNReduceFunc.cpp:8-142: cudnnReduceTensor AVG over the dims where the
+ * output dim is 1. */
+void *dnnrtReduce(dnnrtHandle_t h, int32_t rank, const void *X, const int64_t *dX,
+                  void *Y, const int64_t *dY, int32_t mode, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("reduce: bad dtype");
+  if (mode != DNNRT_REDUCE_AVG) FAIL("reduce: mode %d", mode);
+  if (rank < 1 || rank > 8) FAIL("reduce: rank %d", rank);
+  for (int i = 0; i < rank; i++)
+    if (dY[i] != dX[i] && dY[i] != 1) FAIL("reduce: dimY[%d]", i);
+  const int64_t nx = numel(dX, rank), ny = numel(dY, rank);
+  float *tx, *ty;
+  const float *x = widen(X, nx, dtype, &tx);
+  float *y = outbuf(Y, ny, dtype, &ty);
+  double *acc = (double *)calloc((size_t)ny, sizeof(double));
+  int64_t sY[8], s = 1;
+  for (int i = rank - 1; i >= 0; i--) { sY[i] = dY[i] == 1 ? 0 : s; s *= dY[i]; }
+  for (int64_t i = 0; i < nx; i++) {
+    int64_t rem = i, iy = 0;
+    for (int d = rank - 1; d >= 0; d--) { iy += (rem % dX[d]) * sY[d]; rem /= dX[d]; }
+    acc[iy] += (double)x[i];
+  }
+  const double cnt = (double)(nx / ny);
+  for (int64_t i = 0; i < ny; i++) y[i] = (float)(acc[i] / cnt);
+  free(acc);
+  narrow(Y, ty, ny, dtype); free(tx);
+  return Y;
+}
+
+/* CUDASoftmaxFunc.cu:7-128: exp(x - m) / sum exp(x - m) along `axis`.  The
+ * reference subtracts the tensor-wide max; any per-row constant gives the
+ * same quotient, the row max is used here. */
+void *dnnrtSoftmax(dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
+                   const int64_t *dY, int64_t axis, int64_t rank, int32_t dtype) {
+  (void)h; (void)dY;
+  if (bad_dtype(dtype)) FAIL("softmax: bad dtype");
+  if (axis < 0) axis += rank;
+  if (axis < 0 || axis >= rank) FAIL("softmax: axis");
+  int64_t outer = 1, inner = 1;
+  const int64_t L = dX[axis];
+  for (int64_t i = 0; i < axis; i++) outer *= dX[i];
+  for (int64_t i = axis + 1; i < rank; i++) inner *= dX[i];
+  const int64_t n = outer * L * inner;
+  float *tx, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t o = 0; o < outer; o++)
+    for (int64_t in = 0; in < inner; in++) {
+      const float *xr = x + o * L * inner + in;
+      float *yr = y + o * L * inner + in;
+      float m = xr[0];
+      for (int64_t l = 1; l < L; l++) m = xr[l * inner] > m ? xr[l * inner] : m;
+      double sum = 0;
+      for (int64_t l = 0; l < L; l++) sum += exp((double)xr[l * inner] - (double)m);
+      for (int64_t l = 0; l < L; l++)
+        yr[l * inner] = (float)(exp((double)xr[l * inner] - (double)m) / sum);
+    }
+  narrow(Y, ty, n, dtype); free(tx);
+  return Y;
+}
+
+/* LayerNorm over the last dim, i.e. the chain the reference emits for it:
+ * ReduceMean, Sub, Pow 2, ReduceMean, Add eps, Sqrt, Div, Mul gamma, Add beta. */
+void *dnnrtLayerNorm(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rank,
+                     const void *G, const void *Bt, float eps, void *Y, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("layernorm: bad dtype");
+  const int64_t L = dX[rank - 1], rows = numel(dX, rank - 1), n = rows * L;
+  float *tx, *tg, *tb, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  const float *g = widen(G, L, dtype, &tg);
+  const float *b = widen(Bt, L, dtype, &tb);
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t r = 0; r < rows; r++) {
+    const float *xr = x + r * L;
+    double mu = 0, var = 0;
+    for (int64_t i = 0; i < L; i++) mu += xr[i];
+    mu /= (double)L;
+    for (int64_t i = 0; i < L; i++) { const double d = xr[i] - mu; var += d * d; }
+    var /= (double)L;
+    const double inv = 1.0 / sqrt(var + (double)eps);
+    for (int64_t i = 0; i < L; i++)
+      y[r * L + i] = (float)((xr[i] - mu) * inv * (double)g[i] + (double)b[i]);
+  }
+  narrow(Y, ty, n, dtype); free(tx); free(tg); free(tb);
+  return Y;
+}
+
+/* ---- pooling -------------------------------------------------------------
+ * CUDNNMaxPoolFunc.cpp:8-78 / CUDNNAveragePoolFunc.cpp:8-78:
+ * cudnnPoolingForward, window kernel[0] x kernel[1], vertical pad pads[0],
+ * horizontal pad pads[1] (the lowering hands over ONNX's 4 pads; begin pads
+ * are used for both sides), strides.  Max ignores padding; average divides
+ * by the full window (CUDNN_POOLING_AVERAGE_COUNT_INCLUDE_PADDING, :44).
+ * The reference's beta = 1 accumulate into a zeroed Y is a plain overwrite. */
+static void *pool_entry(const void *X, const int64_t *dX, void *Y, const int64_t *dY,
+                        const int64_t *kr, const int64_t *pads, const int64_t *st,
+                        int is_max, int32_t dtype) {
+  if (bad_dtype(dtype)) FAIL("pool: bad dtype");
+  const int64_t N = dX[0], C = dX[1], H = dX[2], W = dX[3], P = dY[2], Q = dY[3];
+  const int64_t R = kr[0], S = kr[1], ph = pads[0], pw = pads[1];
+  if (dY[0] != N || dY[1] != C) FAIL("pool: dimY");
+  if ((P - 1) * st[0] - ph >= H || (Q - 1) * st[1] - pw >= W) FAIL("pool: window outside");
+  const int64_t nx = N * C * H * W, ny = N * C * P * Q;
+  float *tx, *ty;
+  const float *x = widen(X, nx, dtype, &tx);
+  float *y = outbuf(Y, ny, dtype, &ty);
+#pragma omp parallel for
+  for (int64_t nc = 0; nc < N * C; nc++)
+    for (int64_t p = 0; p < P; p++)
+      for (int64_t q = 0; q < Q; q++) {
+        float m = -INFINITY; double sum = 0; int any_nan = 0;
+        for (int64_t r = 0; r < R; r++)
+          for (int64_t s = 0; s < S; s++) {
+            const int64_t ih = p * st[0] - ph + r, iw = q * st[1] - pw + s;
+            if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+            const float v = x[(nc * H + ih) * W + iw];
+            if (v != v) any_nan = 1;
+            m = v > m ? v : m; sum += v;
+          }
+        y[(nc * P + p) * Q + q] =
+            is_max ? (any_nan ? NAN : m) : (float)(sum / (double)(R * S));
+      }
+  narrow(Y, ty, ny, dtype); free(tx);
+  return Y;
+}
+void *dnnrtMaxPool(dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
+                   const int64_t *dY, const int64_t *k, const int64_t *p,
+                   const int64_t *s, int32_t dtype) {
+  (void)h; return pool_entry(X, dX, Y, dY, k, p, s, 1, dtype);
+}
+void *dnnrtAveragePool(dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
+                       const int64_t *dY, const int64_t *k, const int64_t *p,
+                       const int64_t *s, int32_t dtype) {
+  (void)h; return pool_entry(X, dX, Y, dY, k, p, s, 0, dtype);
+}
+
+/* ---- matrix products ----------------------------------------------------- */
+
+/* C[M,N] = alpha * sum_k A(m,k) B(k,n) (+ beta * Cin), element strides given */
+static void gemm_core(const float *A, int64_t sam, int64_t sak, const float *B,
+                      int64_t sbk, int64_t sbn, const float *Cin, float *C,
+                      int64_t M, int64_t N, int64_t K, float alpha, float beta) {
+#pragma omp parallel for
+  for (int64_t m = 0; m < M; m++)
+    for (int64_t n = 0; n < N; n++) {
+      double acc = 0;
+      for (int64_t k = 0; k < K; k++)
+        acc += (double)A[m * sam + k * sak] * (double)B[k * sbk + n * sbn];
+      double v = (double)alpha * acc;
+      if (beta != 0.0f) v += (double)beta * (double)Cin[m * N + n];
+      C[m * N + n] = (float)v;
+    }
+}
+
+/* CUBLASMatmul2dFunc.cu:9-153: cublasLtMatmul, fp32 compute,
+ * Out = alpha op(A) op(B) + beta C with row-major operands. */
+void *dnnrtMatmul2d(dnnrtHandle_t h, int64_t rank, const void *A, const int64_t *dA,
+                    const void *B, const int64_t *dB, const void *C,
+                    const int64_t *dC, void *Out, const int64_t *dO, float alpha,
+                    float beta, int64_t transA, int64_t transB, int32_t dtype) {
+  (void)h; (void)rank; (void)dC;
+  if (bad_dtype(dtype)) FAIL("matmul2d: bad dtype");
+  const int64_t M = transA ? dA[1] : dA[0], K = transA ? dA[0] : dA[1];
+  const int64_t Kb = transB ? dB[1] : dB[0], N = transB ? dB[0] : dB[1];
+  if (K != Kb || dO[0] != M || dO[1] != N) FAIL("matmul2d: shapes");
+  if (beta != 0.0f && !C) FAIL("matmul2d: beta != 0 needs C");
+  float *ta, *tb, *tc = NULL, *to;
+  const float *a = widen(A, M * K, dtype, &ta);
+  const float *b = widen(B, K * N, dtype, &tb);
+  const float *c = (beta != 0.0f) ? widen(C, M * N, dtype, &tc) : NULL;
+  float *o = outbuf(Out, M * N, dtype, &to);
+  float *cc = NULL;
+  if (c) { /* C may alias Out */
+    cc = (float *)malloc(sizeof(float) * (size_t)(M * N));
+    memcpy(cc, c, sizeof(float) * (size_t)(M * N));
+  }
+  gemm_core(a, transA ? 1 : K, transA ? M : 1, b, transB ? 1 : N, transB ? K : 1,
+            cc, o, M, N, K, alpha, beta);
+  free(cc);
+  narrow(Out, to, M * N, dtype); free(ta); free(tb); free(tc);
+  return Out;
+}
+
+/* CUDAMatmulNdFunc.cu:14-173: numpy.matmul, ranks 2..4; batch dims of the
+ * lower-rank (or size-1) operand are broadcast. */
+void *dnnrtMatmulNd(dnnrtHandle_t h, const void *A, const int64_t *dA, int32_t rA,
+                    const void *B, const int64_t *dB, int32_t rB, void *Y,
+                    const int64_t *dY, int32_t rY, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("matmulNd: bad dtype");
+  if (rA < 2 || rB < 2 || rY < 2 || rA > 4 || rB > 4 || rY > 4 ||
+      rY != (rA > rB ? rA : rB))
+    FAIL("matmulNd: ranks %d %d %d", rA, rB, rY);
+  const int64_t M = dA[rA - 2], K = dA[rA - 1], N = dB[rB - 1];
+  if (dB[rB - 2] != K || dY[rY - 2] != M || dY[rY - 1] != N) FAIL("matmulNd: shapes");
+  const int nb = rY - 2;
+  int64_t bY[2] = {1, 1}, bA[2] = {1, 1}, bB[2] = {1, 1};
+  for (int i = 0; i < nb; i++) {
+    bY[2 - nb + i] = dY[i];
+    const int ia = i - (rY - rA), ib = i - (rY - rB);
+    if (ia >= 0) bA[2 - nb + i] = dA[ia];
+    if (ib >= 0) bB[2 - nb + i] = dB[ib];
+  }
+  for (int i = 0; i < 2; i++)
+    if ((bA[i] != bY[i] && bA[i] != 1) || (bB[i] != bY[i] && bB[i] != 1))
+      FAIL("matmulNd: batch dims do not broadcast");
+  const int64_t na = bA[0] * bA[1] * M * K, nbB = bB[0] * bB[1] * K * N,
+                ny = bY[0] * bY[1] * M * N;
+  float *ta, *tb, *ty;
+  const float *a = widen(A, na, dtype, &ta);
+  const float *b = widen(B, nbB, dtype, &tb);
+  float *y = outbuf(Y, ny, dtype, &ty);
+  for (int64_t i0 = 0; i0 < bY[0]; i0++)
+    for (int64_t i1 = 0; i1 < bY[1]; i1++) {
+      const int64_t a0 = bA[0] == 1 ? 0 : i0, a1 = bA[1] == 1 ? 0 : i1;
+      const int64_t b0 = bB[0] == 1 ? 0 : i0, b1 = bB[1] == 1 ? 0 : i1;
+      gemm_core(a + (a0 * bA[1] + a1) * M * K, K, 1, b + (b0 * bB[1] + b1) * K * N,
+                N, 1, NULL, y + (i0 * bY[1] + i1) * M * N, M, N, K, 1.0f, 0.0f);
+    }
+  narrow(Y, ty, ny, dtype); free(ta); free(tb);
+  return Y;
+}
+
+/* ---- data movement -------------------------------------------------------- */
+
+static int64_t esize(int32_t dtype) {
+  return dtype == DNNRT_F32 ? 4 : dtype == DNNRT_F16 ? 2 : dtype == DNNRT_I64 ? 8 : 0;
+}
+/* CUDAFlattenFunc.cpp:32 / CUDAReshapeFunc.cpp:30: device-to-device copy. */
+void *dnnrtFlatten(dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
+                   const int64_t *dY, int32_t axis, int64_t rank, int32_t dtype) {
+  (void)h; (void)dY; (void)axis;
+  if (!esize(dtype)) FAIL("flatten: bad dtype");
+  memmove(Y, X, (size_t)(numel(dX, rank) * esize(dtype)));
+  return Y;
+}
+void *dnnrtReshape(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rank,
+                   void *Y, int32_t dtype) {
+  (void)h;
+  if (!esize(dtype)) FAIL("reshape: bad dtype");
+  memmove(Y, X, (size_t)(numel(dX, rank) * esize(dtype)));
+  return Y;
+}
+/* CUDATranspose4DFloatFunc.cu: Y[i_perm] = X[i]; dimY[j] = dimX[perm[j]]. */
+void *dnnrtTranspose(dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
+                     const int64_t *dY, const int64_t *perm, int64_t rank,
+                     int32_t dtype) {
+  (void)h;
+  const int64_t es = esize(dtype);
+  if (!es) FAIL("transpose: bad dtype");
+  if (rank < 1 || rank > 6) FAIL("transpose: rank");
+  int64_t sX[6], s = 1;
+  for (int i = (int)rank - 1; i >= 0; i--) { sX[i] = s; s *= dX[i]; }
+  for (int i = 0; i < rank; i++)
+    if (perm[i] < 0 || perm[i] >= rank || dY[i] != dX[perm[i]]) FAIL("transpose: perm/dimY");
+  const int64_t n = numel(dX, rank);
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, ix = 0;
+    for (int d = (int)rank - 1; d >= 0; d--) { ix += (rem % dY[d]) * sX[perm[d]]; rem /= dY[d]; }
+    memcpy((char *)Y + i * es, (const char *)X + ix * es, (size_t)es);
+  }
+  return Y;
+}
+/* CUDAGatherFloatFunc.cu:7-82: numpy.take(X, indices, axis). */
+void *dnnrtGather(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rX,
+                  void *Y, const int64_t *dY, int64_t rY, const int64_t *idx,
+                  const int64_t *dI, int64_t rI, int64_t axis, int32_t dtype) {
+  (void)h; (void)dY; (void)rY;
+  const int64_t es = esize(dtype);
+  if (!es) FAIL("gather: bad dtype");
+  if (axis < 0) axis += rX;
+  if (axis < 0 || axis >= rX) FAIL("gather: axis");
+  int64_t outer = 1, inner = 1;
+  const int64_t ni = numel(dI, rI), L = dX[axis];
+  for (int64_t i = 0; i < axis; i++) outer *= dX[i];
+  for (int64_t i = axis + 1; i < rX; i++) inner *= dX[i];
+  for (int64_t j = 0; j < ni; j++) {
+    int64_t t = idx[j];
+    if (t < 0) t += L;
+    if (t < 0 || t >= L) FAIL("gather: index %ld out of range", (long)idx[j]);
+  }
+  for (int64_t o = 0; o < outer; o++)
+    for (int64_t j = 0; j < ni; j++) {
+      int64_t t = idx[j] < 0 ? idx[j] + L : idx[j];
+      memcpy((char *)Y + ((o * ni + j) * inner) * es,
+             (const char *)X + ((o * L + t) * inner) * es, (size_t)(inner * es));
+    }
+  return Y;
+}

@@ -1,0 +1,164 @@
+"""One function per operator that runs it through a backend (tests/helpers.py)
+on numpy inputs and returns a numpy output.  Used by the oracle tests (oracle
+vs. closed forms / torch CPU) and by the GPU parity tests (HIP vs. oracle)."""
+import numpy as np
+
+from occamy_amd import _abi
+
+DT = {np.dtype(np.float32): _abi.F32, np.dtype(np.float16): _abi.F16, np.dtype(np.int64): _abi.I64}
+
+
+def conv_out_hw(H, W, R, S, pads, strides):
+    return (H + 2 * pads[0] - R) // strides[0] + 1, (W + 2 * pads[1] - S) // strides[1] + 1
+
+
+def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None):
+    N, C, H, W = x.shape
+    K, Cg, R, S = w.shape
+    P, Q = conv_out_hw(H, W, R, S, pads, strides)
+    dt = DT[x.dtype]
+    X, Wt = be.put(x), be.put(w)
+    Y = be.empty((N, K, max(P, 1), max(Q, 1)), x.dtype)  # the call rejects empty outputs itself
+    if b is None:
+        assert activ is None
+        be.ops.conv(be.ptr(X), x.shape, be.ptr(Wt), w.shape, pads, strides, be.ptr(Y), group, dt)
+    else:
+        B = be.put(b)
+        be.ops.conv_bias_activ(be.ptr(X), x.shape, be.ptr(Wt), w.shape, be.ptr(B), pads, strides,
+                               activ if activ is not None else _abi.ACT_IDENTITY, be.ptr(Y), group, dt)
+    be.sync()
+    return be.get(Y)
+
+
+def unary(be, name, x, **kw):
+    X = be.put(x)
+    Y = be.empty(x.shape, x.dtype)
+    dt = DT[x.dtype]
+    if name == "relu":
+        be.ops.active(be.ptr(X), x.shape, _abi.ACT_RELU, be.ptr(Y), dt)
+    elif name == "sigmoid":
+        be.ops.active(be.ptr(X), x.shape, _abi.ACT_SIGMOID, be.ptr(Y), dt)
+    elif name == "tanh":
+        be.ops.active(be.ptr(X), x.shape, _abi.ACT_TANH, be.ptr(Y), dt)
+    elif name == "clip":
+        be.ops.clip(be.ptr(X), be.ptr(Y), x.shape, kw["lo"], kw["hi"], dt)
+    elif name == "sqrt":
+        be.ops.tensor_op(_abi.OP_SQRT, be.ptr(X), x.shape, None, x.shape, be.ptr(Y), 1.0, dt)
+    else:
+        getattr(be.ops, name)(be.ptr(X), be.ptr(Y), x.shape, dt)
+    be.sync()
+    return be.get(Y)
+
+
+def pow_(be, x, e):
+    X, E = be.put(x), be.put(np.array([e], dtype=x.dtype))
+    Y = be.empty(x.shape, x.dtype)
+    be.ops.pow(be.ptr(X), be.ptr(E), be.ptr(Y), x.shape, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def cast(be, x, out_dtype=np.float32):
+    X = be.put(x)
+    Y = be.empty(x.shape, out_dtype)
+    be.ops.cast_i64_to_float(be.ptr(X), be.ptr(Y), x.shape, DT[np.dtype(out_dtype)])
+    be.sync()
+    return be.get(Y)
+
+
+def tensor_op(be, op, a, b, coef=1.0, inplace=False):
+    A, B = be.put(a), be.put(b)
+    O = A if inplace else be.empty(a.shape, a.dtype)
+    be.ops.tensor_op(op, be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(O), coef, DT[a.dtype])
+    be.sync()
+    return be.get(O)
+
+
+def reduce_mean(be, x, out_shape):
+    X = be.put(x)
+    Y = be.empty(out_shape, x.dtype)
+    be.ops.reduce_mean(be.ptr(X), x.shape, be.ptr(Y), out_shape, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def softmax(be, x, axis):
+    X = be.put(x)
+    Y = be.empty(x.shape, x.dtype)
+    be.ops.softmax(be.ptr(X), x.shape, be.ptr(Y), axis, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def layernorm(be, x, g, b, eps):
+    X, G, B = be.put(x), be.put(g), be.put(b)
+    Y = be.empty(x.shape, x.dtype)
+    be.ops.layernorm(be.ptr(X), x.shape, be.ptr(G), be.ptr(B), eps, be.ptr(Y), DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def pool(be, kind, x, kernel, pads, strides):
+    N, C, H, W = x.shape
+    P, Q = conv_out_hw(H, W, kernel[0], kernel[1], pads, strides)
+    X = be.put(x)
+    Y = be.empty((N, C, P, Q), x.dtype)
+    fn = be.ops.maxpool if kind == "max" else be.ops.avgpool
+    fn(be.ptr(X), x.shape, be.ptr(Y), (N, C, P, Q), kernel, [pads[0], pads[1], pads[0], pads[1]],
+       strides, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def matmul2d(be, a, b, c=None, alpha=1.0, beta=0.0, transA=0, transB=0):
+    M = a.shape[1] if transA else a.shape[0]
+    N = b.shape[0] if transB else b.shape[1]
+    A, B = be.put(a), be.put(b)
+    Out = be.put(c) if c is not None else be.empty((M, N), a.dtype)
+    be.ops.matmul2d(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Out), (M, N), alpha, beta, transA,
+                    transB, be.ptr(Out) if c is not None else None, DT[a.dtype])
+    be.sync()
+    return be.get(Out)
+
+
+def matmul_nd(be, a, b):
+    y_shape = np.matmul(np.zeros(a.shape, np.float32), np.zeros(b.shape, np.float32)).shape
+    A, B = be.put(a), be.put(b)
+    Y = be.empty(y_shape, a.dtype)
+    be.ops.matmul_nd(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Y), y_shape, DT[a.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def flatten(be, x, axis):
+    out = (int(np.prod(x.shape[:axis])), int(np.prod(x.shape[axis:])))
+    X = be.put(x)
+    Y = be.empty(out, x.dtype)
+    be.ops.flatten(be.ptr(X), x.shape, be.ptr(Y), out, axis, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def reshape(be, x, out):
+    X = be.put(x)
+    Y = be.empty(out, x.dtype)
+    be.ops.reshape(be.ptr(X), x.shape, be.ptr(Y), DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def transpose(be, x, perm):
+    X = be.put(x)
+    Y = be.empty([x.shape[p] for p in perm], x.dtype)
+    be.ops.transpose(be.ptr(X), x.shape, be.ptr(Y), perm, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def gather(be, x, idx, axis):
+    out = x.shape[:axis] + idx.shape + x.shape[axis + 1:]
+    X, I = be.put(x), be.put(idx.astype(np.int64))
+    Y = be.empty(out, x.dtype)
+    be.ops.gather(be.ptr(X), x.shape, be.ptr(Y), out, be.ptr(I), idx.shape, axis, DT[x.dtype])
+    be.sync()
+    return be.get(Y)

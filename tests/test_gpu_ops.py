@@ -1,0 +1,257 @@
+"""Parity of the gfx950 library with the CPU oracle, operator by operator,
+through the C ABI on the same seeded inputs.
+
+Bars: bit-exact for copies, index work, max, clip, negate, ReLU, two-operand
+add/mul, reciprocal and sqrt (no reassociation is involved); fp32 reductions
+and transcendental functions within rtol 1e-4 / atol 1e-5 of the oracle
+(which accumulates in double); fp16 storage within rtol 2e-2.
+"""
+import numpy as np
+import pytest
+
+import opcases as oc
+from helpers import GpuBackend, OracleBackend, rng
+from occamy_amd import _abi
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return GpuBackend()
+
+
+@pytest.fixture(scope="module")
+def cpu():
+    return OracleBackend()
+
+
+def close(got, ref, rtol=RTOL, atol=ATOL):
+    np.testing.assert_allclose(got, ref, rtol=rtol, atol=atol)
+
+
+# ---- convolution ----------------------------------------------------------------
+
+CONV_CASES = [
+    # N, C, H, W, K, R, S, stride, pad, group
+    (1, 64, 56, 56, 64, 3, 3, 1, 1, 1),     # the single-conv configuration (Kaiming-uniform below)
+    (1, 3, 224, 224, 64, 7, 7, 2, 3, 1),    # ResNet stem
+    (1, 64, 56, 56, 256, 1, 1, 1, 0, 1),
+    (1, 256, 56, 56, 512, 1, 1, 2, 0, 1),   # strided 1x1 downsample
+    (1, 128, 56, 56, 128, 3, 3, 2, 1, 1),
+    (1, 512, 7, 7, 512, 3, 3, 1, 1, 1),     # 49 pixels: ragged column tile
+    (1, 2048, 7, 7, 512, 1, 1, 1, 0, 1),
+    (2, 16, 9, 11, 24, 3, 3, 1, 1, 1),      # batch > 1, ragged everything
+    (3, 5, 8, 8, 7, 2, 3, 1, 0, 1),         # generic filter size, odd channels
+    (1, 8, 12, 12, 16, 5, 5, 1, 2, 1),
+    (1, 16, 10, 10, 32, 3, 3, 1, 1, 4),     # grouped
+    (1, 32, 112, 112, 32, 3, 3, 1, 1, 32),  # MobileNetV2 depthwise
+    (1, 96, 112, 112, 96, 3, 3, 2, 1, 96),  # depthwise stride 2
+    (2, 6, 7, 7, 12, 3, 3, 1, 1, 6),        # depthwise with channel multiplier 2
+    (1, 1, 5, 5, 1, 3, 3, 1, 1, 1),         # smallest
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_conv_f32(gpu, cpu, case):
+    N, C, H, W, K, R, S, st, pd, g = case
+    r = rng(hash(case) % (2 ** 31))
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    bound = np.sqrt(6.0 / (C // g * R * S))
+    w = r.uniform(-bound, bound, (K, C // g, R, S)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, K).astype(np.float32)
+    args = ((pd, pd), (st, st), g)
+    close(oc.conv(gpu, x, w, None, *args), oc.conv(cpu, x, w, None, *args))
+    ref = oc.conv(cpu, x, w, b, *args, _abi.ACT_RELU)
+    got = oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU)
+    close(got, ref)
+    assert (got >= 0).all()
+    close(oc.conv(gpu, x, w, b, *args, _abi.ACT_IDENTITY), oc.conv(cpu, x, w, b, *args, _abi.ACT_IDENTITY))
+
+
+def test_conv_closed_forms(gpu):
+    x = rng(1).standard_normal((1, 3, 8, 8)).astype(np.float32)
+    w = np.zeros((3, 3, 3, 3), np.float32)
+    for c in range(3):
+        w[c, c, 1, 1] = 1
+    np.testing.assert_array_equal(oc.conv(gpu, x, w, None, (1, 1), (1, 1)), x)
+    w = np.zeros((1, 1, 3, 3), np.float32)
+    w[0, 0, 0, 2] = 1
+    xi = np.arange(36, dtype=np.float32).reshape(1, 1, 6, 6)
+    exp = np.zeros((6, 6), np.float32)
+    exp[1:, :-1] = xi[0, 0, :-1, 1:]
+    np.testing.assert_array_equal(oc.conv(gpu, xi, w, None, (1, 1), (1, 1))[0, 0], exp)
+
+
+def test_conv_errors(gpu):
+    x = np.zeros((1, 4, 4, 4), np.float32)
+    with pytest.raises(RuntimeError):
+        oc.conv(gpu, x, np.zeros((4, 3, 1, 1), np.float32))
+    with pytest.raises(RuntimeError):
+        oc.conv(gpu, x, np.zeros((4, 4, 7, 7), np.float32))
+
+
+# ---- elementwise -----------------------------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 3, 255, 256, 1025, 200704])
+def test_unary_exact(gpu, cpu, n):
+    x = np.concatenate([rng(n).standard_normal(n) * 3]).astype(np.float32)
+    x[0] = -0.0
+    for name, kw in [("relu", {}), ("negative", {}), ("clip", {"lo": 0.0, "hi": 6.0})]:
+        np.testing.assert_array_equal(oc.unary(gpu, name, x, **kw), oc.unary(cpu, name, x, **kw))
+    nz = np.where(x == 0, np.float32(1), x)
+    np.testing.assert_array_equal(oc.unary(gpu, "reciprocal", nz), oc.unary(cpu, "reciprocal", nz))
+    np.testing.assert_array_equal(oc.unary(gpu, "sqrt", np.abs(x)), oc.unary(cpu, "sqrt", np.abs(x)))
+    np.testing.assert_array_equal(oc.pow_(gpu, x, 2.0), oc.pow_(cpu, x, 2.0))
+    for name in ("erf", "gelu", "sigmoid", "tanh"):
+        close(oc.unary(gpu, name, x), oc.unary(cpu, name, x))
+    close(oc.pow_(gpu, np.abs(x) + 0.5, 1.5), oc.pow_(cpu, np.abs(x) + 0.5, 1.5))
+
+
+def test_unary_misc(gpu, cpu):
+    assert np.isnan(oc.unary(gpu, "relu", np.array([np.nan, 1.0], np.float32))[0])
+    i = rng(2).integers(-2 ** 40, 2 ** 40, 777)
+    np.testing.assert_array_equal(oc.cast(gpu, i), oc.cast(cpu, i))
+    # 4-D shape through dnnrtActive, and an unaligned view (pointer + 4 bytes)
+    x = rng(3).standard_normal((2, 3, 5, 7)).astype(np.float32)
+    np.testing.assert_array_equal(oc.unary(gpu, "relu", x), oc.unary(cpu, "relu", x))
+    t = gpu.put(rng(4).standard_normal(1030).astype(np.float32))
+    y = gpu.empty(1030)
+    gpu.ops.negative(gpu.ptr(t) + 4, gpu.ptr(y) + 4, [1029])
+    gpu.sync()
+    np.testing.assert_array_equal(gpu.get(y)[1:], -gpu.get(t)[1:])
+    # fp16 storage
+    h = (rng(5).standard_normal(5000) * 4).astype(np.float16)
+    for name, kw in [("relu", {}), ("negative", {}), ("clip", {"lo": 0.0, "hi": 6.0})]:
+        np.testing.assert_array_equal(oc.unary(gpu, name, h, **kw), oc.unary(cpu, name, h, **kw))
+    close(oc.unary(gpu, "gelu", h).astype(np.float32), oc.unary(cpu, "gelu", h).astype(np.float32), 2e-2, 1e-3)
+
+
+def test_tensor_op(gpu, cpu):
+    r = rng(7)
+    shapes = [((2, 5, 3, 4), (2, 5, 3, 4)), ((2, 5, 3, 4), (1, 5, 1, 1)), ((2, 5, 3, 4), (1, 1, 1, 4)),
+              ((2, 5, 3, 4), (2, 1, 3, 1)), ((2, 5, 3, 4), (1, 1, 1, 1)), ((2, 5, 3, 4), (1, 5, 3, 1)),
+              ((1, 256, 56, 56), (1, 256, 56, 56)), ((1, 256, 56, 56), (1, 256, 1, 1)),
+              ((1, 1000), (1, 1000)), ((1, 128, 768), (1, 1, 768)), ((1, 128, 768), (1, 128, 1)),
+              ((3, 7), (1, 7)), ((5,), (5,)), ((5,), (1,))]
+    for sa, sb in shapes:
+        a = r.standard_normal(sa).astype(np.float32)
+        b = r.standard_normal(sb).astype(np.float32)
+        for op in (_abi.OP_ADD, _abi.OP_MUL):
+            np.testing.assert_array_equal(oc.tensor_op(gpu, op, a, b), oc.tensor_op(cpu, op, a, b))
+            np.testing.assert_array_equal(oc.tensor_op(gpu, op, a, b, coef=-2.5), oc.tensor_op(cpu, op, a, b, coef=-2.5))
+        np.testing.assert_array_equal(oc.tensor_op(gpu, _abi.OP_ADD, a, b, inplace=True),
+                                      oc.tensor_op(cpu, _abi.OP_ADD, a, b, inplace=True))
+    with pytest.raises(RuntimeError):
+        oc.tensor_op(gpu, _abi.OP_ADD, np.zeros((2, 4), np.float32), np.zeros((2, 3), np.float32))
+    a = r.standard_normal((2, 3, 4, 8)).astype(np.float16)
+    b = r.standard_normal((1, 3, 1, 1)).astype(np.float16)
+    np.testing.assert_array_equal(oc.tensor_op(gpu, _abi.OP_ADD, a, b), oc.tensor_op(cpu, _abi.OP_ADD, a, b))
+
+
+# ---- reductions --------------------------------------------------------------------
+
+def test_reduce_mean(gpu, cpu):
+    r = rng(9)
+    for shape, out in [((1, 2048, 7, 7), (1, 2048, 1, 1)), ((2, 6, 7, 7), (2, 1, 7, 7)), ((2, 6, 7, 7), (1, 6, 7, 7)),
+                       ((1, 128, 768), (1, 128, 1)), ((3, 1000), (3, 1)), ((1, 1280, 7, 7), (1, 1280, 1, 1))]:
+        x = r.standard_normal(shape).astype(np.float32)
+        close(oc.reduce_mean(gpu, x, out), oc.reduce_mean(cpu, x, out))
+    with pytest.raises(RuntimeError):
+        oc.reduce_mean(gpu, np.zeros((2, 3, 4, 5), np.float32), (1, 3, 1, 5))
+
+
+def test_softmax(gpu, cpu):
+    r = rng(10)
+    x = (r.standard_normal((1, 12, 128, 128)) * 3).astype(np.float32)
+    got = oc.softmax(gpu, x, 3)
+    close(got, oc.softmax(cpu, x, 3), 1e-4, 1e-7)
+    close(got.sum(3), 1.0, 1e-5)
+    x = (r.standard_normal((2, 3, 5, 17)) * 4).astype(np.float32)
+    for axis in (3, -1, 1, 0, 2):
+        close(oc.softmax(gpu, x, axis), oc.softmax(cpu, x, axis), 1e-4, 1e-7)
+    big = np.array([[1000.0, 1000.0, -1000.0]], np.float32)
+    close(oc.softmax(gpu, big, 1), [[0.5, 0.5, 0.0]], 1e-6, 1e-7)
+
+
+def test_layernorm(gpu, cpu):
+    r = rng(12)
+    for shape in [(1, 128, 768), (2, 7, 48), (5, 1000), (3, 1)]:
+        L = shape[-1]
+        x = (r.standard_normal(shape) * 3 + 1).astype(np.float32)
+        g = r.standard_normal(L).astype(np.float32)
+        b = r.standard_normal(L).astype(np.float32)
+        close(oc.layernorm(gpu, x, g, b, 1e-12 if L > 1 else 1e-5), oc.layernorm(cpu, x, g, b, 1e-12 if L > 1 else 1e-5), 1e-4, 1e-4)
+
+
+# ---- pooling ---------------------------------------------------------------------------
+
+def test_pooling(gpu, cpu):
+    r = rng(13)
+    x = r.standard_normal((1, 64, 112, 112)).astype(np.float32)
+    np.testing.assert_array_equal(oc.pool(gpu, "max", x, (3, 3), (1, 1), (2, 2)), oc.pool(cpu, "max", x, (3, 3), (1, 1), (2, 2)))
+    x = r.standard_normal((2, 3, 13, 12)).astype(np.float32)
+    for k, p, s in [(3, 1, 2), (2, 0, 2), (3, 0, 1), (3, 1, 1)]:
+        np.testing.assert_array_equal(oc.pool(gpu, "max", x, (k, k), (p, p), (s, s)), oc.pool(cpu, "max", x, (k, k), (p, p), (s, s)))
+        close(oc.pool(gpu, "avg", x, (k, k), (p, p), (s, s)), oc.pool(cpu, "avg", x, (k, k), (p, p), (s, s)))
+    xn = x.copy()
+    xn[0, 0, 0, 0] = np.nan
+    np.testing.assert_array_equal(np.isnan(oc.pool(gpu, "max", xn, (3, 3), (1, 1), (2, 2))),
+                                  np.isnan(oc.pool(cpu, "max", xn, (3, 3), (1, 1), (2, 2))))
+
+
+# ---- matrix products --------------------------------------------------------------------
+
+def test_matmul2d(gpu, cpu):
+    r = rng(14)
+    for M, K, N in [(1, 2048, 1000), (1, 1280, 1000), (5, 9, 7), (64, 64, 64), (130, 70, 33), (3, 2048, 10), (16, 250, 40)]:
+        a = r.standard_normal((M, K)).astype(np.float32)
+        b = (r.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+        c = r.standard_normal((M, N)).astype(np.float32)
+        ref = oc.matmul2d(cpu, a, b)
+        close(oc.matmul2d(gpu, a, b), ref)
+        close(oc.matmul2d(gpu, a.T.copy(), b, transA=1), ref)
+        close(oc.matmul2d(gpu, a, b.T.copy(), transB=1), ref)
+        close(oc.matmul2d(gpu, a.T.copy(), b.T.copy(), transA=1, transB=1), ref)
+        close(oc.matmul2d(gpu, a, b.T.copy(), c.copy(), alpha=0.5, beta=-2.0, transB=1),
+              oc.matmul2d(cpu, a, b.T.copy(), c.copy(), alpha=0.5, beta=-2.0, transB=1))
+    with pytest.raises(RuntimeError):
+        oc.matmul2d(gpu, np.zeros((5, 9), np.float32), np.zeros((9, 7), np.float32), transB=1)
+
+
+def test_matmul_nd(gpu, cpu):
+    r = rng(15)
+    cases = [((1, 128, 768), (768, 768)), ((1, 12, 128, 64), (1, 12, 64, 128)), ((1, 12, 128, 128), (1, 12, 128, 64)),
+             ((1, 128, 768), (768, 3072)), ((1, 128, 3072), (3072, 768)),
+             ((4, 6), (6, 3)), ((2, 4, 6), (6, 3)), ((2, 3, 4, 6), (2, 3, 6, 5)), ((2, 4, 6), (2, 6, 3)), ((4, 6), (3, 6, 2))]
+    for sa, sb in cases:
+        a = r.standard_normal(sa).astype(np.float32)
+        b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float32)
+        close(oc.matmul_nd(gpu, a, b), oc.matmul_nd(cpu, a, b))
+
+
+# ---- data movement -------------------------------------------------------------------------
+
+def test_data_movement(gpu, cpu):
+    r = rng(16)
+    x = r.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    np.testing.assert_array_equal(oc.flatten(gpu, x, 1), x.reshape(2, 60))
+    np.testing.assert_array_equal(oc.reshape(gpu, x, (6, 20)), x.reshape(6, 20))
+    for perm in [(0, 2, 1, 3), (0, 2, 3, 1), (3, 2, 1, 0), (1, 0, 2, 3)]:
+        np.testing.assert_array_equal(oc.transpose(gpu, x, perm), x.transpose(perm))
+    h = r.standard_normal((1, 128, 12, 64)).astype(np.float32)
+    np.testing.assert_array_equal(oc.transpose(gpu, h, (0, 2, 1, 3)), h.transpose(0, 2, 1, 3))
+    np.testing.assert_array_equal(oc.transpose(gpu, h, (0, 2, 3, 1)), h.transpose(0, 2, 3, 1))
+    np.testing.assert_array_equal(oc.transpose(gpu, x[0], (1, 0, 2)), x[0].transpose(1, 0, 2))
+    xi = r.integers(-5, 5, (3, 4)).astype(np.int64)
+    np.testing.assert_array_equal(oc.transpose(gpu, xi, (1, 0)), xi.T)
+    x6 = r.standard_normal((2, 3, 2, 2, 3, 2)).astype(np.float32)
+    np.testing.assert_array_equal(oc.transpose(gpu, x6, (0, 1, 4, 2, 5, 3)), x6.transpose(0, 1, 4, 2, 5, 3))
+    table = r.standard_normal((30522, 768)).astype(np.float32)
+    idx = r.integers(0, 30522, (1, 128))
+    np.testing.assert_array_equal(oc.gather(gpu, table, idx, 0), np.take(table, idx, 0))
+    np.testing.assert_array_equal(oc.gather(gpu, x, np.array([2, -1]), 2), np.take(x, [2, -1], 2))
+    with pytest.raises(RuntimeError):
+        oc.transpose(gpu, x, (0, 1, 1, 3))

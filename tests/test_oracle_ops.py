@@ -1,0 +1,333 @@
+"""Pins the CPU oracle (oracle/dnnrt_oracle.c).
+
+The reference holds no golden vectors for these operators and its arithmetic
+(cuDNN / cuBLASLt / CUDA kernels) cannot run here, so each oracle function is
+checked against what fixes it independently: an independent library (torch
+CPU / numpy in float64), closed forms, and brute force on tiny shapes -- with
+cases chosen so that a dropped term, a wrong sign or index, or a transposed
+operand fails.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import opcases as oc
+from helpers import OracleBackend, rng
+from occamy_amd import _abi
+
+
+@pytest.fixture(scope="module")
+def be():
+    return OracleBackend()
+
+
+def t64(a):
+    return torch.from_numpy(np.asarray(a, dtype=np.float64))
+
+
+# ---- convolution -----------------------------------------------------------
+
+def brute_conv(x, w, b, pads, strides, group):
+    """7-loop definition in Python floats (float64), tiny shapes only."""
+    N, C, H, W = x.shape
+    K, Cg, R, S = w.shape
+    P, Q = oc.conv_out_hw(H, W, R, S, pads, strides)
+    y = np.zeros((N, K, P, Q))
+    Kg = K // group
+    for n in range(N):
+        for k in range(K):
+            g = k // Kg
+            for p in range(P):
+                for q in range(Q):
+                    acc = 0.0 if b is None else float(b[k])
+                    for c in range(Cg):
+                        for r in range(R):
+                            for s in range(S):
+                                ih, iw = p * strides[0] - pads[0] + r, q * strides[1] - pads[1] + s
+                                if 0 <= ih < H and 0 <= iw < W:
+                                    acc += float(x[n, g * Cg + c, ih, iw]) * float(w[k, c, r, s])
+                    y[n, k, p, q] = acc
+    return y
+
+
+@pytest.mark.parametrize("R,S", [(1, 1), (3, 3), (2, 3)])
+@pytest.mark.parametrize("stride", [(1, 1), (2, 2), (1, 2)])
+@pytest.mark.parametrize("pad", [(0, 0), (1, 1), (2, 1)])
+@pytest.mark.parametrize("group", [1, 2, 4])
+def test_conv_bruteforce_tiny(be, R, S, stride, pad, group):
+    r = rng(R * 100 + S * 10 + stride[0] + pad[0] * 7 + group)
+    x = r.standard_normal((2, 4, 6, 5)).astype(np.float32)
+    w = r.standard_normal((4, 4 // group, R, S)).astype(np.float32)
+    b = r.standard_normal(4).astype(np.float32)
+    if 6 + 2 * pad[0] < R or 5 + 2 * pad[1] < S:
+        pytest.skip("empty output")
+    ref = brute_conv(x, w, b, pad, stride, group)
+    got = oc.conv(be, x, w, b, pad, stride, group, _abi.ACT_IDENTITY)
+    np.testing.assert_allclose(got, ref, rtol=1e-6, atol=1e-6)
+    got_nb = oc.conv(be, x, w, None, pad, stride, group)
+    np.testing.assert_allclose(got_nb, brute_conv(x, w, None, pad, stride, group), rtol=1e-6, atol=1e-6)
+    relu = oc.conv(be, x, w, b, pad, stride, group, _abi.ACT_RELU)
+    np.testing.assert_array_equal(relu, np.maximum(got, 0))
+
+
+@pytest.mark.parametrize("shape", [
+    # (N, C, H, W, K, R, stride, pad, group)
+    (1, 64, 56, 56, 64, 3, 1, 1, 1),     # the single-conv configuration
+    (2, 3, 33, 35, 16, 7, 2, 3, 1),      # stem-like, odd sizes
+    (1, 32, 14, 14, 32, 3, 2, 1, 32),    # depthwise stride 2
+    (1, 24, 9, 9, 48, 1, 2, 0, 1),       # strided 1x1
+])
+def test_conv_vs_torch_float64(be, shape):
+    N, C, H, W, K, R, st, pd, g = shape
+    r = rng(sum(shape))
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((K, C // g, R, R)) * 0.1).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, K).astype(np.float32)
+    ref = F.conv2d(t64(x), t64(w), t64(b), stride=st, padding=pd, groups=g).numpy()
+    got = oc.conv(be, x, w, b, (pd, pd), (st, st), g, _abi.ACT_IDENTITY)
+    np.testing.assert_allclose(got, ref, rtol=2e-6, atol=2e-6)
+
+
+def test_conv_closed_forms(be):
+    r = rng(5)
+    x = r.standard_normal((1, 3, 8, 8)).astype(np.float32)
+    # identity filter: centre tap 1 on the matching channel -> Y == X
+    w = np.zeros((3, 3, 3, 3), np.float32)
+    for c in range(3):
+        w[c, c, 1, 1] = 1
+    np.testing.assert_array_equal(oc.conv(be, x, w, None, (1, 1), (1, 1)), x)
+    # all-ones input and filter: each output counts its in-range taps times C
+    ones = np.ones((1, 2, 5, 5), np.float32)
+    y = oc.conv(be, ones, np.ones((1, 2, 3, 3), np.float32), None, (1, 1), (1, 1))
+    cnt = np.array([[(min(i + 1, 4) - max(i - 1, 0) + 1) * (min(j + 1, 4) - max(j - 1, 0) + 1)
+                     for j in range(5)] for i in range(5)], np.float32)
+    np.testing.assert_array_equal(y[0, 0], 2 * cnt)
+    # a filter with a single off-centre tap shifts the image (catches r/s or
+    # sign mix-ups): tap (r=0, s=2) reads X[p-1, q+1]
+    w = np.zeros((1, 1, 3, 3), np.float32)
+    w[0, 0, 0, 2] = 1
+    xi = np.arange(36, dtype=np.float32).reshape(1, 1, 6, 6)
+    y = oc.conv(be, xi, w, None, (1, 1), (1, 1))[0, 0]
+    exp = np.zeros((6, 6), np.float32)
+    exp[1:, :-1] = xi[0, 0, :-1, 1:]
+    np.testing.assert_array_equal(y, exp)
+    # 1x1 stride-1 convolution is W[K,C] @ X[C,HW]
+    w1 = r.standard_normal((5, 3, 1, 1)).astype(np.float32)
+    y = oc.conv(be, x, w1, None, (0, 0), (1, 1))
+    ref = (w1.reshape(5, 3).astype(np.float64) @ x.reshape(3, 64).astype(np.float64)).reshape(1, 5, 8, 8)
+    np.testing.assert_allclose(y, ref, rtol=1e-6, atol=1e-6)
+
+
+def test_conv_errors(be):
+    x = np.zeros((1, 4, 4, 4), np.float32)
+    with pytest.raises(RuntimeError):
+        oc.conv(be, x, np.zeros((4, 3, 1, 1), np.float32))      # C/g mismatch
+    with pytest.raises(RuntimeError):
+        oc.conv(be, x, np.zeros((4, 4, 7, 7), np.float32))      # empty output
+
+
+def test_conv_fp16_storage(be):
+    r = rng(11)
+    x = r.standard_normal((1, 8, 6, 6)).astype(np.float16)
+    w = (r.standard_normal((4, 8, 3, 3)) * 0.2).astype(np.float16)
+    b = r.uniform(-0.1, 0.1, 4).astype(np.float16)
+    got = oc.conv(be, x, w, b, (1, 1), (1, 1), 1, _abi.ACT_RELU)
+    ref = F.relu(F.conv2d(t64(x), t64(w), t64(b), padding=1)).numpy()
+    assert got.dtype == np.float16
+    # one rounding to fp16 of the exact value
+    np.testing.assert_array_equal(got, ref.astype(np.float32).astype(np.float16))
+
+
+# ---- fp16 conversion -----------------------------------------------------------
+
+def test_fp16_round_trip_all_values(be):
+    """Every finite fp16 value must survive widen -> negate -> negate -> narrow, and
+    float32 -> fp16 rounding must agree with numpy on a sweep incl. subnormals/ties."""
+    allh = np.arange(65536, dtype=np.uint16).view(np.float16)
+    fin = allh[np.isfinite(allh)]
+    np.testing.assert_array_equal(oc.unary(be, "negative", oc.unary(be, "negative", fin)).view(np.uint16),
+                                  fin.view(np.uint16))
+    r = rng(3)
+    f = np.concatenate([r.standard_normal(20000) * 10.0 ** r.integers(-9, 5, 20000),
+                        np.array([65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8,
+                                  6.1035156e-5, 6.0975552e-5, 0.0, -0.0])]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        expect = f.astype(np.float16)
+    got = oc.cast(be, f.astype(np.int64), np.float16)  # integers only; separate path below
+    np.testing.assert_array_equal(got, f.astype(np.int64).astype(np.float32).astype(np.float16))
+    # float path: x * 1 through tensor_op MUL keeps the value, narrowing does the rounding
+    xs = expect  # representable inputs stay fixed
+    np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_MUL, xs, np.ones_like(xs)).view(np.uint16)[np.isfinite(xs)],
+                                  xs.view(np.uint16)[np.isfinite(xs)])
+    # products that need rounding: compare against numpy's float32 -> float16
+    a = (r.standard_normal(5000)).astype(np.float16)
+    b = (r.standard_normal(5000)).astype(np.float16)
+    prod = (a.astype(np.float32) * b.astype(np.float32)).astype(np.float16)
+    np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_MUL, a, b).view(np.uint16), prod.view(np.uint16))
+
+
+# ---- elementwise -------------------------------------------------------------------
+
+def test_unary_ops(be):
+    x = np.concatenate([rng(1).standard_normal(1000) * 3, [0.0, -0.0, 7.5, -7.5]]).astype(np.float32)
+    np.testing.assert_array_equal(oc.unary(be, "relu", x), np.where(x < 0, np.float32(0), x))
+    np.testing.assert_array_equal(oc.unary(be, "negative", x), -x)
+    np.testing.assert_array_equal(oc.unary(be, "clip", x, lo=0.0, hi=6.0), np.clip(x, 0, 6))
+    nz = x[x != 0]
+    np.testing.assert_array_equal(oc.unary(be, "reciprocal", nz), (np.float32(1) / nz))
+    np.testing.assert_array_equal(oc.unary(be, "sqrt", np.abs(x)), np.sqrt(np.abs(x)))
+    ref_erf = np.array([math.erf(float(v)) for v in x])
+    np.testing.assert_allclose(oc.unary(be, "erf", x), ref_erf, rtol=1e-6, atol=1e-7)
+    ref_gelu = np.array([0.5 * float(v) * (1 + math.erf(float(v) / math.sqrt(2))) for v in x])
+    np.testing.assert_allclose(oc.unary(be, "gelu", x), ref_gelu, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(oc.unary(be, "sigmoid", x), 1 / (1 + np.exp(-x.astype(np.float64))), rtol=1e-6)
+    np.testing.assert_allclose(oc.unary(be, "tanh", x), np.tanh(x.astype(np.float64)), rtol=1e-6, atol=1e-7)
+    # NaN goes through ReLU, as with CUDNN_PROPAGATE_NAN
+    assert np.isnan(oc.unary(be, "relu", np.array([np.nan], np.float32))[0])
+    np.testing.assert_array_equal(oc.pow_(be, x, 2.0), x * x)
+    np.testing.assert_allclose(oc.pow_(be, np.abs(x) + 0.5, 1.5), (np.abs(x.astype(np.float64)) + 0.5) ** 1.5, rtol=1e-6)
+    i = rng(2).integers(-2 ** 40, 2 ** 40, 500)
+    np.testing.assert_array_equal(oc.cast(be, i), i.astype(np.float32))
+
+
+def test_tensor_op_broadcast(be):
+    r = rng(7)
+    a = r.standard_normal((2, 5, 3, 4)).astype(np.float32)
+    for bshape in [(2, 5, 3, 4), (1, 5, 1, 1), (1, 1, 1, 4), (2, 1, 3, 1), (1, 1, 1, 1), (1, 5, 3, 1)]:
+        b = r.standard_normal(bshape).astype(np.float32)
+        np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_ADD, a, b), a + b)
+        np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_MUL, a, b), a * b)
+        np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_ADD, a, b, coef=-2.0), a + np.float32(-2) * b)
+        np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_ADD, a, b, inplace=True), a + b)
+    with pytest.raises(RuntimeError):
+        oc.tensor_op(be, _abi.OP_ADD, a, np.zeros((2, 5, 3, 2), np.float32))
+    # rank 2 and 3 (Gemm bias, LayerNorm scale)
+    a2 = r.standard_normal((3, 7)).astype(np.float32)
+    b2 = r.standard_normal((1, 7)).astype(np.float32)
+    np.testing.assert_array_equal(oc.tensor_op(be, _abi.OP_ADD, a2, b2), a2 + b2)
+
+
+# ---- reductions ---------------------------------------------------------------------
+
+def test_reduce_mean(be):
+    r = rng(9)
+    x = r.standard_normal((2, 6, 7, 7)).astype(np.float32)
+    ref = x.astype(np.float64)
+    np.testing.assert_allclose(oc.reduce_mean(be, x, (2, 6, 1, 1)), ref.mean((2, 3), keepdims=True), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(oc.reduce_mean(be, x, (2, 1, 7, 7)), ref.mean(1, keepdims=True), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(oc.reduce_mean(be, x, (1, 6, 7, 7)), ref.mean(0, keepdims=True), rtol=1e-6, atol=1e-7)
+    x3 = r.standard_normal((2, 5, 33)).astype(np.float32)
+    np.testing.assert_allclose(oc.reduce_mean(be, x3, (2, 5, 1)), x3.astype(np.float64).mean(2, keepdims=True), rtol=1e-6, atol=1e-7)
+    # constant tensor: mean is the constant exactly
+    c = np.full((1, 3, 4, 4), 2.5, np.float32)
+    np.testing.assert_array_equal(oc.reduce_mean(be, c, (1, 3, 1, 1)), np.full((1, 3, 1, 1), 2.5, np.float32))
+
+
+def test_softmax(be):
+    r = rng(10)
+    x = (r.standard_normal((2, 3, 5, 16)) * 4).astype(np.float32)
+    for axis in (3, -1, 1, 0):
+        got = oc.softmax(be, x, axis)
+        ref = torch.softmax(t64(x), dim=axis).numpy()
+        np.testing.assert_allclose(got, ref, rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(got.sum(axis), 1.0, rtol=1e-6)
+    # shift invariance and the closed form of a constant row
+    np.testing.assert_allclose(oc.softmax(be, x + 100.0, 3), oc.softmax(be, x, 3), rtol=1e-4)
+    np.testing.assert_allclose(oc.softmax(be, np.full((2, 8), 3.0, np.float32), 1), 1 / 8, rtol=1e-7)
+    # large magnitudes must not overflow
+    big = np.array([[1000.0, 1000.0, -1000.0]], np.float32)
+    np.testing.assert_allclose(oc.softmax(be, big, 1), [[0.5, 0.5, 0.0]], atol=1e-7)
+
+
+def test_layernorm(be):
+    r = rng(12)
+    x = (r.standard_normal((2, 7, 48)) * 3 + 1).astype(np.float32)
+    g = r.standard_normal(48).astype(np.float32)
+    b = r.standard_normal(48).astype(np.float32)
+    got = oc.layernorm(be, x, g, b, 1e-5)
+    ref = F.layer_norm(t64(x), (48,), t64(g), t64(b), 1e-5).numpy()
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+    # gamma 1, beta 0: rows have zero mean and unit (biased) variance
+    y = oc.layernorm(be, x, np.ones(48, np.float32), np.zeros(48, np.float32), 0.0).astype(np.float64)
+    np.testing.assert_allclose(y.mean(-1), 0, atol=1e-6)
+    np.testing.assert_allclose(y.var(-1), 1, rtol=1e-5)
+    # equals the decomposed chain the reference emits, built from the oracle's primitives
+    mu = oc.reduce_mean(be, x, (2, 7, 1))
+    d = oc.tensor_op(be, _abi.OP_ADD, x, oc.unary(be, "negative", mu))
+    var = oc.reduce_mean(be, oc.pow_(be, d, 2.0), (2, 7, 1))
+    std = oc.unary(be, "sqrt", oc.tensor_op(be, _abi.OP_ADD, var, np.full((1, 1, 1), 1e-5, np.float32)))
+    chain = oc.tensor_op(be, _abi.OP_MUL, d, oc.unary(be, "reciprocal", std))
+    chain = oc.tensor_op(be, _abi.OP_ADD, oc.tensor_op(be, _abi.OP_MUL, chain, g.reshape(1, 1, 48)), b.reshape(1, 1, 48))
+    np.testing.assert_allclose(got, chain, rtol=1e-5, atol=2e-6)
+
+
+# ---- pooling -----------------------------------------------------------------------------
+
+def test_pooling(be):
+    r = rng(13)
+    x = r.standard_normal((2, 3, 13, 12)).astype(np.float32)
+    for k, p, s in [(3, 1, 2), (2, 0, 2), (3, 0, 1), (3, 1, 1)]:
+        got = oc.pool(be, "max", x, (k, k), (p, p), (s, s))
+        ref = F.max_pool2d(torch.from_numpy(x), k, s, p).numpy()
+        np.testing.assert_array_equal(got, ref)
+        got = oc.pool(be, "avg", x, (k, k), (p, p), (s, s))
+        ref = F.avg_pool2d(t64(x), k, s, p, count_include_pad=True).numpy()
+        np.testing.assert_allclose(got, ref, rtol=1e-6, atol=1e-7)
+    # negative inputs: padding must not win the max
+    neg = -np.abs(x) - 1
+    assert (oc.pool(be, "max", neg, (3, 3), (1, 1), (2, 2)) < 0).all()
+
+
+# ---- matrix products -------------------------------------------------------------------------
+
+def test_matmul2d(be):
+    r = rng(14)
+    a = r.standard_normal((5, 9)).astype(np.float32)
+    b = r.standard_normal((9, 7)).astype(np.float32)
+    c = r.standard_normal((5, 7)).astype(np.float32)
+    A, B = a.astype(np.float64), b.astype(np.float64)
+    np.testing.assert_allclose(oc.matmul2d(be, a, b), A @ B, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oc.matmul2d(be, a.T.copy(), b, transA=1), A @ B, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oc.matmul2d(be, a, b.T.copy(), transB=1), A @ B, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oc.matmul2d(be, a.T.copy(), b.T.copy(), transA=1, transB=1), A @ B, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oc.matmul2d(be, a, b, c.copy(), alpha=0.5, beta=-2.0), 0.5 * (A @ B) - 2.0 * c, rtol=1e-6, atol=1e-6)
+    # permutation matrix: rows of b reordered exactly
+    perm = np.eye(9, dtype=np.float32)[r.permutation(9)]
+    np.testing.assert_array_equal(oc.matmul2d(be, perm, b), perm @ b)
+    with pytest.raises(RuntimeError):
+        oc.matmul2d(be, a, b, transB=1)
+
+
+def test_matmul_nd(be):
+    r = rng(15)
+    cases = [((4, 6), (6, 3)), ((2, 4, 6), (6, 3)), ((2, 3, 4, 6), (2, 3, 6, 5)), ((1, 3, 4, 6), (1, 3, 6, 4)),
+             ((2, 4, 6), (2, 6, 3)), ((4, 6), (3, 6, 2))]
+    for sa, sb in cases:
+        a = r.standard_normal(sa).astype(np.float32)
+        b = r.standard_normal(sb).astype(np.float32)
+        np.testing.assert_allclose(oc.matmul_nd(be, a, b), np.matmul(a.astype(np.float64), b.astype(np.float64)), rtol=1e-6, atol=1e-6)
+
+
+# ---- data movement --------------------------------------------------------------------------------
+
+def test_data_movement(be):
+    r = rng(16)
+    x = r.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    np.testing.assert_array_equal(oc.flatten(be, x, 1), x.reshape(2, 60))
+    np.testing.assert_array_equal(oc.reshape(be, x, (6, 20)), x.reshape(6, 20))
+    for perm in [(0, 2, 1, 3), (0, 2, 3, 1), (3, 2, 1, 0), (1, 0, 2, 3)]:
+        np.testing.assert_array_equal(oc.transpose(be, x, perm), x.transpose(perm))
+    np.testing.assert_array_equal(oc.transpose(be, x[0], (1, 0, 2)), x[0].transpose(1, 0, 2))
+    np.testing.assert_array_equal(oc.transpose(be, x[0, 0], (1, 0)), x[0, 0].T)
+    xi = r.integers(-5, 5, (3, 4)).astype(np.int64)
+    np.testing.assert_array_equal(oc.transpose(be, xi, (1, 0)), xi.T)
+    table = r.standard_normal((11, 6)).astype(np.float32)
+    idx = r.integers(0, 11, (2, 5))
+    np.testing.assert_array_equal(oc.gather(be, table, idx, 0), np.take(table, idx, 0))
+    np.testing.assert_array_equal(oc.gather(be, table, np.array([-1, 0]), 0), np.take(table, [-1, 0], 0))
+    np.testing.assert_array_equal(oc.gather(be, x, np.array([2, 0]), 2), np.take(x, [2, 0], 2))
+    with pytest.raises(RuntimeError):
+        oc.gather(be, table, np.array([11]), 0)
