@@ -1,0 +1,92 @@
+/* dnnc.h -- C API of the host-side DNN program compiler and executor.
+ *
+ * It stands where the reference's compiler passes and generated model code
+ * stand for the hot path: ONNX-level graph -> DNN program
+ * (src/Conversion/ONNXToDNN), function arguments to device memory
+ * (src/Transform/DNN/FunctionArgument.cpp), removal of unused constant uploads
+ * (eraseDummyConstants.cpp), optional conv+bias+relu fusion
+ * (opFusing/fuseConvBiasRelu.cpp), dealloc placement (DNNDeallocOpt.cpp), the
+ * memory-pool planner (mallocPoolOpt.{hpp,cpp}), and the straight-line call
+ * sequence into the runtime that src/Conversion/DNNToLLVM emits.
+ * All functions return 0 / non-NULL on success; dnncLastError() gives the text
+ * of the calling thread's last failure.
+ */
+#ifndef DNNC_H
+#define DNNC_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dnncGraph dnncGraph;
+typedef struct dnncProgram dnncProgram;
+typedef struct dnncSession dnncSession;
+
+enum { DNNC_F32 = 0, DNNC_F16 = 1, DNNC_I64 = 2 };
+
+const char *dnncLastError(void);
+
+/* ---- graph building (what the ONNX importer hands to the reference) ---- */
+dnncGraph *dnncGraphCreate(void);
+void dnncGraphDestroy(dnncGraph *g);
+int32_t dnncGraphAddInput(dnncGraph *g, const char *name, int32_t dtype, int32_t rank, const int64_t *dims);
+/* the bytes are copied */
+int32_t dnncGraphAddConstant(dnncGraph *g, const char *name, int32_t dtype, int32_t rank, const int64_t *dims, const void *data);
+/* attrs: "key=v1,v2;key2=v" -- integer lists, or a float when the value has a '.' or 'e' */
+int32_t dnncGraphAddNode(dnncGraph *g, const char *op_type, int32_t n_inputs, const char *const *inputs, const char *output, const char *attrs);
+int32_t dnncGraphAddOutput(dnncGraph *g, const char *name);
+
+/* ---- compilation ---- */
+typedef struct {
+  int32_t const_at_use;   /* reference flag --onnx-const-at-use (default 1) */
+  int32_t fusion;         /* --dnn-kernel-fusion (default 0) */
+  int32_t dealloc_opt;    /* --dnn-dealloc-opt (the reference's tests set 1) */
+  int32_t pool_opt;       /* --dnn-malloc-pool-opt (the reference's tests set 1) */
+  int32_t channels_last;  /* fp16 only: rank-4 activations are NHWC on the device */
+} dnncOptions;
+/* the graph must outlive the program: constants are not copied again */
+dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);
+void dnncProgramDestroy(dnncProgram *p);
+/* the program as text, one operation per line (valid until the program is destroyed) */
+const char *dnncProgramText(dnncProgram *p);
+/* pool size as the reference planner reports it (its `maxAllocByte`) */
+int64_t dnncProgramPoolBytes(const dnncProgram *p);
+/* highest planned byte + 1; equal to the above for every trace the emission
+ * rules produce.  The executor allocates the larger of the two. */
+int64_t dnncProgramPoolExtent(const dnncProgram *p);
+/* allocation events in execution order; returns the count (pass NULLs to query).
+ * kind 0 = malloc, 1 = dealloc; bytes = unrounded size (malloc only);
+ * offset = planned pool offset (malloc only, -1 before the pool pass). */
+int64_t dnncProgramEvents(const dnncProgram *p, int32_t *kind, int64_t *id, int64_t *bytes, int64_t *offset, int64_t cap);
+int32_t dnncProgramNumInputs(const dnncProgram *p);
+int32_t dnncProgramNumOutputs(const dnncProgram *p);
+/* rank, dims (up to 8) and dtype of output i */
+int32_t dnncProgramOutputInfo(const dnncProgram *p, int32_t i, int32_t *dtype, int32_t *rank, int64_t *dims);
+int64_t dnncProgramNumOps(const dnncProgram *p, int32_t compute_only);
+
+/* ---- the planner alone (mallocPoolOpt.hpp:21-140, 212-218) ----
+ * kind/id/bytes as above; writes one offset per event (-1 for deallocs) and
+ * returns the pool size, or -1 on a dealloc of a tensor that is not live. */
+int64_t dnncPlanPool(int64_t n, const int32_t *kind, const int64_t *id, const int64_t *bytes, int64_t *offset);
+/* free list after the first `upto + 1` events as (first, last) byte pairs; returns the number of blocks */
+int64_t dnncPlanFreeList(int64_t n, const int32_t *kind, const int64_t *id, const int64_t *bytes, int64_t upto, int64_t *out, int64_t cap);
+
+/* ---- execution ---- */
+enum { DNNC_MODE_OCCAMY = 0, DNNC_MODE_RESIDENT = 1 };
+/* runtime_library: path of a shared object exporting include/dnnrt.h */
+dnncSession *dnncSessionCreate(dnncProgram *p, const char *runtime_library, int32_t mode);
+void dnncSessionDestroy(dnncSession *s);
+/* host buffers in, host buffers out; returns when the results are in `outputs` */
+int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *outputs);
+/* resident mode only.  on_device: inputs/outputs are device buffers and the call does not
+ * wait (dnncSessionSync does); use_graph: replay the kernels from a captured graph */
+int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
+int32_t dnncSessionSync(dnncSession *s);
+int64_t dnncSessionWeightsBytes(const dnncSession *s);
+/* bytes the last occamy-mode run requested from dnnrtMemPoolInit (-1 before any run) */
+int64_t dnncSessionLastPoolBytes(const dnncSession *s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DNNC_H */

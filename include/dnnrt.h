@@ -88,6 +88,14 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format);
  * returns to the host without waiting for its device-to-host copies
  * (src/Tools/dnn-wrapper/cuda/wrapDNNMemcpy.cpp:32). */
 int32_t dnnrtSync(dnnrtHandle_t handle);
+/* New.  Stream capture: the kernels that compute calls launch on the handle's
+ * stream between Begin and End are recorded instead of run, and replayed by
+ * Launch.  The handle must have a stream set (dnnrtSetStream); pointers seen
+ * during capture are baked in.  Not available in a host-only build. */
+int32_t dnnrtGraphBegin(dnnrtHandle_t handle);
+int32_t dnnrtGraphEnd(dnnrtHandle_t handle, void **graph);
+int32_t dnnrtGraphLaunch(dnnrtHandle_t handle, void *graph);
+int32_t dnnrtGraphDestroy(void *graph);
 /* New.  Text of the calling thread's last error ("" if none). */
 const char *dnnrtLastError(void);
 /* New.  0 when built for the GPU, 1 for a host-only build of the same ABI. */

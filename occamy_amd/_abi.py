@@ -23,6 +23,10 @@ SIGNATURES = {
     "dnnrtSetStream": (i32, [P, P]),
     "dnnrtSetTensorFormat": (i32, [P, i32]),
     "dnnrtSync": (i32, [P]),
+    "dnnrtGraphBegin": (i32, [P]),
+    "dnnrtGraphEnd": (i32, [P, C.POINTER(P)]),
+    "dnnrtGraphLaunch": (i32, [P, P]),
+    "dnnrtGraphDestroy": (i32, [P]),
     "dnnrtLastError": (C.c_char_p, []),
     "dnnrtIsHostBackend": (i32, []),
     "dnnrtMemPoolInit": (i32, [C.POINTER(P), i64]),

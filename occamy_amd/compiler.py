@@ -1,0 +1,268 @@
+"""Python front end of the DNN program compiler/executor (include/dnnc.h).
+
+``Graph`` collects an ONNX-level graph (inputs, constants, nodes in ONNX
+operator vocabulary), ``Graph.compile`` runs the reference's pass pipeline on
+it (src/Compiler/CoreDNNPasses.cpp:24-28 and CoreDNNUtils.cpp:773-780: ONNX to
+DNN, function arguments to device, dummy-constant removal, optional fusion,
+dealloc placement, pool planning) and ``Program.session`` binds the result to
+the gfx950 runtime.  The compile flags carry the reference's names and the
+values its own tests use (test/models/simpleconv/run.py:50-54).
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import _abi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+DNNC_PATH = os.path.join(_HERE, "lib", "libdnnc.so")
+
+F32, F16, I64 = 0, 1, 2
+_NP = {F32: np.float32, F16: np.float16, I64: np.int64}
+_DT = {np.dtype(np.float32): F32, np.dtype(np.float16): F16, np.dtype(np.int64): I64}
+MODE_OCCAMY, MODE_RESIDENT = 0, 1
+
+
+class _Options(C.Structure):
+    _fields_ = [("const_at_use", C.c_int32), ("fusion", C.c_int32), ("dealloc_opt", C.c_int32),
+                ("pool_opt", C.c_int32), ("channels_last", C.c_int32)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(DNNC_PATH):
+        raise RuntimeError(f"{DNNC_PATH} is not built; run `make -C occamy_amd/csrc` first")
+    L = C.CDLL(DNNC_PATH)
+    P, I64P, I32P = C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32)
+    sig = {
+        "dnncLastError": (C.c_char_p, []),
+        "dnncGraphCreate": (P, []),
+        "dnncGraphDestroy": (None, [P]),
+        "dnncGraphAddInput": (C.c_int32, [P, C.c_char_p, C.c_int32, C.c_int32, I64P]),
+        "dnncGraphAddConstant": (C.c_int32, [P, C.c_char_p, C.c_int32, C.c_int32, I64P, P]),
+        "dnncGraphAddNode": (C.c_int32, [P, C.c_char_p, C.c_int32, C.POINTER(C.c_char_p), C.c_char_p, C.c_char_p]),
+        "dnncGraphAddOutput": (C.c_int32, [P, C.c_char_p]),
+        "dnncCompile": (P, [P, C.POINTER(_Options)]),
+        "dnncProgramDestroy": (None, [P]),
+        "dnncProgramText": (C.c_char_p, [P]),
+        "dnncProgramPoolBytes": (C.c_int64, [P]),
+        "dnncProgramPoolExtent": (C.c_int64, [P]),
+        "dnncProgramEvents": (C.c_int64, [P, I32P, I64P, I64P, I64P, C.c_int64]),
+        "dnncProgramNumInputs": (C.c_int32, [P]),
+        "dnncProgramNumOutputs": (C.c_int32, [P]),
+        "dnncProgramOutputInfo": (C.c_int32, [P, C.c_int32, I32P, I32P, I64P]),
+        "dnncProgramNumOps": (C.c_int64, [P, C.c_int32]),
+        "dnncPlanPool": (C.c_int64, [C.c_int64, I32P, I64P, I64P, I64P]),
+        "dnncPlanFreeList": (C.c_int64, [C.c_int64, I32P, I64P, I64P, C.c_int64, I64P, C.c_int64]),
+        "dnncSessionCreate": (P, [P, C.c_char_p, C.c_int32]),
+        "dnncSessionDestroy": (None, [P]),
+        "dnncSessionRun": (C.c_int32, [P, C.POINTER(P), C.POINTER(P)]),
+        "dnncSessionRunResident": (C.c_int32, [P, C.POINTER(P), C.POINTER(P), C.c_int32, C.c_int32]),
+        "dnncSessionSync": (C.c_int32, [P]),
+        "dnncSessionWeightsBytes": (C.c_int64, [P]),
+        "dnncSessionLastPoolBytes": (C.c_int64, [P]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = L
+    return L
+
+
+def _err():
+    return lib().dnncLastError().decode()
+
+
+def plan_pool(events):
+    """The planner alone.  events: (kind, id, bytes) with kind 0 = malloc, 1 = dealloc.
+    Returns (offsets per event, pool bytes)."""
+    n = len(events)
+    kind = (C.c_int32 * max(n, 1))(*[e[0] for e in events])
+    ids = (C.c_int64 * max(n, 1))(*[e[1] for e in events])
+    byt = (C.c_int64 * max(n, 1))(*[e[2] for e in events])
+    off = (C.c_int64 * max(n, 1))()
+    peak = lib().dnncPlanPool(n, kind, ids, byt, off)
+    if peak < 0:
+        raise RuntimeError("planner: dealloc of a tensor that is not live")
+    return list(off[:n]), peak
+
+
+def plan_free_list(events, upto):
+    n = len(events)
+    kind = (C.c_int32 * max(n, 1))(*[e[0] for e in events])
+    ids = (C.c_int64 * max(n, 1))(*[e[1] for e in events])
+    byt = (C.c_int64 * max(n, 1))(*[e[2] for e in events])
+    out = (C.c_int64 * 2048)()
+    m = lib().dnncPlanFreeList(n, kind, ids, byt, upto, out, 1024)
+    return [(out[2 * i], out[2 * i + 1]) for i in range(m)]
+
+
+class Graph:
+    """An ONNX-level graph: named tensors, constants, nodes with ONNX operator names."""
+
+    def __init__(self):
+        self._g = lib().dnncGraphCreate()
+        self._n = 0
+        # Python-side mirror of what was added, for inspection and for
+        # evaluating the same graph with another engine
+        self.input_shapes = {}
+        self.constants = {}
+        self.nodes = []
+        self.outputs = []
+
+    def __del__(self):
+        if getattr(self, "_g", None):
+            lib().dnncGraphDestroy(self._g)
+            self._g = None
+
+    def _name(self, prefix):
+        self._n += 1
+        return f"{prefix}_{self._n}"
+
+    def input(self, name, shape, dtype=np.float32):
+        d = _abi.dims(shape)
+        if lib().dnncGraphAddInput(self._g, name.encode(), _DT[np.dtype(dtype)], len(shape), d):
+            raise RuntimeError(_err())
+        self.input_shapes[name] = (tuple(shape), np.dtype(dtype))
+        return name
+
+    def constant(self, array, name=None):
+        a = np.ascontiguousarray(array)
+        name = name or self._name("const")
+        d = _abi.dims(a.shape)
+        if lib().dnncGraphAddConstant(self._g, name.encode(), _DT[a.dtype], a.ndim, d, a.ctypes.data):
+            raise RuntimeError(_err())
+        self.constants[name] = a
+        return name
+
+    def node(self, op_type, inputs, name=None, **attrs):
+        out = name or self._name(op_type.lower())
+        arr = (C.c_char_p * max(len(inputs), 1))(*[(i or "").encode() for i in inputs])
+        parts = []
+        for k, v in attrs.items():
+            if isinstance(v, float):
+                parts.append(f"{k}={v!r}")  # repr of a float always has '.', 'e', 'inf' or 'nan'
+            elif isinstance(v, (list, tuple)):
+                parts.append(f"{k}=" + ",".join(str(int(x)) for x in v))
+            else:
+                parts.append(f"{k}={int(v)}")
+        if lib().dnncGraphAddNode(self._g, op_type.encode(), len(inputs), arr, out.encode(), ";".join(parts).encode()):
+            raise RuntimeError(_err())
+        self.nodes.append((op_type, list(inputs), out, dict(attrs)))
+        return out
+
+    def output(self, name):
+        if lib().dnncGraphAddOutput(self._g, name.encode()):
+            raise RuntimeError(_err())
+        self.outputs.append(name)
+
+    def compile(self, fusion=False, dealloc_opt=True, pool_opt=True, const_at_use=True, channels_last=False):
+        opt = _Options(int(const_at_use), int(fusion), int(dealloc_opt), int(pool_opt), int(channels_last))
+        p = lib().dnncCompile(self._g, C.byref(opt))
+        if not p:
+            raise RuntimeError("compile: " + _err())
+        return Program(p, self)
+
+
+class Program:
+    def __init__(self, handle, graph):
+        self._p = handle
+        self._graph = graph  # owns the constants the program points at
+
+    def __del__(self):
+        if getattr(self, "_p", None):
+            lib().dnncProgramDestroy(self._p)
+            self._p = None
+
+    @property
+    def text(self):
+        return lib().dnncProgramText(self._p).decode()
+
+    @property
+    def pool_bytes(self):
+        return lib().dnncProgramPoolBytes(self._p)
+
+    @property
+    def pool_extent(self):
+        return lib().dnncProgramPoolExtent(self._p)
+
+    def num_ops(self, compute_only=False):
+        return lib().dnncProgramNumOps(self._p, int(compute_only))
+
+    def events(self):
+        """[(kind, id, bytes, offset)] in execution order."""
+        n = lib().dnncProgramEvents(self._p, None, None, None, None, 0)
+        kind = (C.c_int32 * max(n, 1))()
+        ids, byt, off = (C.c_int64 * max(n, 1))(), (C.c_int64 * max(n, 1))(), (C.c_int64 * max(n, 1))()
+        lib().dnncProgramEvents(self._p, kind, ids, byt, off, n)
+        return [(kind[i], ids[i], byt[i], off[i]) for i in range(n)]
+
+    def output_info(self):
+        out = []
+        for i in range(lib().dnncProgramNumOutputs(self._p)):
+            dt, rank, d = C.c_int32(), C.c_int32(), (C.c_int64 * 8)()
+            if lib().dnncProgramOutputInfo(self._p, i, C.byref(dt), C.byref(rank), d):
+                raise RuntimeError(_err())
+            out.append((tuple(d[:rank.value]), _NP[dt.value]))
+        return out
+
+    def session(self, mode=MODE_OCCAMY, runtime_library=None):
+        """Bind to a runtime.  The default, and the only one this package ever
+        chooses, is the gfx950 library; a missing build is an error."""
+        if runtime_library is None:
+            _abi.load_runtime()  # fail loudly when the HIP library is absent
+            runtime_library = _abi.RUNTIME_PATH
+        return Session(self, runtime_library, mode)
+
+
+class Session:
+    def __init__(self, program, runtime_library, mode):
+        self.program = program
+        self.mode = mode
+        self._s = lib().dnncSessionCreate(program._p, runtime_library.encode(), mode)
+        if not self._s:
+            raise RuntimeError("session: " + _err())
+        self._out_info = program.output_info()
+
+    def close(self):
+        if getattr(self, "_s", None):
+            lib().dnncSessionDestroy(self._s)
+            self._s = None
+
+    def __del__(self):
+        self.close()
+
+    def run(self, *inputs):
+        """Host arrays in, host arrays out (the reference's ``sess.run``)."""
+        ins = [np.ascontiguousarray(a) for a in inputs]
+        outs = [np.empty(s, d) for s, d in self._out_info]
+        ip = (C.c_void_p * max(len(ins), 1))(*[a.ctypes.data for a in ins])
+        op = (C.c_void_p * max(len(outs), 1))(*[a.ctypes.data for a in outs])
+        if lib().dnncSessionRun(self._s, ip, op):
+            raise RuntimeError("run: " + _err())
+        return outs
+
+    def run_device(self, in_ptrs, out_ptrs, use_graph=True):
+        """Resident mode: device addresses in and out; returns without waiting."""
+        ip = (C.c_void_p * max(len(in_ptrs), 1))(*in_ptrs)
+        op = (C.c_void_p * max(len(out_ptrs), 1))(*out_ptrs)
+        if lib().dnncSessionRunResident(self._s, ip, op, 1, int(use_graph)):
+            raise RuntimeError("run_device: " + _err())
+
+    def sync(self):
+        if lib().dnncSessionSync(self._s):
+            raise RuntimeError("sync: " + _err())
+
+    @property
+    def weights_bytes(self):
+        return lib().dnncSessionWeightsBytes(self._s)
+
+    @property
+    def last_pool_bytes(self):
+        return lib().dnncSessionLastPoolBytes(self._s)

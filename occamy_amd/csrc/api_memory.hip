@@ -90,6 +90,35 @@ int32_t dnnrtSync(dnnrtHandle_t handle) {
   return 0;
 }
 
+int32_t dnnrtGraphBegin(dnnrtHandle_t handle) {
+  if (!handle || !handle->stream) { set_error("dnnrtGraphBegin: the handle needs a stream of its own"); return 1; }
+  HIP_RET(hipStreamBeginCapture(handle->stream, hipStreamCaptureModeThreadLocal), "dnnrtGraphBegin");
+  return 0;
+}
+
+int32_t dnnrtGraphEnd(dnnrtHandle_t handle, void **graph) {
+  if (!handle || !graph) { set_error("dnnrtGraphEnd: bad arguments"); return 1; }
+  hipGraph_t g = nullptr;
+  HIP_RET(hipStreamEndCapture(handle->stream, &g), "dnnrtGraphEnd: hipStreamEndCapture");
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (e != hipSuccess) { set_error("dnnrtGraphEnd: hipGraphInstantiate: %s", hipGetErrorString(e)); return (int32_t)e; }
+  *graph = exec;
+  return 0;
+}
+
+int32_t dnnrtGraphLaunch(dnnrtHandle_t handle, void *graph) {
+  if (!handle || !graph) { set_error("dnnrtGraphLaunch: bad arguments"); return 1; }
+  HIP_RET(hipGraphLaunch((hipGraphExec_t)graph, handle->stream), "dnnrtGraphLaunch");
+  return 0;
+}
+
+int32_t dnnrtGraphDestroy(void *graph) {
+  if (graph) HIP_RET(hipGraphExecDestroy((hipGraphExec_t)graph), "dnnrtGraphDestroy");
+  return 0;
+}
+
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
   if (!pool || bytes < 0) { set_error("dnnrtMemPoolInit: bad arguments"); return 1; }
   HIP_RET(hipMalloc(pool, (size_t)(bytes > 0 ? bytes : 1)), "dnnrtMemPoolInit: hipMalloc");

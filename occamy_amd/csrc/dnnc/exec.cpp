@@ -1,0 +1,385 @@
+// Executor: walks a compiled DNN program and issues one runtime call per
+// operation, which is what the reference's DNN-to-LLVM lowering turns the
+// program into (src/Conversion/DNNToLLVM/Ops/** build the dims arrays, pass
+// raw device pointers and call the row of DNNAPISpecs.inc).  The runtime is
+// bound at run time from a shared object that exports include/dnnrt.h.
+//
+// Two ways of running a program:
+//   occamy   - the reference's semantics per inference: create the pool,
+//              upload every constant into its pool slot, run, copy results
+//              back, wait, release the pool
+//              (src/Transform/DNN/mallocPoolOpt.hpp:239-265,
+//               src/Conversion/ONNXToDNN/Ops/Constant.cpp:86-90).
+//   resident - the pool and a second arena holding all constants are created
+//              once; an inference is input copy + kernels + output copy, and
+//              the kernels can be replayed from a captured graph.
+#include "exec.h"
+
+#include <dlfcn.h>
+
+#include <algorithm>
+#include <cstring>
+
+namespace dnnc {
+
+#define LOAD(name)                                                            \
+  do {                                                                         \
+    *(void **)(&rt.name) = dlsym(rt.dl, #name);                                \
+    if (!rt.name) { err = std::string("runtime library lacks ") + #name; return false; } \
+  } while (0)
+
+bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
+  rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
+  if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
+  LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
+  LOAD(dnnrtGraphDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
+  LOAD(dnnrtMalloc); LOAD(dnnrtDealloc); LOAD(dnnrtHostAlloc); LOAD(dnnrtHostFree);
+  LOAD(dnnrtConv); LOAD(dnnrtConvBiasActiv); LOAD(dnnrtActive); LOAD(dnnrtTensorOp); LOAD(dnnrtClip);
+  LOAD(dnnrtErf); LOAD(dnnrtNegative); LOAD(dnnrtReciprocal); LOAD(dnnrtPow); LOAD(dnnrtCastI64toFloat);
+  LOAD(dnnrtGelu); LOAD(dnnrtReduce); LOAD(dnnrtSoftmax); LOAD(dnnrtLayerNorm); LOAD(dnnrtMaxPool);
+  LOAD(dnnrtAveragePool); LOAD(dnnrtMatmul2d); LOAD(dnnrtMatmulNd); LOAD(dnnrtFlatten);
+  LOAD(dnnrtReshape); LOAD(dnnrtTranspose); LOAD(dnnrtGather);
+  return true;
+}
+#undef LOAD
+
+static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+Session::~Session() {
+  if (!rt.dl) return;
+  if (graph) rt.dnnrtGraphDestroy(graph);
+  if (handle) rt.dnnrtSync(handle);
+  if (pool) rt.dnnrtDealloc(pool);
+  if (weights) rt.dnnrtDealloc(weights);
+  for (auto &kv : host_const) rt.dnnrtHostFree(kv.second);
+  for (void *p : host_out) rt.dnnrtHostFree(p);
+  for (void *p : host_in) rt.dnnrtHostFree(p);
+  if (handle) rt.dnnrtDestroy(handle);
+  if (stream) rt.dnnrtStreamDestroy(stream);
+}
+
+std::string Session::rt_error(const char *what) const {
+  return std::string(what) + ": " + rt.dnnrtLastError();
+}
+
+// KCRS -> KRSC, element size es
+static void permute_kcrs_to_krsc(const uint8_t *src, uint8_t *dst, const Shape &w, int64_t es) {
+  const int64_t K = w[0], C = w[1], R = w[2], S = w[3];
+  for (int64_t k = 0; k < K; k++)
+    for (int64_t c = 0; c < C; c++)
+      for (int64_t r = 0; r < R; r++)
+        for (int64_t s = 0; s < S; s++)
+          std::memcpy(dst + (((k * R + r) * S + s) * C + c) * es, src + (((k * C + c) * R + r) * S + s) * es, (size_t)es);
+}
+
+bool Session::init(const Program *p, const std::string &runtime_path, int mode_, std::string &err) {
+  prog = p;
+  mode = mode_;
+  if (prog->pool_bytes < 0) { err = "the program was compiled without the pool pass"; return false; }
+  if (!load_runtime(runtime_path, rt, err)) return false;
+  host_backend = rt.dnnrtIsHostBackend() != 0;
+  if (prog->channels_last && host_backend) { err = "channels-last programs need the GPU runtime"; return false; }
+  if (rt.dnnrtCreate(&handle)) { err = rt_error("dnnrtCreate"); return false; }
+  if (rt.dnnrtStreamCreate(&stream)) { err = rt_error("dnnrtStreamCreate"); return false; }
+  if (rt.dnnrtSetStream(handle, stream)) { err = rt_error("dnnrtSetStream"); return false; }
+  ptr.assign(prog->value_store.size(), nullptr);
+
+  // Which constants are convolution filters (they are stored K,R,S,C for a
+  // channels-last program).
+  std::map<std::string, bool> is_filter;
+  if (prog->channels_last)
+    for (const Op *op : prog->ops)
+      if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV) {
+        const Value *w = op->operands[1];
+        if (w->def && w->def->kind == OP_MEM_OFFSET)
+          for (const auto &u : w->uses)
+            if (u.first->kind == OP_MEMCPY && u.first->operands[1]->def &&
+                u.first->operands[1]->def->kind == OP_HOST_CONST)
+              is_filter[u.first->operands[1]->def->const_name] = true;
+      }
+
+  // Constants: one pinned host copy each (the reference keeps them as globals
+  // of the model library); function results: one pinned buffer each.
+  int64_t weight_bytes = 0;
+  for (const Op *op : prog->ops) {
+    if (op->kind == OP_HOST_CONST) {
+      const GTensor &t = prog->graph->tensors.at(op->const_name);
+      void *h = nullptr;
+      if (rt.dnnrtHostAlloc(&h, (int64_t)t.data.size())) { err = rt_error("dnnrtHostAlloc"); return false; }
+      if (is_filter.count(op->const_name) && t.shape.size() == 4)
+        permute_kcrs_to_krsc(t.data.data(), (uint8_t *)h, t.shape, dtype_bytes(t.dtype));
+      else
+        std::memcpy(h, t.data.data(), t.data.size());
+      host_const[op->const_name] = h;
+      ptr[(size_t)op->result->id] = h;
+      weight_bytes += align_up((int64_t)t.data.size(), 256);
+    } else if (op->kind == OP_HOST_ALLOC) {
+      void *h = nullptr;
+      if (rt.dnnrtHostAlloc(&h, op->bytes)) { err = rt_error("dnnrtHostAlloc"); return false; }
+      if ((size_t)op->out_index >= host_out.size()) host_out.resize((size_t)op->out_index + 1, nullptr);
+      host_out[(size_t)op->out_index] = h;
+      ptr[(size_t)op->result->id] = h;
+    }
+  }
+  for (const Value *a : prog->args) {
+    void *h = nullptr;
+    if (rt.dnnrtHostAlloc(&h, shape_numel(a->shape) * dtype_bytes(a->dtype))) { err = rt_error("dnnrtHostAlloc"); return false; }
+    host_in.push_back(h);
+  }
+  weights_bytes = weight_bytes;
+
+  if (mode == MODE_RESIDENT) {
+    if (rt.dnnrtMemPoolInit(&pool, std::max(prog->pool_bytes, prog->pool_extent))) { err = rt_error("dnnrtMemPoolInit"); return false; }
+    if (rt.dnnrtMalloc(&weights, weight_bytes)) { err = rt_error("dnnrtMalloc(weights)"); return false; }
+    // Upload every constant once, into the weights arena; the pool slot the
+    // planner gave it stays unused.
+    int64_t woff = 0;
+    for (const Op *op : prog->ops) {
+      if (op->kind == OP_MEMPOOL_INIT) ptr[(size_t)op->result->id] = pool;
+      else if (op->kind == OP_MEM_OFFSET) ptr[(size_t)op->result->id] = (char *)pool + op->offset;
+    }
+    for (const Op *op : prog->ops) {
+      if (op->kind != OP_MEMCPY || op->mode != 1) continue;
+      const Value *src = op->operands[1];
+      if (!src->def || src->def->kind != OP_HOST_CONST) continue;
+      void *dev = (char *)weights + woff;
+      woff += align_up(op->bytes, 256);
+      if (rt.dnnrtMemcpy(dev, ptr[(size_t)src->id], op->bytes, 1, stream)) { err = rt_error("dnnrtMemcpy(constant)"); return false; }
+      ptr[(size_t)op->operands[0]->id] = dev;
+    }
+    if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
+  }
+  return true;
+}
+
+int Session::format_for(const Op *op) const {
+  if (!prog->channels_last) return 0;  // NCHW
+  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV) {
+    const Value *x = op->operands[0];
+    // the function argument's slot holds what the host sent: NCHW
+    const bool from_arg = x->def && x->def->kind == OP_MEM_OFFSET;
+    return from_arg ? 2 : 1;
+  }
+  return 1;
+}
+
+// One compute operation -> one runtime call.
+bool Session::issue(const Op *op, std::string &err) {
+  auto P = [&](size_t i) { return ptr[(size_t)op->operands[i]->id]; };
+  void *out = op->operands.empty() ? nullptr : P(op->operands.size() - 1);
+  const Value *ov = op->operands.empty() ? nullptr : op->operands.back();
+  const int dt = ov ? (int)ov->dtype : 0;
+  if (prog->channels_last || cur_format != 0) {
+    const int f = format_for(op);
+    if (f != cur_format) {
+      if (rt.dnnrtSetTensorFormat(handle, f)) { err = rt_error("dnnrtSetTensorFormat"); return false; }
+      cur_format = f;
+    }
+  }
+  void *r = nullptr;
+  auto pad4 = [](const Shape &s) { Shape o = s; while (o.size() < 4) o.push_back(1); return o; };
+  switch (op->kind) {
+    case OP_CONVFWD:
+      r = rt.dnnrtConv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), 0, op->algo, op->group,
+                       op->pads.data(), op->strides.data(), out, dt);
+      break;
+    case OP_CONV_BIAS_ACTIV: {
+      const int64_t dimB[4] = {1, op->dimB[0], 1, 1};
+      r = rt.dnnrtConvBiasActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, P(3), 0, 1,
+                                op->group, op->pads.data(), op->strides.data(), op->mode, out, dt);
+      break;
+    }
+    case OP_ACTIVATION: {
+      const Shape d = pad4(op->dimA);  // the lowering pads the dims to 4 with trailing ones
+      if (d.size() > 4) {
+        const int64_t flat[4] = {shape_numel(op->dimA), 1, 1, 1};
+        r = rt.dnnrtActive(handle, P(0), flat, (int32_t)op->mode, out, dt);
+      } else {
+        r = rt.dnnrtActive(handle, P(0), d.data(), (int32_t)op->mode, out, dt);
+      }
+      break;
+    }
+    case OP_ADD:
+    case OP_MUL: {
+      const int32_t rank = (int32_t)op->dimA.size();
+      r = rt.dnnrtTensorOp(handle, op->kind == OP_ADD ? 0 : 1, P(0), op->dimA.data(), rank, P(1), op->dimB.data(),
+                           rank, out, op->dimA.data(), rank, op->coef, dt);
+      break;
+    }
+    case OP_SQRT: {
+      const int32_t rank = (int32_t)op->dimA.size();
+      r = rt.dnnrtTensorOp(handle, 4, P(0), op->dimA.data(), rank, nullptr, op->dimA.data(), rank, out,
+                           op->dimA.data(), rank, 1.f, dt);
+      break;
+    }
+    case OP_NEGATIVE: r = rt.dnnrtNegative(handle, P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
+    case OP_RECIPROCAL: r = rt.dnnrtReciprocal(handle, P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
+    case OP_ERF: r = rt.dnnrtErf(handle, P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
+    case OP_GELU: r = rt.dnnrtGelu(handle, P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
+    case OP_POW: r = rt.dnnrtPow(handle, P(0), P(1), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
+    case OP_CLIP: r = rt.dnnrtClip(handle, P(0), out, op->dimA.data(), op->lo, op->hi, (int64_t)op->dimA.size(), dt); break;
+    case OP_CAST:
+      r = rt.dnnrtCastI64toFloat(handle, (const int64_t *)P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt);
+      break;
+    case OP_REDUCE:
+      r = rt.dnnrtReduce(handle, (int32_t)op->dimA.size(), P(0), op->dimA.data(), out, op->dimOut.data(),
+                         (int32_t)op->mode, dt);
+      break;
+    case OP_MAXPOOL:
+      r = rt.dnnrtMaxPool(handle, P(0), op->dimA.data(), out, op->dimOut.data(), op->kernel.data(), op->pads.data(),
+                          op->strides.data(), dt);
+      break;
+    case OP_AVGPOOL:
+      r = rt.dnnrtAveragePool(handle, P(0), op->dimA.data(), out, op->dimOut.data(), op->kernel.data(),
+                              op->pads.data(), op->strides.data(), dt);
+      break;
+    case OP_SOFTMAX:
+      r = rt.dnnrtSoftmax(handle, P(0), op->dimA.data(), out, op->dimA.data(), op->axis, (int64_t)op->dimA.size(), dt);
+      break;
+    case OP_LAYERNORM:
+      r = rt.dnnrtLayerNorm(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), P(1), P(2), op->eps, out, dt);
+      break;
+    case OP_FLATTEN:
+      r = rt.dnnrtFlatten(handle, P(0), op->dimA.data(), out, op->dimOut.data(), (int32_t)op->axis,
+                          (int64_t)op->dimA.size(), dt);
+      break;
+    case OP_RESHAPE: r = rt.dnnrtReshape(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), out, dt); break;
+    case OP_TRANSPOSE:
+      r = rt.dnnrtTranspose(handle, P(0), op->dimA.data(), out, op->dimOut.data(), op->perm.data(),
+                            (int64_t)op->dimA.size(), dt);
+      break;
+    case OP_GATHER:
+      r = rt.dnnrtGather(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), out, op->dimOut.data(),
+                         (int64_t)op->dimOut.size(), (const int64_t *)P(1), op->dimB.data(), (int64_t)op->dimB.size(),
+                         op->axis, dt);
+      break;
+    case OP_MATMUL2D:
+      r = rt.dnnrtMatmul2d(handle, 2, P(0), op->dimA.data(), P(1), op->dimB.data(), out, op->dimOut.data(), out,
+                           op->dimOut.data(), op->alpha, op->beta, op->trans_a, op->trans_b, dt);
+      break;
+    case OP_MATMULND:
+      r = rt.dnnrtMatmulNd(handle, P(0), op->dimA.data(), (int32_t)op->dimA.size(), P(1), op->dimB.data(),
+                           (int32_t)op->dimB.size(), out, op->dimOut.data(), (int32_t)op->dimOut.size(), dt);
+      break;
+    default: err = std::string("executor: unexpected op ") + op_name(op->kind); return false;
+  }
+  if (!r) { err = std::string(op_name(op->kind)) + ": " + rt.dnnrtLastError(); return false; }
+  ptr[(size_t)op->result->id] = r;
+  return true;
+}
+
+static bool is_compute(OpKind k) { return k >= OP_CONVFWD && k <= OP_GELU; }
+
+// The reference's per-inference sequence, call for call.
+bool Session::run_occamy(const void *const *inputs, void *const *outputs, std::string &err) {
+  void *run_pool = nullptr;
+  for (size_t i = 0; i < prog->args.size(); i++) {
+    std::memcpy(host_in[i], inputs[i], (size_t)(shape_numel(prog->args[i]->shape) * dtype_bytes(prog->args[i]->dtype)));
+    ptr[(size_t)prog->args[i]->id] = host_in[i];
+  }
+  bool ok = true;
+  for (const Op *op : prog->ops) {
+    switch (op->kind) {
+      case OP_MEMPOOL_INIT:
+        if (rt.dnnrtMemPoolInit(&run_pool, op->bytes)) { err = rt_error("dnnrtMemPoolInit"); ok = false; }
+        ptr[(size_t)op->result->id] = run_pool;
+        last_pool_bytes = op->bytes;
+        break;
+      case OP_MEM_OFFSET: {
+        void *q = nullptr;
+        if (rt.dnnrtMemOffset(&q, ptr[(size_t)op->operands[0]->id], op->offset, op->bytes)) { err = rt_error("dnnrtMemOffset"); ok = false; }
+        ptr[(size_t)op->result->id] = q;
+        break;
+      }
+      case OP_MEMCPY:
+        if (rt.dnnrtMemcpy(ptr[(size_t)op->operands[0]->id], ptr[(size_t)op->operands[1]->id], op->bytes, (int32_t)op->mode, stream)) {
+          err = rt_error("dnnrtMemcpy"); ok = false;
+        }
+        break;
+      case OP_DEALLOC:  // only the pool's own release survives the pool pass
+        if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); ok = false; }
+        if (rt.dnnrtDealloc(ptr[(size_t)op->operands[0]->id])) { err = rt_error("dnnrtDealloc"); ok = false; }
+        run_pool = nullptr;
+        break;
+      case OP_HOST_CONST: case OP_HOST_ALLOC: case OP_RETURN: break;
+      default: ok = issue(op, err); break;
+    }
+    if (!ok) break;
+  }
+  if (!ok) {
+    rt.dnnrtSync(handle);
+    if (run_pool) rt.dnnrtDealloc(run_pool);
+    return false;
+  }
+  const Op *ret = prog->ops.back();
+  for (size_t i = 0; i < ret->operands.size(); i++) {
+    const Value *v = ret->operands[i];
+    std::memcpy(outputs[i], ptr[(size_t)v->id], (size_t)(shape_numel(v->shape) * dtype_bytes(v->dtype)));
+  }
+  return true;
+}
+
+bool Session::issue_all_compute(std::string &err) {
+  for (const Op *op : prog->ops)
+    if (is_compute(op->kind) && !issue(op, err)) return false;
+  return true;
+}
+
+// Resident inference.  `on_device` != 0: inputs/outputs are device pointers and
+// the call returns without waiting (sync() does).
+bool Session::run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err) {
+  // 1. inputs into their pool slots
+  for (const Op *op : prog->ops) {
+    if (op->kind != OP_MEMCPY || op->mode != 1) continue;
+    const Value *src = op->operands[1];
+    if (src->arg_index < 0) continue;
+    const size_t ai = (size_t)src->arg_index;
+    const void *from = inputs[ai];
+    if (!on_device) { std::memcpy(host_in[ai], inputs[ai], (size_t)op->bytes); from = host_in[ai]; }
+    if (rt.dnnrtMemcpy(ptr[(size_t)op->operands[0]->id], const_cast<void *>(from), op->bytes, on_device ? 3 : 1, stream)) {
+      err = rt_error("dnnrtMemcpy(input)"); return false;
+    }
+  }
+  // 2. kernels
+  if (use_graph && !host_backend) {
+    if (!graph) {
+      // One eager pass first: it validates every call outside of capture.
+      if (!issue_all_compute(err)) return false;
+      if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
+      if (rt.dnnrtGraphBegin(handle)) { err = rt_error("dnnrtGraphBegin"); return false; }
+      const bool ok = issue_all_compute(err);
+      void *g = nullptr;
+      if (rt.dnnrtGraphEnd(handle, &g)) { if (ok) err = rt_error("dnnrtGraphEnd"); return false; }
+      if (!ok) { rt.dnnrtGraphDestroy(g); return false; }
+      graph = g;
+    }
+    if (rt.dnnrtGraphLaunch(handle, graph)) { err = rt_error("dnnrtGraphLaunch"); return false; }
+  } else {
+    if (!issue_all_compute(err)) return false;
+  }
+  // 3. outputs
+  for (const Op *op : prog->ops) {
+    if (op->kind != OP_MEMCPY || op->mode != 2) continue;
+    const Op *ha = op->operands[0]->def;
+    const size_t oi = (size_t)ha->out_index;
+    void *dst = on_device ? outputs[oi] : host_out[oi];
+    if (rt.dnnrtMemcpy(dst, ptr[(size_t)op->operands[1]->id], op->bytes, on_device ? 3 : 2, stream)) {
+      err = rt_error("dnnrtMemcpy(output)"); return false;
+    }
+  }
+  if (!on_device) {
+    if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
+    for (const Op *op : prog->ops)
+      if (op->kind == OP_HOST_ALLOC) std::memcpy(outputs[(size_t)op->out_index], host_out[(size_t)op->out_index], (size_t)op->bytes);
+  }
+  return true;
+}
+
+bool Session::sync(std::string &err) {
+  if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
+  return true;
+}
+
+}  // namespace dnnc

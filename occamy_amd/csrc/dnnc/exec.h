@@ -1,0 +1,92 @@
+#pragma once
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../../include/dnnrt.h"
+#include "ir.h"
+
+namespace dnnc {
+
+// The runtime's entry points, resolved by name from a shared object.
+struct RuntimeApi {
+  void *dl = nullptr;
+  decltype(&::dnnrtCreate) dnnrtCreate = nullptr;
+  decltype(&::dnnrtDestroy) dnnrtDestroy = nullptr;
+  decltype(&::dnnrtStreamCreate) dnnrtStreamCreate = nullptr;
+  decltype(&::dnnrtStreamDestroy) dnnrtStreamDestroy = nullptr;
+  decltype(&::dnnrtSetStream) dnnrtSetStream = nullptr;
+  decltype(&::dnnrtSetTensorFormat) dnnrtSetTensorFormat = nullptr;
+  decltype(&::dnnrtSync) dnnrtSync = nullptr;
+  decltype(&::dnnrtLastError) dnnrtLastError = nullptr;
+  decltype(&::dnnrtIsHostBackend) dnnrtIsHostBackend = nullptr;
+  decltype(&::dnnrtGraphBegin) dnnrtGraphBegin = nullptr;
+  decltype(&::dnnrtGraphEnd) dnnrtGraphEnd = nullptr;
+  decltype(&::dnnrtGraphLaunch) dnnrtGraphLaunch = nullptr;
+  decltype(&::dnnrtGraphDestroy) dnnrtGraphDestroy = nullptr;
+  decltype(&::dnnrtMemPoolInit) dnnrtMemPoolInit = nullptr;
+  decltype(&::dnnrtMemOffset) dnnrtMemOffset = nullptr;
+  decltype(&::dnnrtMemcpy) dnnrtMemcpy = nullptr;
+  decltype(&::dnnrtMalloc) dnnrtMalloc = nullptr;
+  decltype(&::dnnrtDealloc) dnnrtDealloc = nullptr;
+  decltype(&::dnnrtHostAlloc) dnnrtHostAlloc = nullptr;
+  decltype(&::dnnrtHostFree) dnnrtHostFree = nullptr;
+  decltype(&::dnnrtConv) dnnrtConv = nullptr;
+  decltype(&::dnnrtConvBiasActiv) dnnrtConvBiasActiv = nullptr;
+  decltype(&::dnnrtActive) dnnrtActive = nullptr;
+  decltype(&::dnnrtTensorOp) dnnrtTensorOp = nullptr;
+  decltype(&::dnnrtClip) dnnrtClip = nullptr;
+  decltype(&::dnnrtErf) dnnrtErf = nullptr;
+  decltype(&::dnnrtNegative) dnnrtNegative = nullptr;
+  decltype(&::dnnrtReciprocal) dnnrtReciprocal = nullptr;
+  decltype(&::dnnrtPow) dnnrtPow = nullptr;
+  decltype(&::dnnrtCastI64toFloat) dnnrtCastI64toFloat = nullptr;
+  decltype(&::dnnrtGelu) dnnrtGelu = nullptr;
+  decltype(&::dnnrtReduce) dnnrtReduce = nullptr;
+  decltype(&::dnnrtSoftmax) dnnrtSoftmax = nullptr;
+  decltype(&::dnnrtLayerNorm) dnnrtLayerNorm = nullptr;
+  decltype(&::dnnrtMaxPool) dnnrtMaxPool = nullptr;
+  decltype(&::dnnrtAveragePool) dnnrtAveragePool = nullptr;
+  decltype(&::dnnrtMatmul2d) dnnrtMatmul2d = nullptr;
+  decltype(&::dnnrtMatmulNd) dnnrtMatmulNd = nullptr;
+  decltype(&::dnnrtFlatten) dnnrtFlatten = nullptr;
+  decltype(&::dnnrtReshape) dnnrtReshape = nullptr;
+  decltype(&::dnnrtTranspose) dnnrtTranspose = nullptr;
+  decltype(&::dnnrtGather) dnnrtGather = nullptr;
+};
+
+bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err);
+
+enum { MODE_OCCAMY = 0, MODE_RESIDENT = 1 };
+
+class Session {
+ public:
+  ~Session();
+  bool init(const Program *p, const std::string &runtime_path, int mode, std::string &err);
+  bool run_occamy(const void *const *inputs, void *const *outputs, std::string &err);
+  bool run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err);
+  bool sync(std::string &err);
+
+  const Program *prog = nullptr;
+  int mode = MODE_OCCAMY;
+  int64_t weights_bytes = 0;     // bytes of the constants arena (resident mode)
+  int64_t last_pool_bytes = -1;  // bytes the last occamy-mode run asked the runtime for
+
+ private:
+  RuntimeApi rt;
+  dnnrtHandle_t handle = nullptr;
+  dnnrtStream_t stream = nullptr;
+  bool host_backend = false;
+  int cur_format = 0;
+  void *pool = nullptr, *weights = nullptr, *graph = nullptr;
+  std::vector<void *> ptr;  // value id -> address (host or device)
+  std::map<std::string, void *> host_const;
+  std::vector<void *> host_out, host_in;
+
+  std::string rt_error(const char *what) const;
+  int format_for(const Op *op) const;
+  bool issue(const Op *op, std::string &err);
+  bool issue_all_compute(std::string &err);
+};
+
+}  // namespace dnnc

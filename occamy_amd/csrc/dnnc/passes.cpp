@@ -1,0 +1,164 @@
+// DNN-level passes: conv+bias(+relu) fusion, dealloc placement by last use,
+// and the memory-pool rewrite.  Each restates one pass of the reference:
+//   src/Transform/DNN/opFusing/fuseConvBiasRelu.cpp:35-152
+//   src/Transform/DNN/DNNDeallocOpt.cpp:26-45
+//   src/Transform/DNN/mallocPoolOpt.cpp:41-80 (+ mallocPoolOpt.hpp:239-265)
+#include "ir.h"
+#include "planner.h"
+
+#include <algorithm>
+
+namespace dnnc {
+
+// conv -> add(bias) [-> relu] becomes one conv-bias-relufwd.  With a ReLU the
+// fused op writes the ReLU's buffer and the convolution's own buffer (malloc
+// and dealloc) disappears; without, it writes the convolution's buffer.
+// Unlike the reference the fused op keeps `group`.
+void fuse_conv_bias_activ(Program &p) {
+  std::vector<Op *> convs;
+  for (Op *op : p.ops)
+    if (op->kind == OP_CONVFWD) convs.push_back(op);
+  for (Op *conv : convs) {
+    // every user of the convolution's result must be a dnn.add
+    if (conv->result->uses.empty()) continue;
+    Op *add = nullptr;
+    bool ok = true;
+    for (const auto &u : conv->result->uses) {
+      if (u.first->kind != OP_ADD) { ok = false; break; }
+      add = u.first;
+    }
+    if (!ok || !add) continue;
+    // the add must be the bias add emitted with the convolution: A is the
+    // conv result, the output buffer is the conv's buffer, B is [1,K,1,1]
+    if (add->operands[0] != conv->result || add->operands[2] != conv->operands[3]) continue;
+    if (add->dimB.size() != 4 || add->dimB[0] != 1 || add->dimB[2] != 1 || add->dimB[3] != 1) continue;
+    // first user of the add decides: ReLU -> CONVBIASRELU, anything else -> CONVBIAS
+    Op *relu = nullptr;
+    if (!add->result->uses.empty()) {
+      Op *u0 = add->result->uses.front().first;
+      if (u0->kind == OP_ACTIVATION && u0->mode == 1 && u0->operands[0] == add->result) relu = u0;
+    }
+    // fusing the ReLU away is only sound when nothing else reads the un-activated value
+    if (relu && add->result->uses.size() != 1) relu = nullptr;
+
+    Value *x = conv->operands[0], *w = conv->operands[1], *ws = conv->operands[2], *bias = add->operands[1];
+    Value *out = relu ? relu->operands[1] : conv->operands[3];
+    Op *fused = p.new_op(OP_CONV_BIAS_ACTIV);
+    fused->pads = conv->pads;
+    fused->strides = conv->strides;
+    fused->group = conv->group;
+    fused->dimA = conv->dimA;
+    fused->dimB = conv->dimB;
+    fused->mode = relu ? 1 : 5;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    p.insert_after(fused, out->def);  // right behind the malloc it writes
+    p.set_operands(fused, {x, w, bias, ws, out});
+    if (relu) {
+      p.replace_all_uses(relu->result, fused->result);
+      Value *dead_buf = conv->operands[3];
+      Op *dead_malloc = dead_buf->def;
+      p.erase(relu);
+      p.erase(add);
+      p.erase(conv);
+      std::vector<Op *> deallocs;
+      for (const auto &u : dead_buf->uses)
+        if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+      for (Op *d : deallocs) p.erase(d);
+      if (dead_buf->uses.empty()) p.erase(dead_malloc);
+    } else {
+      p.replace_all_uses(add->result, fused->result);
+      p.erase(add);
+      p.erase(conv);
+    }
+  }
+}
+
+// Each dealloc (visited in block order, i.e. creation order of the parked
+// deallocs) is moved to just after its tensor's last use.  If the last direct
+// user writes the tensor (the malloc is that op's last operand), the tensor
+// lives on under the op's result, and the dealloc goes after the result's last
+// user instead.  One level of aliasing only, as in the reference.
+void dealloc_opt(Program &p) {
+  std::vector<Op *> deallocs;
+  for (Op *op : p.ops)
+    if (op->kind == OP_DEALLOC) deallocs.push_back(op);
+  for (Op *d : deallocs) {
+    Value *buf = d->operands[0];
+    Op *m = buf->def;
+    if (!m) continue;
+    p.move_after(d, m);
+    Op *ldu = p.last_user(buf);
+    if (!ldu || ldu == d) continue;  // nothing but the dealloc uses it
+    // dnn.memcpy carries its byte count as last operand in the reference, so
+    // it never counts as "writes its last operand"
+    const bool writes = ldu->kind != OP_MEMCPY && !ldu->operands.empty() && ldu->operands.back() == buf;
+    if (writes && ldu->result) {
+      Op *last = p.last_user(ldu->result);
+      p.move_after(d, last ? last : ldu);
+    } else {
+      p.move_after(d, ldu);
+    }
+  }
+}
+
+std::vector<PoolEvent> pool_events(const Program &p) {
+  std::vector<PoolEvent> ev;
+  for (const Op *op : p.ops) {
+    if (op->kind == OP_MALLOC)
+      ev.push_back({0, op->result->id, shape_numel(op->result->shape) * dtype_bytes(op->result->dtype), -1});
+    else if (op->kind == OP_DEALLOC && op->operands[0]->def && op->operands[0]->def->kind == OP_MALLOC)
+      ev.push_back({1, op->operands[0]->id, 0, -1});
+  }
+  return ev;
+}
+
+// Every malloc becomes mem-offset(pool, offset, size) with the offset the
+// simulator assigns; all deallocs go; the pool is created once near the top
+// and released in front of the terminator.
+bool malloc_pool_opt(Program &p, std::string &err) {
+  PoolSimulator sim;
+  Op *init = p.new_op(OP_MEMPOOL_INIT);
+  init->result = p.new_value(F32, {1});
+  init->result->def = init;
+  p.insert_before(init, p.ops.front());  // ahead of every mem-offset that will refer to it
+  std::vector<Op *> mallocs, deallocs;
+  for (Op *op : p.ops) {
+    if (op->kind == OP_MALLOC) {
+      const int64_t size = PoolSimulator::round_size(shape_numel(op->result->shape) * dtype_bytes(op->result->dtype));
+      const int64_t off = sim.reserve(op->result->id, size);
+      if (off < 0) { err = "pool simulator ran out of address space"; return false; }
+      p.trace.push_back({0, op->result->id, shape_numel(op->result->shape) * dtype_bytes(op->result->dtype), off});
+      op->offset = off;
+      op->bytes = size;
+      mallocs.push_back(op);
+    } else if (op->kind == OP_DEALLOC) {
+      if (!sim.release(op->operands[0]->id)) { err = "dealloc of a tensor that is not live"; return false; }
+      p.trace.push_back({1, op->operands[0]->id, 0, -1});
+      deallocs.push_back(op);
+    }
+  }
+  for (Op *m : mallocs) {
+    m->kind = OP_MEM_OFFSET;
+    p.set_operands(m, {init->result});
+  }
+  for (Op *d : deallocs) p.erase(d);
+  Op *release = p.new_op(OP_DEALLOC);
+  p.insert_before(release, p.terminator());
+  p.set_operands(release, {init->result});
+  // The reference takes the pool size from the start of the LAST free block.
+  // When an empty (0-byte) tensor is released while it lies inside a free
+  // region, its degenerate block is appended behind the unbounded tail block
+  // and that reading goes stale (too small).  Traces the emission rules
+  // produce never do this (a convolution's empty workspace is released while
+  // its output, at the same address, is live), but the executor must never
+  // under-allocate, so the arena also covers the highest planned byte.
+  int64_t extent = 0;
+  for (Op *m : mallocs) extent = std::max(extent, m->offset + m->bytes);
+  p.pool_bytes = sim.peak();
+  p.pool_extent = extent;
+  init->bytes = std::max(sim.peak(), extent);
+  return true;
+}
+
+}  // namespace dnnc

@@ -121,6 +121,17 @@ static int64_t esize(int32_t dtype) {
   return dtype == DNNRT_F32 ? 4 : dtype == DNNRT_F16 ? 2 : dtype == DNNRT_I64 ? 8 : 0;
 }
 
+// Plain copy, 16 bytes per lane where both pointers allow it.  A kernel rather
+// than a memcpy call so that a captured graph holds kernel nodes only.
+__global__ __launch_bounds__(256) void copy16_kernel(const uint4 *__restrict__ x, uint4 *__restrict__ y, int64_t n16) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) y[i] = x[i];
+}
+__global__ __launch_bounds__(256) void copy1_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ y, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) y[i] = x[i];
+}
+
 static void *copy_entry(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rank,
                         void *Y, int32_t dtype) {
   if (!h) DNNRT_FAIL("%s: null handle", who);
@@ -131,8 +142,15 @@ static void *copy_entry(const char *who, dnnrtHandle_t h, const void *X, const i
     DNNRT_FAIL("%s: a channels-last tensor with spatial extent cannot be re-viewed by a copy", who);
   const int64_t bytes = numel(dX, rank) * es;
   if (bytes > 0 && X != Y) {
-    hipError_t e = hipMemcpyAsync(Y, X, (size_t)bytes, hipMemcpyDeviceToDevice, h->stream);
-    if (e != hipSuccess) DNNRT_FAIL("%s: %s", who, hipGetErrorString(e));
+    const int64_t n16 = (aligned16(X) && aligned16(Y)) ? bytes / 16 : 0, tail = bytes - n16 * 16;
+    if (ceil_div(bytes, 256) > INT32_MAX) DNNRT_FAIL("%s: tensor too large", who);
+    if (n16 > 0)
+      hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)ceil_div(n16, 256)), dim3(256), 0, h->stream,
+                         (const uint4 *)X, (uint4 *)Y, n16);
+    if (tail > 0)
+      hipLaunchKernelGGL(copy1_kernel, dim3((unsigned)ceil_div(tail, 256)), dim3(256), 0, h->stream,
+                         (const uint8_t *)X + n16 * 16, (uint8_t *)Y + n16 * 16, tail);
+    DNNRT_CHECK_LAUNCH(who);
   }
   return Y;
 }

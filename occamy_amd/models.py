@@ -1,0 +1,184 @@
+"""Graph builders for the benchmark configurations: the ONNX graphs a PyTorch
+export of these models gives (node vocabulary and order as in the reference's
+test/models/*/run.py flows), with seeded synthetic weights.
+
+Each builder returns ``(Graph, [input arrays])``.  BatchNorm is folded into
+the convolution bias, as onnx-mlir's ONNX-level rewrites leave it before the
+reference's own passes run.
+"""
+import numpy as np
+
+from . import rng
+from .compiler import Graph
+
+
+class _Init:
+    """Hands out seeded tensors; every tensor gets its own stream number."""
+
+    def __init__(self, seed, dtype):
+        self.seed, self.dtype, self.stream = seed, dtype, 0
+
+    def _next(self):
+        self.stream += 1
+        return self.stream
+
+    def he_normal(self, shape):
+        fan_in = int(np.prod(shape[1:]))
+        return rng.normal(self.seed, self._next(), shape, std=np.sqrt(2.0 / fan_in)).astype(self.dtype)
+
+    def normal(self, shape, std):
+        return rng.normal(self.seed, self._next(), shape, std=std).astype(self.dtype)
+
+    def uniform(self, shape, lo, hi):
+        return rng.uniform(self.seed, self._next(), shape, lo, hi).astype(self.dtype)
+
+
+def single_conv(dtype=np.float32, seed=1):
+    """Conv2d(3x3, 64->64, stride 1, pad 1) + bias + ReLU on 1x64x56x56."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x = rng.normal(seed, 0, (1, 64, 56, 56)).astype(dtype)
+    bound = float(np.sqrt(6.0 / (64 * 9)))  # Kaiming-uniform
+    g.input("X", x.shape, dtype)
+    w = g.constant(init.uniform((64, 64, 3, 3), -bound, bound), "W")
+    b = g.constant(init.uniform((64,), -0.1, 0.1), "B")
+    c = g.node("Conv", ["X", w, b], "conv", kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1], group=1)
+    r = g.node("Relu", [c], "relu")
+    g.output(r)
+    return g, [x]
+
+
+def _conv(g, init, x, cin, cout, k, stride, pad, group=1, bias=True):
+    w = g.constant(init.he_normal((cout, cin // group, k, k)))
+    ins = [x, w]
+    if bias:
+        ins.append(g.constant(init.uniform((cout,), -0.1, 0.1)))
+    return g.node("Conv", ins, kernel_shape=[k, k], pads=[pad] * 4, strides=[stride, stride], group=group)
+
+
+def resnet50(batch=1, dtype=np.float32, seed=2, image=224, classes=1000):
+    """ResNet-50 v1.5: bottlenecks [3,4,6,3], stride on the 3x3, folded BN."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x_np = rng.normal(seed, 0, (batch, 3, image, image)).astype(dtype)
+    g.input("input", x_np.shape, dtype)
+    x = _conv(g, init, "input", 3, 64, 7, 2, 3)
+    x = g.node("Relu", [x])
+    x = g.node("MaxPool", [x], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
+    cin = 64
+    for planes, blocks, stride in [(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)]:
+        for b in range(blocks):
+            s = stride if b == 0 else 1
+            identity = x
+            o = g.node("Relu", [_conv(g, init, x, cin, planes, 1, 1, 0)])
+            o = g.node("Relu", [_conv(g, init, o, planes, planes, 3, s, 1)])
+            o = _conv(g, init, o, planes, planes * 4, 1, 1, 0)
+            if b == 0:
+                identity = _conv(g, init, x, cin, planes * 4, 1, s, 0)
+            x = g.node("Relu", [g.node("Add", [o, identity])])
+            cin = planes * 4
+    x = g.node("GlobalAveragePool", [x])
+    x = g.node("Flatten", [x], axis=1)
+    w = g.constant(init.he_normal((classes, cin)))
+    bias = g.constant(np.zeros((classes,), dtype))
+    y = g.node("Gemm", [x, w, bias], "logits", alpha=1.0, beta=1.0, transB=1)
+    g.output(y)
+    return g, [x_np]
+
+
+def mobilenet_v2(batch=1, dtype=np.float32, seed=3, image=224, classes=1000):
+    """MobileNetV2 width 1.0; ReLU6 is Clip(0, 6) with constant bounds."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x_np = rng.normal(seed, 0, (batch, 3, image, image)).astype(dtype)
+    g.input("input", x_np.shape, dtype)
+
+    def relu6(v):
+        lo = g.constant(np.array(0.0, dtype))
+        hi = g.constant(np.array(6.0, dtype))
+        return g.node("Clip", [v, lo, hi])
+
+    x = relu6(_conv(g, init, "input", 3, 32, 3, 2, 1))
+    cin = 32
+    for t, c, n, s in [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]:
+        for i in range(n):
+            stride = s if i == 0 else 1
+            hidden = cin * t
+            o = x
+            if t != 1:
+                o = relu6(_conv(g, init, o, cin, hidden, 1, 1, 0))
+            o = relu6(_conv(g, init, o, hidden, hidden, 3, stride, 1, group=hidden))
+            o = _conv(g, init, o, hidden, c, 1, 1, 0)
+            x = g.node("Add", [x, o]) if (stride == 1 and cin == c) else o
+            cin = c
+    x = relu6(_conv(g, init, x, cin, 1280, 1, 1, 0))
+    x = g.node("GlobalAveragePool", [x])
+    x = g.node("Flatten", [x], axis=1)
+    w = g.constant(init.he_normal((classes, 1280)))
+    bias = g.constant(np.zeros((classes,), dtype))
+    y = g.node("Gemm", [x, w, bias], "logits", alpha=1.0, beta=1.0, transB=1)
+    g.output(y)
+    return g, [x_np]
+
+
+def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, seq=128, vocab=30522, dtype=np.float32, seed=4,
+                 fused=False):
+    """BERT-base-shaped encoder (post-LayerNorm, GELU(erf)), batch 1.
+
+    With ``fused=False`` LayerNorm and GELU appear as the primitive chains a
+    PyTorch export produces (and the reference lowers op by op); with
+    ``fused=True`` they are single LayerNormalization / Gelu nodes.
+    """
+    init = _Init(seed, dtype)
+    g = Graph()
+    ids = rng.integers(seed, 0, (1, seq), 0, vocab)
+    g.input("input_ids", ids.shape, np.int64)
+    dh = hidden // heads
+    eps = 1e-12
+
+    def scalar(v):
+        return g.constant(np.array(v, dtype))
+
+    def layernorm(x):
+        gamma, beta = g.constant(np.ones((hidden,), dtype)), g.constant(np.zeros((hidden,), dtype))
+        if fused:
+            return g.node("LayerNormalization", [x, gamma, beta], axis=-1, epsilon=eps)
+        mu = g.node("ReduceMean", [x], axes=[-1], keepdims=1)
+        d = g.node("Sub", [x, mu])
+        var = g.node("ReduceMean", [g.node("Pow", [d, scalar(2.0)])], axes=[-1], keepdims=1)
+        std = g.node("Sqrt", [g.node("Add", [var, scalar(eps)])])
+        return g.node("Add", [g.node("Mul", [g.node("Div", [d, std]), gamma]), beta])
+
+    def linear(x, nin, nout):
+        w = g.constant(init.normal((nin, nout), 0.02))
+        b = g.constant(init.normal((nout,), 0.02))
+        return g.node("Add", [b, g.node("MatMul", [x, w])])  # bias first, as the exporter writes it
+
+    def gelu(x):
+        if fused:
+            return g.node("Gelu", [x])
+        e = g.node("Erf", [g.node("Div", [x, scalar(float(np.sqrt(2.0)))])])
+        return g.node("Mul", [g.node("Mul", [x, g.node("Add", [e, scalar(1.0)])]), scalar(0.5)])
+
+    word = g.constant(init.normal((vocab, hidden), 0.02), "word_embeddings")
+    pos = g.constant(init.normal((1, seq, hidden), 0.02), "position_embeddings")
+    tok = g.constant(init.normal((hidden,), 0.02), "token_type_embedding")
+    x = g.node("Gather", [word, "input_ids"], axis=0)
+    x = g.node("Add", [g.node("Add", [x, pos]), tok])
+    x = layernorm(x)
+    for _ in range(layers):
+        def split(v, perm):
+            shp = g.constant(np.array([1, seq, heads, dh], np.int64))
+            return g.node("Transpose", [g.node("Reshape", [v, shp])], perm=perm)
+        q = split(linear(x, hidden, hidden), [0, 2, 1, 3])
+        k = split(linear(x, hidden, hidden), [0, 2, 3, 1])
+        v = split(linear(x, hidden, hidden), [0, 2, 1, 3])
+        s = g.node("Div", [g.node("MatMul", [q, k]), scalar(float(np.sqrt(dh)))])
+        p = g.node("Softmax", [s], axis=-1)
+        c = g.node("Transpose", [g.node("MatMul", [p, v])], perm=[0, 2, 1, 3])
+        c = g.node("Reshape", [c, g.constant(np.array([1, seq, hidden], np.int64))])
+        x = layernorm(g.node("Add", [linear(c, hidden, hidden), x]))
+        h = linear(gelu(linear(x, hidden, ffn)), ffn, hidden)
+        x = layernorm(g.node("Add", [h, x]))
+    g.output(x)
+    return g, [ids]

@@ -147,6 +147,11 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t h, int32_t format) {
   return 0;
 }
 int32_t dnnrtSync(dnnrtHandle_t h) { (void)h; return 0; }
+static int32_t no_graph(void) { snprintf(g_err, sizeof g_err, "oracle: no stream capture on the host"); return 1; }
+int32_t dnnrtGraphBegin(dnnrtHandle_t h) { (void)h; return no_graph(); }
+int32_t dnnrtGraphEnd(dnnrtHandle_t h, void **g) { (void)h; (void)g; return no_graph(); }
+int32_t dnnrtGraphLaunch(dnnrtHandle_t h, void *g) { (void)h; (void)g; return no_graph(); }
+int32_t dnnrtGraphDestroy(void *g) { (void)g; return 0; }
 
 /* wrapDNNMemPoolInit.cpp:19-29 / wrapDNNMalloc.cpp: one allocation. */
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {

@@ -1,0 +1,98 @@
+"""Whole programs on the MI355X: the same compiled DNN program is executed
+through the C ABI against the gfx950 library and against the CPU oracle, on
+the same seeded inputs.  Tolerances: rtol 1e-4 / atol 1e-5 (scaled by the
+output's magnitude) for fp32; rtol 2e-2 for fp16."""
+import numpy as np
+import pytest
+
+from helpers import ORACLE_PATH
+from occamy_amd import compiler, models
+
+pytestmark = pytest.mark.gpu
+
+
+def run(builder, runtime=None, mode=compiler.MODE_OCCAMY, **flags):
+    g, inputs = builder()
+    p = g.compile(**flags)
+    s = p.session(mode, runtime_library=runtime)
+    out = s.run(*inputs)
+    info = dict(pool=p.pool_bytes, requested=s.last_pool_bytes, weights=s.weights_bytes)
+    s.close()
+    return out, info
+
+
+def close(got, ref, rtol=1e-4, atol=1e-5):
+    scale = max(1.0, float(np.abs(ref).max()))
+    np.testing.assert_allclose(got, ref, rtol=rtol, atol=atol * scale)
+
+
+CONFIGS = {
+    "single_conv": models.single_conv,
+    "resnet50": models.resnet50,
+    "mobilenet_v2": models.mobilenet_v2,
+    "bert_2_layers": lambda: models.bert_encoder(layers=2),
+}
+
+
+@pytest.fixture(scope="module")
+def oracle_outputs():
+    return {k: run(b, ORACLE_PATH)[0] for k, b in CONFIGS.items()}
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_occamy_mode_matches_oracle(name, oracle_outputs):
+    out, info = run(CONFIGS[name])
+    assert info["requested"] == info["pool"]  # device arena == planned pool, byte for byte
+    for o, r in zip(out, oracle_outputs[name]):
+        close(o, r)
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_fused_program_matches_oracle(name, oracle_outputs):
+    out, _ = run(CONFIGS[name], fusion=True)
+    for o, r in zip(out, oracle_outputs[name]):
+        close(o, r)
+
+
+@pytest.mark.parametrize("name", ["single_conv", "resnet50", "bert_2_layers"])
+def test_resident_mode_and_graph_replay(name, oracle_outputs):
+    import torch
+    g, inputs = CONFIGS[name]()
+    p = g.compile(fusion=True)
+    s = p.session(compiler.MODE_RESIDENT)
+    out = s.run(*inputs)
+    for o, r in zip(out, oracle_outputs[name]):
+        close(o, r)
+    # device-resident inputs, captured graph, several replays with other work in between
+    dev_in = [torch.from_numpy(a).cuda() for a in inputs]
+    dev_out = [torch.empty(o.shape, dtype=torch.from_numpy(o).dtype, device="cuda") for o in out]
+    torch.cuda.synchronize()
+    for it in range(4):
+        for t in dev_out:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        s.run_device([t.data_ptr() for t in dev_in], [t.data_ptr() for t in dev_out], use_graph=True)
+        s.sync()
+        for t, o in zip(dev_out, out):
+            np.testing.assert_array_equal(t.cpu().numpy(), o)  # replay == eager, bit for bit
+    s.run_device([t.data_ptr() for t in dev_in], [t.data_ptr() for t in dev_out], use_graph=False)
+    s.sync()
+    np.testing.assert_array_equal(dev_out[0].cpu().numpy(), out[0])
+    s.close()
+
+
+def test_bert_fused_layernorm_gelu(oracle_outputs):
+    out, _ = run(lambda: models.bert_encoder(layers=2, fused=True))
+    close(out[0], oracle_outputs["bert_2_layers"][0], 1e-4, 1e-4)
+
+
+def test_new_input_same_session():
+    g, inputs = models.single_conv()
+    p = g.compile()
+    s = p.session()
+    so = p.session(runtime_library=ORACLE_PATH)
+    for seed in (7, 8):
+        x = np.random.default_rng(seed).standard_normal(inputs[0].shape).astype(np.float32)
+        close(s.run(x)[0], so.run(x)[0])
+    s.close()
+    so.close()
