@@ -63,6 +63,11 @@ int32_t dnncProgramNumOutputs(const dnncProgram *p);
 /* rank, dims (up to 8) and dtype of output i */
 int32_t dnncProgramOutputInfo(const dnncProgram *p, int32_t i, int32_t *dtype, int32_t *rank, int64_t *dims);
 int64_t dnncProgramNumOps(const dnncProgram *p, int32_t compute_only);
+/* i-th compute operation in program order: its mnemonic, its work class
+ * (conv_dense, conv_depthwise, gemm, matmul, softmax, layernorm, reduce, pool,
+ * move, elementwise) and its algorithmic FLOPs and bytes (each tensor read or
+ * written counted once at its dense size) */
+int32_t dnncProgramComputeOp(const dnncProgram *p, int64_t i, const char **name, const char **work_class, double *flops, double *bytes);
 
 /* ---- the planner alone (mallocPoolOpt.hpp:21-140, 212-218) ----
  * kind/id/bytes as above; writes one offset per event (-1 for deallocs) and
@@ -82,6 +87,9 @@ int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *o
  * wait (dnncSessionSync does); use_graph: replay the kernels from a captured graph */
 int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
 int32_t dnncSessionSync(dnncSession *s);
+/* resident mode: one eager pass with device timestamps around every compute
+ * operation; ms[i] belongs to dnncProgramComputeOp(i).  Returns the count. */
+int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on_device, float *ms, int64_t cap);
 int64_t dnncSessionWeightsBytes(const dnncSession *s);
 /* bytes the last occamy-mode run requested from dnnrtMemPoolInit (-1 before any run) */
 int64_t dnncSessionLastPoolBytes(const dnncSession *s);

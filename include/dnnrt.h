@@ -96,6 +96,12 @@ int32_t dnnrtGraphBegin(dnnrtHandle_t handle);
 int32_t dnnrtGraphEnd(dnnrtHandle_t handle, void **graph);
 int32_t dnnrtGraphLaunch(dnnrtHandle_t handle, void *graph);
 int32_t dnnrtGraphDestroy(void *graph);
+/* New.  Device-side timestamps on a stream, for per-call timing. */
+int32_t dnnrtEventCreate(void **event);
+int32_t dnnrtEventRecord(void *event, dnnrtStream_t stream);
+/* waits for `stop`, then gives the time from `start` to `stop` in milliseconds */
+int32_t dnnrtEventElapsedMs(void *start, void *stop, float *ms);
+int32_t dnnrtEventDestroy(void *event);
 /* New.  Text of the calling thread's last error ("" if none). */
 const char *dnnrtLastError(void);
 /* New.  0 when built for the GPU, 1 for a host-only build of the same ABI. */

@@ -27,6 +27,10 @@ SIGNATURES = {
     "dnnrtGraphEnd": (i32, [P, C.POINTER(P)]),
     "dnnrtGraphLaunch": (i32, [P, P]),
     "dnnrtGraphDestroy": (i32, [P]),
+    "dnnrtEventCreate": (i32, [C.POINTER(P)]),
+    "dnnrtEventRecord": (i32, [P, P]),
+    "dnnrtEventElapsedMs": (i32, [P, P, C.POINTER(f32)]),
+    "dnnrtEventDestroy": (i32, [P]),
     "dnnrtLastError": (C.c_char_p, []),
     "dnnrtIsHostBackend": (i32, []),
     "dnnrtMemPoolInit": (i32, [C.POINTER(P), i64]),

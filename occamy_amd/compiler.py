@@ -58,6 +58,9 @@ def lib():
         "dnncProgramNumOutputs": (C.c_int32, [P]),
         "dnncProgramOutputInfo": (C.c_int32, [P, C.c_int32, I32P, I32P, I64P]),
         "dnncProgramNumOps": (C.c_int64, [P, C.c_int32]),
+        "dnncProgramComputeOp": (C.c_int32, [P, C.c_int64, C.POINTER(C.c_char_p), C.POINTER(C.c_char_p),
+                                 C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+        "dnncSessionProfile": (C.c_int64, [P, C.POINTER(P), C.c_int32, C.POINTER(C.c_float), C.c_int64]),
         "dnncPlanPool": (C.c_int64, [C.c_int64, I32P, I64P, I64P, I64P]),
         "dnncPlanFreeList": (C.c_int64, [C.c_int64, I32P, I64P, I64P, C.c_int64, I64P, C.c_int64]),
         "dnncSessionCreate": (P, [P, C.c_char_p, C.c_int32]),
@@ -195,6 +198,16 @@ class Program:
     def num_ops(self, compute_only=False):
         return lib().dnncProgramNumOps(self._p, int(compute_only))
 
+    def compute_ops(self):
+        """[(mnemonic, work class, algorithmic FLOPs, algorithmic bytes)] per compute op, program order."""
+        out = []
+        for i in range(self.num_ops(compute_only=True)):
+            name, cls, fl, by = C.c_char_p(), C.c_char_p(), C.c_double(), C.c_double()
+            if lib().dnncProgramComputeOp(self._p, i, C.byref(name), C.byref(cls), C.byref(fl), C.byref(by)):
+                raise RuntimeError(_err())
+            out.append((name.value.decode(), cls.value.decode(), fl.value, by.value))
+        return out
+
     def events(self):
         """[(kind, id, bytes, offset)] in execution order."""
         n = lib().dnncProgramEvents(self._p, None, None, None, None, 0)
@@ -254,6 +267,19 @@ class Session:
         op = (C.c_void_p * max(len(out_ptrs), 1))(*out_ptrs)
         if lib().dnncSessionRunResident(self._s, ip, op, 1, int(use_graph)):
             raise RuntimeError("run_device: " + _err())
+
+    def profile(self, in_ptrs_or_arrays, on_device=False):
+        """Resident mode: milliseconds per compute op (device timestamps), program order."""
+        if on_device:
+            ip = (C.c_void_p * max(len(in_ptrs_or_arrays), 1))(*in_ptrs_or_arrays)
+        else:
+            keep = [np.ascontiguousarray(a) for a in in_ptrs_or_arrays]
+            ip = (C.c_void_p * max(len(keep), 1))(*[a.ctypes.data for a in keep])
+        n = self.program.num_ops(compute_only=True)
+        ms = (C.c_float * max(n, 1))()
+        if lib().dnncSessionProfile(self._s, ip, int(on_device), ms, n) < 0:
+            raise RuntimeError("profile: " + _err())
+        return list(ms[:n])
 
     def sync(self):
         if lib().dnncSessionSync(self._s):

@@ -119,6 +119,31 @@ int32_t dnnrtGraphDestroy(void *graph) {
   return 0;
 }
 
+int32_t dnnrtEventCreate(void **event) {
+  if (!event) { set_error("dnnrtEventCreate: null pointer"); return 1; }
+  hipEvent_t e;
+  HIP_RET(hipEventCreate(&e), "dnnrtEventCreate");
+  *event = e;
+  return 0;
+}
+
+int32_t dnnrtEventRecord(void *event, dnnrtStream_t stream) {
+  HIP_RET(hipEventRecord((hipEvent_t)event, (hipStream_t)stream), "dnnrtEventRecord");
+  return 0;
+}
+
+int32_t dnnrtEventElapsedMs(void *start, void *stop, float *ms) {
+  if (!ms) { set_error("dnnrtEventElapsedMs: null pointer"); return 1; }
+  HIP_RET(hipEventSynchronize((hipEvent_t)stop), "dnnrtEventElapsedMs: hipEventSynchronize");
+  HIP_RET(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "dnnrtEventElapsedMs");
+  return 0;
+}
+
+int32_t dnnrtEventDestroy(void *event) {
+  if (event) HIP_RET(hipEventDestroy((hipEvent_t)event), "dnnrtEventDestroy");
+  return 0;
+}
+
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
   if (!pool || bytes < 0) { set_error("dnnrtMemPoolInit: bad arguments"); return 1; }
   HIP_RET(hipMalloc(pool, (size_t)(bytes > 0 ? bytes : 1)), "dnnrtMemPoolInit: hipMalloc");

@@ -178,6 +178,20 @@ int64_t dnncProgramNumOps(const dnncProgram *p, int32_t compute_only) {
   return n;
 }
 
+int32_t dnncProgramComputeOp(const dnncProgram *p, int64_t i, const char **name, const char **work_class, double *flops, double *bytes) {
+  if (!p || !name || !work_class || !flops || !bytes) return fail("dnncProgramComputeOp: bad arguments");
+  int64_t n = 0;
+  for (const Op *op : p->p.ops) {
+    if (op->kind < OP_CONVFWD || op->kind > OP_GELU) continue;
+    if (n++ != i) continue;
+    *name = op_name(op->kind);
+    *work_class = op_class(op);
+    op_work(op, *flops, *bytes);
+    return 0;
+  }
+  return fail("dnncProgramComputeOp: index out of range");
+}
+
 int64_t dnncPlanPool(int64_t n, const int32_t *kind, const int64_t *id, const int64_t *bytes, int64_t *offset) {
   PoolSimulator sim;
   for (int64_t i = 0; i < n; i++) {
@@ -231,6 +245,15 @@ int32_t dnncSessionSync(dnncSession *s) {
   if (!s) return fail("dnncSessionSync: null session");
   std::string err;
   return s->s.sync(err) ? 0 : fail(err);
+}
+
+int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on_device, float *ms, int64_t cap) {
+  if (!s || !inputs) { fail("dnncSessionProfile: bad arguments"); return -1; }
+  std::vector<float> t;
+  std::string err;
+  if (!s->s.profile_resident(inputs, on_device, t, err)) { fail(err); return -1; }
+  for (size_t i = 0; i < t.size() && (int64_t)i < cap && ms; i++) ms[i] = t[i];
+  return (int64_t)t.size();
 }
 
 int64_t dnncSessionWeightsBytes(const dnncSession *s) { return s ? s->s.weights_bytes : -1; }

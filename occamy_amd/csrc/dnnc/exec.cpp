@@ -34,7 +34,8 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
   LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
-  LOAD(dnnrtGraphDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
+  LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
+  LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
   LOAD(dnnrtMalloc); LOAD(dnnrtDealloc); LOAD(dnnrtHostAlloc); LOAD(dnnrtHostFree);
   LOAD(dnnrtConv); LOAD(dnnrtConvBiasActiv); LOAD(dnnrtActive); LOAD(dnnrtTensorOp); LOAD(dnnrtClip);
   LOAD(dnnrtErf); LOAD(dnnrtNegative); LOAD(dnnrtReciprocal); LOAD(dnnrtPow); LOAD(dnnrtCastI64toFloat);
@@ -330,31 +331,38 @@ bool Session::issue_all_compute(std::string &err) {
 // Resident inference.  `on_device` != 0: inputs/outputs are device pointers and
 // the call returns without waiting (sync() does).
 bool Session::run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err) {
-  // 1. inputs into their pool slots
-  for (const Op *op : prog->ops) {
-    if (op->kind != OP_MEMCPY || op->mode != 1) continue;
-    const Value *src = op->operands[1];
-    if (src->arg_index < 0) continue;
-    const size_t ai = (size_t)src->arg_index;
-    const void *from = inputs[ai];
-    if (!on_device) { std::memcpy(host_in[ai], inputs[ai], (size_t)op->bytes); from = host_in[ai]; }
-    if (rt.dnnrtMemcpy(ptr[(size_t)op->operands[0]->id], const_cast<void *>(from), op->bytes, on_device ? 3 : 1, stream)) {
-      err = rt_error("dnnrtMemcpy(input)"); return false;
+  // The pool reuses the inputs' slots for later tensors, so every pass over
+  // the kernels must be preceded by a fresh copy of the inputs.
+  auto copy_inputs = [&]() -> bool {
+    for (const Op *op : prog->ops) {
+      if (op->kind != OP_MEMCPY || op->mode != 1) continue;
+      const Value *src = op->operands[1];
+      if (src->arg_index < 0) continue;
+      const size_t ai = (size_t)src->arg_index;
+      const void *from = inputs[ai];
+      if (!on_device) { std::memcpy(host_in[ai], inputs[ai], (size_t)op->bytes); from = host_in[ai]; }
+      if (rt.dnnrtMemcpy(ptr[(size_t)op->operands[0]->id], const_cast<void *>(from), op->bytes, on_device ? 3 : 1, stream)) {
+        err = rt_error("dnnrtMemcpy(input)"); return false;
+      }
     }
+    return true;
+  };
+  const bool graphed = use_graph && !host_backend;
+  if (graphed && !graph) {
+    // One eager pass on real data first: it validates every call outside of
+    // capture.  Then the same call sequence is recorded (nothing runs).
+    if (!copy_inputs() || !issue_all_compute(err)) return false;
+    if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
+    if (rt.dnnrtGraphBegin(handle)) { err = rt_error("dnnrtGraphBegin"); return false; }
+    const bool ok = issue_all_compute(err);
+    void *g = nullptr;
+    if (rt.dnnrtGraphEnd(handle, &g)) { if (ok) err = rt_error("dnnrtGraphEnd"); return false; }
+    if (!ok) { rt.dnnrtGraphDestroy(g); return false; }
+    graph = g;
   }
-  // 2. kernels
-  if (use_graph && !host_backend) {
-    if (!graph) {
-      // One eager pass first: it validates every call outside of capture.
-      if (!issue_all_compute(err)) return false;
-      if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
-      if (rt.dnnrtGraphBegin(handle)) { err = rt_error("dnnrtGraphBegin"); return false; }
-      const bool ok = issue_all_compute(err);
-      void *g = nullptr;
-      if (rt.dnnrtGraphEnd(handle, &g)) { if (ok) err = rt_error("dnnrtGraphEnd"); return false; }
-      if (!ok) { rt.dnnrtGraphDestroy(g); return false; }
-      graph = g;
-    }
+  // 1. inputs into their pool slots  2. kernels
+  if (!copy_inputs()) return false;
+  if (graphed) {
     if (rt.dnnrtGraphLaunch(handle, graph)) { err = rt_error("dnnrtGraphLaunch"); return false; }
   } else {
     if (!issue_all_compute(err)) return false;
@@ -375,6 +383,39 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
       if (op->kind == OP_HOST_ALLOC) std::memcpy(outputs[(size_t)op->out_index], host_out[(size_t)op->out_index], (size_t)op->bytes);
   }
   return true;
+}
+
+bool Session::profile_resident(const void *const *inputs, int on_device, std::vector<float> &ms, std::string &err) {
+  if (mode != MODE_RESIDENT) { err = "profiling needs a resident session"; return false; }
+  std::vector<const Op *> compute;
+  for (const Op *op : prog->ops)
+    if (is_compute(op->kind)) compute.push_back(op);
+  std::vector<void *> ev(compute.size() + 1, nullptr);
+  bool ok = true;
+  for (void *&e : ev)
+    if (rt.dnnrtEventCreate(&e)) { err = rt_error("dnnrtEventCreate"); ok = false; break; }
+  if (ok) {
+    for (const Op *op : prog->ops) {  // inputs into their pool slots
+      if (op->kind != OP_MEMCPY || op->mode != 1 || op->operands[1]->arg_index < 0) continue;
+      const size_t ai = (size_t)op->operands[1]->arg_index;
+      const void *from = inputs[ai];
+      if (!on_device) { std::memcpy(host_in[ai], inputs[ai], (size_t)op->bytes); from = host_in[ai]; }
+      if (rt.dnnrtMemcpy(ptr[(size_t)op->operands[0]->id], const_cast<void *>(from), op->bytes, on_device ? 3 : 1, stream)) {
+        err = rt_error("dnnrtMemcpy(input)"); ok = false; break;
+      }
+    }
+  }
+  if (ok && rt.dnnrtEventRecord(ev[0], stream)) { err = rt_error("dnnrtEventRecord"); ok = false; }
+  for (size_t i = 0; ok && i < compute.size(); i++) {
+    ok = issue(compute[i], err);
+    if (ok && rt.dnnrtEventRecord(ev[i + 1], stream)) { err = rt_error("dnnrtEventRecord"); ok = false; }
+  }
+  if (rt.dnnrtSync(handle) && ok) { err = rt_error("dnnrtSync"); ok = false; }
+  ms.assign(compute.size(), 0.f);
+  for (size_t i = 0; ok && i < compute.size(); i++)
+    if (rt.dnnrtEventElapsedMs(ev[i], ev[i + 1], &ms[i])) { err = rt_error("dnnrtEventElapsedMs"); ok = false; }
+  for (void *e : ev) rt.dnnrtEventDestroy(e);
+  return ok;
 }
 
 bool Session::sync(std::string &err) {

@@ -24,6 +24,10 @@ struct RuntimeApi {
   decltype(&::dnnrtGraphEnd) dnnrtGraphEnd = nullptr;
   decltype(&::dnnrtGraphLaunch) dnnrtGraphLaunch = nullptr;
   decltype(&::dnnrtGraphDestroy) dnnrtGraphDestroy = nullptr;
+  decltype(&::dnnrtEventCreate) dnnrtEventCreate = nullptr;
+  decltype(&::dnnrtEventRecord) dnnrtEventRecord = nullptr;
+  decltype(&::dnnrtEventElapsedMs) dnnrtEventElapsedMs = nullptr;
+  decltype(&::dnnrtEventDestroy) dnnrtEventDestroy = nullptr;
   decltype(&::dnnrtMemPoolInit) dnnrtMemPoolInit = nullptr;
   decltype(&::dnnrtMemOffset) dnnrtMemOffset = nullptr;
   decltype(&::dnnrtMemcpy) dnnrtMemcpy = nullptr;
@@ -66,6 +70,9 @@ class Session {
   bool run_occamy(const void *const *inputs, void *const *outputs, std::string &err);
   bool run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err);
   bool sync(std::string &err);
+  // Resident mode: one eager pass with a device timestamp around every compute
+  // operation; ms[i] is the time of the i-th compute op in program order.
+  bool profile_resident(const void *const *inputs, int on_device, std::vector<float> &ms, std::string &err);
 
   const Program *prog = nullptr;
   int mode = MODE_OCCAMY;

@@ -152,6 +152,9 @@ void constant_at_use(Graph &g);
 bool emit_program(const Graph &g, Program &p, std::string &err);
 void func_args_to_device(Program &p);
 void erase_dummy_constants(Program &p);
+// work.cpp
+const char *op_class(const Op *op);
+void op_work(const Op *op, double &flops, double &bytes);
 // passes.cpp
 void fuse_conv_bias_activ(Program &p);
 void dealloc_opt(Program &p);

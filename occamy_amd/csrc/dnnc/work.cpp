@@ -1,0 +1,87 @@
+// Algorithmic work of one compute operation: the FLOP and byte counts that
+// roofline figures are computed from.  Every tensor an operation reads or
+// writes is counted once at its dense size; nothing here depends on how a
+// kernel is implemented.
+#include "ir.h"
+
+namespace dnnc {
+
+const char *op_class(const Op *op) {
+  switch (op->kind) {
+    case OP_CONVFWD:
+    case OP_CONV_BIAS_ACTIV: return (op->dimB[1] == 1 && op->group > 1) ? "conv_depthwise" : "conv_dense";
+    case OP_MATMUL2D: return "gemm";
+    case OP_MATMULND: return "matmul";
+    case OP_SOFTMAX: return "softmax";
+    case OP_LAYERNORM: return "layernorm";
+    case OP_REDUCE: return "reduce";
+    case OP_MAXPOOL:
+    case OP_AVGPOOL: return "pool";
+    case OP_FLATTEN:
+    case OP_RESHAPE:
+    case OP_TRANSPOSE:
+    case OP_GATHER: return "move";
+    default: return "elementwise";
+  }
+}
+
+void op_work(const Op *op, double &flops, double &bytes) {
+  flops = 0;
+  bytes = 0;
+  const Value *out = op->operands.back();
+  const double es = (double)dtype_bytes(out->dtype);
+  const double n_out = (double)shape_numel(op->result ? op->result->shape : out->shape);
+  auto n_in = [&](size_t i) { return (double)shape_numel(op->operands[i]->shape); };
+  switch (op->kind) {
+    case OP_CONVFWD:
+    case OP_CONV_BIAS_ACTIV: {
+      const double crs = (double)(op->dimB[1] * op->dimB[2] * op->dimB[3]);
+      flops = 2.0 * n_out * crs;
+      bytes = ((double)shape_numel(op->dimA) + (double)shape_numel(op->dimB) + n_out +
+               (op->kind == OP_CONV_BIAS_ACTIV ? (double)op->dimB[0] : 0.0)) * es;
+      break;
+    }
+    case OP_MATMUL2D: {
+      const double k = (double)(op->trans_a ? op->dimA[0] : op->dimA[1]);
+      flops = 2.0 * n_out * k;
+      bytes = (n_in(0) + n_in(1) + n_out) * es;
+      break;
+    }
+    case OP_MATMULND: {
+      flops = 2.0 * n_out * (double)op->dimA.back();
+      bytes = (n_in(0) + n_in(1) + n_out) * es;
+      break;
+    }
+    case OP_ADD:
+    case OP_MUL:
+      flops = n_out;
+      bytes = (n_out + (double)shape_numel(op->dimB) + n_out) * es;
+      break;
+    case OP_GATHER:
+      bytes = 2.0 * n_out * es + n_in(1) * 8.0;
+      break;
+    case OP_LAYERNORM:
+      flops = 8.0 * n_out;
+      bytes = (2.0 * n_out + 2.0 * (double)op->dimA.back()) * es;
+      break;
+    case OP_SOFTMAX:
+      flops = 5.0 * n_out;
+      bytes = 2.0 * n_out * es;
+      break;
+    case OP_REDUCE:
+    case OP_MAXPOOL:
+    case OP_AVGPOOL:
+      flops = (double)shape_numel(op->dimA);
+      bytes = ((double)shape_numel(op->dimA) + n_out) * es;
+      break;
+    case OP_CAST:
+      bytes = n_out * (8.0 + es);
+      break;
+    default:  // unary elementwise and copies: one read, one write
+      flops = n_out;
+      bytes = 2.0 * n_out * es;
+      break;
+  }
+}
+
+}  // namespace dnnc

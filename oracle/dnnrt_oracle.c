@@ -23,6 +23,7 @@
  * Layout is dense NCHW / row-major, as in the reference
  * (src/Tools/dnn-wrapper/cudnn/CUDNNConvFunc.cpp:48-60).
  */
+#define _POSIX_C_SOURCE 200809L
 #include "../include/dnnrt.h"
 
 #include <math.h>
@@ -152,6 +153,19 @@ int32_t dnnrtGraphBegin(dnnrtHandle_t h) { (void)h; return no_graph(); }
 int32_t dnnrtGraphEnd(dnnrtHandle_t h, void **g) { (void)h; (void)g; return no_graph(); }
 int32_t dnnrtGraphLaunch(dnnrtHandle_t h, void *g) { (void)h; (void)g; return no_graph(); }
 int32_t dnnrtGraphDestroy(void *g) { (void)g; return 0; }
+
+/* host stand-in for stream timestamps: the wall clock at record time */
+#include <time.h>
+int32_t dnnrtEventCreate(void **e) { *e = calloc(1, sizeof(double)); return *e ? 0 : 1; }
+int32_t dnnrtEventRecord(void *e, dnnrtStream_t s) {
+  (void)s;
+  struct timespec t;
+  clock_gettime(CLOCK_MONOTONIC, &t);
+  *(double *)e = (double)t.tv_sec * 1e3 + (double)t.tv_nsec * 1e-6;
+  return 0;
+}
+int32_t dnnrtEventElapsedMs(void *a, void *b, float *ms) { *ms = (float)(*(double *)b - *(double *)a); return 0; }
+int32_t dnnrtEventDestroy(void *e) { free(e); return 0; }
 
 /* wrapDNNMemPoolInit.cpp:19-29 / wrapDNNMalloc.cpp: one allocation. */
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
