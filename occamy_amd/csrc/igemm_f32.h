@@ -37,5 +37,8 @@ struct IgemmArgs {
 // Launches the kernel on `stream`; returns false (with the error text set) if
 // the shape cannot be handled.
 bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a);
+// The variant for problems too small to fill the chip with LDS-staged tiles
+// (igemm_f32_direct.hip); rsmode / layout as computed by launch_igemm_f32.
+bool launch_igemm_f32_direct(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout);
 
 }  // namespace dnnrt

@@ -273,8 +273,8 @@ bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a) {
   auto wgs = [&](int bm, int bn) { return ceil_div(a.M, bm) * ceil_div(a.Ncols, bn) * a.Z; };
   if (wgs(128, 128) >= want) return launch_tile<128, 128, 2, 2>(ctx, a, rsmode, layout);
   if (wgs(64, 64) >= want) return launch_tile<64, 64, 2, 2>(ctx, a, rsmode, layout);
-  if (wgs(32, 64) >= want) return launch_tile<32, 64, 1, 2>(ctx, a, rsmode, layout);
-  return launch_tile<32, 32, 1, 1>(ctx, a, rsmode, layout);
+  // Too small to fill the chip with LDS-staged tiles: latency-bound territory.
+  return launch_igemm_f32_direct(ctx, a, rsmode, layout);
 }
 
 }  // namespace dnnrt
