@@ -96,3 +96,36 @@ def test_new_input_same_session():
         close(s.run(x)[0], so.run(x)[0])
     s.close()
     so.close()
+
+
+@pytest.mark.parametrize("batch,image", [(2, 64), (4, 224)])
+def test_resnet50_fp16_channels_last(batch, image):
+    """fp16 weights/activations, fp32 accumulation, NHWC on the device, against
+    the fp32 oracle on the same (fp16-representable) weights and input."""
+    build16 = lambda: models.resnet50(batch, np.float16, seed=5, image=image)  # noqa: E731
+    out16, info = run(build16, fusion=True, channels_last=True)
+    assert info["requested"] == info["pool"]
+
+    def build32():
+        g16, inputs = build16()
+        g = compiler.Graph()
+        for name, (shape, _) in g16.input_shapes.items():
+            g.input(name, shape, np.float32)
+        for name, arr in g16.constants.items():
+            g.constant(arr.astype(np.float32), name)
+        for op, ins, out, at in g16.nodes:
+            g.node(op, ins, out, **at)
+        for o in g16.outputs:
+            g.output(o)
+        return g, [a.astype(np.float32) for a in inputs]
+
+    ref, _ = run(build32, ORACLE_PATH, fusion=True)
+    got, want = out16[0].astype(np.float32), ref[0]
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    # resident + graph replay gives the same bits as the per-inference mode
+    g, inputs = build16()
+    p = g.compile(fusion=True, channels_last=True)
+    s = p.session(compiler.MODE_RESIDENT)
+    np.testing.assert_array_equal(s.run(*inputs)[0], out16[0])
+    s.close()

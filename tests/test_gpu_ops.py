@@ -255,3 +255,93 @@ def test_data_movement(gpu, cpu):
     np.testing.assert_array_equal(oc.gather(gpu, x, np.array([2, -1]), 2), np.take(x, [2, -1], 2))
     with pytest.raises(RuntimeError):
         oc.transpose(gpu, x, (0, 1, 1, 3))
+
+
+# ---- fp16, channels-last -----------------------------------------------------------------
+
+def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt):
+    """x, w in logical NCHW / KCRS order; returns logical NCHW."""
+    N, C, H, W = x.shape
+    K, Cg, R, S = w.shape
+    P, Q = oc.conv_out_hw(H, W, R, S, pads, strides)
+    xin = x if fmt != _abi.NHWC else np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    win = w if fmt == _abi.NCHW else np.ascontiguousarray(w.transpose(0, 2, 3, 1))  # K,R,S,C
+    X, Wt, B = gpu.put(xin), gpu.put(win), gpu.put(b)
+    Y = gpu.empty((N * K * P * Q,), np.float16)
+    gpu.ops.set_format(fmt)
+    try:
+        gpu.ops.conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), pads, strides, activ, gpu.ptr(Y),
+                                group, _abi.F16)
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    y = gpu.get(Y)
+    return y.reshape(N, K, P, Q) if fmt == _abi.NCHW else y.reshape(N, P, Q, K).transpose(0, 3, 1, 2)
+
+
+F16_CASES = [
+    # N, C, H, W, K, R, stride, pad
+    (2, 64, 56, 56, 64, 3, 1, 1),      # fast path, K_out = 64 tile
+    (2, 64, 56, 56, 256, 1, 1, 0),
+    (2, 256, 28, 28, 128, 3, 2, 1),    # strided 3x3
+    (3, 512, 7, 7, 512, 3, 1, 1),      # ragged pixel tile (147 pixels)
+    (2, 256, 14, 14, 1000, 1, 1, 0),   # K_out not a multiple of the tile
+    (1, 1024, 14, 14, 2048, 1, 2, 0),
+    (2, 32, 9, 11, 40, 3, 1, 1),       # smallest C the fast path takes
+    (2, 3, 32, 32, 64, 7, 2, 3),       # generic path: 3 channels
+    (1, 20, 9, 9, 24, 3, 1, 1),        # generic path: C % 32 != 0
+]
+
+
+@pytest.mark.parametrize("case", F16_CASES, ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("fmt", [_abi.NHWC, _abi.NCHW_TO_NHWC, _abi.NCHW])
+def test_conv_f16(gpu, cpu, case, fmt):
+    N, C, H, W, K, R, st, pd = case
+    r = rng(sum(case) + fmt)
+    x = r.standard_normal((N, C, H, W)).astype(np.float16)
+    w = (r.standard_normal((K, C, R, R)) * np.sqrt(2.0 / (C * R * R))).astype(np.float16)
+    b = r.uniform(-0.1, 0.1, K).astype(np.float16)
+    ref = oc.conv(cpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU)          # fp16 storage, exact accumulate
+    got = conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, fmt)
+    # fp32 accumulation then one rounding to fp16: within 1 fp16 ulp of the oracle
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3)
+    if fmt == _abi.NHWC:
+        ident = conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_IDENTITY, fmt)
+        refi = oc.conv(cpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_IDENTITY)
+        np.testing.assert_allclose(ident.astype(np.float32), refi.astype(np.float32), rtol=2e-3, atol=2e-3)
+
+
+def test_f16_channels_last_ops(gpu, cpu):
+    r = rng(77)
+    x = r.standard_normal((2, 64, 28, 28)).astype(np.float16)
+    xl = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    gpu.ops.set_format(_abi.NHWC)
+    try:
+        X = gpu.put(xl)
+        Y = gpu.empty((2 * 64 * 14 * 14,), np.float16)
+        gpu.ops.maxpool(gpu.ptr(X), x.shape, gpu.ptr(Y), (2, 64, 14, 14), (3, 3), (1, 1, 1, 1), (2, 2), _abi.F16)
+        G = gpu.empty((2 * 64,), np.float16)
+        gpu.ops.reduce_mean(gpu.ptr(X), x.shape, gpu.ptr(G), (2, 64, 1, 1), _abi.F16)
+        bias = r.standard_normal((1, 64, 1, 1)).astype(np.float16)
+        Bv = gpu.put(bias.reshape(64))
+        O = gpu.empty(xl.shape, np.float16)
+        gpu.ops.tensor_op(_abi.OP_ADD, gpu.ptr(X), x.shape, gpu.ptr(Bv), (1, 64, 1, 1), gpu.ptr(O), 1.0, _abi.F16)
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    np.testing.assert_array_equal(gpu.get(Y).reshape(2, 14, 14, 64).transpose(0, 3, 1, 2),
+                                  oc.pool(cpu, "max", x, (3, 3), (1, 1), (2, 2)))
+    np.testing.assert_allclose(gpu.get(G).reshape(2, 64, 1, 1).astype(np.float32),
+                               oc.reduce_mean(cpu, x, (2, 64, 1, 1)).astype(np.float32), rtol=2e-3, atol=1e-3)
+    np.testing.assert_array_equal(gpu.get(O).transpose(0, 3, 1, 2), oc.tensor_op(cpu, _abi.OP_ADD, x, bias))
+
+
+def test_matmul2d_f16(gpu, cpu):
+    r = rng(78)
+    for M, K, N in [(64, 2048, 1000), (2, 64, 8), (130, 96, 72)]:
+        a = r.standard_normal((M, K)).astype(np.float16)
+        b = (r.standard_normal((N, K)) / np.sqrt(K)).astype(np.float16)
+        np.testing.assert_allclose(oc.matmul2d(gpu, a, b, transB=1).astype(np.float32),
+                                   oc.matmul2d(cpu, a, b, transB=1).astype(np.float32), rtol=2e-3, atol=2e-3)
+    with pytest.raises(RuntimeError):
+        oc.matmul2d(gpu, np.zeros((4, 8), np.float16), np.zeros((8, 4), np.float16))  # layout not built: loud
