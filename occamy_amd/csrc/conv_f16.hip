@@ -27,6 +27,13 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// 16-byte load through an explicitly GLOBAL pointer.  Left to itself the
+// compiler emits flat loads here, which count against the LDS counter as well
+// and so serialise the prefetch behind every LDS operand fetch.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const u32x4 *global_u32x4_ptr;
+__device__ __forceinline__ u32x4 load_global_16(const void *p) { return *(global_u32x4_ptr)p; }
+
 constexpr int BK16 = 32;      // k per step
 constexpr int LDS_ROW = 40;   // halfs per LDS row: 32 + 8 pad (80 bytes)
 
@@ -56,18 +63,21 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
 
   // ---- loader constants ------------------------------------------------
   // A (filters): chunk id -> (row, 16-byte chunk of the 64-byte k slice)
-  const _Float16 *a_ptr[A_CH];
+  // element OFFSETS, not pointers, are kept across the loop: the address is
+  // formed from the kernel-argument base at each load, which keeps the loads
+  // in the global address space (flat loads would tie them to the LDS counter)
+  int64_t a_off[A_CH];
   bool a_ok[A_CH];
 #pragma unroll
   for (int i = 0; i < A_CH; i++) {
     const int id = tid + i * 256, row = id >> 2, ch = id & 3;
     const int k_out = m0 + row;
     a_ok[i] = k_out < a.K;
-    a_ptr[i] = Wg + (int64_t)(a_ok[i] ? k_out : 0) * CRS + ch * 8;
+    a_off[i] = (int64_t)(a_ok[i] ? k_out : 0) * CRS + ch * 8;
   }
   // B (im2col): each chunk belongs to one output pixel
   int b_ih0[B_CH], b_iw0[B_CH];
-  const _Float16 *b_ptr[B_CH];
+  int64_t b_off[B_CH];
   bool b_ok[B_CH];
 #pragma unroll
   for (int i = 0; i < B_CH; i++) {
@@ -79,35 +89,48 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
     const int p = pq / a.Q, q = pq - p * a.Q;
     b_ih0[i] = p * a.sh - a.ph;
     b_iw0[i] = q * a.sw - a.pw;
-    b_ptr[i] = Xg + (int64_t)n * a.H * a.W * a.C + ch * 8;
+    b_off[i] = (int64_t)n * a.H * a.W * a.C + ch * 8;
   }
 
-  uint4 ra[A_CH], rb[B_CH];
-  const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+  // Register ring: the loads of DEPTH future steps are in flight while the
+  // MFMAs of the current one run (a step is ~0.1 us of MFMA work, a global
+  // load takes several times that).  Slots are indexed with compile-time
+  // constants: the step loop is unrolled DEPTH times.
+  constexpr int DEPTH = 4;
+  u32x4 ra[DEPTH][A_CH], rb[DEPTH][B_CH];
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
 
-  auto load_step = [&](int r, int s, int c0) {
-    const int kk = (r * a.S + s) * a.C + c0;
+  const int steps_c = a.C / BK16, nk = a.R * a.S * steps_c;
+  int lr = 0, ls = 0, lc0 = 0, lstep = 0;  // cursor of the next step to load
+
+  auto load_step = [&](u32x4 (&qa)[A_CH], u32x4 (&qb)[B_CH]) {
+    if (lstep < nk) {
+      const int kk = (lr * a.S + ls) * a.C + lc0;
 #pragma unroll
-    for (int i = 0; i < A_CH; i++)
-      ra[i] = a_ok[i] ? *reinterpret_cast<const uint4 *>(a_ptr[i] + kk) : zero4;
+      for (int i = 0; i < A_CH; i++)
+        qa[i] = a_ok[i] ? load_global_16(Wg + (a_off[i] + kk)) : zero4;
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) {
-      const int ih = b_ih0[i] + r, iw = b_iw0[i] + s;
-      const bool ok = b_ok[i] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
-      rb[i] = ok ? *reinterpret_cast<const uint4 *>(b_ptr[i] + ((int64_t)ih * a.W + iw) * a.C + c0) : zero4;
+      for (int i = 0; i < B_CH; i++) {
+        const int ih = b_ih0[i] + lr, iw = b_iw0[i] + ls;
+        const bool ok = b_ok[i] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+        qb[i] = ok ? load_global_16(Xg + (b_off[i] + ((int64_t)ih * a.W + iw) * a.C + lc0)) : zero4;
+      }
+      lc0 += BK16;
+      if (lc0 == a.C) { lc0 = 0; if (++ls == a.S) { ls = 0; ++lr; } }
     }
+    lstep++;
   };
-  auto store_step = [&](int buf) {
+  auto store_step = [&](int buf, const u32x4 (&qa)[A_CH], const u32x4 (&qb)[B_CH]) {
     _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
 #pragma unroll
     for (int i = 0; i < A_CH; i++) {
       const int id = tid + i * 256, row = id >> 2, ch = id & 3;
-      *reinterpret_cast<uint4 *>(As + row * LDS_ROW + ch * 8) = ra[i];
+      *reinterpret_cast<u32x4 *>(As + row * LDS_ROW + ch * 8) = qa[i];
     }
 #pragma unroll
     for (int i = 0; i < B_CH; i++) {
       const int id = tid + i * 256, row = id >> 2, ch = id & 3;
-      *reinterpret_cast<uint4 *>(Bs + row * LDS_ROW + ch * 8) = rb[i];
+      *reinterpret_cast<u32x4 *>(Bs + row * LDS_ROW + ch * 8) = qb[i];
     }
   };
 
@@ -119,36 +142,41 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  const int steps_c = a.C / BK16, nk = a.R * a.S * steps_c;
-  int r = 0, s = 0, c0 = 0;
-  load_step(0, 0, 0);
-  store_step(0);
+  // prologue: step 0 into LDS, steps 1 .. DEPTH-1 in flight in slots 1 .. DEPTH-1
+  load_step(ra[0], rb[0]);
+#pragma unroll
+  for (int d = 1; d < DEPTH; d++) load_step(ra[d], rb[d]);
+  store_step(0, ra[0], rb[0]);
   __syncthreads();
 
-  for (int kt = 0; kt < nk; kt++) {
-    const int buf = kt & 1;
-    // advance (r, s, c0) to the next step
-    c0 += BK16;
-    if (c0 == a.C) { c0 = 0; if (++s == a.S) { s = 0; ++r; } }
-    if (kt + 1 < nk) load_step(r, s, c0);
-    const _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
+  for (int kt0 = 0; kt0 < nk; kt0 += DEPTH) {
 #pragma unroll
-    for (int ks = 0; ks < BK16; ks += 16) {
-      half8 av[TM], bv[TN];
+    for (int u = 0; u < DEPTH; u++) {
+      const int kt = kt0 + u;
+      if (kt < nk) {
+        const int buf = kt & 1;
+        // slot u held step kt (already in LDS): reuse it for step kt + DEPTH
+        load_step(ra[u], rb[u]);
+        const _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
 #pragma unroll
-      for (int i = 0; i < TM; i++)
-        av[i] = *reinterpret_cast<const half8 *>(As + (wm0 + i * 32 + l32) * LDS_ROW + ks + half * 8);
+        for (int ks = 0; ks < BK16; ks += 16) {
+          half8 av[TM], bv[TN];
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-        bv[j] = *reinterpret_cast<const half8 *>(Bs + (wn0 + j * 32 + l32) * LDS_ROW + ks + half * 8);
+          for (int i = 0; i < TM; i++)
+            av[i] = *reinterpret_cast<const half8 *>(As + (wm0 + i * 32 + l32) * LDS_ROW + ks + half * 8);
 #pragma unroll
-      for (int i = 0; i < TM; i++)
+          for (int j = 0; j < TN; j++)
+            bv[j] = *reinterpret_cast<const half8 *>(Bs + (wn0 + j * 32 + l32) * LDS_ROW + ks + half * 8);
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+          for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) store_step(buf ^ 1, ra[(u + 1) % DEPTH], rb[(u + 1) % DEPTH]);
+        __syncthreads();
+      }
     }
-    if (kt + 1 < nk) store_step(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue: bias, activation, fp16, transpose through LDS ------------
@@ -271,15 +299,25 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
   const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 32 == 0 && a.K % 8 == 0 &&
                     aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y);
   if (fast) {
+    // Largest tile that still gives every CU two workgroups to overlap.
+    const int64_t want = 2 * (int64_t)ctx->num_cu;
+    auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
+#define LAUNCH_FAST(BM_, BN_, WM_, WN_)                                                                    \
+  do {                                                                                                     \
+    const int64_t tiles = tiles_of(BM_, BN_);                                                              \
+    if (tiles > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                      \
+    hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_>), dim3((unsigned)tiles), dim3(256), 0,    \
+                       ctx->stream, a);                                                                    \
+  } while (0)
     if (a.K <= 64) {
-      const int64_t tiles = ceil_div(a.K, 64) * ceil_div(NPQ, 128);
-      if (tiles > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<64, 128, 1, 4>), dim3((unsigned)tiles), dim3(256), 0, ctx->stream, a);
+      if (tiles_of(64, 128) >= want) LAUNCH_FAST(64, 128, 1, 4);
+      else LAUNCH_FAST(64, 64, 2, 2);
     } else {
-      const int64_t tiles = ceil_div(a.K, 128) * ceil_div(NPQ, 128);
-      if (tiles > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<128, 128, 2, 2>), dim3((unsigned)tiles), dim3(256), 0, ctx->stream, a);
+      if (tiles_of(128, 128) >= want) LAUNCH_FAST(128, 128, 2, 2);
+      else if (tiles_of(128, 64) >= want) LAUNCH_FAST(128, 64, 2, 2);
+      else LAUNCH_FAST(64, 64, 2, 2);
     }
+#undef LAUNCH_FAST
   } else {
     const int Kg = a.K / a.group;
     const int64_t tiles = ceil_div(Kg, 64) * ceil_div(NPQ, 64);
