@@ -23,7 +23,8 @@
  *     src/Tools/dnn-wrapper/cuda/wrapDNNMemOffset.cpp:27); every kernel here
  *     fully overwrites its output.
  *   - one dnnrtTranspose replaces the per-rank Transpose{2,3,4,6}D symbols.
- *   - new: dnnrtSync, dnnrtSetStream, dnnrtSetTensorFormat, dnnrtLayerNorm,
+ *   - new: dnnrtSync, dnnrtSetStream, dnnrtSetTensorFormat,
+ *     dnnrtSetFilterLayout, dnnrtLayerNorm,
  *     dnnrtGelu, dnnrtHostAlloc/Free, dnnrtLastError.
  *
  * The library is not re-entrant per handle; calls on one handle must come
@@ -50,6 +51,14 @@ enum { DNNRT_F32 = 0, DNNRT_F16 = 1, DNNRT_I64 = 2 };
  * NCHW, Y is written as NHWC (used for the first convolution of an fp16
  * channels-last program, whose input arrives from the host as NCHW). */
 enum { DNNRT_NCHW = 0, DNNRT_NHWC = 1, DNNRT_NCHW_TO_NHWC = 2 };
+
+/* Physical layout of fp32 convolution filters.  dimW is always passed in
+ * logical K,C/group,R,S order.  KCRS is the reference's (ONNX initializers as
+ * they come).  CRSK stores element (k, c, r, s) at ((c*R + r)*S + s)*K + k, so
+ * consecutive output channels are adjacent: a caller that owns the constants
+ * permutes them once on the host and the batch-1 kernels read them coalesced.
+ * fp16 filters follow the tensor format instead (NHWC => K,R,S,C). */
+enum { DNNRT_FILTER_KCRS = 0, DNNRT_FILTER_CRSK = 1 };
 
 /* activation modes: cudnnActivationMode_t values the reference emits
  * (src/Tools/dnn-wrapper/cudnn/CUDNNActiveFunc.cpp:8-91;
@@ -84,6 +93,9 @@ int32_t dnnrtStreamDestroy(dnnrtStream_t stream);
 int32_t dnnrtSetStream(dnnrtHandle_t handle, dnnrtStream_t stream);
 /* New.  Physical layout of rank-4 activations for subsequent calls. */
 int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format);
+/* New.  Physical layout of fp32 convolution filters for subsequent calls
+ * (DNNRT_FILTER_KCRS is the default and the reference's). */
+int32_t dnnrtSetFilterLayout(dnnrtHandle_t handle, int32_t layout);
 /* New.  Blocks until all work on the handle's stream is done; the reference
  * returns to the host without waiting for its device-to-host copies
  * (src/Tools/dnn-wrapper/cuda/wrapDNNMemcpy.cpp:32). */

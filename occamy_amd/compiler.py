@@ -120,7 +120,7 @@ class Graph:
         self.outputs = []
 
     def __del__(self):
-        if getattr(self, "_g", None):
+        if getattr(self, "_g", None) and lib is not None:  # module globals are gone at interpreter exit
             lib().dnncGraphDestroy(self._g)
             self._g = None
 
@@ -179,7 +179,7 @@ class Program:
         self._graph = graph  # owns the constants the program points at
 
     def __del__(self):
-        if getattr(self, "_p", None):
+        if getattr(self, "_p", None) and lib is not None:
             lib().dnncProgramDestroy(self._p)
             self._p = None
 
@@ -244,7 +244,7 @@ class Session:
         self._out_info = program.output_info()
 
     def close(self):
-        if getattr(self, "_s", None):
+        if getattr(self, "_s", None) and lib is not None:
             lib().dnncSessionDestroy(self._s)
             self._s = None
 

@@ -45,6 +45,7 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
   dnnrtContext *c = new dnnrtContext();
   c->stream = nullptr;
   c->format = DNNRT_NCHW;
+  c->filter_layout = DNNRT_FILTER_KCRS;
   c->device = dev;
   c->num_cu = prop.multiProcessorCount;
   *handle = c;
@@ -81,6 +82,16 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format) {
     return 1;
   }
   handle->format = format;
+  return 0;
+}
+
+int32_t dnnrtSetFilterLayout(dnnrtHandle_t handle, int32_t layout) {
+  if (!handle) { set_error("dnnrtSetFilterLayout: null handle"); return 1; }
+  if (layout != DNNRT_FILTER_KCRS && layout != DNNRT_FILTER_CRSK) {
+    set_error("dnnrtSetFilterLayout: unknown layout %d", layout);
+    return 1;
+  }
+  handle->filter_layout = layout;
   return 0;
 }
 

@@ -13,6 +13,7 @@
 struct dnnrtContext {
   hipStream_t stream;  // kernels of this handle are launched here
   int format;          // DNNRT_NCHW / DNNRT_NHWC / DNNRT_NCHW_TO_NHWC
+  int filter_layout;   // DNNRT_FILTER_KCRS / DNNRT_FILTER_CRSK (fp32 convolutions)
   int device;
   int num_cu;
 };

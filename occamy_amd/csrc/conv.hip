@@ -19,7 +19,7 @@ template <int R, int S>
 __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
     const float *__restrict__ X, const float *__restrict__ Wt, const float *__restrict__ bias,
     float *__restrict__ Y, int C, int H, int W, int K, int Kg, int P, int Q, int ph, int pw,
-    int sh, int sw, int rr, int ss, int act, int64_t total) {
+    int sh, int sw, int rr, int ss, int act, int64_t total, int w_k_stride, int w_tap_stride) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
   const int q = (int)(i % Q);
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
   const int c = k / Kg;
   const int Rr = R ? R : rr, Ss = S ? S : ss;
   const float *x = X + ((int64_t)n * C + c) * H * W;
-  const float *w = Wt + (int64_t)k * Rr * Ss;
+  const float *w = Wt + (int64_t)k * w_k_stride;  // tap (r, s) at w[(r * S + s) * w_tap_stride]
   const int ih0 = p * sh - ph, iw0 = q * sw - pw;
   float acc = 0.f;
 #pragma unroll
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
 #pragma unroll
     for (int s = 0; s < Ss; s++) {
       const int iw = iw0 + s;
-      if ((unsigned)iw < (unsigned)W) acc = fmaf(x[(int64_t)ih * W + iw], w[r * Ss + s], acc);
+      if ((unsigned)iw < (unsigned)W) acc = fmaf(x[(int64_t)ih * W + iw], w[(r * Ss + s) * w_tap_stride], acc);
     }
   }
   if (bias) acc += bias[k];
@@ -87,17 +87,22 @@ static bool parse_conv(const char *who, const int64_t *dX, const int64_t *dW, in
 
 static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const float *X,
                            const float *Wt, const float *bias, int act, float *Y) {
+  // Filter storage: K,C,R,S (the reference's) or C,R,S,K (k_out contiguous),
+  // which lets 32 lanes that own 32 consecutive output channels read one
+  // contiguous 128-byte line per reduction element.
+  const bool crsk = ctx->filter_layout == DNNRT_FILTER_CRSK;
   if (s.Cg == 1 && s.group > 1) {  // depthwise
     const int64_t total = (int64_t)s.N * s.K * s.P * s.Q;
     const int Kg = s.K / s.group;
     dim3 grid((unsigned)ceil_div(total, 256)), block(256);
     if (ceil_div(total, 256) > INT32_MAX) DNNRT_FAIL("conv: depthwise output too large");
+    const int w_k = crsk ? 1 : s.R * s.S, w_tap = crsk ? s.K : 1;
     if (s.R == 3 && s.S == 3)
       hipLaunchKernelGGL((dwconv_f32_nchw_kernel<3, 3>), grid, block, 0, ctx->stream, X, Wt, bias, Y,
-                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, total);
+                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, total, w_k, w_tap);
     else
       hipLaunchKernelGGL((dwconv_f32_nchw_kernel<0, 0>), grid, block, 0, ctx->stream, X, Wt, bias, Y,
-                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, total);
+                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, total, w_k, w_tap);
     DNNRT_CHECK_LAUNCH("conv(depthwise)");
     return Y;
   }
@@ -112,12 +117,15 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
   a.y_img_stride = (int64_t)s.K * s.P * s.Q;
   a.y_row_stride = (int64_t)s.P * s.Q;
   a.Z = s.group;
-  a.a_z_stride = (int64_t)Kg * a.Kdim;
+  // K,C,R,S: group g owns rows [g*Kg, (g+1)*Kg) of Kdim words each;
+  // C,R,S,K: element (m, k) of group g sits at k * K + g * Kg + m.
+  a.a_z_stride = crsk ? Kg : (int64_t)Kg * a.Kdim;
+  a.a_ld = s.K;
   a.x_z_stride = (int64_t)s.Cg * s.H * s.W;
   a.y_z_stride = (int64_t)Kg * s.P * s.Q;
   a.bias_z_stride = Kg;
-  a.b_kcontig = false; a.a_mcontig = false;
-  a.a_vec4 = (a.Kdim % 4 == 0) && aligned16(Wt);
+  a.b_kcontig = false; a.a_mcontig = crsk;
+  a.a_vec4 = !crsk && (a.Kdim % 4 == 0) && aligned16(Wt);
   a.b_vec4 = false;
   if (!launch_igemm_f32(ctx, a)) return nullptr;
   return Y;

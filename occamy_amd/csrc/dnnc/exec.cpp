@@ -32,7 +32,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
   if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
   LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
-  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
@@ -75,7 +75,17 @@ static void permute_kcrs_to_krsc(const uint8_t *src, uint8_t *dst, const Shape &
           std::memcpy(dst + (((k * R + r) * S + s) * C + c) * es, src + (((k * C + c) * R + r) * S + s) * es, (size_t)es);
 }
 
-bool Session::init(const Program *p, const std::string &runtime_path, int mode_, std::string &err) {
+// KCRS -> CRSK, element size es
+static void permute_kcrs_to_crsk(const uint8_t *src, uint8_t *dst, const Shape &w, int64_t es) {
+  const int64_t K = w[0], CRS = w[1] * w[2] * w[3];
+  for (int64_t k = 0; k < K; k++)
+    for (int64_t j = 0; j < CRS; j++)
+      std::memcpy(dst + (j * K + k) * es, src + (k * CRS + j) * es, (size_t)es);
+}
+
+static bool is_compute(OpKind k) { return k >= OP_CONVFWD && k <= OP_GELU; }
+
+bool Session::init(const Program *p,const std::string &runtime_path, int mode_, std::string &err) {
   prog = p;
   mode = mode_;
   if (prog->pool_bytes < 0) { err = "the program was compiled without the pool pass"; return false; }
@@ -87,19 +97,27 @@ bool Session::init(const Program *p, const std::string &runtime_path, int mode_,
   if (rt.dnnrtSetStream(handle, stream)) { err = rt_error("dnnrtSetStream"); return false; }
   ptr.assign(prog->value_store.size(), nullptr);
 
-  // Which constants are convolution filters (they are stored K,R,S,C for a
-  // channels-last program).
+  // Which constants are convolution filters and nothing else.  They are
+  // re-laid once, in the pinned host copy: K,R,S,C for a channels-last (fp16)
+  // program, C,R,S,K for fp32 programs on the GPU runtime.
   std::map<std::string, bool> is_filter;
-  if (prog->channels_last)
-    for (const Op *op : prog->ops)
-      if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV) {
-        const Value *w = op->operands[1];
-        if (w->def && w->def->kind == OP_MEM_OFFSET)
-          for (const auto &u : w->uses)
-            if (u.first->kind == OP_MEMCPY && u.first->operands[1]->def &&
-                u.first->operands[1]->def->kind == OP_HOST_CONST)
-              is_filter[u.first->operands[1]->def->const_name] = true;
-      }
+  for (const Op *op : prog->ops) {
+    if (op->kind != OP_MEMCPY || op->mode != 1) continue;
+    const Value *src = op->operands[1];
+    if (!src->def || src->def->kind != OP_HOST_CONST) continue;
+    const std::string &name = src->def->const_name;
+    bool only_filter = true, any = false;
+    for (const auto &u : op->operands[0]->uses) {
+      if (u.first == op) continue;
+      const bool conv = u.first->kind == OP_CONVFWD || u.first->kind == OP_CONV_BIAS_ACTIV;
+      if (conv && u.second == 1) any = true;
+      else if (is_compute(u.first->kind)) only_filter = false;
+    }
+    const bool f = any && only_filter;
+    auto it = is_filter.find(name);
+    if (it == is_filter.end()) is_filter[name] = f;
+    else it->second = it->second && f;
+  }
 
   // Constants: one pinned host copy each (the reference keeps them as globals
   // of the model library); function results: one pinned buffer each.
@@ -109,10 +127,16 @@ bool Session::init(const Program *p, const std::string &runtime_path, int mode_,
       const GTensor &t = prog->graph->tensors.at(op->const_name);
       void *h = nullptr;
       if (rt.dnnrtHostAlloc(&h, (int64_t)t.data.size())) { err = rt_error("dnnrtHostAlloc"); return false; }
-      if (is_filter.count(op->const_name) && t.shape.size() == 4)
+      const auto fit = is_filter.find(op->const_name);
+      const bool filter = fit != is_filter.end() && fit->second && t.shape.size() == 4;
+      if (filter && prog->channels_last) {
         permute_kcrs_to_krsc(t.data.data(), (uint8_t *)h, t.shape, dtype_bytes(t.dtype));
-      else
+      } else if (filter && !host_backend && t.dtype == F32) {
+        permute_kcrs_to_crsk(t.data.data(), (uint8_t *)h, t.shape, dtype_bytes(t.dtype));
+        crsk_const[op->const_name] = true;
+      } else {
         std::memcpy(h, t.data.data(), t.data.size());
+      }
       host_const[op->const_name] = h;
       ptr[(size_t)op->result->id] = h;
       weight_bytes += align_up((int64_t)t.data.size(), 256);
@@ -123,6 +147,13 @@ bool Session::init(const Program *p, const std::string &runtime_path, int mode_,
       host_out[(size_t)op->out_index] = h;
       ptr[(size_t)op->result->id] = h;
     }
+  }
+  filter_crsk.assign(prog->value_store.size(), 0);
+  for (const Op *op : prog->ops) {
+    if (op->kind != OP_MEMCPY || op->mode != 1) continue;
+    const Value *src = op->operands[1];
+    if (src->def && src->def->kind == OP_HOST_CONST && crsk_const.count(src->def->const_name))
+      filter_crsk[(size_t)op->operands[0]->id] = 1;
   }
   for (const Value *a : prog->args) {
     void *h = nullptr;
@@ -179,8 +210,15 @@ bool Session::issue(const Op *op, std::string &err) {
       cur_format = f;
     }
   }
+  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV) {
+    const int lay = filter_crsk[(size_t)op->operands[1]->id] ? DNNRT_FILTER_CRSK : DNNRT_FILTER_KCRS;
+    if (lay != cur_filter_layout) {
+      if (rt.dnnrtSetFilterLayout(handle, lay)) { err = rt_error("dnnrtSetFilterLayout"); return false; }
+      cur_filter_layout = lay;
+    }
+  }
   void *r = nullptr;
-  auto pad4 = [](const Shape &s) { Shape o = s; while (o.size() < 4) o.push_back(1); return o; };
+  auto pad4 =[](const Shape &s) { Shape o = s; while (o.size() < 4) o.push_back(1); return o; };
   switch (op->kind) {
     case OP_CONVFWD:
       r = rt.dnnrtConv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), 0, op->algo, op->group,
@@ -270,8 +308,6 @@ bool Session::issue(const Op *op, std::string &err) {
   ptr[(size_t)op->result->id] = r;
   return true;
 }
-
-static bool is_compute(OpKind k) { return k >= OP_CONVFWD && k <= OP_GELU; }
 
 // The reference's per-inference sequence, call for call.
 bool Session::run_occamy(const void *const *inputs, void *const *outputs, std::string &err) {

@@ -17,6 +17,7 @@ struct RuntimeApi {
   decltype(&::dnnrtStreamDestroy) dnnrtStreamDestroy = nullptr;
   decltype(&::dnnrtSetStream) dnnrtSetStream = nullptr;
   decltype(&::dnnrtSetTensorFormat) dnnrtSetTensorFormat = nullptr;
+  decltype(&::dnnrtSetFilterLayout) dnnrtSetFilterLayout = nullptr;
   decltype(&::dnnrtSync) dnnrtSync = nullptr;
   decltype(&::dnnrtLastError) dnnrtLastError = nullptr;
   decltype(&::dnnrtIsHostBackend) dnnrtIsHostBackend = nullptr;
@@ -84,7 +85,9 @@ class Session {
   dnnrtHandle_t handle = nullptr;
   dnnrtStream_t stream = nullptr;
   bool host_backend = false;
-  int cur_format = 0;
+  int cur_format = 0, cur_filter_layout = 0;
+  std::map<std::string, bool> crsk_const;  // constants re-laid C,R,S,K on the host
+  std::vector<char> filter_crsk;           // value id -> its device copy is C,R,S,K
   void *pool = nullptr, *weights = nullptr, *graph = nullptr;
   std::vector<void *> ptr;  // value id -> address (host or device)
   std::map<std::string, void *> host_const;

@@ -12,7 +12,8 @@
 namespace dnnrt {
 
 struct IgemmArgs {
-  const float *A;     // [M][Kdim] (k contiguous), or [Kdim][M] when a_mcontig
+  const float *A;     // [M][Kdim] (k contiguous), or [Kdim][a_ld] when a_mcontig
+  int64_t a_ld;       // a_mcontig: elements between consecutive k (>= M)
   const float *X;     // conv input / right matrix
   float *Y;
   const float *bias;  // per row m, may be null
@@ -40,5 +41,7 @@ bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a);
 // The variant for problems too small to fill the chip with LDS-staged tiles
 // (igemm_f32_direct.hip); rsmode / layout as computed by launch_igemm_f32.
 bool launch_igemm_f32_direct(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout);
+// 3x3 / 1x1 specialisations of the above (igemm_f32_small.hip); `launched` says whether one applied.
+bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout, bool &launched);
 
 }  // namespace dnnrt

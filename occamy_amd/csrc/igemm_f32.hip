@@ -108,7 +108,7 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
       for (int i = 0; i < AM_PER; i++) {
         const int idx = tid + i * NT, mm = idx % BM, kk = idx / BM;
         const int m = m0 + mm, k = k0 + kk;
-        ram[i] = (m < a.M && k < a.Kdim) ? Ag[(int64_t)k * a.M + m] : 0.f;
+        ram[i] = (m < a.M && k < a.Kdim) ? Ag[(int64_t)k * a.a_ld + m] : 0.f;
       }
     }
     // B
@@ -249,8 +249,14 @@ static bool launch_tile(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode,
       default: LAUNCH(0, 0); break;
     }
   } else if (layout == 1) LAUNCH(1, 1);
-  else if (layout == 2) LAUNCH(1, 2);
-  else LAUNCH(1, 3);
+  else if (layout == 2) {  // m-contiguous A: transposed left matrix, or filters stored C,R,S,K
+    switch (rsmode) {
+      case 1: LAUNCH(1, 2); break;
+      case 3: LAUNCH(3, 2); break;
+      case 7: LAUNCH(7, 2); break;
+      default: LAUNCH(0, 2); break;
+    }
+  } else LAUNCH(1, 3);
 #undef LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("igemm_f32: launch failed: %s", hipGetErrorString(e)); return false; }
@@ -265,7 +271,7 @@ bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a) {
   else if (a.R == 3 && a.S == 3) rsmode = 3;
   else if (a.R == 7 && a.S == 7) rsmode = 7;
   const int layout = (a.b_kcontig ? 1 : 0) | (a.a_mcontig ? 2 : 0);
-  if (layout != 0 && rsmode != 1) { set_error("igemm_f32: transposed operands need a 1x1 geometry"); return false; }
+  if ((layout & 1) && rsmode != 1) { set_error("igemm_f32: a k-contiguous right operand needs a 1x1 geometry"); return false; }
 
   // Largest tile that still gives every CU a workgroup; small problems fall
   // through to the one-wave 32x32 tile.

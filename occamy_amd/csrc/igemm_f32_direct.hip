@@ -76,7 +76,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; j++) av[j] = (m_ok && ka + j < kend) ? Ag[(int64_t)(ka + j) * a.M + m] : 0.f;
+      for (int j = 0; j < 4; j++) av[j] = (m_ok && ka + j < kend) ? Ag[(int64_t)(ka + j) * a.a_ld + m] : 0.f;
     }
     // ---- B ----
     if (B_KC) {
@@ -159,12 +159,21 @@ static void launch_ks(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, i
       default: LAUNCH(0, 0); break;
     }
   } else if (layout == 1) LAUNCH(1, 1);
-  else if (layout == 2) LAUNCH(1, 2);
-  else LAUNCH(1, 3);
+  else if (layout == 2) {
+    switch (rsmode) {
+      case 1: LAUNCH(1, 2); break;
+      case 3: LAUNCH(3, 2); break;
+      case 7: LAUNCH(7, 2); break;
+      default: LAUNCH(0, 2); break;
+    }
+  } else LAUNCH(1, 3);
 #undef LAUNCH
 }
 
 bool launch_igemm_f32_direct(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout) {
+  bool launched = false;
+  if (!launch_igemm_f32_small(ctx, a, rsmode, layout, launched)) return false;
+  if (launched) return true;
   const int64_t tiles64 = ceil_div(a.M, 32) * ceil_div(a.Ncols, 32);
   if (tiles64 > INT32_MAX) { set_error("igemm_f32: too many tiles"); return false; }
   const int tiles = (int)tiles64;

@@ -1,0 +1,246 @@
+// Two specialisations of the small-problem fp32 implicit GEMM
+// (igemm_f32_direct.hip) for the shapes that make up a batch-1 CNN or a short
+// transformer: 3x3 convolutions and 1x1 convolutions / plain matrix products.
+//
+// Same decomposition -- one 32x32 tile of D per workgroup, KS wavefronts
+// splitting the reduction, operands straight from global memory into MFMA
+// registers -- but the per-element index arithmetic is gone (a wave64 VALU
+// instruction costs 4 cycles, and ~30 of them per loaded element made the
+// general kernel issue-bound):
+//   3x3: a lane owns one output pixel; its nine tap offsets and nine validity
+//        masks are computed once.  One iteration = 2 channels x 9 taps
+//        (half-wave h takes channel c+h), i.e. nine MFMAs fed by nine
+//        contiguous filter words and nine input words at base + tap_off[j].
+//   1x1: the reduction index is the channel; addresses advance by a constant.
+// All loads are unconditional (clamped addresses; what must not contribute is
+// masked on the B side at the time of use), so the compiler can track the
+// hardware load counter and the register ring keeps several iterations of
+// loads in flight.  Offsets are 32-bit: the dispatcher only takes these
+// kernels when every operand is below 2^31 elements.
+#include "igemm_f32.h"
+
+namespace dnnrt {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float mask_f(float v, unsigned m) { return __uint_as_float(__float_as_uint(v) & m); }
+
+// Sum the KS partial tiles in LDS, then bias / residual / activation / store by wavefront 0.
+template <int KS>
+__device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, float (*red)[16][64], int wave, int lane,
+                                                 int m0, int col, bool col_ok, int z) {
+  if (KS > 1) {
+    if (wave > 0) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) red[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < KS - 1; w++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] += red[w][r][lane];
+  }
+  if (!col_ok) return;
+  const int half = lane >> 5, PQ = a.P * a.Q;
+  float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
+  const float *__restrict__ Cg = a.Cin ? a.Cin + (int64_t)z * a.y_z_stride : nullptr;
+  const float *__restrict__ biasg = a.bias ? a.bias + (int64_t)z * a.bias_z_stride : nullptr;
+  const int img = col / PQ, pq = col - img * PQ;
+  const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const int mm = m0 + 8 * (r >> 2) + 4 * half + (r & 3);
+    if (mm >= a.M) continue;
+    const int64_t off = ycol + (int64_t)mm * a.y_row_stride;
+    float v = a.alpha * acc[r];
+    if (biasg) v += biasg[mm];
+    if (Cg) v += a.beta * Cg[off];
+    if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+    Yg[off] = v;
+  }
+}
+
+template <int KS, bool AMC>
+__global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmArgs a, const int c_per_wave) {
+  __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
+  const int tiles_n = (a.Ncols + 31) / 32;
+  const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+  const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
+  const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
+  const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
+
+  const int m = m0 + l32, mrow = m < a.M ? m : 0;
+  const int col = n0 + l32;
+  const bool col_ok = col < a.Ncols;
+  const int PQ = a.P * a.Q, HW = a.H * a.W, C = a.Kdim / 9;
+  const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
+  const int p = pq / a.Q, q = pq - p * a.Q;
+  const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
+  unsigned tap_off[9], tap_mask[9];
+#pragma unroll
+  for (int j = 0; j < 9; j++) {
+    const int ih = ih0 + j / 3, iw = iw0 + j % 3;
+    const bool ok = col_ok && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+    tap_off[j] = ok ? (unsigned)(ih * a.W + iw) : 0u;
+    tap_mask[j] = ok ? 0xffffffffu : 0u;
+  }
+  const unsigned x_img = (unsigned)((int64_t)img * a.x_img_stride);
+  const unsigned a_row = (unsigned)mrow * (unsigned)a.Kdim, lda = (unsigned)a.a_ld;
+
+  const int cbeg = wave * c_per_wave, cend = min(C, cbeg + c_per_wave);
+  const int niter = c_per_wave >> 1;
+
+  constexpr int DEPTH = 2;
+  float ra[DEPTH][9], rb[DEPTH][9];
+  unsigned cm[DEPTH];
+  auto load_iter = [&](int i, float (&av)[9], float (&bv)[9], unsigned &cmask) {
+    const int c = cbeg + 2 * i + half;
+    const unsigned cc = (unsigned)min(c, C - 1);
+    cmask = c < cend ? 0xffffffffu : 0u;
+    const unsigned bo = x_img + cc * (unsigned)HW;
+    if (AMC) {  // filter stored [k][K_out]: 32 lanes read 32 consecutive words
+      const unsigned ao = cc * 9u * lda + (unsigned)mrow;
+#pragma unroll
+      for (int j = 0; j < 9; j++) av[j] = Ag[ao + (unsigned)j * lda];
+    } else {
+      const unsigned ao = a_row + cc * 9u;
+#pragma unroll
+      for (int j = 0; j < 9; j++) av[j] = Ag[ao + j];
+    }
+#pragma unroll
+    for (int j = 0; j < 9; j++) bv[j] = Xg[bo + tap_off[j]];
+  };
+
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++) load_iter(d, ra[d], rb[d], cm[d]);
+  for (int i0 = 0; i0 < niter; i0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; u++) {
+      if (i0 + u < niter) {
+#pragma unroll
+        for (int j = 0; j < 9; j++)
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u][j], mask_f(rb[u][j], tap_mask[j] & cm[u]), acc, 0, 0, 0);
+        load_iter(i0 + u + DEPTH, ra[u], rb[u], cm[u]);
+      }
+    }
+  }
+  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z);
+}
+
+// 1x1 geometry (convolution, possibly strided, or matrix product with A rows
+// k-contiguous and B columns contiguous); Kdim % 4 == 0, A rows 16-byte aligned.
+template <int KS, bool AMC>
+__global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmArgs a, const int k_per_wave) {
+  __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
+  const int tiles_n = (a.Ncols + 31) / 32;
+  const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+  const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
+  const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
+  const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
+
+  const int m = m0 + l32, mrow = m < a.M ? m : 0;
+  const int col = n0 + l32;
+  const bool col_ok = col < a.Ncols;
+  const int PQ = a.P * a.Q, HW = a.H * a.W;
+  const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
+  const int p = pq / a.Q, q = pq - p * a.Q;
+  const unsigned x_pix = (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
+  const unsigned a_row = (unsigned)mrow * (unsigned)a.Kdim, lda = (unsigned)a.a_ld;
+
+  const int kbeg = wave * k_per_wave, kend = min(a.Kdim, kbeg + k_per_wave);
+  const int niter = k_per_wave >> 3;
+
+  constexpr int DEPTH = 4;
+  float4 ra[DEPTH];
+  float rb[DEPTH][4];
+  unsigned km[DEPTH];
+  auto load_iter = [&](int i, float4 &av, float (&bv)[4], unsigned &kmask) {
+    const int ka = kbeg + 8 * i + 4 * half;
+    const unsigned kc = (unsigned)min(ka, a.Kdim - 4);
+    kmask = ka < kend ? 0xffffffffu : 0u;
+    if (AMC) {
+      const unsigned ao = kc * lda + (unsigned)mrow;
+      av.x = Ag[ao]; av.y = Ag[ao + lda]; av.z = Ag[ao + 2u * lda]; av.w = Ag[ao + 3u * lda];
+    } else {
+      av = *reinterpret_cast<const float4 *>(Ag + (a_row + kc));
+    }
+    const unsigned bo = x_pix + kc * (unsigned)HW;
+#pragma unroll
+    for (int j = 0; j < 4; j++) bv[j] = Xg[bo + (unsigned)(j * HW)];
+  };
+
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++) load_iter(d, ra[d], rb[d], km[d]);
+  for (int i0 = 0; i0 < niter; i0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; u++) {
+      if (i0 + u < niter) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].x, mask_f(rb[u][0], km[u]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].y, mask_f(rb[u][1], km[u]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].z, mask_f(rb[u][2], km[u]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].w, mask_f(rb[u][3], km[u]), acc, 0, 0, 0);
+        load_iter(i0 + u + DEPTH, ra[u], rb[u], km[u]);
+      }
+    }
+  }
+  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z);
+}
+
+// Returns true if one of the specialised kernels took the problem.
+bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout, bool &launched) {
+  launched = false;
+  if (layout != 0 && layout != 2) return true;
+  const bool amc = layout == 2;
+  // 32-bit element offsets inside the kernels
+  const int64_t a_elems = amc ? (int64_t)a.Kdim * a.a_ld : (int64_t)a.M * a.Kdim;
+  const int64_t x_elems = (int64_t)((a.Ncols + a.P * a.Q - 1) / (a.P * a.Q)) * a.x_img_stride + (int64_t)a.Kdim * a.H * a.W;
+  if (a_elems >= (1ll << 31) || x_elems >= (1ll << 31)) return true;
+  const bool is3x3 = rsmode == 3 && a.Kdim % 9 == 0;
+  const bool is1x1 = rsmode == 1 && (amc || a.a_vec4) && a.Kdim % 4 == 0 && a.Kdim >= 4;
+  if (!is3x3 && !is1x1) return true;
+
+  const int64_t tiles64 = ceil_div(a.M, 32) * ceil_div(a.Ncols, 32);
+  if (tiles64 > INT32_MAX) return true;
+  const int tiles = (int)tiles64;
+  const int64_t want_waves = (int64_t)ctx->num_cu * 8;
+  const int red_len = is3x3 ? a.Kdim / 9 : a.Kdim;   // channels
+  const int min_slice = is3x3 ? 4 : 32;              // reduction slice worth a wavefront
+  int ks = 1;
+  while (ks < 8 && (int64_t)tiles * a.Z * ks < want_waves && ceil_div(red_len, ks * 2) >= min_slice) ks *= 2;
+  dim3 grid(tiles, 1, a.Z);
+#define LAUNCH_KS2(KERNEL, AMC_, ARG)                                                                  \
+  switch (ks) {                                                                                          \
+    case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, a, ARG); break;        \
+    case 2: hipLaunchKernelGGL((KERNEL<2, AMC_>), grid, dim3(128), 0, ctx->stream, a, ARG); break;       \
+    case 4: hipLaunchKernelGGL((KERNEL<4, AMC_>), grid, dim3(256), 0, ctx->stream, a, ARG); break;       \
+    default: hipLaunchKernelGGL((KERNEL<8, AMC_>), grid, dim3(512), 0, ctx->stream, a, ARG); break;      \
+  }
+#define LAUNCH_KS(KERNEL, ARG)                                                                         \
+  do {                                                                                                 \
+    if (amc) { LAUNCH_KS2(KERNEL, true, ARG) } else { LAUNCH_KS2(KERNEL, false, ARG) }                 \
+  } while (0)
+  if (is3x3) {
+    const int c_per_wave = (int)(ceil_div(ceil_div(red_len, ks), 2) * 2);
+    LAUNCH_KS(conv3x3_f32_small_kernel, c_per_wave);
+  } else {
+    const int k_per_wave = (int)(ceil_div(ceil_div(red_len, ks), 8) * 8);
+    LAUNCH_KS(conv1x1_f32_small_kernel, k_per_wave);
+  }
+#undef LAUNCH_KS
+#undef LAUNCH_KS2
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_error("igemm_f32(small): launch failed: %s", hipGetErrorString(e)); return false; }
+  launched = true;
+  return true;
+}
+
+}  // namespace dnnrt

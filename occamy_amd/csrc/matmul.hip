@@ -77,7 +77,7 @@ static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, co
   a.H = 1; a.W = N; a.R = 1; a.S = 1; a.P = 1; a.Q = N; a.ph = 0; a.pw = 0; a.sh = 1; a.sw = 1;
   a.x_img_stride = 0; a.y_img_stride = 0; a.y_row_stride = N;
   a.Z = Z; a.a_z_stride = az; a.x_z_stride = bz; a.y_z_stride = yz; a.bias_z_stride = 0;
-  a.b_kcontig = transB; a.a_mcontig = transA;
+  a.b_kcontig = transB; a.a_mcontig = transA; a.a_ld = M;
   a.a_vec4 = !transA && (K % 4 == 0) && aligned16(A) && (az % 4 == 0);
   a.b_vec4 = transB && (K % 4 == 0) && aligned16(B) && (bz % 4 == 0);
   return launch_igemm_f32(ctx, a);

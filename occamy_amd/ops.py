@@ -48,6 +48,9 @@ class Ops:
     def set_format(self, fmt):
         self._check(self.lib.dnnrtSetTensorFormat(self.handle, fmt), "dnnrtSetTensorFormat")
 
+    def set_filter_layout(self, layout):
+        self._check(self.lib.dnnrtSetFilterLayout(self.handle, layout), "dnnrtSetFilterLayout")
+
     def sync(self):
         self._check(self.lib.dnnrtSync(self.handle), "dnnrtSync")
 

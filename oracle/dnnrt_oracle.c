@@ -147,6 +147,14 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t h, int32_t format) {
   h->format = format;
   return 0;
 }
+int32_t dnnrtSetFilterLayout(dnnrtHandle_t h, int32_t layout) {
+  (void)h;
+  if (layout != DNNRT_FILTER_KCRS) {
+    snprintf(g_err, sizeof g_err, "oracle: only K,C,R,S filters are implemented");
+    return 1;
+  }
+  return 0;
+}
 int32_t dnnrtSync(dnnrtHandle_t h) { (void)h; return 0; }
 static int32_t no_graph(void) { snprintf(g_err, sizeof g_err, "oracle: no stream capture on the host"); return 1; }
 int32_t dnnrtGraphBegin(dnnrtHandle_t h) { (void)h; return no_graph(); }

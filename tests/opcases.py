@@ -12,20 +12,28 @@ def conv_out_hw(H, W, R, S, pads, strides):
     return (H + 2 * pads[0] - R) // strides[0] + 1, (W + 2 * pads[1] - S) // strides[1] + 1
 
 
-def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None):
+def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crsk=False):
+    """crsk: hand the filter over stored C,R,S,K (the dims stay logical K,C,R,S)."""
     N, C, H, W = x.shape
     K, Cg, R, S = w.shape
     P, Q = conv_out_hw(H, W, R, S, pads, strides)
     dt = DT[x.dtype]
-    X, Wt = be.put(x), be.put(w)
+    X = be.put(x)
+    Wt = be.put(np.ascontiguousarray(w.transpose(1, 2, 3, 0)) if crsk else w)
     Y = be.empty((N, K, max(P, 1), max(Q, 1)), x.dtype)  # the call rejects empty outputs itself
-    if b is None:
-        assert activ is None
-        be.ops.conv(be.ptr(X), x.shape, be.ptr(Wt), w.shape, pads, strides, be.ptr(Y), group, dt)
-    else:
-        B = be.put(b)
-        be.ops.conv_bias_activ(be.ptr(X), x.shape, be.ptr(Wt), w.shape, be.ptr(B), pads, strides,
-                               activ if activ is not None else _abi.ACT_IDENTITY, be.ptr(Y), group, dt)
+    if crsk:
+        be.ops.set_filter_layout(_abi.FILTER_CRSK)
+    try:
+        if b is None:
+            assert activ is None
+            be.ops.conv(be.ptr(X), x.shape, be.ptr(Wt), w.shape, pads, strides, be.ptr(Y), group, dt)
+        else:
+            B = be.put(b)
+            be.ops.conv_bias_activ(be.ptr(X), x.shape, be.ptr(Wt), w.shape, be.ptr(B), pads, strides,
+                                   activ if activ is not None else _abi.ACT_IDENTITY, be.ptr(Y), group, dt)
+    finally:
+        if crsk:
+            be.ops.set_filter_layout(_abi.FILTER_KCRS)
     be.sync()
     return be.get(Y)
 

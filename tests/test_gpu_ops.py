@@ -69,6 +69,10 @@ def test_conv_f32(gpu, cpu, case):
     close(got, ref)
     assert (got >= 0).all()
     close(oc.conv(gpu, x, w, b, *args, _abi.ACT_IDENTITY), oc.conv(cpu, x, w, b, *args, _abi.ACT_IDENTITY))
+    # the same filter handed over C,R,S,K: same kernels' K,C,R,S result up to
+    # the summation order of the tile shapes each layout selects
+    close(oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, crsk=True), ref)
+    close(oc.conv(gpu, x, w, None, *args, crsk=True), oc.conv(cpu, x, w, None, *args))
 
 
 def test_conv_closed_forms(gpu):

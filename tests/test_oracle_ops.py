@@ -331,3 +331,14 @@ def test_data_movement(be):
     np.testing.assert_array_equal(oc.gather(be, x, np.array([2, 0]), 2), np.take(x, [2, 0], 2))
     with pytest.raises(RuntimeError):
         oc.gather(be, table, np.array([11]), 0)
+
+
+def test_layouts_the_oracle_lacks_are_refused(be):
+    # The oracle restates the reference, which knows N,C,H,W tensors and
+    # K,C,R,S filters only; asking it for anything else must fail, not drift.
+    with pytest.raises(RuntimeError):
+        be.ops.set_format(_abi.NHWC)
+    with pytest.raises(RuntimeError):
+        be.ops.set_filter_layout(_abi.FILTER_CRSK)
+    be.ops.set_format(_abi.NCHW)
+    be.ops.set_filter_layout(_abi.FILTER_KCRS)
