@@ -28,11 +28,11 @@ PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
 def build_workload(name):
     from occamy_amd import models
     if name == "resnet50_fp32_bs1":
-        return models.resnet50(1, np.float32), dict(fusion=True), 1, "img/s", "f32"
+        return models.resnet50(1, np.float32), dict(fusion=True, fuse_residual=True), 1, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
-        return models.resnet50(64, np.float16, seed=5), dict(fusion=True, channels_last=True), 64, "img/s", "f16"
+        return models.resnet50(64, np.float16, seed=5), dict(fusion=True, fuse_residual=True, channels_last=True), 64, "img/s", "f16"
     if name == "mobilenet_v2_fp32_bs1":
-        return models.mobilenet_v2(1, np.float32), dict(fusion=True), 1, "img/s", "f32"
+        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
         return models.bert_encoder(), dict(), 1, "seq/s", "f32"
     if name == "single_conv_fp32":
@@ -99,7 +99,11 @@ def main():
                 c["ms"] += float(ms)
             res["by_class"] = by_class
         # the reference's per-inference semantics: pool alloc, all weights H2D, kernels, D2H, sync, pool free
-        so = prog.session(compiler.MODE_OCCAMY)
+        # (compiled with the reference's own flags: no residual fusion)
+        (ref_graph, _), _, _, _, _ = build_workload(name)  # a graph compiles once; the builders are seeded
+        ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k != "fuse_residual"})
+        res["pool_bytes_reference_flags"] = ref_prog.pool_bytes
+        so = ref_prog.session(compiler.MODE_OCCAMY)
         so.run(*inputs)
         n = max(3, min(20, steps // 10))
         t0 = time.perf_counter()
@@ -151,14 +155,16 @@ def main():
         "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic",
-        "config": {"workload": args.workload, "batch": main_res["batch"], "fusion": "conv+bias+relu",
+        "config": {"workload": args.workload, "batch": main_res["batch"],
+                   "fusion": "conv+bias+relu, conv+bias+residual add+relu",
                    "mode": "weights and input resident in HBM, kernels replayed from a captured graph",
                    "kernels_per_step": main_res["kernels_per_step"]},
         "roofline": roof,
         "cpu_baseline": cpu,
-        "pool_bytes": main_res["pool_bytes"], "weights_bytes": main_res["weights_bytes"],
+        "pool_bytes": main_res["pool_bytes"], "pool_bytes_reference_flags": main_res["pool_bytes_reference_flags"],
+        "weights_bytes": main_res["weights_bytes"],
         "occamy_semantics": {"value": main_res["occamy_semantics_value"], "unit": main_res["unit"],
-                             "what": "per inference: pool hipMalloc, every weight H2D into its pool slot, kernels, D2H, sync, pool free"},
+                             "what": "reference flags (no residual fusion); per inference: pool hipMalloc, every weight H2D into its pool slot, kernels, D2H, sync, pool free"},
         "by_class": {k: {"launches": v["launches"], "ms": round(v["ms"], 4),
                          "TFLOP/s": round(v["flops"] / max(v["ms"], 1e-9) / 1e9, 3),
                          "GB/s": round(v["bytes"] / max(v["ms"], 1e-9) / 1e6, 1)} for k, v in main_res["by_class"].items()},

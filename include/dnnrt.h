@@ -160,6 +160,21 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X,
                          int64_t workspaceBytes, int64_t algo, int64_t group,
                          const int64_t *pads, const int64_t *strides,
                          int64_t activMode, void *Y, int32_t dtype);
+/* New: the same call with the residual operand that
+ * cudnnConvolutionBiasActivationForward has and the reference passes with a
+ * zero weight (CUDNNConvBiasReluFunc.cpp:94-112: alpha2 = 0, z = y).
+ * Y = act((conv(X, W) + B) + Z), Z shaped and laid out like Y, not
+ * overlapping it.
+ * It replaces the conv -> add -> relu chain that closes a residual block; the
+ * sums are formed in that chain's order. */
+void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X,
+                            const int64_t *dimX, const void *W,
+                            const int64_t *dimW, const void *B,
+                            const int64_t *dimB, const void *Z,
+                            void *workspace, int64_t workspaceBytes,
+                            int64_t algo, int64_t group, const int64_t *pads,
+                            const int64_t *strides, int64_t activMode, void *Y,
+                            int32_t dtype);
 
 /* ---- elementwise / broadcast ----------------------------------------- */
 

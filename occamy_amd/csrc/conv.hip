@@ -18,7 +18,7 @@ namespace dnnrt {
 template <int R, int S>
 __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
     const float *__restrict__ X, const float *__restrict__ Wt, const float *__restrict__ bias,
-    float *__restrict__ Y, int C, int H, int W, int K, int Kg, int P, int Q, int ph, int pw,
+    const float *__restrict__ Zr, float *__restrict__ Y, int C, int H, int W, int K, int Kg, int P, int Q, int ph, int pw,
     int sh, int sw, int rr, int ss, int act, int64_t total, int w_k_stride, int w_tap_stride) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
@@ -45,6 +45,7 @@ __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
     }
   }
   if (bias) acc += bias[k];
+  if (Zr) acc += Zr[i];
   if (act == DNNRT_ACT_RELU) acc = acc < 0.f ? 0.f : acc;
   Y[i] = acc;
 }
@@ -86,7 +87,7 @@ static bool parse_conv(const char *who, const int64_t *dX, const int64_t *dW, in
 }
 
 static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const float *X,
-                           const float *Wt, const float *bias, int act, float *Y) {
+                           const float *Wt, const float *bias, const float *Z, int act, float *Y) {
   // Filter storage: K,C,R,S (the reference's) or C,R,S,K (k_out contiguous),
   // which lets 32 lanes that own 32 consecutive output channels read one
   // contiguous 128-byte line per reduction element.
@@ -98,18 +99,18 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
     if (ceil_div(total, 256) > INT32_MAX) DNNRT_FAIL("conv: depthwise output too large");
     const int w_k = crsk ? 1 : s.R * s.S, w_tap = crsk ? s.K : 1;
     if (s.R == 3 && s.S == 3)
-      hipLaunchKernelGGL((dwconv_f32_nchw_kernel<3, 3>), grid, block, 0, ctx->stream, X, Wt, bias, Y,
+      hipLaunchKernelGGL((dwconv_f32_nchw_kernel<3, 3>), grid, block, 0, ctx->stream, X, Wt, bias, Z, Y,
                          s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, total, w_k, w_tap);
     else
-      hipLaunchKernelGGL((dwconv_f32_nchw_kernel<0, 0>), grid, block, 0, ctx->stream, X, Wt, bias, Y,
+      hipLaunchKernelGGL((dwconv_f32_nchw_kernel<0, 0>), grid, block, 0, ctx->stream, X, Wt, bias, Z, Y,
                          s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, total, w_k, w_tap);
     DNNRT_CHECK_LAUNCH("conv(depthwise)");
     return Y;
   }
   IgemmArgs a{};
   const int Kg = s.K / s.group;
-  a.A = Wt; a.X = X; a.Y = Y; a.bias = bias; a.Cin = nullptr;
-  a.alpha = 1.f; a.beta = 0.f; a.act = act;
+  a.A = Wt; a.X = X; a.Y = Y; a.bias = bias; a.Cin = Z;  // residual: (acc + bias) + Z
+  a.alpha = 1.f; a.beta = Z ? 1.f : 0.f; a.act = act;
   a.M = Kg; a.Kdim = s.Cg * s.R * s.S; a.Ncols = s.N * s.P * s.Q;
   a.H = s.H; a.W = s.W; a.R = s.R; a.S = s.S; a.P = s.P; a.Q = s.Q;
   a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw;
@@ -132,7 +133,7 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
 }
 
 static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX,
-                           const void *W, const int64_t *dW, const void *B, int64_t group,
+                           const void *W, const int64_t *dW, const void *B, const void *Z, int64_t group,
                            const int64_t *pads, const int64_t *strides, int act, void *Y,
                            int32_t dtype) {
   if (!h) DNNRT_FAIL("%s: null handle", who);
@@ -141,11 +142,11 @@ static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, cons
   if (!parse_conv(who, dX, dW, group, pads, strides, s)) return nullptr;
   if (dtype == DNNRT_F32) {
     if (h->format != DNNRT_NCHW) DNNRT_FAIL("%s: fp32 tensors are NCHW only", who);
-    return conv_f32_nchw(h, s, (const float *)X, (const float *)W, (const float *)B, act, (float *)Y);
+    return conv_f32_nchw(h, s, (const float *)X, (const float *)W, (const float *)B, (const float *)Z, act, (float *)Y);
   }
   if (dtype == DNNRT_F16) {
     ConvF16Args a{};
-    a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Y = (__half *)Y;
+    a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Z = (const __half *)Z; a.Y = (__half *)Y;
     a.N = s.N; a.C = s.C; a.H = s.H; a.W = s.W; a.K = s.K; a.Cg = s.Cg; a.R = s.R; a.S = s.S;
     a.P = s.P; a.Q = s.Q; a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw; a.group = s.group;
     a.act = act; a.format = h->format;
@@ -163,7 +164,7 @@ void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const 
                 const int64_t *dimW, void *workspace, int64_t workspaceBytes, int64_t algo,
                 int64_t group, const int64_t *pads, const int64_t *strides, void *Y, int32_t dtype) {
   (void)workspace; (void)workspaceBytes; (void)algo;
-  return dnnrt::conv_dispatch("dnnrtConv", handle, X, dimX, W, dimW, nullptr, group, pads, strides,
+  return dnnrt::conv_dispatch("dnnrtConv", handle, X, dimX, W, dimW, nullptr, nullptr, group, pads, strides,
                               DNNRT_ACT_IDENTITY, Y, dtype);
 }
 
@@ -176,7 +177,22 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dim
     DNNRT_FAIL("dnnrtConvBiasActiv: activMode %ld (1 = ReLU, 5 = identity)", (long)activMode);
   if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
     DNNRT_FAIL("dnnrtConvBiasActiv: bias must hold K values");
-  return dnnrt::conv_dispatch("dnnrtConvBiasActiv", handle, X, dimX, W, dimW, B, group, pads,
+  return dnnrt::conv_dispatch("dnnrtConvBiasActiv", handle, X, dimX, W, dimW, B, nullptr, group, pads,
+                              strides, (int)activMode, Y, dtype);
+}
+
+void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
+                            const int64_t *dimW, const void *B, const int64_t *dimB, const void *Z,
+                            void *workspace, int64_t workspaceBytes, int64_t algo, int64_t group,
+                            const int64_t *pads, const int64_t *strides, int64_t activMode, void *Y,
+                            int32_t dtype) {
+  (void)workspace; (void)workspaceBytes; (void)algo;
+  if (activMode != DNNRT_ACT_RELU && activMode != DNNRT_ACT_IDENTITY)
+    DNNRT_FAIL("dnnrtConvBiasAddActiv: activMode %ld (1 = ReLU, 5 = identity)", (long)activMode);
+  if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
+    DNNRT_FAIL("dnnrtConvBiasAddActiv: bias must hold K values");
+  if (!Z) DNNRT_FAIL("dnnrtConvBiasAddActiv: null residual tensor");
+  return dnnrt::conv_dispatch("dnnrtConvBiasAddActiv", handle, X, dimX, W, dimW, B, Z, group, pads,
                               strides, (int)activMode, Y, dtype);
 }
 

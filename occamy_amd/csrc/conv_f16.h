@@ -6,6 +6,7 @@ namespace dnnrt {
 
 struct ConvF16Args {
   const __half *X, *Wt, *bias;
+  const __half *Z;  // residual tensor laid out like Y, or null
   __half *Y;
   int N, C, H, W, K, Cg, R, S, P, Q, ph, pw, sh, sw, group;
   int act;     // DNNRT_ACT_RELU / DNNRT_ACT_IDENTITY

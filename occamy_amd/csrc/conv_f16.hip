@@ -183,6 +183,8 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
   // register r of lane l in block (i, j): k_out = 8*(r/4) + 4*(l/32) + r%4,
   // pixel = l%32 -> four consecutive k_out per register group.
   const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
+  const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
+  const bool relu_now = a.act == DNNRT_ACT_RELU && !Zg;  // with a residual the activation comes after the sum
   _Float16 *Cs = smem;  // [BN pixels][CROW]
 #pragma unroll
   for (int i = 0; i < TM; i++)
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
           float v = acc[i][j][4 * g + e];
           const int k_out = m0 + kl + e;
           if (biasg && k_out < a.K) v += (float)biasg[k_out];
-          if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+          if (relu_now) v = v < 0.f ? 0.f : v;
           o[e] = (_Float16)v;
         }
         *reinterpret_cast<half4 *>(Cs + (wn0 + j * 32 + l32) * CROW + kl) = o;
@@ -209,8 +211,21 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
   for (int id = tid; id < BN * CH_PER_ROW; id += 256) {
     const int row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
     const int pix = n0 + row, k_out = m0 + ch * 8;
-    if (pix < NPQ && k_out < a.K)
-      *reinterpret_cast<uint4 *>(Yg + (int64_t)pix * a.K + k_out) = *reinterpret_cast<const uint4 *>(Cs + row * CROW + ch * 8);
+    if (pix < NPQ && k_out < a.K) {
+      half8 o = *reinterpret_cast<const half8 *>(Cs + row * CROW + ch * 8);
+      if (Zg) {
+        // conv + bias was rounded to fp16 above, as a separate convolution
+        // would have stored it; the residual sum follows in fp32
+        const half8 zv = *reinterpret_cast<const half8 *>(Zg + (int64_t)pix * a.K + k_out);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          float v = (float)o[e] + (float)zv[e];
+          if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+          o[e] = (_Float16)v;
+        }
+      }
+      *reinterpret_cast<half8 *>(Yg + (int64_t)pix * a.K + k_out) = o;
+    }
   }
 }
 
@@ -277,6 +292,7 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
   }
 
   const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
+  const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
   _Float16 *__restrict__ Yg = reinterpret_cast<_Float16 *>(a.Y);
   const int opix = n0 + wn0 + l32;
   if (opix >= NPQ) return;
@@ -288,8 +304,9 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
     const int ko = g * Kg + ml;
     float v = acc[r];
     if (biasg) v += (float)biasg[ko];
-    if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
     const int64_t off = out_nhwc ? (int64_t)opix * a.K + ko : ((int64_t)on * a.K + ko) * PQ + opq;
+    if (Zg) v = (float)(_Float16)v + (float)Zg[off];
+    if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
     Yg[off] = (_Float16)v;
   }
 }
@@ -297,7 +314,7 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
   const int64_t NPQ = (int64_t)a.N * a.P * a.Q;
   const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 32 == 0 && a.K % 8 == 0 &&
-                    aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y);
+                    aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) && aligned16(a.Z);
   if (fast) {
     // Largest tile that still gives every CU two workgroups to overlap.
     const int64_t want = 2 * (int64_t)ctx->num_cu;

@@ -102,6 +102,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   func_args_to_device(p);
   erase_dummy_constants(p);
   if (opt->fusion) fuse_conv_bias_activ(p);
+  if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {
     // Only fp16 programs whose rank-4 tensors flow through layout-aware calls
@@ -112,7 +113,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
       if (!r4) continue;
       if (op->result->dtype != F16) { g_err = "channels_last needs an fp16 graph"; delete pp; return nullptr; }
       switch (op->kind) {
-        case OP_MALLOC: case OP_HOST_ALLOC: case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_ACTIVATION: case OP_ADD:
+        case OP_MALLOC: case OP_HOST_ALLOC: case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_ACTIVATION: case OP_ADD:
         case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE: break;
         default: g_err = std::string("channels_last: ") + op_name(op->kind) + " has no channels-last form"; delete pp; return nullptr;
       }
@@ -122,7 +123,8 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
     for (const Op *op : p.ops)
       if (op->kind == OP_MEMCPY && op->mode == 1 && op->operands[1]->arg_index >= 0 && op->operands[0]->shape.size() == 4)
         for (const auto &u : op->operands[0]->uses)
-          if (u.first->kind != OP_MEMCPY && u.first->kind != OP_DEALLOC && u.first->kind != OP_CONVFWD && u.first->kind != OP_CONV_BIAS_ACTIV) {
+          if (u.first->kind != OP_MEMCPY && u.first->kind != OP_DEALLOC && u.first->kind != OP_CONVFWD && u.first->kind != OP_CONV_BIAS_ACTIV &&
+              !(u.first->kind == OP_CONV_BIAS_ADD_ACTIV && u.second == 0)) {
             g_err = "channels_last: a rank-4 function argument may only feed convolutions"; delete pp; return nullptr;
           }
     p.channels_last = true;
@@ -174,7 +176,7 @@ int64_t dnncProgramNumOps(const dnncProgram *p, int32_t compute_only) {
   if (!p) return -1;
   int64_t n = 0;
   for (const Op *op : p->p.ops)
-    if (!compute_only || (op->kind >= OP_CONVFWD && op->kind <= OP_GELU)) n++;
+    if (!compute_only || (op->kind >= OP_CONVFWD && op->kind < OP_RETURN)) n++;
   return n;
 }
 
@@ -182,7 +184,7 @@ int32_t dnncProgramComputeOp(const dnncProgram *p, int64_t i, const char **name,
   if (!p || !name || !work_class || !flops || !bytes) return fail("dnncProgramComputeOp: bad arguments");
   int64_t n = 0;
   for (const Op *op : p->p.ops) {
-    if (op->kind < OP_CONVFWD || op->kind > OP_GELU) continue;
+    if (op->kind < OP_CONVFWD || op->kind >= OP_RETURN) continue;
     if (n++ != i) continue;
     *name = op_name(op->kind);
     *work_class = op_class(op);

@@ -38,6 +38,7 @@ struct RuntimeApi {
   decltype(&::dnnrtHostFree) dnnrtHostFree = nullptr;
   decltype(&::dnnrtConv) dnnrtConv = nullptr;
   decltype(&::dnnrtConvBiasActiv) dnnrtConvBiasActiv = nullptr;
+  decltype(&::dnnrtConvBiasAddActiv) dnnrtConvBiasAddActiv = nullptr;
   decltype(&::dnnrtActive) dnnrtActive = nullptr;
   decltype(&::dnnrtTensorOp) dnnrtTensorOp = nullptr;
   decltype(&::dnnrtClip) dnnrtClip = nullptr;

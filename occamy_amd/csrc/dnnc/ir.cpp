@@ -39,6 +39,7 @@ const char *op_name(OpKind k) {
     case OP_CLIP: return "dnn.clip";
     case OP_LAYERNORM: return "dnn.layernorm";
     case OP_GELU: return "dnn.gelu";
+    case OP_CONV_BIAS_ADD_ACTIV: return "dnn.conv-bias-add-relufwd";
     case OP_RETURN: return "return";
   }
   return "?";
@@ -164,12 +165,13 @@ std::string Program::to_text() const {
       case OP_HOST_ALLOC: os << " {result=" << op->out_index << "}"; break;
       case OP_CONVFWD:
       case OP_CONV_BIAS_ACTIV:
+      case OP_CONV_BIAS_ADD_ACTIV:
         os << " {pads=";
         print_shape(os, op->pads);
         os << ", strides=";
         print_shape(os, op->strides);
         os << ", group=" << op->group;
-        if (op->kind == OP_CONV_BIAS_ACTIV) os << ", activMode=" << op->mode;
+        if (op->kind != OP_CONVFWD) os << ", activMode=" << op->mode;
         os << "}";
         break;
       case OP_ACTIVATION: os << " {mode=" << op->mode << "}"; break;

@@ -63,6 +63,7 @@ enum OpKind {
   OP_TRANSPOSE, OP_GATHER, OP_MATMUL2D, OP_MATMULND, OP_POW, OP_ERF, OP_CAST, OP_CLIP,
   // fused operators that have no counterpart in DNN.td
   OP_LAYERNORM, OP_GELU,
+  OP_CONV_BIAS_ADD_ACTIV,  // conv + bias + residual tensor + activation (cuDNN's z operand)
   OP_RETURN
 };
 const char *op_name(OpKind k);
@@ -157,6 +158,7 @@ const char *op_class(const Op *op);
 void op_work(const Op *op, double &flops, double &bytes);
 // passes.cpp
 void fuse_conv_bias_activ(Program &p);
+void fuse_residual_add(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);
 bool malloc_pool_opt(Program &p, std::string &err);

@@ -74,6 +74,55 @@ void fuse_conv_bias_activ(Program &p) {
   }
 }
 
+// conv+bias (identity) -> add(full-shape tensor Z) -> relu, each intermediate
+// read by nothing else, becomes one conv-bias-add-relu writing the ReLU's
+// buffer.  The reference has no such pattern; cuDNN's fused call has the z
+// operand for it (the reference passes it with weight 0,
+// src/Tools/dnn-wrapper/cudnn/fusedOp/CUDNNConvBiasReluFunc.cpp:94-112).
+void fuse_residual_add(Program &p) {
+  std::vector<Op *> convs;
+  for (Op *op : p.ops)
+    if (op->kind == OP_CONV_BIAS_ACTIV && op->mode == 5) convs.push_back(op);
+  auto drop_buffer = [&](Value *buf) {
+    std::vector<Op *> deallocs;
+    for (const auto &u : buf->uses)
+      if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+    for (Op *d : deallocs) p.erase(d);
+    if (buf->uses.empty() && buf->def) p.erase(buf->def);
+  };
+  for (Op *conv : convs) {
+    if (conv->result->uses.size() != 1) continue;
+    Op *add = conv->result->uses.front().first;
+    if (add->kind != OP_ADD || add->coef != 1.f || add->dimA != add->dimB) continue;
+    Value *z = add->operands[0] == conv->result ? add->operands[1] : add->operands[0];
+    if (z == conv->result || z->shape != conv->result->shape) continue;
+    if (add->result->uses.size() != 1) continue;
+    Op *relu = add->result->uses.front().first;
+    if (relu->kind != OP_ACTIVATION || relu->mode != 1 || relu->operands[0] != add->result) continue;
+
+    Value *out = relu->operands[1];
+    Op *fused = p.new_op(OP_CONV_BIAS_ADD_ACTIV);
+    fused->pads = conv->pads;
+    fused->strides = conv->strides;
+    fused->group = conv->group;
+    fused->dimA = conv->dimA;
+    fused->dimB = conv->dimB;
+    fused->mode = 1;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    // where the ReLU stood: Z and the ReLU's buffer both exist by then
+    p.insert_after(fused, relu);
+    p.set_operands(fused, {conv->operands[0], conv->operands[1], conv->operands[2], conv->operands[3], z, out});
+    p.replace_all_uses(relu->result, fused->result);
+    Value *conv_buf = conv->operands[4], *add_buf = add->operands[2];
+    p.erase(relu);
+    p.erase(add);
+    p.erase(conv);
+    drop_buffer(conv_buf);
+    if (add_buf != conv_buf) drop_buffer(add_buf);
+  }
+}
+
 // Each dealloc (visited in block order, i.e. creation order of the parked
 // deallocs) is moved to just after its tensor's last use.  If the last direct
 // user writes the tensor (the malloc is that op's last operand), the tensor

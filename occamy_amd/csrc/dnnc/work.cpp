@@ -9,7 +9,8 @@ namespace dnnc {
 const char *op_class(const Op *op) {
   switch (op->kind) {
     case OP_CONVFWD:
-    case OP_CONV_BIAS_ACTIV: return (op->dimB[1] == 1 && op->group > 1) ? "conv_depthwise" : "conv_dense";
+    case OP_CONV_BIAS_ACTIV:
+    case OP_CONV_BIAS_ADD_ACTIV: return (op->dimB[1] == 1 && op->group > 1) ? "conv_depthwise" : "conv_dense";
     case OP_MATMUL2D: return "gemm";
     case OP_MATMULND: return "matmul";
     case OP_SOFTMAX: return "softmax";
@@ -34,11 +35,13 @@ void op_work(const Op *op, double &flops, double &bytes) {
   auto n_in = [&](size_t i) { return (double)shape_numel(op->operands[i]->shape); };
   switch (op->kind) {
     case OP_CONVFWD:
-    case OP_CONV_BIAS_ACTIV: {
+    case OP_CONV_BIAS_ACTIV:
+    case OP_CONV_BIAS_ADD_ACTIV: {
       const double crs = (double)(op->dimB[1] * op->dimB[2] * op->dimB[3]);
       flops = 2.0 * n_out * crs;
       bytes = ((double)shape_numel(op->dimA) + (double)shape_numel(op->dimB) + n_out +
-               (op->kind == OP_CONV_BIAS_ACTIV ? (double)op->dimB[0] : 0.0)) * es;
+               (op->kind != OP_CONVFWD ? (double)op->dimB[0] : 0.0) +
+               (op->kind == OP_CONV_BIAS_ADD_ACTIV ? n_out : 0.0)) * es;
       break;
     }
     case OP_MATMUL2D: {

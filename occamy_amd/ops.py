@@ -88,6 +88,13 @@ class Ops:
                                                      dims(strides), activ, Y, dtype),
                          "dnnrtConvBiasActiv")
 
+    def conv_bias_add_activ(self, X, dimX, W, dimW, B, Z, pads, strides, activ, Y, group=1, dtype=_abi.F32):
+        dimB = [1, dimW[0], 1, 1]
+        return self._ret(self.lib.dnnrtConvBiasAddActiv(self.handle, X, dims(dimX), W, dims(dimW), B,
+                                                        dims(dimB), Z, None, 0, 1, group, dims(pads),
+                                                        dims(strides), activ, Y, dtype),
+                         "dnnrtConvBiasAddActiv")
+
     def active(self, X, dimX, mode, Y, dtype=_abi.F32):
         d = list(dimX) + [1] * (4 - len(dimX))
         return self._ret(self.lib.dnnrtActive(self.handle, X, dims(d), mode, Y, dtype), "dnnrtActive")

@@ -296,6 +296,37 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
   if (numel(dB, 4) != dW[0]) FAIL("convBiasActiv: bias must hold K values");
   return conv_entry(X, dX, W, dW, B, group, pads, strides, act, Y, dtype);
 }
+/* No reference wrapper of its own: the reference runs this as three calls,
+ * conv+bias (CUDNNConvBiasReluFunc.cpp, identity), cudnnAddTensor
+ * (CUDNNAddFunc.cpp) and cudnnActivationForward (CUDNNActiveFunc.cpp), each
+ * storing its result in the tensor's type.  Restated as exactly that chain. */
+void *dnnrtConvBiasAddActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
+                            const void *W, const int64_t *dW, const void *B,
+                            const int64_t *dB, const void *Z, void *ws,
+                            int64_t wsBytes, int64_t algo, int64_t group,
+                            const int64_t *pads, const int64_t *strides,
+                            int64_t act, void *Y, int32_t dtype) {
+  (void)h; (void)ws; (void)wsBytes; (void)algo;
+  if (act != DNNRT_ACT_RELU && act != DNNRT_ACT_IDENTITY)
+    FAIL("convBiasAddActiv: activMode %ld", (long)act);
+  if (numel(dB, 4) != dW[0]) FAIL("convBiasAddActiv: bias must hold K values");
+  if (!Z) FAIL("convBiasAddActiv: null residual tensor");
+  if (!conv_entry(X, dX, W, dW, B, group, pads, strides, DNNRT_ACT_IDENTITY, Y, dtype))
+    return NULL;
+  const int64_t P = (dX[2] + 2 * pads[0] - dW[2]) / strides[0] + 1,
+                Q = (dX[3] + 2 * pads[1] - dW[3]) / strides[1] + 1;
+  const int64_t ny = dX[0] * dW[0] * P * Q;
+  float *ty, *tz, *to;
+  const float *y = widen(Y, ny, dtype, &ty);
+  const float *z = widen(Z, ny, dtype, &tz);
+  float *o = outbuf(Y, ny, dtype, &to);
+  /* rounding to the tensor's type commutes with ReLU, so one narrow() at the
+   * end stands for the add's and the activation's stores */
+  for (int64_t i = 0; i < ny; i++) o[i] = act_apply(y[i] + z[i], act);
+  narrow(Y, to, ny, dtype);
+  free(ty); free(tz);
+  return Y;
+}
 
 /* ---- elementwise -------------------------------------------------------- */
 

@@ -190,3 +190,27 @@ def test_compile_errors():
     g.output(g.node("Conv", ["x", w], pads=[1, 0, 0, 1]))
     with pytest.raises(RuntimeError, match="asymmetric"):
         g.compile()
+
+
+def test_residual_fusion_flag():
+    g, _ = models.resnet50()
+    pf = g.compile(fusion=True)
+    g2, _ = models.resnet50()
+    pr = g2.compile(fusion=True, fuse_residual=True)
+    planned_vs_oracle(pr)
+    txt = pr.text
+    # every bottleneck ends conv3 (+ shortcut) -> add -> relu: 16 blocks, 16 fused closers
+    assert txt.count("dnn.conv-bias-add-relufwd") == 16
+    assert txt.count("dnn.conv-bias-relufwd") == 53 - 16
+    assert "dnn.add" in txt and txt.count("dnn.add") == 1             # the classifier's bias add stays
+    assert txt.count("dnn.activationfwd") == 0
+    assert pr.num_ops(compute_only=True) == pf.num_ops(compute_only=True) - 32
+    # two intermediate tensors per block are never allocated
+    assert len(pr.events()) == len(pf.events()) - 2 * 2 * 16
+    # (first fit is not monotonic: fewer tensors need not mean a smaller pool)
+    # the flag alone (without conv+bias fusion) changes nothing
+    g3, _ = models.resnet50(**SMALL)
+    g4, _ = models.resnet50(**SMALL)
+    assert g3.compile(fuse_residual=True).text == g4.compile().text
+    check_lifetimes(lambda: models.resnet50(**SMALL), fusion=True, fuse_residual=True)
+    check_lifetimes(lambda: models.mobilenet_v2(**SMALL), fusion=True, fuse_residual=True)

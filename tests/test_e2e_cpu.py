@@ -114,3 +114,17 @@ def test_executor_errors():
     s = p.session(runtime_library=ORACLE_PATH)
     with pytest.raises(RuntimeError, match="occamy mode"):
         s.run_device([0], [0])
+
+
+def test_residual_fusion_matches_unfused_chain():
+    # The oracle runs the fused closer of a residual block as the reference's
+    # three calls, so the flag must not change a single bit on the CPU.
+    small = lambda: models.resnet50(batch=2, image=32, classes=10)  # noqa: E731
+    _, _, a = run_oracle(small, fusion=True)
+    _, _, b = run_oracle(small, fusion=True, fuse_residual=True)
+    np.testing.assert_array_equal(a[0], b[0])
+    check(small, fusion=True, fuse_residual=True)
+    mb = lambda: models.mobilenet_v2(image=32, classes=10)  # noqa: E731
+    _, _, a = run_oracle(mb, fusion=True)
+    _, _, b = run_oracle(mb, fusion=True, fuse_residual=True)
+    np.testing.assert_array_equal(a[0], b[0])

@@ -129,3 +129,26 @@ def test_resnet50_fp16_channels_last(batch, image):
     s = p.session(compiler.MODE_RESIDENT)
     np.testing.assert_array_equal(s.run(*inputs)[0], out16[0])
     s.close()
+
+
+@pytest.mark.parametrize("name", ["resnet50", "mobilenet_v2"])
+def test_residual_fusion_fp32(name, oracle_outputs):
+    """conv+bias -> add -> relu as one call: against the oracle, and bit for
+    bit against this library's own three-call chain (same sums, same order)."""
+    fused, _ = run(CONFIGS[name], fusion=True, fuse_residual=True)
+    close(fused[0], oracle_outputs[name][0])
+    chain, _ = run(CONFIGS[name], fusion=True)
+    np.testing.assert_array_equal(fused[0], chain[0])
+    res, _ = run(CONFIGS[name], mode=compiler.MODE_RESIDENT, fusion=True, fuse_residual=True)
+    np.testing.assert_array_equal(res[0], fused[0])
+
+
+def test_residual_fusion_fp16_channels_last():
+    build16 = lambda: models.resnet50(2, np.float16, seed=5, image=64)  # noqa: E731
+    chain, _ = run(build16, fusion=True, channels_last=True)
+    fused, _ = run(build16, fusion=True, channels_last=True, fuse_residual=True)
+    # the fused closer rounds conv+bias to fp16 exactly where the chain stores
+    # it, so only the final fp32->fp16 rounding of the sum can differ (the chain
+    # adds in fp16 arithmetic): a few fp16 ulps after 16 blocks
+    np.testing.assert_allclose(fused[0].astype(np.float32), chain[0].astype(np.float32), rtol=2e-2,
+                               atol=2e-2 * float(np.abs(chain[0].astype(np.float32)).max()))

@@ -73,6 +73,14 @@ def test_conv_f32(gpu, cpu, case):
     # the summation order of the tile shapes each layout selects
     close(oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, crsk=True), ref)
     close(oc.conv(gpu, x, w, None, *args, crsk=True), oc.conv(cpu, x, w, None, *args))
+    # residual operand: relu((conv + b) + z); bit-equal to this library's own
+    # conv -> add -> relu chain, which forms the same sums in the same order
+    z = r.standard_normal(ref.shape).astype(np.float32)
+    fused = oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, z=z)
+    close(fused, oc.conv(cpu, x, w, b, *args, _abi.ACT_RELU, z=z))
+    lin = oc.conv(gpu, x, w, b, *args, _abi.ACT_IDENTITY)
+    np.testing.assert_array_equal(fused, oc.unary(gpu, "relu", oc.tensor_op(gpu, _abi.OP_ADD, lin, z)))
+    close(oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, crsk=True, z=z), fused)
 
 
 def test_conv_closed_forms(gpu):
@@ -263,8 +271,8 @@ def test_data_movement(gpu, cpu):
 
 # ---- fp16, channels-last -----------------------------------------------------------------
 
-def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt):
-    """x, w in logical NCHW / KCRS order; returns logical NCHW."""
+def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt, z=None):
+    """x, w (and the residual z) in logical NCHW / KCRS order; returns logical NCHW."""
     N, C, H, W = x.shape
     K, Cg, R, S = w.shape
     P, Q = oc.conv_out_hw(H, W, R, S, pads, strides)
@@ -274,8 +282,13 @@ def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt):
     Y = gpu.empty((N * K * P * Q,), np.float16)
     gpu.ops.set_format(fmt)
     try:
-        gpu.ops.conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), pads, strides, activ, gpu.ptr(Y),
-                                group, _abi.F16)
+        if z is None:
+            gpu.ops.conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), pads, strides, activ,
+                                    gpu.ptr(Y), group, _abi.F16)
+        else:  # laid out like Y
+            Z = gpu.put(z if fmt == _abi.NCHW else np.ascontiguousarray(z.transpose(0, 2, 3, 1)))
+            gpu.ops.conv_bias_add_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), gpu.ptr(Z), pads, strides,
+                                        activ, gpu.ptr(Y), group, _abi.F16)
         gpu.sync()
     finally:
         gpu.ops.set_format(_abi.NCHW)
@@ -313,6 +326,10 @@ def test_conv_f16(gpu, cpu, case, fmt):
         ident = conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_IDENTITY, fmt)
         refi = oc.conv(cpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_IDENTITY)
         np.testing.assert_allclose(ident.astype(np.float32), refi.astype(np.float32), rtol=2e-3, atol=2e-3)
+    z = r.standard_normal(ref.shape).astype(np.float16)
+    refz = oc.conv(cpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, z=z)
+    gotz = conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, fmt, z=z)
+    np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
 
 
 def test_f16_channels_last_ops(gpu, cpu):

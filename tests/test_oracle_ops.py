@@ -89,6 +89,14 @@ def test_conv_vs_torch_float64(be, shape):
     ref = F.conv2d(t64(x), t64(w), t64(b), stride=st, padding=pd, groups=g).numpy()
     got = oc.conv(be, x, w, b, (pd, pd), (st, st), g, _abi.ACT_IDENTITY)
     np.testing.assert_allclose(got, ref, rtol=2e-6, atol=2e-6)
+    # with a residual tensor: relu(conv + b + z), and exactly the three-call chain
+    z = r.standard_normal(ref.shape).astype(np.float32)
+    fused = oc.conv(be, x, w, b, (pd, pd), (st, st), g, _abi.ACT_RELU, z=z)
+    np.testing.assert_allclose(fused, np.maximum(ref + z.astype(np.float64), 0), rtol=2e-6, atol=2e-6)
+    chain = oc.unary(be, "relu", oc.tensor_op(be, _abi.OP_ADD, got, z))
+    np.testing.assert_array_equal(fused, chain)
+    lin = oc.conv(be, x, w, b, (pd, pd), (st, st), g, _abi.ACT_IDENTITY, z=z)
+    np.testing.assert_array_equal(lin, oc.tensor_op(be, _abi.OP_ADD, got, z))
 
 
 def test_conv_closed_forms(be):
