@@ -48,6 +48,8 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
   c->filter_layout = DNNRT_FILTER_KCRS;
   c->device = dev;
   c->num_cu = prop.multiProcessorCount;
+  const char *tile = getenv("DNNRT_F16_TILE");
+  c->f16_tile = tile ? atoi(tile) : 0;
   *handle = c;
   return 0;
 }

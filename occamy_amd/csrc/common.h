@@ -16,6 +16,8 @@ struct dnnrtContext {
   int filter_layout;   // DNNRT_FILTER_KCRS / DNNRT_FILTER_CRSK (fp32 convolutions)
   int device;
   int num_cu;
+  int f16_tile;        // 0 = pick the fp16 convolution tile by problem size; 1..7 force one
+                       // (environment variable DNNRT_F16_TILE at dnnrtCreate; for tuning)
 };
 
 namespace dnnrt {

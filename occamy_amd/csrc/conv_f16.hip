@@ -8,8 +8,9 @@
 //
 // Fast kernel (NHWC in, NHWC out, C % 32 == 0, K % 8 == 0, group 1):
 //   tile BM k_out x BN pixels, BK = 32; per step every thread moves 16-byte
-//   chunks global -> registers -> LDS (rows padded to 80 bytes, which makes
-//   the ds_read_b128 operand fetches conflict-free); registers prefetch the
+//   chunks global -> registers -> LDS (64-byte rows with an XOR swizzle of the
+//   chunk position, which makes both the stores and the ds_read_b128 operand
+//   fetches conflict-free); registers prefetch the
 //   next step while the MFMAs of the current one run; LDS is double-buffered,
 //   one barrier per step.  A BK step lies inside one (r, s) tap, so the tap
 //   and its bounds check are wave-uniform.  The epilogue adds bias, applies the
@@ -35,102 +36,151 @@ typedef __attribute__((address_space(1))) const u32x4 *global_u32x4_ptr;
 __device__ __forceinline__ u32x4 load_global_16(const void *p) { return *(global_u32x4_ptr)p; }
 
 constexpr int BK16 = 32;      // k per step
-constexpr int LDS_ROW = 40;   // halfs per LDS row: 32 + 8 pad (80 bytes)
+constexpr int LDS_ROW = 32;   // halfs per LDS row of the fast kernel: 64 bytes, no padding
+constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 
-template <int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a) {
+// Fast kernel.  Tile BM k_out x BN pixels, four wavefronts in a WM x WN grid,
+// each owning (BM/WM) x (BN/WN) of the tile as 32x32 MFMA blocks.
+//
+// Everything inside the K loop is branch-free on the vector side: every load
+// is issued unconditionally from a clamped address and what must not
+// contribute (padding taps, rows past the end of the tensor) is zeroed by an
+// AND when the chunk goes to LDS.  Only then can the compiler count the
+// outstanding loads exactly and wait for just the stage it is about to store
+// (a load under a divergent branch forces a wait for ALL outstanding loads,
+// which exposes the full memory latency at every step).
+//
+// Pipeline, one barrier per step.  Three LDS stages and two sets of MFMA
+// operand registers: in step kt a wavefront
+//   1. issues the global loads of step kt + 1 + DEPTH (register ring),
+//   2. issues the LDS reads of step kt + 1's operands (written a step ago),
+//   3. runs the MFMAs of step kt on operands read during step kt - 1,
+//   4. stores step kt + 2 (loaded DEPTH steps ago) into the third LDS stage.
+// No MFMA ever waits on an LDS read issued in its own step.
+//
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its
+// own: the kernel renumbers them so that one XCD works on a contiguous run of
+// tiles (k_out tiles of one pixel tile first), which then share their
+// operands in that L2.
+template <int BM, int BN, int WM, int WN, int DEPTH, int MINWG, bool MASKED>
+__global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   constexpr int A_CH = BM * 4 / 256, B_CH = BN * 4 / 256;  // 16-byte chunks per thread per step
   static_assert(A_CH >= 1 && B_CH >= 1, "tile too small");
   constexpr int STAGE = (BM + BN) * LDS_ROW;               // halfs per pipeline stage
   constexpr int CROW = BM + 8;                             // halfs per row of the output staging tile
-  constexpr int SMEM = (2 * STAGE > BN * CROW) ? 2 * STAGE : BN * CROW;
+  constexpr int SMEM = (3 * STAGE > BN * CROW) ? 3 * STAGE : BN * CROW;
+  static_assert(DEPTH == 2 || DEPTH == 4, "ring slots and operand sets are indexed at compile time");
   __shared__ __attribute__((aligned(16))) _Float16 smem[SMEM];
+
+  const int per_xcd = (tiles_total + 7) >> 3;
+  const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+  if (tile >= tiles_total) return;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
 
   const int tiles_m = (a.K + BM - 1) / BM;
-  const int tile_n = blockIdx.x / tiles_m, tile_m = blockIdx.x - tile_n * tiles_m;
+  const int tile_n = tile / tiles_m, tile_m = tile - tile_n * tiles_m;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int NPQ = a.N * a.P * a.Q, PQ = a.P * a.Q;
   const int CRS = a.C * a.R * a.S;
 
-  const _Float16 *__restrict__ Xg = reinterpret_cast<const _Float16 *>(a.X);
-  const _Float16 *__restrict__ Wg = reinterpret_cast<const _Float16 *>(a.Wt);
+  const char *__restrict__ Xg = reinterpret_cast<const char *>(a.X);
+  const char *__restrict__ Wg = reinterpret_cast<const char *>(a.Wt);
 
   // ---- loader constants ------------------------------------------------
-  // A (filters): chunk id -> (row, 16-byte chunk of the 64-byte k slice)
-  // element OFFSETS, not pointers, are kept across the loop: the address is
-  // formed from the kernel-argument base at each load, which keeps the loads
-  // in the global address space (flat loads would tie them to the LDS counter)
-  int64_t a_off[A_CH];
-  bool a_ok[A_CH];
+  // chunk id -> (row of the tile, 16-byte chunk of the row's 64-byte k slice).
+  // Unsigned 32-bit BYTE offsets from the kernel-argument bases (the
+  // dispatcher checks the tensors are below 4 GiB), so the loads use the
+  // scalar-base + 32-bit vector-offset form: no 64-bit address arithmetic and
+  // no address registers that outlive the load.
+  unsigned a_off[A_CH], a_msk[A_CH];
 #pragma unroll
   for (int i = 0; i < A_CH; i++) {
     const int id = tid + i * 256, row = id >> 2, ch = id & 3;
     const int k_out = m0 + row;
-    a_ok[i] = k_out < a.K;
-    a_off[i] = (int64_t)(a_ok[i] ? k_out : 0) * CRS + ch * 8;
+    const bool ok = k_out < a.K;
+    a_off[i] = 2u * (unsigned)((ok ? k_out : 0) * CRS + ch * 8);
+    a_msk[i] = ok ? 0xffffffffu : 0u;
   }
-  // B (im2col): each chunk belongs to one output pixel
-  int b_ih0[B_CH], b_iw0[B_CH];
-  int64_t b_off[B_CH];
-  bool b_ok[B_CH];
+  // B (im2col): a chunk belongs to one output pixel; bit (r * S + s) of
+  // b_taps says whether that tap reads inside the image.
+  int b_pix[B_CH];
+  unsigned b_taps[B_CH];
 #pragma unroll
   for (int i = 0; i < B_CH; i++) {
     const int id = tid + i * 256, row = id >> 2, ch = id & 3;
     const int pix = n0 + row;
-    b_ok[i] = pix < NPQ;
-    const int n = b_ok[i] ? pix / PQ : 0;
-    const int pq = b_ok[i] ? pix - n * PQ : 0;
+    const bool ok = pix < NPQ;
+    const int n = ok ? pix / PQ : 0;
+    const int pq = ok ? pix - n * PQ : 0;
     const int p = pq / a.Q, q = pq - p * a.Q;
-    b_ih0[i] = p * a.sh - a.ph;
-    b_iw0[i] = q * a.sw - a.pw;
-    b_off[i] = (int64_t)n * a.H * a.W * a.C + ch * 8;
+    const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
+    b_pix[i] = 2 * (((n * a.H + ih0) * a.W + iw0) * a.C + ch * 8);  // bytes; negative inside the padding
+    unsigned taps = 0;
+    if (MASKED) {
+      for (int r = 0; r < a.R; r++)
+        for (int s = 0; s < a.S; s++)
+          if (ok && (unsigned)(ih0 + r) < (unsigned)a.H && (unsigned)(iw0 + s) < (unsigned)a.W)
+            taps |= 1u << (r * a.S + s);
+    }
+    b_taps[i] = taps;
   }
 
-  // Register ring: the loads of DEPTH future steps are in flight while the
-  // MFMAs of the current one run (a step is ~0.1 us of MFMA work, a global
-  // load takes several times that).  Slots are indexed with compile-time
-  // constants: the step loop is unrolled DEPTH times.
-  constexpr int DEPTH = 4;
   u32x4 ra[DEPTH][A_CH], rb[DEPTH][B_CH];
-  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  unsigned rm[DEPTH][B_CH];
 
   const int steps_c = a.C / BK16, nk = a.R * a.S * steps_c;
-  int lr = 0, ls = 0, lc0 = 0, lstep = 0;  // cursor of the next step to load
+  // cursor of the next step to load (wave-uniform); it stops at the last step,
+  // so loads issued past the end re-read that step and are never used
+  int lj = 0, l_r = 0, l_s = 0, l_c0 = 0;
 
-  auto load_step = [&](u32x4 (&qa)[A_CH], u32x4 (&qb)[B_CH]) {
-    if (lstep < nk) {
-      const int kk = (lr * a.S + ls) * a.C + lc0;
+  auto load_step = [&](u32x4 (&qa)[A_CH], u32x4 (&qb)[B_CH], unsigned (&qm)[B_CH]) {
+    const unsigned w_off = 2u * (unsigned)lj * BK16;
+    const int x_off = 2 * ((l_r * a.W + l_s) * a.C + l_c0);
+    const int tap = l_r * a.S + l_s;
 #pragma unroll
-      for (int i = 0; i < A_CH; i++)
-        qa[i] = a_ok[i] ? load_global_16(Wg + (a_off[i] + kk)) : zero4;
+    for (int i = 0; i < A_CH; i++) qa[i] = load_global_16(Wg + (a_off[i] + w_off));
 #pragma unroll
-      for (int i = 0; i < B_CH; i++) {
-        const int ih = b_ih0[i] + lr, iw = b_iw0[i] + ls;
-        const bool ok = b_ok[i] && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
-        qb[i] = ok ? load_global_16(Xg + (b_off[i] + ((int64_t)ih * a.W + iw) * a.C + lc0)) : zero4;
+    for (int i = 0; i < B_CH; i++) {
+      if (MASKED) {
+        const unsigned m = 0u - ((b_taps[i] >> tap) & 1u);
+        qm[i] = m;
+        qb[i] = load_global_16(Xg + ((unsigned)(b_pix[i] + x_off) & m));
+      } else {
+        qb[i] = load_global_16(Xg + (unsigned)(b_pix[i] + x_off));
       }
-      lc0 += BK16;
-      if (lc0 == a.C) { lc0 = 0; if (++ls == a.S) { ls = 0; ++lr; } }
     }
-    lstep++;
+    if (lj + 1 < nk) {
+      lj++;
+      l_c0 += BK16;
+      if (l_c0 == a.C) { l_c0 = 0; if (++l_s == a.S) { l_s = 0; ++l_r; } }
+    }
   };
-  auto store_step = [&](int buf, const u32x4 (&qa)[A_CH], const u32x4 (&qb)[B_CH]) {
+  // LDS rows are 64 bytes (four 16-byte chunks) and chunk c of row r lives at
+  // position c ^ ((r >> 1) & 3).  Eight consecutive lanes then always cover all
+  // 32 banks once, both when a step is stored (two rows x four chunks) and when
+  // MFMA operands are read (eight rows, one chunk each).
+  const int st_swz = (tid >> 3) & 3;   // store side: row = tid / 4 + 64 * i
+  const int ld_swz = (l32 >> 1) & 3;   // operand side: row = 32 * block + l32
+  auto store_step = [&](int buf, const u32x4 (&qa)[A_CH], const u32x4 (&qb)[B_CH], const unsigned (&qm)[B_CH]) {
     _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
 #pragma unroll
     for (int i = 0; i < A_CH; i++) {
       const int id = tid + i * 256, row = id >> 2, ch = id & 3;
-      *reinterpret_cast<u32x4 *>(As + row * LDS_ROW + ch * 8) = qa[i];
+      u32x4 v = qa[i];
+      if (MASKED) v &= a_msk[i];
+      *reinterpret_cast<u32x4 *>(As + row * LDS_ROW + ((ch ^ st_swz) * 8)) = v;
     }
 #pragma unroll
     for (int i = 0; i < B_CH; i++) {
       const int id = tid + i * 256, row = id >> 2, ch = id & 3;
-      *reinterpret_cast<u32x4 *>(Bs + row * LDS_ROW + ch * 8) = qb[i];
+      u32x4 v = qb[i];
+      if (MASKED) v &= qm[i];
+      *reinterpret_cast<u32x4 *>(Bs + row * LDS_ROW + ((ch ^ st_swz) * 8)) = v;
     }
   };
 
@@ -142,39 +192,74 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  // prologue: step 0 into LDS, steps 1 .. DEPTH-1 in flight in slots 1 .. DEPTH-1
-  load_step(ra[0], rb[0]);
+  // Bias of the k_out this lane will hold in its accumulators: four
+  // consecutive values per register group, fetched once, up front, as 8-byte
+  // loads from clamped addresses (K is a multiple of 8, so a group of four is
+  // inside the tensor or outside it as a whole; rows outside are never stored).
+  half4 bias4[TM][4];
+  {
+    const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
 #pragma unroll
-  for (int d = 1; d < DEPTH; d++) load_step(ra[d], rb[d]);
-  store_step(0, ra[0], rb[0]);
-  __syncthreads();
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int k_out = m0 + wm0 + i * 32 + 8 * g + 4 * half;
+        const half4 zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+        bias4[i][g] = biasg ? *reinterpret_cast<const half4 *>(biasg + (k_out < a.K ? k_out : 0)) : zero;
+      }
+  }
 
+  half8 fa[2][TM], fb[2][TN];
+  auto read_frags = [&](int stage, half8 (&qa)[TM], half8 (&qb)[TN], int ks) {
+    const _Float16 *As = smem + stage * STAGE, *Bs = As + BM * LDS_ROW;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+      qa[i] = *reinterpret_cast<const half8 *>(As + (wm0 + i * 32 + l32) * LDS_ROW + ((((ks >> 3) + half) ^ ld_swz) * 8));
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+      qb[j] = *reinterpret_cast<const half8 *>(Bs + (wn0 + j * 32 + l32) * LDS_ROW + ((((ks >> 3) + half) ^ ld_swz) * 8));
+  };
+  auto mfma_frags = [&](const half8 (&qa)[TM], const half8 (&qb)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[i], qb[j], acc[i][j], 0, 0, 0);
+  };
+
+  // prologue: steps 0 .. DEPTH-1 in flight; steps 0 and 1 into LDS stages 0
+  // and 1; slot 0 refilled with step DEPTH; operands of step 0 (first half of
+  // its k range) into set 0
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++) load_step(ra[d], rb[d], rm[d]);
+  store_step(0, ra[0], rb[0], rm[0]);
+  load_step(ra[0], rb[0], rm[0]);
+  store_step(1, ra[1], rb[1], rm[1]);
+  __syncthreads();
+  read_frags(0, fa[0], fb[0], 0);
+
+  // A step has two k16 halves; operand set 0 carries the first, set 1 the
+  // second, each read while the other half's MFMAs run.
+  int stage = 0;  // LDS stage of step kt
   for (int kt0 = 0; kt0 < nk; kt0 += DEPTH) {
 #pragma unroll
     for (int u = 0; u < DEPTH; u++) {
       const int kt = kt0 + u;
+      // slot (u + 1) % DEPTH held step kt + 1, in LDS since the last step
+      load_step(ra[(u + 1) % DEPTH], rb[(u + 1) % DEPTH], rm[(u + 1) % DEPTH]);
       if (kt < nk) {
-        const int buf = kt & 1;
-        // slot u held step kt (already in LDS): reuse it for step kt + DEPTH
-        load_step(ra[u], rb[u]);
-        const _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
-#pragma unroll
-        for (int ks = 0; ks < BK16; ks += 16) {
-          half8 av[TM], bv[TN];
-#pragma unroll
-          for (int i = 0; i < TM; i++)
-            av[i] = *reinterpret_cast<const half8 *>(As + (wm0 + i * 32 + l32) * LDS_ROW + ks + half * 8);
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-            bv[j] = *reinterpret_cast<const half8 *>(Bs + (wn0 + j * 32 + l32) * LDS_ROW + ks + half * 8);
-#pragma unroll
-          for (int i = 0; i < TM; i++)
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) store_step(buf ^ 1, ra[(u + 1) % DEPTH], rb[(u + 1) % DEPTH]);
+        const int next = stage == 2 ? 0 : stage + 1, after = next == 2 ? 0 : next + 1;
+        read_frags(stage, fa[1], fb[1], 16);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_frags(fa[0], fb[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 1 < nk) read_frags(next, fa[0], fb[0], 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_frags(fa[1], fb[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 2 < nk) store_step(after, ra[(u + 2) % DEPTH], rb[(u + 2) % DEPTH], rm[(u + 2) % DEPTH]);
         __syncthreads();
+        stage = next;
       }
     }
   }
@@ -182,7 +267,6 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
   // ---- epilogue: bias, activation, fp16, transpose through LDS ------------
   // register r of lane l in block (i, j): k_out = 8*(r/4) + 4*(l/32) + r%4,
   // pixel = l%32 -> four consecutive k_out per register group.
-  const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
   const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
   const bool relu_now = a.act == DNNRT_ACT_RELU && !Zg;  // with a residual the activation comes after the sum
   _Float16 *Cs = smem;  // [BN pixels][CROW]
@@ -196,9 +280,7 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
         half4 o;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          float v = acc[i][j][4 * g + e];
-          const int k_out = m0 + kl + e;
-          if (biasg && k_out < a.K) v += (float)biasg[k_out];
+          float v = acc[i][j][4 * g + e] + (float)bias4[i][g][e];
           if (relu_now) v = v < 0.f ? 0.f : v;
           o[e] = (_Float16)v;
         }
@@ -234,8 +316,8 @@ __global__ __launch_bounds__(256) void conv_f16_nhwc_kernel(const ConvF16Args a)
 // stage, element-wise gathers.  Layout flags are runtime values.
 __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args a, const int in_nchw,
                                                                const int out_nhwc, const int w_krsc) {
-  __shared__ __attribute__((aligned(16))) _Float16 As[64 * LDS_ROW];
-  __shared__ __attribute__((aligned(16))) _Float16 Bs[64 * LDS_ROW];
+  __shared__ __attribute__((aligned(16))) _Float16 As[64 * LDS_ROW_G];
+  __shared__ __attribute__((aligned(16))) _Float16 Bs[64 * LDS_ROW_G];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm0 = (wave >> 1) * 32, wn0 = (wave & 1) * 32;
@@ -278,14 +360,14 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
           bv = in_nchw ? Xg[(((int64_t)n * a.C + cc) * a.H + ih) * a.W + iw]
                        : Xg[(((int64_t)n * a.H + ih) * a.W + iw) * a.C + cc];
       }
-      As[lrow * LDS_ROW + lk0 + e] = av;
-      Bs[lrow * LDS_ROW + lk0 + e] = bv;
+      As[lrow * LDS_ROW_G + lk0 + e] = av;
+      Bs[lrow * LDS_ROW_G + lk0 + e] = bv;
     }
     __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < BK16; ks += 16) {
-      const half8 av = *reinterpret_cast<const half8 *>(As + (wm0 + l32) * LDS_ROW + ks + half * 8);
-      const half8 bv = *reinterpret_cast<const half8 *>(Bs + (wn0 + l32) * LDS_ROW + ks + half * 8);
+      const half8 av = *reinterpret_cast<const half8 *>(As + (wm0 + l32) * LDS_ROW_G + ks + half * 8);
+      const half8 bv = *reinterpret_cast<const half8 *>(Bs + (wn0 + l32) * LDS_ROW_G + ks + half * 8);
       acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, acc, 0, 0, 0);
     }
     __syncthreads();
@@ -313,26 +395,44 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
   const int64_t NPQ = (int64_t)a.N * a.P * a.Q;
-  const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 32 == 0 && a.K % 8 == 0 &&
-                    aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) && aligned16(a.Z);
+  const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 32 == 0 && a.K % 8 == 0 && a.R * a.S <= 32 &&
+                    (int64_t)a.N * a.H * a.W * a.C < (1ll << 31) && (int64_t)a.K * a.C * a.R * a.S < (1ll << 31) &&
+                    aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) && aligned16(a.Z) &&
+                    (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0;
   if (fast) {
-    // Largest tile that still gives every CU two workgroups to overlap.
-    const int64_t want = 2 * (int64_t)ctx->num_cu;
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
-#define LAUNCH_FAST(BM_, BN_, WM_, WN_)                                                                    \
+    const bool pad = a.ph != 0 || a.pw != 0;
+#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MINWG_)                                                    \
   do {                                                                                                     \
     const int64_t tiles = tiles_of(BM_, BN_);                                                              \
-    if (tiles > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                      \
-    hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_>), dim3((unsigned)tiles), dim3(256), 0,    \
-                       ctx->stream, a);                                                                    \
+    if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                  \
+    const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                              \
+    if (pad || NPQ % BN_ != 0 || a.K % BM_ != 0)                                                           \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, true>), dim3(grid),     \
+                         dim3(256), 0, ctx->stream, a, (int)tiles);                                        \
+    else                                                                                                   \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, false>), dim3(grid),    \
+                         dim3(256), 0, ctx->stream, a, (int)tiles);                                        \
   } while (0)
-    if (a.K <= 64) {
-      if (tiles_of(64, 128) >= want) LAUNCH_FAST(64, 128, 1, 4);
-      else LAUNCH_FAST(64, 64, 2, 2);
-    } else {
-      if (tiles_of(128, 128) >= want) LAUNCH_FAST(128, 128, 2, 2);
-      else if (tiles_of(128, 64) >= want) LAUNCH_FAST(128, 64, 2, 2);
-      else LAUNCH_FAST(64, 64, 2, 2);
+    // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64:
+    // 128x128 as soon as it yields about one workgroup per two CUs (two or
+    // three are resident per CU, so fewer, larger tiles still fill the chip);
+    // below that, 64x64 tiles for parallelism; 64-row tiles when K_out <= 64.
+    const int tile_sel = ctx->f16_tile;  // 0 = automatic; otherwise forced (tuning and tests)
+    int sel = tile_sel;
+    if (sel == 0) {
+      if (a.K <= 64) sel = 6;
+      else if (tiles_of(128, 128) >= (3 * (int64_t)ctx->num_cu) / 5) sel = 3;
+      else sel = 4;
+    }
+    switch (sel) {
+      case 1: LAUNCH_FAST(256, 128, 2, 2, 2, 1); break;
+      case 2: LAUNCH_FAST(128, 256, 2, 2, 2, 1); break;
+      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2); break;
+      case 5: LAUNCH_FAST(64, 256, 1, 4, 2, 2); break;
+      case 6: LAUNCH_FAST(64, 128, 1, 4, 4, 2); break;
+      case 7: LAUNCH_FAST(128, 64, 2, 2, 4, 2); break;
+      default: LAUNCH_FAST(64, 64, 2, 2, 4, 2); break;
     }
 #undef LAUNCH_FAST
   } else {
