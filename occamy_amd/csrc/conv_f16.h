@@ -14,5 +14,7 @@ struct ConvF16Args {
 };
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a);
+// The 3-channel 7x7 stride-2 first layer (NCHW in, NHWC out); `launched` says whether it took the problem.
+bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 
 }  // namespace dnnrt

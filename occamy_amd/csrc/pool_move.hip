@@ -52,6 +52,50 @@ __global__ __launch_bounds__(256) void pool_kernel(const T *__restrict__ x, T *_
   pl_st(y + i, out);
 }
 
+// Channels-last fp16, C % 8 == 0: one thread per output pixel and group of
+// eight channels, 16-byte loads and stores (the scalar kernel above reads two
+// bytes per lane).  Same arithmetic: fp32 max / sum, NaN propagates.
+typedef _Float16 pl_half8 __attribute__((ext_vector_type(8)));
+template <bool IS_MAX>
+__global__ __launch_bounds__(256) void pool_nhwc_f16x8_kernel(const _Float16 *__restrict__ x, _Float16 *__restrict__ y,
+                                                              PoolGeom g, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c8 = g.C >> 3;
+  int64_t t = i;
+  const int cg = (int)(t % c8); t /= c8;
+  const int q = (int)(t % g.Q); t /= g.Q;
+  const int p = (int)(t % g.P);
+  const int n = (int)(t / g.P);
+  const _Float16 *xb = x + (int64_t)n * g.H * g.W * g.C + cg * 8;
+  const int ih0 = p * g.sh - g.ph, iw0 = q * g.sw - g.pw;
+  float m[8], s[8];
+  bool nan[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) { m[e] = -INFINITY; s[e] = 0.f; nan[e] = false; }
+  for (int r = 0; r < g.R; r++) {
+    const int ih = ih0 + r;
+    if ((unsigned)ih >= (unsigned)g.H) continue;
+    for (int ss = 0; ss < g.S; ss++) {
+      const int iw = iw0 + ss;
+      if ((unsigned)iw >= (unsigned)g.W) continue;
+      const pl_half8 v8 = *reinterpret_cast<const pl_half8 *>(xb + ((int64_t)ih * g.W + iw) * g.C);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float v = (float)v8[e];
+        nan[e] = nan[e] || (v != v);
+        m[e] = v > m[e] ? v : m[e];
+        s[e] += v;
+      }
+    }
+  }
+  pl_half8 o;
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    o[e] = (_Float16)(IS_MAX ? (nan[e] ? __builtin_nanf("") : m[e]) : s[e] / (float)(g.R * g.S));
+  *reinterpret_cast<pl_half8 *>(y + i * 8) = o;
+}
+
 static void *pool_entry(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
                         const int64_t *dY, const int64_t *kr, const int64_t *pads, const int64_t *st,
                         bool is_max, int32_t dtype) {
@@ -73,6 +117,17 @@ static void *pool_entry(const char *who, dnnrtHandle_t h, const void *X, const i
     DNNRT_FAIL("%s: a pooling window lies outside the input", who);
   const int64_t total = numel(dY, 4), blocks = ceil_div(total, 256);
   if (blocks > INT32_MAX) DNNRT_FAIL("%s: tensor too large", who);
+  if (dtype == DNNRT_F16 && g.nhwc && g.C % 8 == 0 && aligned16(X) && aligned16(Y)) {
+    const int64_t tot8 = total / 8, blocks8 = ceil_div(tot8, 256);
+    if (is_max)
+      hipLaunchKernelGGL((pool_nhwc_f16x8_kernel<true>), dim3((unsigned)blocks8), dim3(256), 0, h->stream,
+                         (const _Float16 *)X, (_Float16 *)Y, g, tot8);
+    else
+      hipLaunchKernelGGL((pool_nhwc_f16x8_kernel<false>), dim3((unsigned)blocks8), dim3(256), 0, h->stream,
+                         (const _Float16 *)X, (_Float16 *)Y, g, tot8);
+    DNNRT_CHECK_LAUNCH(who);
+    return Y;
+  }
 #define POOL_LAUNCH(T, MX)                                                                       \
   hipLaunchKernelGGL((pool_kernel<T, MX>), dim3((unsigned)blocks), dim3(256), 0, h->stream,      \
                      (const T *)X, (T *)Y, g, total)

@@ -305,7 +305,9 @@ F16_CASES = [
     (2, 256, 14, 14, 1000, 1, 1, 0),   # K_out not a multiple of the tile
     (1, 1024, 14, 14, 2048, 1, 2, 0),
     (2, 32, 9, 11, 40, 3, 1, 1),       # smallest C the fast path takes
-    (2, 3, 32, 32, 64, 7, 2, 3),       # generic path: 3 channels
+    (2, 3, 32, 32, 64, 7, 2, 3),       # 3 channels: first-layer kernel (NCHW in, NHWC out), generic otherwise
+    (2, 3, 45, 37, 64, 7, 2, 3),       # first-layer kernel, ragged tiles (23 x 19 output pixels)
+    (1, 3, 224, 224, 64, 7, 2, 3),     # the ResNet first layer at full size
     (1, 20, 9, 9, 24, 3, 1, 1),        # generic path: C % 32 != 0
 ]
 
@@ -355,6 +357,31 @@ def test_f16_channels_last_ops(gpu, cpu):
     np.testing.assert_allclose(gpu.get(G).reshape(2, 64, 1, 1).astype(np.float32),
                                oc.reduce_mean(cpu, x, (2, 64, 1, 1)).astype(np.float32), rtol=2e-3, atol=1e-3)
     np.testing.assert_array_equal(gpu.get(O).transpose(0, 3, 1, 2), oc.tensor_op(cpu, _abi.OP_ADD, x, bias))
+
+
+@pytest.mark.parametrize("C", [64, 12])          # 16-byte vector kernel / scalar kernel
+@pytest.mark.parametrize("kind", ["max", "avg"])
+def test_pooling_f16_channels_last(gpu, cpu, C, kind):
+    r = rng(79 + C)
+    x = r.standard_normal((3, C, 15, 13)).astype(np.float16)
+    x[1, 3, 4, 5] = np.nan                        # NaN must reach every window that sees it
+    for kernel, pads, strides in [((3, 3), (1, 1), (2, 2)), ((2, 2), (0, 0), (2, 2)), ((3, 2), (1, 0), (1, 2))]:
+        P, Q = oc.conv_out_hw(15, 13, kernel[0], kernel[1], pads, strides)
+        gpu.ops.set_format(_abi.NHWC)
+        try:
+            X = gpu.put(np.ascontiguousarray(x.transpose(0, 2, 3, 1)))
+            Y = gpu.empty((3 * C * P * Q,), np.float16)
+            fn = gpu.ops.maxpool if kind == "max" else gpu.ops.avgpool
+            fn(gpu.ptr(X), x.shape, gpu.ptr(Y), (3, C, P, Q), kernel, [pads[0], pads[1], pads[0], pads[1]], strides, _abi.F16)
+            gpu.sync()
+        finally:
+            gpu.ops.set_format(_abi.NCHW)
+        got = gpu.get(Y).reshape(3, P, Q, C).transpose(0, 3, 1, 2)
+        ref = oc.pool(cpu, kind, x, kernel, pads, strides)
+        if kind == "max":
+            np.testing.assert_array_equal(got, ref)
+        else:
+            np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=1e-3)
 
 
 def test_matmul2d_f16(gpu, cpu):
