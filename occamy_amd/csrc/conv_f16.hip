@@ -247,7 +247,9 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
       const int kt = kt0 + u;
       // slot (u + 1) % DEPTH held step kt + 1, in LDS since the last step
       load_step(ra[(u + 1) % DEPTH], rb[(u + 1) % DEPTH], rm[(u + 1) % DEPTH]);
-      if (kt < nk) {
+      // DEPTH == 2 kernels are only launched with an even number of steps (C % 64 == 0):
+      // no branch around the MFMAs, so the accumulators never pass through a merge
+      if (DEPTH == 2 || kt < nk) {
         const int next = stage == 2 ? 0 : stage + 1, after = next == 2 ? 0 : next + 1;
         read_frags(stage, fa[1], fb[1], 16);
         __builtin_amdgcn_sched_barrier(0);
@@ -428,6 +430,8 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       else if (tiles_of(128, 128) >= (3 * (int64_t)ctx->num_cu) / 5) sel = 3;
       else sel = 4;
     }
+    // tiles 1, 2, 3, 5 run two steps per loop trip and need an even step count
+    if (a.C % 64 != 0 && (sel == 1 || sel == 2 || sel == 3 || sel == 5)) sel = a.K <= 64 ? 6 : 4;
     switch (sel) {
       case 1: LAUNCH_FAST(256, 128, 2, 2, 2, 1); break;
       case 2: LAUNCH_FAST(128, 256, 2, 2, 2, 1); break;
