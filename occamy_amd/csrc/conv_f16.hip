@@ -6,9 +6,9 @@
 // the im2col operand so: with k ordered (r, s, c) a run of 8 k is 8 adjacent
 // channels of one input pixel, and the filter is stored K,R,S,C to match.
 //
-// Fast kernel (NHWC in, NHWC out, C % 32 == 0, K % 8 == 0, group 1):
-//   tile BM k_out x BN pixels, BK = 32; per step every thread moves 16-byte
-//   chunks global -> registers -> LDS (64-byte rows with an XOR swizzle of the
+// Fast kernel (NHWC in, NHWC out, C % 64 == 0, K % 8 == 0, group 1):
+//   tile BM k_out x BN pixels, BK = 64; per step every thread moves 16-byte
+//   chunks global -> registers -> LDS (128-byte rows with an XOR swizzle of the
 //   chunk position, which makes both the stores and the ds_read_b128 operand
 //   fetches conflict-free); registers prefetch the
 //   next step while the MFMAs of the current one run; LDS is double-buffered,
@@ -21,6 +21,8 @@
 // with element-wise gathers; it serves the first convolution of a network
 // (3 input channels, NCHW from the host) and odd shapes.
 #include "conv_f16.h"
+
+#include <type_traits>
 
 namespace dnnrt {
 
@@ -35,8 +37,9 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const u32x4 *global_u32x4_ptr;
 __device__ __forceinline__ u32x4 load_global_16(const void *p) { return *(global_u32x4_ptr)p; }
 
-constexpr int BK16 = 32;      // k per step
-constexpr int LDS_ROW = 32;   // halfs per LDS row of the fast kernel: 64 bytes, no padding
+constexpr int BK16 = 32;      // k per step of the generic kernel
+constexpr int BKF = 64;       // k per step of the fast kernel: a row's slice is one 128-byte line
+constexpr int LDS_ROW = 64;   // halfs per LDS row of the fast kernel: 128 bytes, no padding
 constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 
 // Fast kernel.  Tile BM k_out x BN pixels, four wavefronts in a WM x WN grid,
@@ -50,13 +53,11 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // (a load under a divergent branch forces a wait for ALL outstanding loads,
 // which exposes the full memory latency at every step).
 //
-// Pipeline, one barrier per step.  Three LDS stages and two sets of MFMA
-// operand registers: in step kt a wavefront
-//   1. issues the global loads of step kt + 1 + DEPTH (register ring),
-//   2. issues the LDS reads of step kt + 1's operands (written a step ago),
-//   3. runs the MFMAs of step kt on operands read during step kt - 1,
-//   4. stores step kt + 2 (loaded DEPTH steps ago) into the third LDS stage.
-// No MFMA ever waits on an LDS read issued in its own step.
+// Pipeline, one barrier per step of 64 k: two register stages of global
+// loads in flight (a step's loads are issued two steps before it is
+// computed), LDS double buffered, MFMA operands double buffered inside the
+// step.  A row's slice of a step is one full 128-byte line: half-line requests
+// cost the L2 a full slot each, and the L2 is what bounds this kernel.
 //
 // Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its
 // own: the kernel renumbers them so that one XCD works on a contiguous run of
@@ -66,12 +67,12 @@ template <int BM, int BN, int WM, int WN, int DEPTH, int MINWG, bool MASKED>
 __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  constexpr int A_CH = BM * 4 / 256, B_CH = BN * 4 / 256;  // 16-byte chunks per thread per step
+  constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;  // 16-byte chunks per thread per step
   static_assert(A_CH >= 1 && B_CH >= 1, "tile too small");
   constexpr int STAGE = (BM + BN) * LDS_ROW;               // halfs per pipeline stage
   constexpr int CROW = BM + 8;                             // halfs per row of the output staging tile
-  constexpr int SMEM = (3 * STAGE > BN * CROW) ? 3 * STAGE : BN * CROW;
-  static_assert(DEPTH == 2 || DEPTH == 4, "ring slots and operand sets are indexed at compile time");
+  constexpr int SMEM = (2 * STAGE > BN * CROW) ? 2 * STAGE : BN * CROW;
+  static_assert(DEPTH == 2, "two register stages: ring slots and operand sets are indexed at compile time");
   __shared__ __attribute__((aligned(16))) _Float16 smem[SMEM];
 
   const int per_xcd = (tiles_total + 7) >> 3;
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   unsigned a_off[A_CH], a_msk[A_CH];
 #pragma unroll
   for (int i = 0; i < A_CH; i++) {
-    const int id = tid + i * 256, row = id >> 2, ch = id & 3;
+    const int id = tid + i * 256, row = id >> 3, ch = id & 7;
     const int k_out = m0 + row;
     const bool ok = k_out < a.K;
     a_off[i] = 2u * (unsigned)((ok ? k_out : 0) * CRS + ch * 8);
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   unsigned b_taps[B_CH];
 #pragma unroll
   for (int i = 0; i < B_CH; i++) {
-    const int id = tid + i * 256, row = id >> 2, ch = id & 3;
+    const int id = tid + i * 256, row = id >> 3, ch = id & 7;
     const int pix = n0 + row;
     const bool ok = pix < NPQ;
     const int n = ok ? pix / PQ : 0;
@@ -133,13 +134,13 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   u32x4 ra[DEPTH][A_CH], rb[DEPTH][B_CH];
   unsigned rm[DEPTH][B_CH];
 
-  const int steps_c = a.C / BK16, nk = a.R * a.S * steps_c;
+  const int steps_c = a.C / BKF, nk = a.R * a.S * steps_c;
   // cursor of the next step to load (wave-uniform); it stops at the last step,
   // so loads issued past the end re-read that step and are never used
   int lj = 0, l_r = 0, l_s = 0, l_c0 = 0;
 
   auto load_step = [&](u32x4 (&qa)[A_CH], u32x4 (&qb)[B_CH], unsigned (&qm)[B_CH]) {
-    const unsigned w_off = 2u * (unsigned)lj * BK16;
+    const unsigned w_off = 2u * (unsigned)lj * BKF;
     const int x_off = 2 * ((l_r * a.W + l_s) * a.C + l_c0);
     const int tap = l_r * a.S + l_s;
 #pragma unroll
@@ -154,30 +155,36 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
         qb[i] = load_global_16(Xg + (unsigned)(b_pix[i] + x_off));
       }
     }
-    if (lj + 1 < nk) {
-      lj++;
-      l_c0 += BK16;
-      if (l_c0 == a.C) { l_c0 = 0; if (++l_s == a.S) { l_s = 0; ++l_r; } }
-    }
+    // advance, without branches (selects on the scalar unit)
+    const bool more = lj + 1 < nk;
+    const int c0n = l_c0 + BKF, sn = l_s + 1;
+    const bool wrap_c = c0n == a.C, wrap_s = wrap_c && sn == a.S;
+    lj = more ? lj + 1 : lj;
+    l_c0 = more ? (wrap_c ? 0 : c0n) : l_c0;
+    l_s = more ? (wrap_c ? (wrap_s ? 0 : sn) : l_s) : l_s;
+    l_r = (more && wrap_s) ? l_r + 1 : l_r;
   };
-  // LDS rows are 64 bytes (four 16-byte chunks) and chunk c of row r lives at
-  // position c ^ ((r >> 1) & 3).  Eight consecutive lanes then always cover all
-  // 32 banks once, both when a step is stored (two rows x four chunks) and when
-  // MFMA operands are read (eight rows, one chunk each).
-  const int st_swz = (tid >> 3) & 3;   // store side: row = tid / 4 + 64 * i
-  const int ld_swz = (l32 >> 1) & 3;   // operand side: row = 32 * block + l32
+  // LDS rows are 128 bytes (eight 16-byte chunks) and chunk c of row r lives at
+  // position c ^ ((r >> 1) & 7).  The LDS has 64 four-byte banks and serves a
+  // 16-byte access for 16 lanes per clock: with this placement 16 consecutive
+  // lanes always cover all 64 banks once, both when a step is stored (two
+  // rows x eight chunks) and when MFMA operands are read (16 rows, one chunk
+  // each).  Measured on the same 16-byte reads: 240 B/clk per CU conflict-free,
+  // 126 with two lanes per bank, 63 with four.
+  const int st_swz = (tid >> 4) & 7;   // store side: row = tid / 8 + 32 * i
+  const int ld_swz = (l32 >> 1) & 7;   // operand side: row = 32 * block + l32
   auto store_step = [&](int buf, const u32x4 (&qa)[A_CH], const u32x4 (&qb)[B_CH], const unsigned (&qm)[B_CH]) {
     _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
 #pragma unroll
     for (int i = 0; i < A_CH; i++) {
-      const int id = tid + i * 256, row = id >> 2, ch = id & 3;
+      const int id = tid + i * 256, row = id >> 3, ch = id & 7;
       u32x4 v = qa[i];
       if (MASKED) v &= a_msk[i];
       *reinterpret_cast<u32x4 *>(As + row * LDS_ROW + ((ch ^ st_swz) * 8)) = v;
     }
 #pragma unroll
     for (int i = 0; i < B_CH; i++) {
-      const int id = tid + i * 256, row = id >> 2, ch = id & 3;
+      const int id = tid + i * 256, row = id >> 3, ch = id & 7;
       u32x4 v = qb[i];
       if (MASKED) v &= qm[i];
       *reinterpret_cast<u32x4 *>(Bs + row * LDS_ROW + ((ch ^ st_swz) * 8)) = v;
@@ -210,14 +217,14 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   }
 
   half8 fa[2][TM], fb[2][TN];
-  auto read_frags = [&](int stage, half8 (&qa)[TM], half8 (&qb)[TN], int ks) {
+  auto read_frags = [&](int stage, half8 (&qa)[TM], half8 (&qb)[TN], int sub) {  // sub: which k16 of the step
     const _Float16 *As = smem + stage * STAGE, *Bs = As + BM * LDS_ROW;
 #pragma unroll
     for (int i = 0; i < TM; i++)
-      qa[i] = *reinterpret_cast<const half8 *>(As + (wm0 + i * 32 + l32) * LDS_ROW + ((((ks >> 3) + half) ^ ld_swz) * 8));
+      qa[i] = *reinterpret_cast<const half8 *>(As + (wm0 + i * 32 + l32) * LDS_ROW + (((2 * sub + half) ^ ld_swz) * 8));
 #pragma unroll
     for (int j = 0; j < TN; j++)
-      qb[j] = *reinterpret_cast<const half8 *>(Bs + (wn0 + j * 32 + l32) * LDS_ROW + ((((ks >> 3) + half) ^ ld_swz) * 8));
+      qb[j] = *reinterpret_cast<const half8 *>(Bs + (wn0 + j * 32 + l32) * LDS_ROW + (((2 * sub + half) ^ ld_swz) * 8));
   };
   auto mfma_frags = [&](const half8 (&qa)[TM], const half8 (&qb)[TN]) {
 #pragma unroll
@@ -227,44 +234,38 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[i], qb[j], acc[i][j], 0, 0, 0);
   };
 
-  // prologue: steps 0 .. DEPTH-1 in flight; steps 0 and 1 into LDS stages 0
-  // and 1; slot 0 refilled with step DEPTH; operands of step 0 (first half of
-  // its k range) into set 0
-#pragma unroll
-  for (int d = 0; d < DEPTH; d++) load_step(ra[d], rb[d], rm[d]);
-  store_step(0, ra[0], rb[0], rm[0]);
+  // prologue: steps 0 and 1 in flight, step 0 into LDS stage 0
   load_step(ra[0], rb[0], rm[0]);
-  store_step(1, ra[1], rb[1], rm[1]);
+  load_step(ra[1], rb[1], rm[1]);
+  store_step(0, ra[0], rb[0], rm[0]);
   __syncthreads();
-  read_frags(0, fa[0], fb[0], 0);
 
-  // A step has two k16 halves; operand set 0 carries the first, set 1 the
-  // second, each read while the other half's MFMAs run.
-  int stage = 0;  // LDS stage of step kt
-  for (int kt0 = 0; kt0 < nk; kt0 += DEPTH) {
-#pragma unroll
-    for (int u = 0; u < DEPTH; u++) {
-      const int kt = kt0 + u;
-      // slot (u + 1) % DEPTH held step kt + 1, in LDS since the last step
-      load_step(ra[(u + 1) % DEPTH], rb[(u + 1) % DEPTH], rm[(u + 1) % DEPTH]);
-      // DEPTH == 2 kernels are only launched with an even number of steps (C % 64 == 0):
-      // no branch around the MFMAs, so the accumulators never pass through a merge
-      if (DEPTH == 2 || kt < nk) {
-        const int next = stage == 2 ? 0 : stage + 1, after = next == 2 ? 0 : next + 1;
-        read_frags(stage, fa[1], fb[1], 16);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_frags(fa[0], fb[0]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 1 < nk) read_frags(next, fa[0], fb[0], 0);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_frags(fa[1], fb[1]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kt + 2 < nk) store_step(after, ra[(u + 2) % DEPTH], rb[(u + 2) % DEPTH], rm[(u + 2) % DEPTH]);
-        __syncthreads();
-        stage = next;
-      }
-    }
+  // Step kt (LDS stage and register slot U = kt & 1): refill slot U with step
+  // kt + 2; four k16 sub-steps, the operands of each read from LDS while the
+  // MFMAs of the one before run; half way, step kt + 1 goes from slot U ^ 1
+  // into the other LDS stage (nobody reads that stage during this step); one
+  // barrier.  The body has no branch, so the scheduler is free to spread the
+  // loads, LDS traffic and address arithmetic between the MFMAs.  Steps past
+  // the end are harmless (the cursor stops, LDS rows written are never read).
+  auto step = [&](auto slot_c) {
+    constexpr int U = decltype(slot_c)::value;
+    load_step(ra[U], rb[U], rm[U]);
+    read_frags(U, fa[0], fb[0], 0);
+    read_frags(U, fa[1], fb[1], 1);
+    mfma_frags(fa[0], fb[0]);
+    read_frags(U, fa[0], fb[0], 2);
+    mfma_frags(fa[1], fb[1]);
+    store_step(U ^ 1, ra[U ^ 1], rb[U ^ 1], rm[U ^ 1]);
+    read_frags(U, fa[1], fb[1], 3);
+    mfma_frags(fa[0], fb[0]);
+    mfma_frags(fa[1], fb[1]);
+    __syncthreads();
+  };
+  for (int kt = 0; kt + 1 < nk; kt += 2) {
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
   }
+  if (nk & 1) step(std::integral_constant<int, 0>{});
 
   // ---- epilogue: bias, activation, fp16, transpose through LDS ------------
   // register r of lane l in block (i, j): k_out = 8*(r/4) + 4*(l/32) + r%4,
@@ -400,7 +401,7 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
   if (!launch_conv_f16_stem(ctx, a, stem_launched)) return false;
   if (stem_launched) return true;
   const int64_t NPQ = (int64_t)a.N * a.P * a.Q;
-  const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 32 == 0 && a.K % 8 == 0 && a.R * a.S <= 32 &&
+  const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 64 == 0 && a.K % 8 == 0 && a.R * a.S <= 32 &&
                     (int64_t)a.N * a.H * a.W * a.C < (1ll << 31) && (int64_t)a.K * a.C * a.R * a.S < (1ll << 31) &&
                     aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) && aligned16(a.Z) &&
                     (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0;
@@ -419,27 +420,27 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, false>), dim3(grid),    \
                          dim3(256), 0, ctx->stream, a, (int)tiles);                                        \
   } while (0)
-    // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64:
-    // 128x128 as soon as it yields about one workgroup per two CUs (two or
-    // three are resident per CU, so fewer, larger tiles still fill the chip);
-    // below that, 64x64 tiles for parallelism; 64-row tiles when K_out <= 64.
+    // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
+    // (14.8 GFLOP 3x3 layers run in 28-38 us, 1x1 layers near their HBM time):
+    // 128x128 when it yields at least ~0.6 workgroups per CU and the reduction
+    // is long enough to amortise the larger tile's prologue and epilogue;
+    // 128x64 for few-tile or short-reduction problems; 64x64 when K_out <= 64.
     const int tile_sel = ctx->f16_tile;  // 0 = automatic; otherwise forced (tuning and tests)
     int sel = tile_sel;
     if (sel == 0) {
-      if (a.K <= 64) sel = 6;
-      else if (tiles_of(128, 128) >= (3 * (int64_t)ctx->num_cu) / 5) sel = 3;
-      else sel = 4;
+      const int nk = a.R * a.S * (a.C / BKF);
+      if (a.K <= 64) sel = 4;
+      else if (nk <= 2 || tiles_of(128, 128) < (3 * (int64_t)ctx->num_cu) / 5) sel = 7;
+      else sel = 3;
     }
-    // tiles 1, 2, 3, 5 run two steps per loop trip and need an even step count
-    if (a.C % 64 != 0 && (sel == 1 || sel == 2 || sel == 3 || sel == 5)) sel = a.K <= 64 ? 6 : 4;
     switch (sel) {
       case 1: LAUNCH_FAST(256, 128, 2, 2, 2, 1); break;
       case 2: LAUNCH_FAST(128, 256, 2, 2, 2, 1); break;
       case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2); break;
       case 5: LAUNCH_FAST(64, 256, 1, 4, 2, 2); break;
-      case 6: LAUNCH_FAST(64, 128, 1, 4, 4, 2); break;
-      case 7: LAUNCH_FAST(128, 64, 2, 2, 4, 2); break;
-      default: LAUNCH_FAST(64, 64, 2, 2, 4, 2); break;
+      case 6: LAUNCH_FAST(64, 128, 1, 4, 2, 2); break;
+      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2); break;
+      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2); break;
     }
 #undef LAUNCH_FAST
   } else {
