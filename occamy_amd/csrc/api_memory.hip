@@ -48,6 +48,17 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
   c->filter_layout = DNNRT_FILTER_KCRS;
   c->device = dev;
   c->num_cu = prop.multiProcessorCount;
+  c->splitk_partials = nullptr;
+  c->splitk_counters = nullptr;
+  if (hipMalloc((void **)&c->splitk_partials, dnnrt::SPLITK_PARTIAL_BYTES) != hipSuccess ||
+      hipMalloc((void **)&c->splitk_counters, dnnrt::SPLITK_MAX_TILES * sizeof(unsigned)) != hipSuccess ||
+      hipMemset(c->splitk_counters, 0, dnnrt::SPLITK_MAX_TILES * sizeof(unsigned)) != hipSuccess) {
+    set_error("dnnrtCreate: cannot allocate the handle's reduction scratch");
+    (void)hipFree(c->splitk_partials);
+    (void)hipFree(c->splitk_counters);
+    delete c;
+    return 1;
+  }
   const char *tile = getenv("DNNRT_F16_TILE");
   c->f16_tile = tile ? atoi(tile) : 0;
   *handle = c;
@@ -55,6 +66,10 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
 }
 
 int32_t dnnrtDestroy(dnnrtHandle_t handle) {
+  if (handle) {
+    (void)hipFree(handle->splitk_partials);
+    (void)hipFree(handle->splitk_counters);
+  }
   delete handle;
   return 0;
 }

@@ -16,11 +16,19 @@ struct dnnrtContext {
   int filter_layout;   // DNNRT_FILTER_KCRS / DNNRT_FILTER_CRSK (fp32 convolutions)
   int device;
   int num_cu;
+  // Scratch for reductions split over workgroups: partial tiles and one
+  // arrival counter per output tile (all zero between kernels).  Allocated with
+  // the handle; kernels of one handle run in stream order, so they share it.
+  float *splitk_partials;
+  unsigned *splitk_counters;
   int f16_tile;        // 0 = pick the fp16 convolution tile by problem size; 1..7 force one
                        // (environment variable DNNRT_F16_TILE at dnnrtCreate; for tuning)
 };
 
 namespace dnnrt {
+
+constexpr int64_t SPLITK_PARTIAL_BYTES = 8ll << 20;  // 2048 partial 32x32 fp32 tiles
+constexpr int SPLITK_MAX_TILES = 16384;               // arrival counters
 
 void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 

@@ -26,9 +26,15 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ float mask_f(float v, unsigned m) { return __uint_as_float(__float_as_uint(v) & m); }
 
 // Sum the KS partial tiles in LDS, then bias / residual / activation / store by wavefront 0.
+// The reduction may also be split over gridDim.y workgroups.  Each of them
+// leaves its partial tile in `partials` and bumps the tile's arrival counter;
+// whoever arrives last adds the partials up in split order -- the order of
+// arrival does not matter, so the result is the same bits on every run -- and
+// finishes the tile.  Nobody waits for anybody.  The last arriver puts the
+// counter back to zero for the next kernel on the stream.
 template <int KS>
 __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, float (*red)[16][64], int wave, int lane,
-                                                 int m0, int col, bool col_ok, int z) {
+                                                 int m0, int col, bool col_ok, int z, float *partials, unsigned *counters) {
   if (KS > 1) {
     if (wave > 0) {
 #pragma unroll
@@ -40,6 +46,31 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     for (int w = 0; w < KS - 1; w++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[r] += red[w][r][lane];
+  }
+  const int splits = (int)gridDim.y;
+  if (splits > 1) {
+    const unsigned tile = blockIdx.z * gridDim.x + blockIdx.x;
+    float *mine = partials + ((size_t)tile * splits + blockIdx.y) * 1024;
+#pragma unroll
+    for (int r = 0; r < 16; r++) __hip_atomic_store(&mine[r * 64 + lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // Partials are written and read with device-scope atomic accesses, which
+    // go past the per-XCD L2 to where all XCDs agree.  A release fence here
+    // would also write back every dirty line of this XCD's L2 (the previous
+    // layer's output), which costs more than the split saves; waiting for the
+    // stores' acknowledgements orders them before the arrival just as well.
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0)
+    unsigned arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    if (arrived != (unsigned)splits - 1) return;
+    const float *all = partials + (size_t)tile * splits * 1024;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    for (int y = 0; y < splits; y++)
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        acc[r] += __hip_atomic_load(all + (size_t)y * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (!col_ok) return;
   const int half = lane >> 5, PQ = a.P * a.Q;
@@ -62,7 +93,8 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
 }
 
 template <int KS, bool AMC>
-__global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmArgs a, const int c_per_wave) {
+__global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmArgs a, const int c_per_wave, float *partials,
+                                                                    unsigned *counters) {
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
   const int tiles_n = (a.Ncols + 31) / 32;
@@ -89,7 +121,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   const unsigned x_img = (unsigned)((int64_t)img * a.x_img_stride);
   const unsigned a_row = (unsigned)mrow * (unsigned)a.Kdim, lda = (unsigned)a.a_ld;
 
-  const int cbeg = wave * c_per_wave, cend = min(C, cbeg + c_per_wave);
+  const int cbeg = ((int)blockIdx.y * KS + wave) * c_per_wave, cend = min(C, cbeg + c_per_wave);
   const int niter = c_per_wave >> 1;
 
   constexpr int DEPTH = 2;
@@ -129,13 +161,14 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z);
+  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, partials, counters);
 }
 
 // 1x1 geometry (convolution, possibly strided, or matrix product with A rows
 // k-contiguous and B columns contiguous); Kdim % 4 == 0, A rows 16-byte aligned.
 template <int KS, bool AMC>
-__global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmArgs a, const int k_per_wave) {
+__global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmArgs a, const int k_per_wave, float *partials,
+                                                                    unsigned *counters) {
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
   const int tiles_n = (a.Ncols + 31) / 32;
@@ -153,7 +186,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   const unsigned x_pix = (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
   const unsigned a_row = (unsigned)mrow * (unsigned)a.Kdim, lda = (unsigned)a.a_ld;
 
-  const int kbeg = wave * k_per_wave, kend = min(a.Kdim, kbeg + k_per_wave);
+  const int kbeg = ((int)blockIdx.y * KS + wave) * k_per_wave, kend = min(a.Kdim, kbeg + k_per_wave);
   const int niter = k_per_wave >> 3;
 
   constexpr int DEPTH = 4;
@@ -192,7 +225,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z);
+  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, partials, counters);
 }
 
 // Returns true if one of the specialised kernels took the problem.
@@ -216,23 +249,30 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
   const int min_slice = is3x3 ? 4 : 32;              // reduction slice worth a wavefront
   int ks = 1;
   while (ks < 8 && (int64_t)tiles * a.Z * ks < want_waves && ceil_div(red_len, ks * 2) >= min_slice) ks *= 2;
-  dim3 grid(tiles, 1, a.Z);
+  // Still far from filling the chip (deep layers at batch 1: a few dozen tiles
+  // over a reduction of thousands): split the reduction over workgroups too.
+  int splits = 1;
+  while (splits < 16 && (int64_t)tiles * a.Z * splits * 2 <= ctx->num_cu &&
+         ceil_div(red_len, ks * splits * 2) >= min_slice &&
+         (int64_t)tiles * a.Z * splits * 2 * 4096 <= SPLITK_PARTIAL_BYTES && (int64_t)tiles * a.Z <= SPLITK_MAX_TILES)
+    splits *= 2;
+  dim3 grid(tiles, splits, a.Z);
 #define LAUNCH_KS2(KERNEL, AMC_, ARG)                                                                  \
   switch (ks) {                                                                                          \
-    case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, a, ARG); break;        \
-    case 2: hipLaunchKernelGGL((KERNEL<2, AMC_>), grid, dim3(128), 0, ctx->stream, a, ARG); break;       \
-    case 4: hipLaunchKernelGGL((KERNEL<4, AMC_>), grid, dim3(256), 0, ctx->stream, a, ARG); break;       \
-    default: hipLaunchKernelGGL((KERNEL<8, AMC_>), grid, dim3(512), 0, ctx->stream, a, ARG); break;      \
+    case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break;  \
+    case 2: hipLaunchKernelGGL((KERNEL<2, AMC_>), grid, dim3(128), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
+    case 4: hipLaunchKernelGGL((KERNEL<4, AMC_>), grid, dim3(256), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
+    default: hipLaunchKernelGGL((KERNEL<8, AMC_>), grid, dim3(512), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
   }
 #define LAUNCH_KS(KERNEL, ARG)                                                                         \
   do {                                                                                                 \
     if (amc) { LAUNCH_KS2(KERNEL, true, ARG) } else { LAUNCH_KS2(KERNEL, false, ARG) }                 \
   } while (0)
   if (is3x3) {
-    const int c_per_wave = (int)(ceil_div(ceil_div(red_len, ks), 2) * 2);
+    const int c_per_wave = (int)(ceil_div(ceil_div(red_len, ks * splits), 2) * 2);
     LAUNCH_KS(conv3x3_f32_small_kernel, c_per_wave);
   } else {
-    const int k_per_wave = (int)(ceil_div(ceil_div(red_len, ks), 8) * 8);
+    const int k_per_wave = (int)(ceil_div(ceil_div(red_len, ks * splits), 8) * 8);
     LAUNCH_KS(conv1x1_f32_small_kernel, k_per_wave);
   }
 #undef LAUNCH_KS
