@@ -40,6 +40,20 @@ def build_workload(name):
     raise SystemExit(f"unknown workload {name}")
 
 
+def recorded_traffic(workload, cls):
+    """HBM bytes per launch of kernel class `cls`, from the counter runs whose
+    summary is kept under profiles/ (FETCH_SIZE and WRITE_SIZE scaled by the
+    copy-kernel calibration); None if no such summary exists for the workload."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith(f"traffic_bytes_per_launch[{cls}]:"):
+                return float(line.split(":", 1)[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -49,6 +63,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU-baseline leg")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time the other workloads (reported under 'extra')")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only launch the library's plain copy kernel on 256 MiB a few times: the run that the "
+                         "FETCH_SIZE / WRITE_SIZE counters of the other runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path has no exchange step between devices, "
@@ -59,6 +76,20 @@ def main():
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
+
+    if args.calibrate_copy:
+        from occamy_amd import _abi
+        from occamy_amd.ops import Ops
+        n = 64 << 20  # floats: 256 MiB read + 256 MiB written per launch
+        src = torch.ones(n, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        ops = Ops()
+        for _ in range(5):
+            ops.reshape(src.data_ptr(), (n,), dst.data_ptr(), _abi.F32)
+        ops.sync()
+        print(json.dumps({"calibration": "copy16_kernel", "launches": 5, "bytes_read_per_launch": 4 * n,
+                          "bytes_written_per_launch": 4 * n}))
+        return
 
     def measure(name, steps, warmup, want_profile):
         (graph, inputs), flags, batch, unit, dtype = build_workload(name)
@@ -126,7 +157,8 @@ def main():
     else:
         achieved = c["bytes"] / (c["ms"] * 1e-3)
         roof = dict(bound="hbm", achieved=achieved / 1e9, peak=PEAK["hbm"] / 1e9, unit="GB/s", frac=achieved / PEAK["hbm"])
-    roof.update(kernel=cls, launches_per_step=c["launches"], avg_launch_us=1e3 * c["ms"] / c["launches"], traffic=None)
+    roof.update(kernel=cls, launches_per_step=c["launches"], avg_launch_us=1e3 * c["ms"] / c["launches"],
+                traffic=recorded_traffic(args.workload, cls))
 
     cpu = None
     if not args.no_cpu:

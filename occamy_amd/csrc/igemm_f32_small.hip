@@ -34,7 +34,7 @@ __device__ __forceinline__ float mask_f(float v, unsigned m) { return __uint_as_
 // counter back to zero for the next kernel on the stream.
 template <int KS>
 __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, float (*red)[16][64], int wave, int lane,
-                                                 int m0, int col, bool col_ok, int z, float *partials, unsigned *counters) {
+                                                 int m0, int col, bool col_ok, int z, unsigned tile, float *partials, unsigned *counters) {
   if (KS > 1) {
     if (wave > 0) {
 #pragma unroll
@@ -49,7 +49,6 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
   }
   const int splits = (int)gridDim.y;
   if (splits > 1) {
-    const unsigned tile = blockIdx.z * gridDim.x + blockIdx.x;
     float *mine = partials + ((size_t)tile * splits + blockIdx.y) * 1024;
 #pragma unroll
     for (int r = 0; r < 16; r++) __hip_atomic_store(&mine[r * 64 + lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -97,8 +96,15 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
                                                                     unsigned *counters) {
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
-  const int tiles_n = (a.Ncols + 31) / 32;
-  const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+  // Workgroup ids go round-robin over the 8 XCDs (gridDim.x is a multiple of 8,
+  // so that holds for every y and z as well).  Renumbered so that one XCD owns
+  // a contiguous run of tiles, column tiles of one filter-row tile first: a
+  // slice of the filter is then fetched into one L2 instead of all eight.
+  const int tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * ((a.M + 31) / 32);
+  const int per_xcd = (int)(gridDim.x >> 3);
+  const int tile_id = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+  if (tile_id >= tiles) return;
+  const int tile_m = tile_id / tiles_n, tile_n = tile_id - tile_m * tiles_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
   const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
   const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
@@ -161,7 +167,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, partials, counters);
+  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // 1x1 geometry (convolution, possibly strided, or matrix product with A rows
@@ -171,8 +177,15 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
                                                                     unsigned *counters) {
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
-  const int tiles_n = (a.Ncols + 31) / 32;
-  const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+  // Workgroup ids go round-robin over the 8 XCDs (gridDim.x is a multiple of 8,
+  // so that holds for every y and z as well).  Renumbered so that one XCD owns
+  // a contiguous run of tiles, column tiles of one filter-row tile first: a
+  // slice of the filter is then fetched into one L2 instead of all eight.
+  const int tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * ((a.M + 31) / 32);
+  const int per_xcd = (int)(gridDim.x >> 3);
+  const int tile_id = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+  if (tile_id >= tiles) return;
+  const int tile_m = tile_id / tiles_n, tile_n = tile_id - tile_m * tiles_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
   const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
   const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
@@ -225,7 +238,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, partials, counters);
+  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // Returns true if one of the specialised kernels took the problem.
@@ -256,7 +269,7 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
          ceil_div(red_len, ks * splits * 2) >= min_slice &&
          (int64_t)tiles * a.Z * splits * 2 * 4096 <= SPLITK_PARTIAL_BYTES && (int64_t)tiles * a.Z <= SPLITK_MAX_TILES)
     splits *= 2;
-  dim3 grid(tiles, splits, a.Z);
+  dim3 grid((unsigned)(ceil_div(tiles, 8) * 8), splits, a.Z);
 #define LAUNCH_KS2(KERNEL, AMC_, ARG)                                                                  \
   switch (ks) {                                                                                          \
     case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break;  \
