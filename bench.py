@@ -168,7 +168,13 @@ def main():
         olib = ctypes.CDLL(oracle_path)
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
         olib.dnnrtOracleSetThreads(cores)
-        so = prog.session(compiler.MODE_RESIDENT, runtime_library=oracle_path)
+        cpu_prog = prog
+        _, wl_flags, _, _, _ = build_workload(args.workload)
+        if wl_flags.get("channels_last"):
+            # the oracle keeps the reference's N,C,H,W layout: same graph, same flags otherwise
+            (cpu_graph, _), _, _, _, _ = build_workload(args.workload)
+            cpu_prog = cpu_graph.compile(**{k: v for k, v in wl_flags.items() if k != "channels_last"})
+        so = cpu_prog.session(compiler.MODE_RESIDENT, runtime_library=oracle_path)
         t0 = time.perf_counter()
         so.run(*inputs)
         first = time.perf_counter() - t0
