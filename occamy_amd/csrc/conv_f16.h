@@ -11,6 +11,7 @@ struct ConvF16Args {
   int N, C, H, W, K, Cg, R, S, P, Q, ph, pw, sh, sw, group;
   int act;     // DNNRT_ACT_RELU / DNNRT_ACT_IDENTITY
   int format;  // physical layout of X and Y (DNNRT_NCHW / NHWC / NCHW_TO_NHWC)
+  unsigned magic_pq, magic_q;  // filled in by the launcher: ceil(2^32 / (P*Q)), ceil(2^32 / Q)
 };
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a);

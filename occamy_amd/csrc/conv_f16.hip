@@ -63,6 +63,16 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // own: the kernel renumbers them so that one XCD works on a contiguous run of
 // tiles (k_out tiles of one pixel tile first), which then share their
 // operands in that L2.
+// x / d for 0 <= x < 2^31 with magic = ceil(2^32 / d) from the host: one
+// multiply-high and a correction instead of ~40 instructions of integer division.
+__device__ __forceinline__ int div_magic(int x, int d, unsigned magic) {
+  int q = (int)__umulhi((unsigned)x, magic);
+  int r = x - q * d;
+  if (r < 0) { q--; r += d; }
+  if (r >= d) q++;
+  return q;
+}
+
 template <int BM, int BN, int WM, int WN, int DEPTH, int MINWG, bool MASKED>
 __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
@@ -116,17 +126,19 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
     const int id = tid + i * 256, row = id >> 3, ch = id & 7;
     const int pix = n0 + row;
     const bool ok = pix < NPQ;
-    const int n = ok ? pix / PQ : 0;
+    const int n = ok ? div_magic(pix, PQ, a.magic_pq) : 0;
     const int pq = ok ? pix - n * PQ : 0;
-    const int p = pq / a.Q, q = pq - p * a.Q;
+    const int p = div_magic(pq, a.Q, a.magic_q), q = pq - p * a.Q;
     const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
     b_pix[i] = 2 * (((n * a.H + ih0) * a.W + iw0) * a.C + ch * 8);  // bytes; negative inside the padding
     unsigned taps = 0;
-    if (MASKED) {
+    if (MASKED && ok) {
+      // taps (r, s) inside the image: r in [r_lo, r_hi), s in [s_lo, s_hi)
+      const int r_lo = max(0, -ih0), r_hi = min(a.R, a.H - ih0);
+      const int s_lo = max(0, -iw0), s_hi = min(a.S, a.W - iw0);
+      const unsigned row_bits = s_hi > s_lo ? ((1u << (s_hi - s_lo)) - 1u) << s_lo : 0u;
       for (int r = 0; r < a.R; r++)
-        for (int s = 0; s < a.S; s++)
-          if (ok && (unsigned)(ih0 + r) < (unsigned)a.H && (unsigned)(iw0 + s) < (unsigned)a.W)
-            taps |= 1u << (r * a.S + s);
+        if (r >= r_lo && r < r_hi) taps |= row_bits << (r * a.S);
     }
     b_taps[i] = taps;
   }
@@ -273,6 +285,18 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
   const bool relu_now = a.act == DNNRT_ACT_RELU && !Zg;  // with a residual the activation comes after the sum
   _Float16 *Cs = smem;  // [BN pixels][CROW]
+  // the residual chunks this thread will need, requested now (clamped
+  // addresses) so that they arrive while the tile is staged through LDS
+  constexpr int CH_PER_ROW = BM / 8, OUT_IT = BN * CH_PER_ROW / 256;
+  half8 zpre[OUT_IT];
+  if (Zg) {
+#pragma unroll
+    for (int it = 0; it < OUT_IT; it++) {
+      const int id = tid + it * 256, row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
+      const int pix = min(n0 + row, NPQ - 1), k_out = min(m0 + ch * 8, a.K - 8);
+      zpre[it] = *reinterpret_cast<const half8 *>(Zg + (int64_t)pix * a.K + k_out);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -291,9 +315,9 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
       }
   __syncthreads();
   _Float16 *__restrict__ Yg = reinterpret_cast<_Float16 *>(a.Y);
-  constexpr int CH_PER_ROW = BM / 8;
 #pragma unroll
-  for (int id = tid; id < BN * CH_PER_ROW; id += 256) {
+  for (int it = 0; it < OUT_IT; it++) {
+    const int id = tid + it * 256;
     const int row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
     const int pix = n0 + row, k_out = m0 + ch * 8;
     if (pix < NPQ && k_out < a.K) {
@@ -301,7 +325,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
       if (Zg) {
         // conv + bias was rounded to fp16 above, as a separate convolution
         // would have stored it; the residual sum follows in fp32
-        const half8 zv = *reinterpret_cast<const half8 *>(Zg + (int64_t)pix * a.K + k_out);
+        const half8 zv = zpre[it];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           float v = (float)o[e] + (float)zv[e];
@@ -406,6 +430,11 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
                     aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) && aligned16(a.Z) &&
                     (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0;
   if (fast) {
+    ConvF16Args am = a;
+    auto magic_of = [](int d) { return (unsigned)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d > 0xffffffffull
+                                                   ? 0xffffffffull : (((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d); };
+    am.magic_pq = magic_of(a.P * a.Q);
+    am.magic_q = magic_of(a.Q);
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
     const bool pad = a.ph != 0 || a.pw != 0;
 #define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MINWG_)                                                    \
@@ -415,10 +444,10 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                              \
     if (pad || NPQ % BN_ != 0 || a.K % BM_ != 0)                                                           \
       hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, true>), dim3(grid),     \
-                         dim3(256), 0, ctx->stream, a, (int)tiles);                                        \
+                         dim3(256), 0, ctx->stream, am, (int)tiles);                                       \
     else                                                                                                   \
       hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, false>), dim3(grid),    \
-                         dim3(256), 0, ctx->stream, a, (int)tiles);                                        \
+                         dim3(256), 0, ctx->stream, am, (int)tiles);                                       \
   } while (0)
     // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
     // (14.8 GFLOP 3x3 layers run in 28-38 us, 1x1 layers near their HBM time):
