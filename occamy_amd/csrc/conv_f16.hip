@@ -73,11 +73,21 @@ __device__ __forceinline__ int div_magic(int x, int d, unsigned magic) {
   return q;
 }
 
-template <int BM, int BN, int WM, int WN, int DEPTH, int MINWG, bool MASKED>
-__global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
+//
+// KG = 2 doubles the workgroup to eight wavefronts: wavefronts 4-7 own the
+// same output blocks as 0-3 and take the second half of every 64-k step (the
+// partial sums meet in LDS once, at the end).  Same tile, same traffic, but
+// two wavefronts per SIMD: a wavefront cannot overlap its own vector
+// arithmetic with its MFMAs, so where a CU holds a single workgroup (few
+// tiles: the 14x14 and 7x7 layers) the MFMA pipe otherwise idles during all
+// address, mask and LDS work.
+template <int BM, int BN, int WM, int WN, int DEPTH, int MINWG, bool MASKED, int KG>
+__global__ __launch_bounds__(256 * KG, MINWG) void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  constexpr int A_CH = BM * 8 / 256, B_CH = BN * 8 / 256;  // 16-byte chunks per thread per step
+  static_assert(KG == 1 || KG == 2, "one or two k groups");
+  constexpr int NT = 256 * KG;
+  constexpr int A_CH = BM * 8 / NT, B_CH = BN * 8 / NT;  // 16-byte chunks per thread per step
   static_assert(A_CH >= 1 && B_CH >= 1, "tile too small");
   constexpr int STAGE = (BM + BN) * LDS_ROW;               // halfs per pipeline stage
   constexpr int CROW = BM + 8;                             // halfs per row of the output staging tile
@@ -89,7 +99,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
   if (tile >= tiles_total) return;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3, kg = tid >> 8;
   const int l32 = lane & 31, half = lane >> 5;
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
 
@@ -111,7 +121,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   unsigned a_off[A_CH], a_msk[A_CH];
 #pragma unroll
   for (int i = 0; i < A_CH; i++) {
-    const int id = tid + i * 256, row = id >> 3, ch = id & 7;
+    const int id = tid + i * NT, row = id >> 3, ch = id & 7;
     const int k_out = m0 + row;
     const bool ok = k_out < a.K;
     a_off[i] = 2u * (unsigned)((ok ? k_out : 0) * CRS + ch * 8);
@@ -123,7 +133,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   unsigned b_taps[B_CH];
 #pragma unroll
   for (int i = 0; i < B_CH; i++) {
-    const int id = tid + i * 256, row = id >> 3, ch = id & 7;
+    const int id = tid + i * NT, row = id >> 3, ch = id & 7;
     const int pix = n0 + row;
     const bool ok = pix < NPQ;
     const int n = ok ? div_magic(pix, PQ, a.magic_pq) : 0;
@@ -189,14 +199,14 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
     _Float16 *As = smem + buf * STAGE, *Bs = As + BM * LDS_ROW;
 #pragma unroll
     for (int i = 0; i < A_CH; i++) {
-      const int id = tid + i * 256, row = id >> 3, ch = id & 7;
+      const int id = tid + i * NT, row = id >> 3, ch = id & 7;
       u32x4 v = qa[i];
       if (MASKED) v &= a_msk[i];
       *reinterpret_cast<u32x4 *>(As + row * LDS_ROW + ((ch ^ st_swz) * 8)) = v;
     }
 #pragma unroll
     for (int i = 0; i < B_CH; i++) {
-      const int id = tid + i * 256, row = id >> 3, ch = id & 7;
+      const int id = tid + i * NT, row = id >> 3, ch = id & 7;
       u32x4 v = qb[i];
       if (MASKED) v &= qm[i];
       *reinterpret_cast<u32x4 *>(Bs + row * LDS_ROW + ((ch ^ st_swz) * 8)) = v;
@@ -264,15 +274,23 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   auto step = [&](auto slot_c) {
     constexpr int U = decltype(slot_c)::value, S = U & 1, N = (U + 1) % DEPTH;
     load_step(ra[U], rb[U], rm[U]);
-    read_frags(S, fa[0], fb[0], 0);
-    read_frags(S, fa[1], fb[1], 1);
-    mfma_frags(fa[0], fb[0]);
-    read_frags(S, fa[0], fb[0], 2);
-    mfma_frags(fa[1], fb[1]);
-    store_step(S ^ 1, ra[N], rb[N], rm[N]);
-    read_frags(S, fa[1], fb[1], 3);
-    mfma_frags(fa[0], fb[0]);
-    mfma_frags(fa[1], fb[1]);
+    if constexpr (KG == 1) {
+      read_frags(S, fa[0], fb[0], 0);
+      read_frags(S, fa[1], fb[1], 1);
+      mfma_frags(fa[0], fb[0]);
+      read_frags(S, fa[0], fb[0], 2);
+      mfma_frags(fa[1], fb[1]);
+      store_step(S ^ 1, ra[N], rb[N], rm[N]);
+      read_frags(S, fa[1], fb[1], 3);
+      mfma_frags(fa[0], fb[0]);
+      mfma_frags(fa[1], fb[1]);
+    } else {  // this k group's half of the step: sub-steps 2 kg and 2 kg + 1
+      read_frags(S, fa[0], fb[0], 2 * kg);
+      read_frags(S, fa[1], fb[1], 2 * kg + 1);
+      mfma_frags(fa[0], fb[0]);
+      store_step(S ^ 1, ra[N], rb[N], rm[N]);
+      mfma_frags(fa[1], fb[1]);
+    }
     __syncthreads();
   };
   using std::integral_constant;
@@ -295,21 +313,46 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   // ---- epilogue: bias, activation, fp16, transpose through LDS ------------
   // register r of lane l in block (i, j): k_out = 8*(r/4) + 4*(l/32) + r%4,
   // pixel = l%32 -> four consecutive k_out per register group.
+  if constexpr (KG == 2) {
+    // the second k group hands its partial sums over through LDS (the step
+    // loop ended on a barrier: nobody reads the operand stages any more)
+    static_assert(4 * TM * TN * 16 * 64 * 2 <= SMEM, "partial sums must fit in the operand stages");
+    float *red = reinterpret_cast<float *>(smem);
+    if (kg == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) red[(((wave * TM + i) * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+    }
+    __syncthreads();
+    if (kg == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][j][r] += red[(((wave * TM + i) * TN + j) * 16 + r) * 64 + lane];
+    }
+    __syncthreads();  // the output staging below reuses the same LDS
+  }
   const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
   const bool relu_now = a.act == DNNRT_ACT_RELU && !Zg;  // with a residual the activation comes after the sum
   _Float16 *Cs = smem;  // [BN pixels][CROW]
   // the residual chunks this thread will need, requested now (clamped
   // addresses) so that they arrive while the tile is staged through LDS
-  constexpr int CH_PER_ROW = BM / 8, OUT_IT = BN * CH_PER_ROW / 256;
+  constexpr int CH_PER_ROW = BM / 8, OUT_IT = BN * CH_PER_ROW / NT;
   half8 zpre[OUT_IT];
   if (Zg) {
 #pragma unroll
     for (int it = 0; it < OUT_IT; it++) {
-      const int id = tid + it * 256, row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
+      const int id = tid + it * NT, row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
       const int pix = min(n0 + row, NPQ - 1), k_out = min(m0 + ch * 8, a.K - 8);
       zpre[it] = *reinterpret_cast<const half8 *>(Zg + (int64_t)pix * a.K + k_out);
     }
   }
+  if (KG == 1 || kg == 0)
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -330,7 +373,7 @@ __global__ __launch_bounds__(256, MINWG) void conv_f16_nhwc_kernel(const ConvF16
   _Float16 *__restrict__ Yg = reinterpret_cast<_Float16 *>(a.Y);
 #pragma unroll
   for (int it = 0; it < OUT_IT; it++) {
-    const int id = tid + it * 256;
+    const int id = tid + it * NT;
     const int row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
     const int pix = n0 + row, k_out = m0 + ch * 8;
     if (pix < NPQ && k_out < a.K) {
@@ -450,39 +493,45 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     am.magic_q = magic_of(a.Q);
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
     const bool pad = a.ph != 0 || a.pw != 0;
-#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MINWG_)                                                    \
+#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MINWG_, KG_)                                                    \
   do {                                                                                                     \
     const int64_t tiles = tiles_of(BM_, BN_);                                                              \
     if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                  \
     const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                              \
     if (pad || NPQ % BN_ != 0 || a.K % BM_ != 0)                                                           \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, true>), dim3(grid),     \
-                         dim3(256), 0, ctx->stream, am, (int)tiles);                                       \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, true, KG_>), dim3(grid), \
+                         dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
     else                                                                                                   \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, false>), dim3(grid),    \
-                         dim3(256), 0, ctx->stream, am, (int)tiles);                                       \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, false, KG_>), dim3(grid), \
+                         dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
   } while (0)
     // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
-    // (14.8 GFLOP 3x3 layers run in 28-38 us, 1x1 layers near their HBM time):
-    // 128x128 when it yields at least ~0.6 workgroups per CU and the reduction
-    // is long enough to amortise the larger tile's prologue and epilogue;
-    // 128x64 for few-tile or short-reduction problems; 64x64 when K_out <= 64.
+    // (14.8 GFLOP 3x3 layers run in 25-35 us, 1x1 layers near their HBM time):
+    // 128x128 when there are enough tiles for more than one workgroup per CU;
+    // with about one per CU or fewer, the eight-wavefront variants (128x128,
+    // then 128x64), which keep two wavefronts on every SIMD; 128x64 for very
+    // short reductions; 64x64 when K_out <= 64.
     const int tile_sel = ctx->f16_tile;  // 0 = automatic; otherwise forced (tuning and tests)
     int sel = tile_sel;
     if (sel == 0) {
       const int nk = a.R * a.S * (a.C / BKF);
+      const int64_t t128 = tiles_of(128, 128), cus = ctx->num_cu;
       if (a.K <= 64) sel = 4;
-      else if (nk <= 2 || tiles_of(128, 128) < (3 * (int64_t)ctx->num_cu) / 5) sel = 7;
-      else sel = 3;
+      else if (nk <= 2) sel = 7;
+      else if (4 * t128 >= 5 * cus) sel = 3;
+      else if (5 * t128 >= 3 * cus) sel = 12;
+      else sel = 11;
     }
     switch (sel) {
-      case 1: LAUNCH_FAST(256, 128, 2, 2, 2, 1); break;
-      case 2: LAUNCH_FAST(128, 256, 2, 2, 2, 1); break;
-      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2); break;
-      case 5: LAUNCH_FAST(64, 256, 1, 4, 2, 2); break;
-      case 6: LAUNCH_FAST(64, 128, 1, 4, 2, 2); break;
-      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2); break;
-      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2); break;
+      case 1: LAUNCH_FAST(256, 128, 2, 2, 2, 1, 1); break;
+      case 2: LAUNCH_FAST(128, 256, 2, 2, 2, 1, 1); break;
+      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1); break;
+      case 5: LAUNCH_FAST(64, 256, 1, 4, 2, 2, 1); break;
+      case 6: LAUNCH_FAST(64, 128, 1, 4, 2, 2, 1); break;
+      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1); break;
+      case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2); break;
+      case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2); break;
+      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1); break;
     }
 #undef LAUNCH_FAST
   } else {
