@@ -10,16 +10,16 @@
 //   tile BM k_out x BN pixels, BK = 64; per step every thread moves 16-byte
 //   chunks global -> registers -> LDS (128-byte rows with an XOR swizzle of the
 //   chunk position, which makes both the stores and the ds_read_b128 operand
-//   fetches conflict-free); registers prefetch the
-//   next step while the MFMAs of the current one run; LDS is double-buffered,
-//   one barrier per step.  A BK step lies inside one (r, s) tap, so the tap
-//   and its bounds check are wave-uniform.  The epilogue adds bias, applies the
-//   activation, converts to fp16 and goes through LDS once more so that global
-//   stores are full 16-byte chunks of a pixel's channel vector.
+//   fetches conflict-free); two register stages of loads in flight, LDS
+//   double buffered, one barrier per step.  A step lies inside one (r, s) tap,
+//   so the tap and its bounds check are wave-uniform.  The epilogue adds bias,
+//   applies the activation (after the residual sum, if there is one), converts
+//   to fp16 and goes through LDS once more so that global stores are full
+//   16-byte chunks of a pixel's channel vector.
 //
-// Generic kernel (any C, NCHW or NHWC on either side): same MFMA structure
-// with element-wise gathers; it serves the first convolution of a network
-// (3 input channels, NCHW from the host) and odd shapes.
+// Generic kernel (any C, groups, NCHW or NHWC on either side): same MFMA
+// structure with element-wise gathers, for the shapes neither the fast kernel
+// nor the first-layer kernel (conv_f16_stem.hip) takes.
 #include "conv_f16.h"
 
 #include <type_traits>
