@@ -35,6 +35,17 @@ int32_t dnncGraphAddConstant(dnncGraph *g, const char *name, int32_t dtype, int3
 /* attrs: "key=v1,v2;key2=v" -- integer lists, or a float when the value has a '.' or 'e' */
 int32_t dnncGraphAddNode(dnncGraph *g, const char *op_type, int32_t n_inputs, const char *const *inputs, const char *output, const char *attrs);
 int32_t dnncGraphAddOutput(dnncGraph *g, const char *name);
+/* The reference's own input format: an ONNX model file
+ * (`core-dnn --EmitLib ... model.onnx`, test/models/simpleconv/run.py:56-60 of
+ * the reference).  `bytes` is the whole file (a serialized ModelProto); the
+ * tensors are copied.  Static shapes, float / float16 / int64 tensors, one
+ * output per node; NULL on error (dnncLastError says which construct). */
+dnncGraph *dnncGraphFromOnnx(const void *bytes, int64_t nbytes);
+int32_t dnncGraphNumInputs(const dnncGraph *g);
+int32_t dnncGraphNumOutputs(const dnncGraph *g);
+const char *dnncGraphInputName(const dnncGraph *g, int32_t i);   /* valid while the graph lives */
+const char *dnncGraphOutputName(const dnncGraph *g, int32_t i);
+int32_t dnncGraphInputInfo(const dnncGraph *g, int32_t i, int32_t *dtype, int32_t *rank, int64_t *dims, int32_t cap);
 
 /* ---- compilation ---- */
 typedef struct {

@@ -1,0 +1,58 @@
+"""``python -m occamy_amd model.onnx``: compile an ONNX file with the reference's
+flags and time it, the way the reference's test scripts do
+(test/models/*/run.py: export, ``core-dnn --EmitLib --dnn-dealloc-opt=true
+--dnn-malloc-pool-opt=true model.onnx``, run N times discarding the first,
+report mean / P90 / P95 / P99 in milliseconds)."""
+import argparse
+import time
+
+import numpy as np
+
+from . import compiler
+
+
+def main():
+    ap = argparse.ArgumentParser(prog="python -m occamy_amd")
+    ap.add_argument("model", help="ONNX model file (static shapes)")
+    ap.add_argument("--dnn-kernel-fusion", dest="fusion", action="store_true")
+    ap.add_argument("--fuse-residual", action="store_true", help="with fusion: conv+bias -> add -> relu as one call")
+    ap.add_argument("--no-dnn-dealloc-opt", dest="dealloc_opt", action="store_false")
+    ap.add_argument("--no-onnx-const-at-use", dest="const_at_use", action="store_false")
+    ap.add_argument("--channels-last", action="store_true", help="fp16 graphs: NHWC on the device")
+    ap.add_argument("--resident", action="store_true", help="keep pool and weights on the device between runs")
+    ap.add_argument("--runtime", default=None, help="shared object exporting include/dnnrt.h (default: the gfx950 library)")
+    ap.add_argument("--iterations", type=int, default=100)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--emit", action="store_true", help="print the DNN program and stop")
+    args = ap.parse_args()
+
+    graph = compiler.load_onnx(args.model)
+    prog = graph.compile(fusion=args.fusion, fuse_residual=args.fuse_residual, dealloc_opt=args.dealloc_opt,
+                         const_at_use=args.const_at_use, channels_last=args.channels_last)
+    print(f"inputs: {graph.input_shapes}")
+    print(f"pool: {prog.pool_bytes} bytes (maxAllocByte); {prog.num_ops(compute_only=True)} runtime calls per inference")
+    if args.emit:
+        print(prog.text)
+        return
+    rng = np.random.default_rng(args.seed)
+    inputs = []
+    for name, (shape, dt) in graph.input_shapes.items():
+        inputs.append(rng.integers(0, 100, shape).astype(dt) if dt == np.int64 else rng.standard_normal(shape).astype(dt))
+    sess = prog.session(compiler.MODE_RESIDENT if args.resident else compiler.MODE_OCCAMY, runtime_library=args.runtime)
+    times = []
+    for i in range(args.iterations + 1):
+        t0 = time.perf_counter()
+        out = sess.run(*inputs)
+        dt = (time.perf_counter() - t0) * 1e3
+        if i:
+            times.append(dt)
+        else:
+            print(f"first run: {dt:.3f} ms")
+    sess.close()
+    t = np.array(times)
+    print(f"outputs: {[o.shape for o in out]}")
+    print(f"mean {t.mean():.3f} ms  P90 {np.percentile(t, 90):.3f}  P95 {np.percentile(t, 95):.3f}  P99 {np.percentile(t, 99):.3f}")
+
+
+if __name__ == "__main__":
+    main()

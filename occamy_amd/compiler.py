@@ -48,6 +48,12 @@ def lib():
         "dnncGraphAddConstant": (C.c_int32, [P, C.c_char_p, C.c_int32, C.c_int32, I64P, P]),
         "dnncGraphAddNode": (C.c_int32, [P, C.c_char_p, C.c_int32, C.POINTER(C.c_char_p), C.c_char_p, C.c_char_p]),
         "dnncGraphAddOutput": (C.c_int32, [P, C.c_char_p]),
+        "dnncGraphFromOnnx": (P, [C.c_char_p, C.c_int64]),
+        "dnncGraphNumInputs": (C.c_int32, [P]),
+        "dnncGraphNumOutputs": (C.c_int32, [P]),
+        "dnncGraphInputName": (C.c_char_p, [P, C.c_int32]),
+        "dnncGraphOutputName": (C.c_char_p, [P, C.c_int32]),
+        "dnncGraphInputInfo": (C.c_int32, [P, C.c_int32, I32P, I32P, I64P, C.c_int32]),
         "dnncCompile": (P, [P, C.POINTER(_Options)]),
         "dnncProgramDestroy": (None, [P]),
         "dnncProgramText": (C.c_char_p, [P]),
@@ -106,11 +112,29 @@ def plan_free_list(events, upto):
     return [(out[2 * i], out[2 * i + 1]) for i in range(m)]
 
 
+def load_onnx(source):
+    """An ONNX model file (a path, or the file's bytes) as a Graph: what the
+    reference is given on its command line (``core-dnn --EmitLib model.onnx``).
+    The Python-side mirror holds the inputs and outputs only."""
+    data = source if isinstance(source, (bytes, bytearray)) else open(source, "rb").read()
+    h = lib().dnncGraphFromOnnx(bytes(data), len(data))
+    if not h:
+        raise RuntimeError(_err())
+    g = Graph(_handle=h)
+    for i in range(lib().dnncGraphNumInputs(h)):
+        dt, rank, d = C.c_int32(), C.c_int32(), (C.c_int64 * 8)()
+        if lib().dnncGraphInputInfo(h, i, C.byref(dt), C.byref(rank), d, 8):
+            raise RuntimeError(_err())
+        g.input_shapes[lib().dnncGraphInputName(h, i).decode()] = (tuple(d[:rank.value]), np.dtype(_NP[dt.value]))
+    g.outputs = [lib().dnncGraphOutputName(h, i).decode() for i in range(lib().dnncGraphNumOutputs(h))]
+    return g
+
+
 class Graph:
     """An ONNX-level graph: named tensors, constants, nodes with ONNX operator names."""
 
-    def __init__(self):
-        self._g = lib().dnncGraphCreate()
+    def __init__(self, _handle=None):
+        self._g = _handle if _handle is not None else lib().dnncGraphCreate()
         self._n = 0
         # Python-side mirror of what was added, for inspection and for
         # evaluating the same graph with another engine

@@ -81,8 +81,9 @@ __device__ __forceinline__ int div_magic(int x, int d, unsigned magic) {
 // arithmetic with its MFMAs, so where a CU holds a single workgroup (few
 // tiles: the 14x14 and 7x7 layers) the MFMA pipe otherwise idles during all
 // address, mask and LDS work.
-template <int BM, int BN, int WM, int WN, int DEPTH, int MINWG, bool MASKED, int KG>
-__global__ __launch_bounds__(256 * KG, MINWG) void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
+template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG>
+__global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefronts per SIMD the register budget must allow
+ void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(KG == 1 || KG == 2, "one or two k groups");
@@ -493,16 +494,16 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     am.magic_q = magic_of(a.Q);
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
     const bool pad = a.ph != 0 || a.pw != 0;
-#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MINWG_, KG_)                                                    \
+#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, KG_)                                                    \
   do {                                                                                                     \
     const int64_t tiles = tiles_of(BM_, BN_);                                                              \
     if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                  \
     const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                              \
     if (pad || NPQ % BN_ != 0 || a.K % BM_ != 0)                                                           \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, true, KG_>), dim3(grid), \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, true, KG_>), dim3(grid), \
                          dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
     else                                                                                                   \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MINWG_, false, KG_>), dim3(grid), \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, false, KG_>), dim3(grid), \
                          dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
   } while (0)
     // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
@@ -523,11 +524,7 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       else sel = 11;
     }
     switch (sel) {
-      case 1: LAUNCH_FAST(256, 128, 2, 2, 2, 1, 1); break;
-      case 2: LAUNCH_FAST(128, 256, 2, 2, 2, 1, 1); break;
       case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1); break;
-      case 5: LAUNCH_FAST(64, 256, 1, 4, 2, 2, 1); break;
-      case 6: LAUNCH_FAST(64, 128, 1, 4, 2, 2, 1); break;
       case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1); break;
       case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2); break;
       case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2); break;

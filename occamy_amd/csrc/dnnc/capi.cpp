@@ -25,6 +25,34 @@ const char *dnncLastError(void) { return g_err.c_str(); }
 dnncGraph *dnncGraphCreate(void) { return new dnncGraph(); }
 void dnncGraphDestroy(dnncGraph *g) { delete g; }
 
+dnncGraph *dnncGraphFromOnnx(const void *bytes, int64_t nbytes) {
+  if (!bytes || nbytes <= 0) { g_err = "dnncGraphFromOnnx: empty buffer"; return nullptr; }
+  dnncGraph *g = new dnncGraph();
+  std::string err;
+  if (!graph_from_onnx((const uint8_t *)bytes, (size_t)nbytes, g->g, err)) {
+    g_err = "dnncGraphFromOnnx: " + err;
+    delete g;
+    return nullptr;
+  }
+  return g;
+}
+int32_t dnncGraphNumInputs(const dnncGraph *g) { return g ? (int32_t)g->g.inputs.size() : 0; }
+int32_t dnncGraphNumOutputs(const dnncGraph *g) { return g ? (int32_t)g->g.outputs.size() : 0; }
+const char *dnncGraphInputName(const dnncGraph *g, int32_t i) {
+  return (g && i >= 0 && (size_t)i < g->g.inputs.size()) ? g->g.inputs[(size_t)i].c_str() : nullptr;
+}
+const char *dnncGraphOutputName(const dnncGraph *g, int32_t i) {
+  return (g && i >= 0 && (size_t)i < g->g.outputs.size()) ? g->g.outputs[(size_t)i].c_str() : nullptr;
+}
+int32_t dnncGraphInputInfo(const dnncGraph *g, int32_t i, int32_t *dtype, int32_t *rank, int64_t *dims, int32_t cap) {
+  if (!g || i < 0 || (size_t)i >= g->g.inputs.size()) return fail("dnncGraphInputInfo: no such input");
+  const GTensor &t = g->g.tensors.at(g->g.inputs[(size_t)i]);
+  if (dtype) *dtype = (int32_t)t.dtype;
+  if (rank) *rank = (int32_t)t.shape.size();
+  if (dims) for (int32_t d = 0; d < cap && (size_t)d < t.shape.size(); d++) dims[d] = t.shape[(size_t)d];
+  return 0;
+}
+
 static bool valid_dtype(int32_t dt) { return dt >= 0 && dt <= 2; }
 
 int32_t dnncGraphAddInput(dnncGraph *g, const char *name, int32_t dtype, int32_t rank, const int64_t *dims) {

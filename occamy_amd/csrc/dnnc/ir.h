@@ -156,6 +156,8 @@ void erase_dummy_constants(Program &p);
 // work.cpp
 const char *op_class(const Op *op);
 void op_work(const Op *op, double &flops, double &bytes);
+// onnx_reader.cpp: an ONNX ModelProto (the reference's input format) -> Graph
+bool graph_from_onnx(const uint8_t *data, size_t nbytes, Graph &g, std::string &err);
 // passes.cpp
 void fuse_conv_bias_activ(Program &p);
 void fuse_residual_add(Program &p);

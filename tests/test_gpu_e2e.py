@@ -152,3 +152,18 @@ def test_residual_fusion_fp16_channels_last():
     # adds in fp16 arithmetic): a few fp16 ulps after 16 blocks
     np.testing.assert_allclose(fused[0].astype(np.float32), chain[0].astype(np.float32), rtol=2e-2,
                                atol=2e-2 * float(np.abs(chain[0].astype(np.float32)).max()))
+
+
+def test_model_from_an_onnx_file_runs_like_the_built_graph(tmp_path):
+    """ResNet-50 through a file: ONNX bytes -> reader -> compiler -> gfx950."""
+    import onnx_writer
+    g0, inputs = models.resnet50()
+    path = tmp_path / "resnet50.onnx"
+    path.write_bytes(onnx_writer.model_bytes(g0))
+    g1 = compiler.load_onnx(str(path))
+    p0, p1 = g0.compile(fusion=True), g1.compile(fusion=True)
+    assert p1.text == p0.text and p1.pool_bytes == p0.pool_bytes
+    s0, s1 = p0.session(), p1.session()
+    np.testing.assert_array_equal(s1.run(*inputs)[0], s0.run(*inputs)[0])
+    s0.close()
+    s1.close()

@@ -1,0 +1,170 @@
+"""The ONNX reader (the reference's input format, `core-dnn ... model.onnx`).
+
+No `onnx` package or exporter exists offline, so the files come from
+tests/onnx_writer.py, written from the same published onnx.proto3 as the reader
+but independently of it (Python, emitting; the reader is C++, parsing), plus one
+model assembled by hand below.  A graph that went through a file must compile to
+the very same DNN program (text, pool layout) as the graph built in memory."""
+import numpy as np
+import pytest
+
+import onnx_writer as ow
+from helpers import ORACLE_PATH
+from occamy_amd import compiler, models
+
+SMALL = {
+    "single_conv": models.single_conv,
+    "resnet50": lambda: models.resnet50(image=32, classes=10),
+    "mobilenet_v2": lambda: models.mobilenet_v2(image=32, classes=10),
+    "bert": lambda: models.bert_encoder(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100),
+    "bert_fused": lambda: models.bert_encoder(layers=1, hidden=64, heads=4, ffn=128, seq=16, vocab=100, fused=True),
+    "resnet50_fp16": lambda: models.resnet50(2, np.float16, image=32, classes=10),
+}
+
+# x: float[1,2] -> Relu -> y, by hand from onnx.proto3:
+#   ModelProto  08 08            ir_version = 8
+#               3A 28            graph (field 7), 40 bytes
+#   GraphProto  0A 0C            node (field 1), 12 bytes
+#     NodeProto 0A 01 78           input "x"
+#               12 01 79           output "y"
+#               22 04 52 65 6C 75  op_type "Relu"
+#               5A 13            input (field 11), 19 bytes
+#     ValueInfo 0A 01 78           name "x"
+#               12 0E              type, 14 bytes
+#       Type    0A 0C                tensor_type, 12 bytes
+#         Tensor 08 01                 elem_type = FLOAT
+#                12 08                 shape, 8 bytes
+#                   0A 02 08 01          dim { dim_value: 1 }
+#                   0A 02 08 02          dim { dim_value: 2 }
+#               62 03            output (field 12), 3 bytes
+#     ValueInfo 0A 01 79           name "y"
+HAND_MADE_RELU = bytes.fromhex(
+    "0808" "3A28"
+    "0A0C" "0A0178" "120179" "220452656C75"
+    "5A13" "0A0178" "120E" "0A0C" "0801" "1208" "0A020801" "0A020802"
+    "6203" "0A0179")
+
+
+def test_hand_assembled_model():
+    g = compiler.load_onnx(HAND_MADE_RELU)
+    assert g.input_shapes == {"x": ((1, 2), np.dtype(np.float32))} and g.outputs == ["y"]
+    p = g.compile()
+    assert "dnn.activationfwd" in p.text and p.text.count("dnn.malloc") == 0  # pooled
+    s = p.session(runtime_library=ORACLE_PATH)
+    np.testing.assert_array_equal(s.run(np.array([[-1.5, 2.0]], np.float32))[0], [[0.0, 2.0]])
+    s.close()
+
+
+LAYOUTS = [
+    dict(),                                            # raw_data, packed repeated fields
+    dict(typed_fields=True),                           # float_data / int64_data / int32_data
+    dict(typed_fields=True, packed=False),             # one element per tag
+    dict(initializers_as_inputs=True),                 # IR < 4 style
+    dict(constants_as_nodes=True),                     # Constant nodes instead of initializers
+]
+
+
+def tiny_fp16():
+    g = compiler.Graph()
+    r = np.random.default_rng(3)
+    x = g.input("x", (1, 8, 6, 6), np.float16)
+    w = g.constant((r.standard_normal((4, 8, 3, 3)) * 0.2).astype(np.float16), "w")
+    b = g.constant(r.uniform(-0.1, 0.1, 4).astype(np.float16), "b")
+    g.output(g.node("Relu", [g.node("Conv", [x, w, b], "c", kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1])], "y"))
+    return g, [r.standard_normal((1, 8, 6, 6)).astype(np.float16)]
+
+
+SMALL["tiny_fp16"] = tiny_fp16
+BIG = {"resnet50", "mobilenet_v2", "resnet50_fp16"}  # millions of weights: per-element encodings are left to the small ones
+
+
+@pytest.mark.parametrize("layout", range(len(LAYOUTS)))
+@pytest.mark.parametrize("name", list(SMALL))
+def test_file_round_trip_gives_the_same_program(name, layout):
+    if name in BIG and LAYOUTS[layout].get("typed_fields"):
+        pytest.skip("typed data fields are exercised on the small models")
+    g0, inputs = SMALL[name]()
+    data = ow.model_bytes(g0, **LAYOUTS[layout])
+    g1 = compiler.load_onnx(data)
+    assert g1.input_shapes == g0.input_shapes and g1.outputs == g0.outputs
+    flags = dict(fusion=True) if "bert" not in name else {}
+    p0, p1 = g0.compile(**flags), g1.compile(**flags)
+    assert p1.text == p0.text
+    assert p1.pool_bytes == p0.pool_bytes and p1.events() == p0.events()
+    if layout == 0:  # the tensors themselves arrived intact: same numbers out
+        s0, s1 = p0.session(runtime_library=ORACLE_PATH), p1.session(runtime_library=ORACLE_PATH)
+        for a, b in zip(s0.run(*inputs), s1.run(*inputs)):
+            np.testing.assert_array_equal(a, b)
+        s0.close(); s1.close()
+
+
+def test_file_on_disk(tmp_path):
+    g0, inputs = models.single_conv()
+    path = tmp_path / "single_conv.onnx"
+    path.write_bytes(ow.model_bytes(g0))
+    p = compiler.load_onnx(str(path)).compile()
+    assert p.pool_bytes == 1753344  # the single-conv configuration's planned pool
+
+
+def test_negative_and_large_integers_survive():
+    g = compiler.Graph()
+    x = g.input("x", (2, 3, 4), np.float32)
+    idx = g.constant(np.array([-1, 0, 2 ** 40 % 3], np.int64), "idx")   # -1: ten-byte varint
+    y = g.node("Gather", [x, idx], "y", axis=1)
+    g.output(y)
+    for layout in (dict(), dict(typed_fields=True), dict(typed_fields=True, packed=False)):
+        g1 = compiler.load_onnx(ow.model_bytes(g, **layout))
+        s = g1.compile().session(runtime_library=ORACLE_PATH)
+        xv = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+        np.testing.assert_array_equal(s.run(xv)[0], xv[:, [-1, 0, 1], :])
+        s.close()
+
+
+def _single(op, **attrs):
+    g = compiler.Graph()
+    x = g.input("x", (1, 4, 8, 8), np.float32)
+    g.output(g.node(op, [x], "y", **attrs))
+    return g
+
+
+def test_what_the_reader_refuses():
+    g0, _ = models.single_conv()
+    good = ow.model_bytes(g0)
+    with pytest.raises(RuntimeError, match="static shape"):
+        compiler.load_onnx(ow.model_bytes(g0, dynamic_batch="N"))
+    with pytest.raises(RuntimeError, match="auto_pad"):
+        compiler.load_onnx(ow.model_bytes(g0, auto_pad="SAME_UPPER"))
+    compiler.load_onnx(ow.model_bytes(g0, auto_pad="NOTSET"))           # the default spelled out is fine
+    for cut in (1, 7, len(good) // 2, len(good) - 1):                   # truncated files
+        with pytest.raises(RuntimeError):
+            compiler.load_onnx(good[:cut]).compile()
+    with pytest.raises(RuntimeError):
+        compiler.load_onnx(b"")
+    with pytest.raises(RuntimeError, match="no graph"):
+        compiler.load_onnx(ow.f_varint(1, 8))
+    # a double tensor
+    t = ow.f_bytes(1, ow.varint(1)) + ow.f_varint(2, 11) + ow.f_string(8, "w") + ow.f_bytes(9, b"\0" * 8)
+    with pytest.raises(RuntimeError, match="data type 11"):
+        compiler.load_onnx(ow.f_bytes(7, ow.f_bytes(5, t)))
+    # raw_data of the wrong length
+    t = ow.f_bytes(1, ow.varint(3)) + ow.f_varint(2, 1) + ow.f_string(8, "w") + ow.f_bytes(9, b"\0" * 8)
+    with pytest.raises(RuntimeError, match="raw_data"):
+        compiler.load_onnx(ow.f_bytes(7, ow.f_bytes(5, t)))
+    # an operator the DNN dialect has no lowering for is reported by name at compile time
+    with pytest.raises(RuntimeError, match="Selu"):
+        compiler.load_onnx(ow.model_bytes(_single("Selu"))).compile()
+    # two outputs on one node
+    n = ow.f_string(1, "x") + ow.f_string(2, "y") + ow.f_string(2, "mask") + ow.f_string(4, "MaxPool")
+    vi = ow.value_info("x", (1, 1, 4, 4), np.float32)
+    with pytest.raises(RuntimeError, match="more than one output"):
+        compiler.load_onnx(ow.f_bytes(7, ow.f_bytes(1, n) + ow.f_bytes(11, vi) + ow.f_bytes(12, ow.f_string(1, "y"))))
+
+
+def test_unknown_fields_are_skipped():
+    g0, _ = models.single_conv()
+    data = ow.model_bytes(g0)
+    # doc_string (6), model_version (5), metadata_props (14) and a 64-bit field in front
+    junk = ow.f_string(6, "doc") + ow.f_varint(5, 3) + ow.f_bytes(14, ow.f_string(1, "k") + ow.f_string(2, "v")) + \
+        ow.tag(31, 1) + b"\1\2\3\4\5\6\7\x08"
+    p = compiler.load_onnx(junk + data).compile()
+    assert p.pool_bytes == 1753344
