@@ -37,6 +37,12 @@ def build_workload(name):
         return models.bert_encoder(), dict(), 1, "seq/s", "f32"
     if name == "single_conv_fp32":
         return models.single_conv(), dict(fusion=True), 1, "img/s", "f32"
+    if name == "alexnet_fp32_bs1":
+        return models.alexnet(1, np.float32), dict(fusion=True), 1, "img/s", "f32"
+    if name == "yolo_v1_fp32_bs2":
+        return models.yolo_v1(2, np.float32), dict(fusion=True), 2, "img/s", "f32"
+    if name == "srgan_fp32_96x96":
+        return models.srgan_generator(1, np.float32, height=96, width=96), dict(fusion=True), 1, "img/s", "f32"
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -209,7 +215,8 @@ def main():
     }
     if args.extra:
         extra = {}
-        for name in ["resnet50_fp16_bs64", "mobilenet_v2_fp32_bs1", "bert_base_fp32_seq128", "single_conv_fp32"]:
+        for name in ["resnet50_fp16_bs64", "mobilenet_v2_fp32_bs1", "bert_base_fp32_seq128", "single_conv_fp32",
+                     "alexnet_fp32_bs1", "yolo_v1_fp32_bs2", "srgan_fp32_96x96"]:
             if name == args.workload:
                 continue
             try:

@@ -195,6 +195,20 @@ void *dnnrtTensorOp(dnnrtHandle_t handle, int64_t op, const void *A,
 void *dnnrtClip(dnnrtHandle_t handle, const void *X, void *Y,
                 const int64_t *dimY, float lo, float hi, int64_t rank,
                 int32_t dtype);
+/* DNNAPISpecs.inc:38 "CUDALeakyReluFunc" (cuda/CUDALeakyReluFunc.cu:4-34):
+ * Y = X < 0 ? alpha * X : X. */
+void *dnnrtLeakyRelu(dnnrtHandle_t handle, const void *X, void *Y,
+                     const int64_t *dimY, float alpha, int64_t rank,
+                     int32_t dtype);
+/* DNNAPISpecs.inc:58 "CUDAPReluFunc" (cuda/CUDAPReluFunc.cu:4-34):
+ * Y = X < 0 ? slope * X : X.  The reference kernel reads slope[0] only (one
+ * slope for the whole tensor); here the slope tensor carries its dims
+ * (`rank` entries, right-aligned to dimY by the caller) and is broadcast
+ * along every dim where dimSlope[i] == 1, as ONNX PRelu specifies -- a
+ * one-element slope gives the reference's result. */
+void *dnnrtPRelu(dnnrtHandle_t handle, const void *X, void *Y,
+                 const int64_t *dimY, const void *slope,
+                 const int64_t *dimSlope, int64_t rank, int32_t dtype);
 /* DNNAPISpecs.inc:30 "CUDAErfFunc" (cuda/CUDAErfFunc.cu:4-27). */
 void *dnnrtErf(dnnrtHandle_t handle, const void *X, void *Y,
                const int64_t *dim, int64_t rank, int32_t dtype);
@@ -280,6 +294,26 @@ void *dnnrtFlatten(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
 /* DNNAPISpecs.inc:62 "CUDAReshapeFunc" (cuda/CUDAReshapeFunc.cpp): copy. */
 void *dnnrtReshape(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
                    int64_t rankX, void *Y, int32_t dtype);
+/* DNNAPISpecs.inc:66-69 "CUDASqueeze{Int64,Float}Func"
+ * (cuda/CUDASqueezeFloatFunc.cpp:6-45) and :86-89
+ * "CUDAUnsqueeze{Int64,Float}Func": copies; dimY must be dimX with size-1
+ * dims removed / inserted (the reference passes the axes and ignores them). */
+void *dnnrtSqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                   int64_t rankX, void *Y, const int64_t *dimY, int64_t rankY,
+                   int32_t dtype);
+void *dnnrtUnsqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                     int64_t rankX, void *Y, const int64_t *dimY,
+                     int64_t rankY, int32_t dtype);
+/* DNNAPISpecs.inc:15-18 "CUDAConcat{Int64,Float}Func"
+ * (cuda/CUDAConcatFloatFunc.cu:64-99): Y = concatenation of numInputs tensors
+ * along `axis`.  X and dimX are HOST arrays (of device pointers / of host dim
+ * arrays with `rank` entries each); nothing is allocated per call, where the
+ * reference uploads both lists with cudaMalloc on every call.  Up to 16
+ * inputs (reference: 10) of rank <= 8 (reference: 4). */
+void *dnnrtConcat(dnnrtHandle_t handle, const void *const *X,
+                  const int64_t *const *dimX, void *Y, const int64_t *dimY,
+                  int64_t axis, int64_t numInputs, int32_t rank,
+                  int32_t dtype);
 /* DNNAPISpecs.inc:72-87 "CUDATranspose{2,3,4,6}D{Float,Int64}Func"
  * (cuda/CUDATranspose4DFloatFunc.cu): Y = numpy.transpose(X, perm), rank <= 6;
  * dtype DNNRT_I64 selects the Int64 variants. */

@@ -47,6 +47,8 @@ SIGNATURES = {
     "dnnrtActive": (P, [P, P, I64P, i32, P, i32]),
     "dnnrtTensorOp": (P, [P, i64, P, I64P, i32, P, I64P, i32, P, I64P, i32, f32, i32]),
     "dnnrtClip": (P, [P, P, P, I64P, f32, f32, i64, i32]),
+    "dnnrtLeakyRelu": (P, [P, P, P, I64P, f32, i64, i32]),
+    "dnnrtPRelu": (P, [P, P, P, I64P, P, I64P, i64, i32]),
     "dnnrtErf": (P, [P, P, P, I64P, i64, i32]),
     "dnnrtNegative": (P, [P, P, P, I64P, i64, i32]),
     "dnnrtReciprocal": (P, [P, P, P, I64P, i64, i32]),
@@ -62,6 +64,9 @@ SIGNATURES = {
     "dnnrtMatmulNd": (P, [P, P, I64P, i32, P, I64P, i32, P, I64P, i32, i32]),
     "dnnrtFlatten": (P, [P, P, I64P, P, I64P, i32, i64, i32]),
     "dnnrtReshape": (P, [P, P, I64P, i64, P, i32]),
+    "dnnrtSqueeze": (P, [P, P, I64P, i64, P, I64P, i64, i32]),
+    "dnnrtUnsqueeze": (P, [P, P, I64P, i64, P, I64P, i64, i32]),
+    "dnnrtConcat": (P, [P, P, P, P, I64P, i64, i64, i32, i32]),
     "dnnrtTranspose": (P, [P, P, I64P, P, I64P, I64P, i64, i32]),
     "dnnrtGather": (P, [P, P, I64P, i64, P, I64P, i64, P, I64P, i64, i64, i32]),
 }

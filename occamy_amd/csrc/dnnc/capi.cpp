@@ -142,7 +142,8 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
       if (op->result->dtype != F16) { g_err = "channels_last needs an fp16 graph"; delete pp; return nullptr; }
       switch (op->kind) {
         case OP_MALLOC: case OP_HOST_ALLOC: case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_ACTIVATION: case OP_ADD:
-        case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE: break;
+        case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE: case OP_LEAKYRELU: case OP_PRELU:
+        case OP_CONCAT: break;
         default: g_err = std::string("channels_last: ") + op_name(op->kind) + " has no channels-last form"; delete pp; return nullptr;
       }
       if (op->kind == OP_HOST_ALLOC) { g_err = "channels_last: a returned rank-4 tensor would come back in NHWC order"; delete pp; return nullptr; }

@@ -227,6 +227,45 @@ struct Emitter {
       o->dimA = ot.shape;
       result = o->result;
       park_dealloc(out_buf);
+    } else if (t == "LeakyRelu") {  // Ops/cuda/LeakyRelu.cpp
+      out_buf = malloc_(ot.dtype, ot.shape);
+      Op *o = compute(OP_LEAKYRELU, {x, out_buf});
+      o->alpha = (float)flt("alpha", 0.01);
+      o->dimA = ot.shape;
+      result = o->result;
+      park_dealloc(out_buf);
+    } else if (t == "PRelu") {  // Ops/cuda/PRelu.cpp: the slope stays a device tensor
+      Value *sl = in(1);
+      if (!sl) { err = "PRelu: slope not available"; return false; }
+      out_buf = malloc_(ot.dtype, ot.shape);
+      Op *o = compute(OP_PRELU, {x, sl, out_buf});
+      o->dimA = ot.shape;
+      o->dimB = pad_front(sl->shape, ot.shape.size());
+      result = o->result;
+      park_dealloc(out_buf);
+    } else if (t == "Concat") {  // Ops/cuda/Concat.cpp: all inputs, then the output buffer
+      std::vector<Value *> operands;
+      for (size_t i = 0; i < n.inputs.size(); i++) {
+        Value *v = in(i);
+        if (!v) { err = "Concat: input not available"; return false; }
+        operands.push_back(v);
+      }
+      if (operands.size() > 16) { err = "Concat: more than 16 inputs"; return false; }
+      out_buf = malloc_(ot.dtype, ot.shape);
+      operands.push_back(out_buf);
+      Op *o = compute(OP_CONCAT, operands);
+      o->dimOut = ot.shape;
+      o->axis = int1("axis", 0);
+      result = o->result;
+      park_dealloc(out_buf);
+    } else if (t == "Squeeze" || t == "Unsqueeze" || t == "Identity") {  // Ops/cuda/Squeeze.cpp, Unsqueeze.cpp
+      out_buf = malloc_(ot.dtype, ot.shape);
+      Op *o = compute(t == "Squeeze" ? OP_SQUEEZE : t == "Unsqueeze" ? OP_UNSQUEEZE : OP_RESHAPE, {x, out_buf});
+      o->dimA = x->shape;
+      o->dimOut = ot.shape;
+      o->perm = ints("axes", {});
+      result = o->result;
+      park_dealloc(out_buf);
     } else if (t == "Cast") {
       if (x->dtype != I64 || ot.dtype == I64) { err = "Cast: only int64 -> float is covered"; return false; }
       out_buf = malloc_(ot.dtype, ot.shape);

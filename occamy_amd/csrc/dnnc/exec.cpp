@@ -42,6 +42,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   LOAD(dnnrtGelu); LOAD(dnnrtReduce); LOAD(dnnrtSoftmax); LOAD(dnnrtLayerNorm); LOAD(dnnrtMaxPool);
   LOAD(dnnrtAveragePool); LOAD(dnnrtMatmul2d); LOAD(dnnrtMatmulNd); LOAD(dnnrtFlatten);
   LOAD(dnnrtReshape); LOAD(dnnrtTranspose); LOAD(dnnrtGather);
+  LOAD(dnnrtLeakyRelu); LOAD(dnnrtPRelu); LOAD(dnnrtConcat); LOAD(dnnrtSqueeze); LOAD(dnnrtUnsqueeze);
   return true;
 }
 #undef LOAD
@@ -54,6 +55,7 @@ Session::~Session() {
   if (handle) rt.dnnrtSync(handle);
   if (pool) rt.dnnrtDealloc(pool);
   if (weights) rt.dnnrtDealloc(weights);
+  for (auto &kv : staged_out) rt.dnnrtDealloc(kv.second);
   for (auto &kv : host_const) rt.dnnrtHostFree(kv.second);
   for (void *p : host_out) rt.dnnrtHostFree(p);
   for (void *p : host_in) rt.dnnrtHostFree(p);
@@ -183,6 +185,16 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
       ptr[(size_t)op->operands[0]->id] = dev;
     }
     if (rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); return false; }
+    // a result that is copied out before the last compute operation
+    bool compute_later = false;
+    for (auto it = prog->ops.rbegin(); it != prog->ops.rend(); ++it) {
+      const Op *op = *it;
+      if (is_compute(op->kind)) compute_later = true;
+      if (op->kind != OP_MEMCPY || op->mode != 2 || !compute_later) continue;
+      void *stage = nullptr;
+      if (rt.dnnrtMalloc(&stage, op->bytes)) { err = rt_error("dnnrtMalloc(result staging)"); return false; }
+      staged_out[op] = stage;
+    }
   }
   return true;
 }
@@ -266,6 +278,28 @@ bool Session::issue(const Op *op, std::string &err) {
     case OP_GELU: r = rt.dnnrtGelu(handle, P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
     case OP_POW: r = rt.dnnrtPow(handle, P(0), P(1), out, op->dimA.data(), (int64_t)op->dimA.size(), dt); break;
     case OP_CLIP: r = rt.dnnrtClip(handle, P(0), out, op->dimA.data(), op->lo, op->hi, (int64_t)op->dimA.size(), dt); break;
+    case OP_LEAKYRELU:
+      r = rt.dnnrtLeakyRelu(handle, P(0), out, op->dimA.data(), op->alpha, (int64_t)op->dimA.size(), dt);
+      break;
+    case OP_PRELU:
+      r = rt.dnnrtPRelu(handle, P(0), out, op->dimA.data(), P(1), op->dimB.data(), (int64_t)op->dimA.size(), dt);
+      break;
+    case OP_CONCAT: {
+      const size_t n_in = op->operands.size() - 1;
+      const void *xs[16];
+      const int64_t *ds[16];
+      for (size_t i = 0; i < n_in; i++) { xs[i] = P(i); ds[i] = op->operands[i]->shape.data(); }
+      r = rt.dnnrtConcat(handle, xs, ds, out, op->dimOut.data(), op->axis, (int64_t)n_in, (int32_t)op->dimOut.size(), dt);
+      break;
+    }
+    case OP_SQUEEZE:
+      r = rt.dnnrtSqueeze(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), out, op->dimOut.data(),
+                          (int64_t)op->dimOut.size(), dt);
+      break;
+    case OP_UNSQUEEZE:
+      r = rt.dnnrtUnsqueeze(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), out, op->dimOut.data(),
+                            (int64_t)op->dimOut.size(), dt);
+      break;
     case OP_CAST:
       r = rt.dnnrtCastI64toFloat(handle, (const int64_t *)P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt);
       break;
@@ -366,8 +400,21 @@ bool Session::run_occamy(const void *const *inputs, void *const *outputs, std::s
 }
 
 bool Session::issue_all_compute(std::string &err) {
-  for (const Op *op : prog->ops)
-    if (is_compute(op->kind) && !issue(op, err)) return false;
+  for (const Op *op : prog->ops) {
+    if (is_compute(op->kind)) {
+      if (!issue(op, err)) return false;
+    } else if (op->kind == OP_MEMCPY && op->mode == 2) {
+      auto st = staged_out.find(op);
+      if (st == staged_out.end()) continue;
+      // a copy kernel, so that a captured graph holds it too
+      const Value *v = op->operands[1];
+      const int64_t n = shape_numel(v->shape);
+      if (!rt.dnnrtReshape(handle, ptr[(size_t)v->id], &n, 1, st->second, (int32_t)v->dtype)) {
+        err = rt_error("dnnrtReshape(result staging)");
+        return false;
+      }
+    }
+  }
   return true;
 }
 
@@ -416,7 +463,9 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
     const Op *ha = op->operands[0]->def;
     const size_t oi = (size_t)ha->out_index;
     void *dst = on_device ? outputs[oi] : host_out[oi];
-    if (rt.dnnrtMemcpy(dst, ptr[(size_t)op->operands[1]->id], op->bytes, on_device ? 3 : 2, stream)) {
+    auto st = staged_out.find(op);
+    void *src = st != staged_out.end() ? st->second : ptr[(size_t)op->operands[1]->id];
+    if (rt.dnnrtMemcpy(dst, src, op->bytes, on_device ? 3 : 2, stream)) {
       err = rt_error("dnnrtMemcpy(output)"); return false;
     }
   }

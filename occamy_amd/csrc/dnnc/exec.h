@@ -59,6 +59,11 @@ struct RuntimeApi {
   decltype(&::dnnrtReshape) dnnrtReshape = nullptr;
   decltype(&::dnnrtTranspose) dnnrtTranspose = nullptr;
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
+  decltype(&::dnnrtLeakyRelu) dnnrtLeakyRelu = nullptr;
+  decltype(&::dnnrtPRelu) dnnrtPRelu = nullptr;
+  decltype(&::dnnrtConcat) dnnrtConcat = nullptr;
+  decltype(&::dnnrtSqueeze) dnnrtSqueeze = nullptr;
+  decltype(&::dnnrtUnsqueeze) dnnrtUnsqueeze = nullptr;
 };
 
 bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err);
@@ -93,6 +98,9 @@ class Session {
   std::vector<void *> ptr;  // value id -> address (host or device)
   std::map<std::string, void *> host_const;
   std::vector<void *> host_out, host_in;
+  // resident mode: results produced mid-program, whose pool bytes a later
+  // tensor may take over, are copied aside (on the device, in program order)
+  std::map<const Op *, void *> staged_out;  // the device-to-host memcpy op -> its staging buffer
 
   std::string rt_error(const char *what) const;
   int format_for(const Op *op) const;

@@ -1,9 +1,12 @@
 // ONNX-level graph: shape inference for the operator subset the DNN dialect
-// covers, and the two ONNX-level rewrites that shape the event trace:
-// GlobalAveragePool -> ReduceMean over (H, W) (done by onnx-mlir ahead of the
-// reference's own passes) and "constant at use"
-// (src/Transform/ONNX/ONNXConstantAtUsePass.cpp:29-58).
+// covers, and the ONNX-level rewrites that shape the event trace:
+// GlobalAveragePool -> ReduceMean over (H, W), Identity / inference-mode
+// Dropout removal and inference-mode BatchNormalization folded into the
+// preceding convolution or turned into Mul + Add (all done by onnx-mlir's
+// canonicalisation ahead of the reference's own passes), and "constant at
+// use" (src/Transform/ONNX/ONNXConstantAtUsePass.cpp:29-58).
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 
 #include "ir.h"
@@ -33,7 +36,169 @@ static bool broadcast_shape(const Shape &a, const Shape &b, Shape &out) {
   return true;
 }
 
-bool infer_shapes(Graph &g, std::string &err) {
+// ---- float <-> stored element, for constants rewritten at compile time
+static float half_to_float(uint16_t h) {
+  const int s = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+  const float v = e == 0 ? std::ldexp((float)m, -24) : e == 31 ? (m ? NAN : INFINITY) : std::ldexp((float)(m + 1024), e - 25);
+  return s ? -v : v;
+}
+static uint16_t float_to_half(float f) {  // round to nearest even
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7FFFFFFFu;
+  if (x >= 0x7F800000u) return (uint16_t)(sign | (x > 0x7F800000u ? 0x7E00u : 0x7C00u));
+  if (x >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);  // rounds to >= 65520: infinity
+  if (x < 0x33000001u) return (uint16_t)sign;                // below half of the smallest subnormal
+  const int e = (int)(x >> 23) - 127;
+  uint32_t m = (x & 0x7FFFFFu) | 0x800000u;
+  int shift = e < -14 ? 13 + (-14 - e) : 13;
+  uint32_t q = m >> shift;
+  const uint32_t rem = m & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+  if (rem > halfway || (rem == halfway && (q & 1))) q++;
+  // q carries the implicit one for normals; adding the exponent field lets a carry ripple into it
+  const uint32_t h = e < -14 ? q : ((uint32_t)(e + 15 - 1) << 10) + q;
+  return (uint16_t)(sign | h);
+}
+static double load_elem(const GTensor &t, int64_t i) {
+  if (t.dtype == F32) { float v; std::memcpy(&v, t.data.data() + i * 4, 4); return v; }
+  if (t.dtype == F16) { uint16_t h; std::memcpy(&h, t.data.data() + i * 2, 2); return half_to_float(h); }
+  int64_t v; std::memcpy(&v, t.data.data() + i * 8, 8); return (double)v;
+}
+static void store_elem(GTensor &t, int64_t i, double v) {
+  if (t.dtype == F32) { const float f = (float)v; std::memcpy(t.data.data() + i * 4, &f, 4); }
+  else if (t.dtype == F16) { const uint16_t h = float_to_half((float)v); std::memcpy(t.data.data() + i * 2, &h, 2); }
+  else { const int64_t q = (int64_t)v; std::memcpy(t.data.data() + i * 8, &q, 8); }
+}
+
+static int count_uses(const Graph &g, const std::string &name) {
+  int n = 0;
+  for (const GNode &m : g.nodes)
+    for (const std::string &i : m.inputs) n += i == name;
+  for (const std::string &o : g.outputs) n += o == name;
+  return n;
+}
+
+// Identity and inference-mode Dropout forward their input: later nodes read
+// the input directly.  One that produces a graph output stays, as a copy.
+static void forward_aliases(Graph &g) {
+  std::map<std::string, std::string> alias;
+  std::vector<GNode> kept;
+  for (GNode &n : g.nodes) {
+    for (std::string &i : n.inputs) {
+      auto it = alias.find(i);
+      if (it != alias.end()) i = it->second;
+    }
+    const bool fwd = (n.op_type == "Identity" || n.op_type == "Dropout") && !n.inputs.empty() && !n.inputs[0].empty();
+    if (fwd && std::find(g.outputs.begin(), g.outputs.end(), n.output) == g.outputs.end()) {
+      alias[n.output] = n.inputs[0];
+      continue;
+    }
+    if (fwd) { n.op_type = "Identity"; n.inputs.resize(1); }
+    kept.push_back(n);
+  }
+  g.nodes.swap(kept);
+}
+
+// BatchNormalization with constant statistics at g.nodes[at] (shapes are
+// known):  y = x * s[c] + t[c],  s = scale / sqrt(var + eps),  t = bias - mean * s.
+// Folded into the producing Conv when x has no other reader (w' = w * s[k],
+// b' = b * s + t), else replaced by Mul and Add with [C,1,..] constants.
+static bool rewrite_batchnorm(Graph &g, size_t at, std::string &err) {
+  const GNode bn = g.nodes[at];
+  auto fail = [&](const std::string &m) { err = "BatchNormalization '" + bn.output + "': " + m; return false; };
+  if (bn.inputs.size() < 5) return fail("needs X, scale, B, mean and var");
+  const GTensor *c[4];
+  for (int i = 0; i < 4; i++) {
+    auto it = g.tensors.find(bn.inputs[(size_t)i + 1]);
+    if (it == g.tensors.end() || !it->second.is_const) return fail("scale, B, mean and var must be constants (inference mode)");
+    c[i] = &it->second;
+  }
+  const GTensor x = g.tensors.at(bn.inputs[0]);
+  if (x.shape.size() < 2) return fail("input rank < 2");
+  const int64_t C = x.shape[1];
+  for (int i = 0; i < 4; i++)
+    if (shape_numel(c[i]->shape) != C || c[i]->dtype == I64) return fail("statistics must be float tensors with one entry per channel");
+  auto ef = bn.floats.find("epsilon");
+  const double eps = ef == bn.floats.end() ? 1e-5 : ef->second;
+  std::vector<double> s((size_t)C), t((size_t)C);
+  for (int64_t k = 0; k < C; k++) {
+    s[(size_t)k] = load_elem(*c[0], k) / std::sqrt(load_elem(*c[3], k) + eps);
+    t[(size_t)k] = load_elem(*c[1], k) - load_elem(*c[2], k) * s[(size_t)k];
+  }
+  auto new_const = [&](const std::string &name, DType dt, const Shape &shape) -> GTensor & {
+    GTensor ct;
+    ct.name = name; ct.dtype = dt; ct.shape = shape; ct.is_const = true;
+    ct.data.assign((size_t)(shape_numel(shape) * dtype_bytes(dt)), 0);
+    return g.tensors[name] = ct;
+  };
+  auto const_node = [](const std::string &name) { GNode cn; cn.op_type = "Constant"; cn.output = name; return cn; };
+  size_t prod = at;  // the producer of x
+  for (size_t i = 0; i < at; i++)
+    if (g.nodes[i].output == bn.inputs[0]) prod = i;
+  bool fold = prod != at && g.nodes[prod].op_type == "Conv" && count_uses(g, bn.inputs[0]) == 1;
+  if (fold) {
+    const GNode &cv = g.nodes[prod];
+    auto wt = g.tensors.find(cv.inputs[1]);
+    fold = wt != g.tensors.end() && wt->second.is_const && wt->second.dtype != I64 && wt->second.shape.size() == 4 && wt->second.shape[0] == C;
+    if (fold && cv.inputs.size() > 2 && !cv.inputs[2].empty()) {
+      auto bt = g.tensors.find(cv.inputs[2]);
+      fold = bt != g.tensors.end() && bt->second.is_const && shape_numel(bt->second.shape) == C;
+    }
+  }
+  std::vector<std::string> maybe_dead{bn.inputs[1], bn.inputs[2], bn.inputs[3], bn.inputs[4]};
+  std::vector<GNode> fresh;  // what replaces the BN node (and, when folding, precedes the conv)
+  if (fold) {
+    const GNode cv = g.nodes[prod];
+    const GTensor w = g.tensors.at(cv.inputs[1]);
+    const bool has_b = cv.inputs.size() > 2 && !cv.inputs[2].empty();
+    const GTensor b = has_b ? g.tensors.at(cv.inputs[2]) : GTensor();
+    const std::string wn = bn.output + "_folded_w", bname = bn.output + "_folded_b";
+    if (g.tensors.count(wn) || g.tensors.count(bname)) return fail("name clash with a folded constant");
+    GTensor &nw = new_const(wn, w.dtype, w.shape);
+    const int64_t per_k = shape_numel(w.shape) / C;
+    for (int64_t k = 0; k < C; k++)
+      for (int64_t j = 0; j < per_k; j++) store_elem(nw, k * per_k + j, load_elem(w, k * per_k + j) * s[(size_t)k]);
+    GTensor &nb = new_const(bname, w.dtype, {C});
+    for (int64_t k = 0; k < C; k++) store_elem(nb, k, (has_b ? load_elem(b, k) : 0.0) * s[(size_t)k] + t[(size_t)k]);
+    maybe_dead.push_back(cv.inputs[1]);
+    if (has_b) maybe_dead.push_back(cv.inputs[2]);
+    g.nodes.erase(g.nodes.begin() + (long)at);
+    GNode &conv = g.nodes[prod];
+    conv.inputs.resize(3);
+    conv.inputs[1] = wn;
+    conv.inputs[2] = bname;
+    conv.output = bn.output;
+    g.nodes.insert(g.nodes.begin() + (long)prod, const_node(bname));
+    g.nodes.insert(g.nodes.begin() + (long)prod, const_node(wn));
+  } else {
+    Shape cs(x.shape.size() - 1, 1);
+    cs[0] = C;
+    const std::string sn = bn.output + "_bn_scale", tn = bn.output + "_bn_shift", mid = bn.output + "_bn_scaled";
+    if (g.tensors.count(sn) || g.tensors.count(tn) || g.tensors.count(mid)) return fail("name clash with a derived constant");
+    GTensor &st = new_const(sn, x.dtype, cs);
+    for (int64_t k = 0; k < C; k++) store_elem(st, k, s[(size_t)k]);
+    GTensor &tt = new_const(tn, x.dtype, cs);
+    for (int64_t k = 0; k < C; k++) store_elem(tt, k, t[(size_t)k]);
+    GNode mul, add;
+    mul.op_type = "Mul"; mul.inputs = {bn.inputs[0], sn}; mul.output = mid;
+    add.op_type = "Add"; add.inputs = {mid, tn}; add.output = bn.output;
+    g.nodes[at] = add;
+    g.nodes.insert(g.nodes.begin() + (long)at, mul);
+    g.nodes.insert(g.nodes.begin() + (long)at, const_node(tn));
+    g.nodes.insert(g.nodes.begin() + (long)at, const_node(sn));
+  }
+  // constants that fed only the replaced nodes go away with them
+  for (const std::string &d : maybe_dead) {
+    if (count_uses(g, d) != 0) continue;
+    for (size_t j = 0; j < g.nodes.size(); j++)
+      if (g.nodes[j].op_type == "Constant" && g.nodes[j].output == d) { g.nodes.erase(g.nodes.begin() + (long)j); break; }
+    g.tensors.erase(d);
+  }
+  return true;
+}
+
+static bool infer_pass(Graph &g, std::string &err) {
   for (GNode &n : g.nodes) {
     if (n.op_type == "Constant") continue;
     // onnx-mlir rewrites GlobalAveragePool to ReduceMean(axes = spatial dims, keepdims = 1)
@@ -79,8 +244,59 @@ bool infer_shapes(Graph &g, std::string &err) {
       if (P < 1 || Q < 1) return fail("empty output");
       out.shape = {x[0], w[0], P, Q};
     } else if (t == "Relu" || t == "Sigmoid" || t == "Tanh" || t == "Sqrt" || t == "Erf" || t == "Clip" ||
-               t == "Gelu" || t == "Pow" || t == "Softmax" || t == "LayerNormalization") {
+               t == "Gelu" || t == "Pow" || t == "Softmax" || t == "LayerNormalization" || t == "LeakyRelu" ||
+               t == "Identity" || t == "BatchNormalization") {
       out.shape = x;
+    } else if (t == "PRelu") {
+      if (in.size() < 2 || !in[1]) return fail("needs a slope");
+      Shape b;
+      if (!broadcast_shape(x, in[1]->shape, b) || b != x) return fail("the slope does not broadcast to X");
+      out.shape = x;
+    } else if (t == "Concat") {
+      int64_t axis = get_int(n, "axis", 0);
+      if (axis < 0) axis += (int64_t)x.size();
+      if (axis < 0 || axis >= (int64_t)x.size()) return fail("axis out of range");
+      out.shape = x;
+      for (size_t i = 1; i < in.size(); i++) {
+        if (!in[i] || in[i]->shape.size() != x.size() || in[i]->dtype != out.dtype) return fail("inputs differ in rank or type");
+        for (size_t d = 0; d < x.size(); d++)
+          if ((int64_t)d != axis && in[i]->shape[d] != x[d]) return fail("inputs differ off the axis");
+        out.shape[(size_t)axis] += in[i]->shape[(size_t)axis];
+      }
+      n.ints["axis"] = {axis};
+    } else if (t == "Squeeze" || t == "Unsqueeze") {
+      // axes: an attribute up to opset 12, a constant input from opset 13 on
+      std::vector<int64_t> axes;
+      bool have = get_ints(n, "axes", axes);
+      if (!have && in.size() > 1 && in[1]) {
+        if (!in[1]->is_const || in[1]->dtype != I64) return fail("axes must be an int64 constant");
+        const int64_t *a = reinterpret_cast<const int64_t *>(in[1]->data.data());
+        axes.assign(a, a + in[1]->data.size() / 8);
+        have = true;
+      }
+      const int64_t rank_out = t == "Squeeze" ? (int64_t)x.size() : (int64_t)(x.size() + axes.size());
+      const int64_t rank_ref = t == "Squeeze" ? (int64_t)x.size() : rank_out;
+      std::vector<bool> mark((size_t)rank_ref, false);
+      if (t == "Unsqueeze" && !have) return fail("needs axes");
+      for (int64_t &a : axes) {
+        if (a < 0) a += rank_ref;
+        if (a < 0 || a >= rank_ref || mark[(size_t)a]) return fail("axis out of range or repeated");
+        mark[(size_t)a] = true;
+      }
+      if (t == "Squeeze") {
+        for (size_t d = 0; d < x.size(); d++) {
+          if (have ? mark[d] : x[d] == 1) {
+            if (x[d] != 1) return fail("squeezed dim is not 1");
+            if (!have) axes.push_back((int64_t)d);
+          } else {
+            out.shape.push_back(x[d]);
+          }
+        }
+      } else {
+        size_t src = 0;
+        for (int64_t d = 0; d < rank_out; d++) out.shape.push_back(mark[(size_t)d] ? 1 : x[src++]);
+      }
+      n.ints["axes"] = axes;
     } else if (t == "Add" || t == "Sub" || t == "Mul" || t == "Div") {
       if (in.size() < 2 || !in[1]) return fail("needs two inputs");
       if (!broadcast_shape(x, in[1]->shape, out.shape)) return fail("operands do not broadcast");
@@ -174,6 +390,22 @@ bool infer_shapes(Graph &g, std::string &err) {
   for (const std::string &o : g.outputs)
     if (!g.tensors.count(o)) { err = "graph output '" + o + "' is never produced"; return false; }
   return true;
+}
+
+bool infer_shapes(Graph &g, std::string &err) {
+  forward_aliases(g);
+  if (!infer_pass(g, err)) return false;
+  bool rewritten = false;
+  for (size_t i = 0; i < g.nodes.size();) {
+    if (g.nodes[i].op_type != "BatchNormalization") { i++; continue; }
+    if (!rewrite_batchnorm(g, i, err)) return false;
+    rewritten = true;
+    i = 0;
+  }
+  if (!rewritten) return true;
+  for (auto it = g.tensors.begin(); it != g.tensors.end();)  // derived shapes: inferred again
+    it = (it->second.is_input || it->second.is_const) ? std::next(it) : g.tensors.erase(it);
+  return infer_pass(g, err);
 }
 
 // Each constant is moved to just before its first user; constants sharing a

@@ -37,6 +37,11 @@ const char *op_name(OpKind k) {
     case OP_ERF: return "dnn.erf";
     case OP_CAST: return "dnn.cast";
     case OP_CLIP: return "dnn.clip";
+    case OP_LEAKYRELU: return "dnn.leakyrelu";
+    case OP_PRELU: return "dnn.prelu";
+    case OP_CONCAT: return "dnn.concat";
+    case OP_SQUEEZE: return "dnn.squeeze";
+    case OP_UNSQUEEZE: return "dnn.unsqueeze";
     case OP_LAYERNORM: return "dnn.layernorm";
     case OP_GELU: return "dnn.gelu";
     case OP_CONV_BIAS_ADD_ACTIV: return "dnn.conv-bias-add-relufwd";
@@ -190,7 +195,11 @@ std::string Program::to_text() const {
         break;
       case OP_SOFTMAX:
       case OP_FLATTEN:
+      case OP_CONCAT:
       case OP_GATHER: os << " {axis=" << op->axis << "}"; break;
+      case OP_LEAKYRELU: os << " {alpha=" << op->alpha << "}"; break;
+      case OP_SQUEEZE:
+      case OP_UNSQUEEZE: os << " {axes="; print_shape(os, op->perm); os << "}"; break;
       case OP_TRANSPOSE: os << " {perm="; print_shape(os, op->perm); os << "}"; break;
       case OP_MATMUL2D:
         os << " {alpha=" << op->alpha << ", beta=" << op->beta << ", transA=" << op->trans_a

@@ -265,7 +265,10 @@ bool parse_node(Reader r, Graph &g, std::string &err) {
   if (!r.ok) { err = "malformed NodeProto"; return false; }
   if (!domain.empty() && domain != "ai.onnx") { err = "operator '" + n.op_type + "' of domain '" + domain + "'"; return false; }
   if (outputs.empty() || outputs[0].empty()) { err = "node '" + n.op_type + "' has no output"; return false; }
-  for (size_t i = 1; i < outputs.size(); i++)
+  // Dropout's mask and BatchNormalization's running statistics are training
+  // outputs: they stay undefined, so a node that reads one is refused later
+  const bool extra_ok = n.op_type == "Dropout" || n.op_type == "BatchNormalization";
+  for (size_t i = 1; i < outputs.size() && !extra_ok; i++)
     if (!outputs[i].empty()) { err = "node '" + n.op_type + "' has more than one output ('" + outputs[i] + "')"; return false; }
   n.output = outputs[0];
   if (n.op_type == "Constant") {
@@ -281,9 +284,9 @@ bool parse_node(Reader r, Graph &g, std::string &err) {
     g.nodes.push_back(c);
     return true;
   }
-  if (n.op_type == "Identity" || n.op_type == "Dropout") {  // inference: the value itself
-    err = "operator " + n.op_type + " is not supported (simplify the model at export)";
-    return false;
+  if (n.op_type == "BatchNormalization") {
+    auto tm = n.ints.find("training_mode");
+    if (tm != n.ints.end() && !tm->second.empty() && tm->second[0] != 0) { err = "BatchNormalization in training mode"; return false; }
   }
   if (n.op_type == "Cast") {  // attribute `to` is a TensorProto.DataType
     auto it = n.ints.find("to");

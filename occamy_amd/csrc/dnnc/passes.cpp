@@ -127,7 +127,15 @@ void fuse_residual_add(Program &p) {
 // deallocs) is moved to just after its tensor's last use.  If the last direct
 // user writes the tensor (the malloc is that op's last operand), the tensor
 // lives on under the op's result, and the dealloc goes after the result's last
-// user instead.  One level of aliasing only, as in the reference.
+// user instead (src/Transform/DNN/DNNDeallocOpt.cpp:24-43).
+//
+// One case is handled differently from the reference, on purpose: a tensor
+// that the function returns AND a later operation reads (SRGAN's feature map).
+// There the last direct user is the device-to-host copy, which does not write
+// the tensor, so the reference frees it right after the copy although the
+// producer's result is still read afterwards; with the pool pass a later
+// tensor can then land on it.  Here the readers of every writer's result
+// count as uses, which gives the reference's placement in every other case.
 void dealloc_opt(Program &p) {
   std::vector<Op *> deallocs;
   for (Op *op : p.ops)
@@ -141,13 +149,19 @@ void dealloc_opt(Program &p) {
     if (!ldu || ldu == d) continue;  // nothing but the dealloc uses it
     // dnn.memcpy carries its byte count as last operand in the reference, so
     // it never counts as "writes its last operand"
-    const bool writes = ldu->kind != OP_MEMCPY && !ldu->operands.empty() && ldu->operands.back() == buf;
-    if (writes && ldu->result) {
-      Op *last = p.last_user(ldu->result);
-      p.move_after(d, last ? last : ldu);
+    auto writes = [&](const Op *u) { return u->kind != OP_MEMCPY && u->kind != OP_DEALLOC && !u->operands.empty() && u->operands.back() == buf; };
+    Op *last = ldu;
+    if (writes(ldu) && ldu->result) {
+      Op *r = p.last_user(ldu->result);
+      if (r) last = r;
     } else {
-      p.move_after(d, ldu);
+      for (const auto &u : buf->uses) {
+        if (!writes(u.first) || !u.first->result) continue;
+        Op *r = p.last_user(u.first->result);
+        if (r && p.order(r) > p.order(last)) last = r;
+      }
     }
+    p.move_after(d, last);
   }
 }
 

@@ -21,6 +21,9 @@ const char *op_class(const Op *op) {
     case OP_FLATTEN:
     case OP_RESHAPE:
     case OP_TRANSPOSE:
+    case OP_CONCAT:
+    case OP_SQUEEZE:
+    case OP_UNSQUEEZE:
     case OP_GATHER: return "move";
     default: return "elementwise";
   }
@@ -62,6 +65,10 @@ void op_work(const Op *op, double &flops, double &bytes) {
       break;
     case OP_GATHER:
       bytes = 2.0 * n_out * es + n_in(1) * 8.0;
+      break;
+    case OP_PRELU:
+      flops = n_out;
+      bytes = (2.0 * n_out + n_in(1)) * es;
       break;
     case OP_LAYERNORM:
       flops = 8.0 * n_out;

@@ -5,7 +5,8 @@
 // Reference wrappers replaced here:
 //   cudnn/CUDNNActiveFunc.cpp, cudnn/CUDNNTensorOpFunc.cpp,
 //   cuda/CUDAClipFunc.cu, CUDAErfFunc.cu, CUDANegativeFunc.cu,
-//   CUDAReciprocalFunc.cu, CUDAPowFunc.cu, CUDACastI64toFloatFunc.cu
+//   CUDAReciprocalFunc.cu, CUDAPowFunc.cu, CUDACastI64toFloatFunc.cu,
+//   CUDALeakyReluFunc.cu, CUDAPReluFunc.cu
 // (all under src/Tools/dnn-wrapper/).
 #include "common.h"
 
@@ -127,6 +128,13 @@ struct FClip {
     v = v < lo ? lo : v;
     return v > hi ? hi : v;
   }
+};
+struct FLeaky {
+  float alpha;
+  __device__ float operator()(float v) const { return v < 0.f ? __fmul_rn(alpha, v) : v; }
+};
+struct FPRelu {
+  __device__ float operator()(float v, float slope) const { return v < 0.f ? __fmul_rn(slope, v) : v; }
 };
 struct FPow {
   float e;
@@ -252,6 +260,34 @@ void *dnnrtReciprocal(dnnrtHandle_t handle, const void *X, void *Y, const int64_
 void *dnnrtGelu(dnnrtHandle_t handle, const void *X, void *Y, const int64_t *dim, int64_t rank,
                 int32_t dtype) {
   return unary_entry("dnnrtGelu", handle, X, Y, dim, rank, dtype, FGelu{});
+}
+
+void *dnnrtLeakyRelu(dnnrtHandle_t handle, const void *X, void *Y, const int64_t *dimY, float alpha,
+                     int64_t rank, int32_t dtype) {
+  return unary_entry("dnnrtLeakyRelu", handle, X, Y, dimY, rank, dtype, FLeaky{alpha});
+}
+
+void *dnnrtPRelu(dnnrtHandle_t handle, const void *X, void *Y, const int64_t *dimY, const void *slope,
+                 const int64_t *dimSlope, int64_t rank, int32_t dtype) {
+  if (!handle) DNNRT_FAIL("dnnrtPRelu: null handle");
+  if (!X || !Y || !dimY || !slope || !dimSlope) DNNRT_FAIL("dnnrtPRelu: null argument");
+  if (rank < 1 || rank > 8) DNNRT_FAIL("dnnrtPRelu: rank %ld (1..8)", (long)rank);
+  for (int i = 0; i < rank; i++) {
+    if (dimY[i] < 0) DNNRT_FAIL("dnnrtPRelu: negative dim");
+    if (dimSlope[i] != dimY[i] && dimSlope[i] != 1)
+      DNNRT_FAIL("dnnrtPRelu: dimSlope[%d]=%ld cannot broadcast to %ld", i, (long)dimSlope[i], (long)dimY[i]);
+  }
+  int64_t dy[8], ds[8];
+  for (int i = 0; i < rank; i++) { dy[i] = dimY[i]; ds[i] = dimSlope[i]; }
+  if (handle->format != DNNRT_NCHW && rank == 4) {  // dense [N,H,W,C] arrays
+    dy[1] = dimY[2]; dy[2] = dimY[3]; dy[3] = dimY[1];
+    ds[1] = dimSlope[2]; ds[2] = dimSlope[3]; ds[3] = dimSlope[1];
+  }
+  bool ok;
+  if (dtype == DNNRT_F32) ok = run_binary<float>(handle, X, slope, Y, dy, ds, (int)rank, FPRelu{});
+  else if (dtype == DNNRT_F16) ok = run_binary<__half>(handle, X, slope, Y, dy, ds, (int)rank, FPRelu{});
+  else DNNRT_FAIL("dnnrtPRelu: dtype %d", dtype);
+  return ok ? Y : nullptr;
 }
 
 void *dnnrtPow(dnnrtHandle_t handle, const void *X, const void *exponent, void *Y, const int64_t *dimY,

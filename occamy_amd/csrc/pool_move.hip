@@ -2,7 +2,8 @@
 // Reference wrappers replaced (under src/Tools/dnn-wrapper/):
 //   cudnn/CUDNNMaxPoolFunc.cpp, cudnn/CUDNNAveragePoolFunc.cpp,
 //   cuda/CUDAFlattenFunc.cpp, CUDAReshapeFunc.cpp,
-//   CUDATranspose{2,3,4,6}D{Float,Int64}Func.cu, CUDAGatherFloatFunc.cu.
+//   CUDATranspose{2,3,4,6}D{Float,Int64}Func.cu, CUDAGatherFloatFunc.cu,
+//   CUDAConcat{Float,Int64}Func.cu, CUDA{Squeeze,Unsqueeze}{Float,Int64}Func.cpp.
 #include "common.h"
 
 namespace dnnrt {
@@ -210,6 +211,28 @@ static void *copy_entry(const char *who, dnnrtHandle_t h, const void *X, const i
   return Y;
 }
 
+// Concatenation along one axis.  Every tensor is seen as [outer][row] with
+// row = dim[axis] * inner; output row j comes from the input whose span of
+// the output row holds j.  U is the copy unit: 16 bytes when every row length
+// and pointer allows it, else one element.
+constexpr int CONCAT_MAX_INPUTS = 16;
+struct ConcatGeom {
+  const void *x[CONCAT_MAX_INPUTS];
+  int64_t begin[CONCAT_MAX_INPUTS + 1];  // prefix sums of the input rows, in units
+  int n;
+};
+template <typename U>
+__global__ __launch_bounds__(256) void concat_kernel(ConcatGeom g, U *__restrict__ y, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t row = g.begin[g.n], o = i / row, j = i - o * row;
+  int s = 0;
+#pragma unroll 1
+  for (int k = 1; k < g.n; k++) s += j >= g.begin[k] ? 1 : 0;
+  const int64_t len = g.begin[s + 1] - g.begin[s];
+  y[i] = static_cast<const U *>(g.x[s])[o * len + (j - g.begin[s])];
+}
+
 }  // namespace dnnrt
 
 using namespace dnnrt;
@@ -234,6 +257,85 @@ void *dnnrtFlatten(dnnrtHandle_t handle, const void *X, const int64_t *dimX, voi
 void *dnnrtReshape(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
                    int32_t dtype) {
   return copy_entry("dnnrtReshape", handle, X, dimX, rankX, Y, dtype);
+}
+
+// Squeeze / Unsqueeze move no data around: dimY must be dimX with size-1 dims
+// removed or inserted.
+static void *same_order_copy(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rX,
+                             void *Y, const int64_t *dY, int64_t rY, int32_t dtype) {
+  if (!h) DNNRT_FAIL("%s: null handle", who);
+  if (!X || !Y || !dX || !dY || rX < 0 || rY < 0) DNNRT_FAIL("%s: null argument", who);
+  int64_t i = 0, j = 0;
+  while (true) {
+    while (i < rX && dX[i] == 1) i++;
+    while (j < rY && dY[j] == 1) j++;
+    if (i == rX || j == rY) break;
+    if (dX[i] != dY[j]) DNNRT_FAIL("%s: dims differ beyond size-1 axes (%ld vs %ld)", who, (long)dX[i], (long)dY[j]);
+    i++; j++;
+  }
+  if (i != rX || j != rY) DNNRT_FAIL("%s: dims differ beyond size-1 axes", who);
+  if (h->format != DNNRT_NCHW && (rX == 4 || rY == 4)) DNNRT_FAIL("%s: channels-last tensors are not supported", who);
+  return copy_entry(who, h, X, dX, rX, Y, dtype);
+}
+
+void *dnnrtSqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
+                   const int64_t *dimY, int64_t rankY, int32_t dtype) {
+  return same_order_copy("dnnrtSqueeze", handle, X, dimX, rankX, Y, dimY, rankY, dtype);
+}
+void *dnnrtUnsqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
+                     const int64_t *dimY, int64_t rankY, int32_t dtype) {
+  return same_order_copy("dnnrtUnsqueeze", handle, X, dimX, rankX, Y, dimY, rankY, dtype);
+}
+
+void *dnnrtConcat(dnnrtHandle_t handle, const void *const *X, const int64_t *const *dimX, void *Y,
+                  const int64_t *dimY, int64_t axis, int64_t numInputs, int32_t rank, int32_t dtype) {
+  if (!handle) DNNRT_FAIL("dnnrtConcat: null handle");
+  if (!X || !dimX || !Y || !dimY) DNNRT_FAIL("dnnrtConcat: null argument");
+  if (rank < 1 || rank > 8) DNNRT_FAIL("dnnrtConcat: rank %d (1..8)", rank);
+  if (numInputs < 1 || numInputs > CONCAT_MAX_INPUTS) DNNRT_FAIL("dnnrtConcat: %ld inputs (1..%d)", (long)numInputs, CONCAT_MAX_INPUTS);
+  if (axis < 0) axis += rank;
+  if (axis < 0 || axis >= rank) DNNRT_FAIL("dnnrtConcat: axis out of range");
+  const int64_t es = esize(dtype);
+  if (!es) DNNRT_FAIL("dnnrtConcat: dtype %d", dtype);
+  int64_t along = 0;
+  for (int64_t k = 0; k < numInputs; k++) {
+    if (!X[k] || !dimX[k]) DNNRT_FAIL("dnnrtConcat: null input %ld", (long)k);
+    for (int i = 0; i < rank; i++)
+      if (dimX[k][i] < 0 || (i != axis && dimX[k][i] != dimY[i])) DNNRT_FAIL("dnnrtConcat: input %ld dim %d differs from the output's", (long)k, i);
+    along += dimX[k][axis];
+  }
+  if (along != dimY[axis]) DNNRT_FAIL("dnnrtConcat: the inputs' dims along the axis sum to %ld, dimY has %ld", (long)along, (long)dimY[axis]);
+  // memory order of the dims: a channels-last [N,C,H,W] tensor is a dense [N,H,W,C] array
+  int order[8];
+  for (int i = 0; i < rank; i++) order[i] = i;
+  if (handle->format != DNNRT_NCHW && rank == 4) { order[1] = 2; order[2] = 3; order[3] = 1; }
+  int64_t outer = 1, inner = 1;
+  bool before = true;
+  for (int i = 0; i < rank; i++) {
+    if (order[i] == axis) { before = false; continue; }
+    (before ? outer : inner) *= dimY[order[i]];
+  }
+  ConcatGeom g;
+  g.n = (int)numInputs;
+  bool vec = aligned16(Y);
+  for (int64_t k = 0; k < numInputs; k++) {
+    vec = vec && aligned16(X[k]) && (dimX[k][axis] * inner * es) % 16 == 0;
+    g.x[k] = X[k];
+  }
+  const int64_t unit = vec ? 16 : es;
+  g.begin[0] = 0;
+  for (int64_t k = 0; k < numInputs; k++) g.begin[k + 1] = g.begin[k] + dimX[k][axis] * inner * es / unit;
+  const int64_t total = outer * g.begin[numInputs];
+  if (total == 0) return Y;
+  const int64_t blocks = ceil_div(total, 256);
+  if (blocks > INT32_MAX) DNNRT_FAIL("dnnrtConcat: tensor too large");
+  const dim3 grid((unsigned)blocks), block(256);
+  if (unit == 16) hipLaunchKernelGGL((concat_kernel<uint4>), grid, block, 0, handle->stream, g, (uint4 *)Y, total);
+  else if (unit == 8) hipLaunchKernelGGL((concat_kernel<uint64_t>), grid, block, 0, handle->stream, g, (uint64_t *)Y, total);
+  else if (unit == 4) hipLaunchKernelGGL((concat_kernel<uint32_t>), grid, block, 0, handle->stream, g, (uint32_t *)Y, total);
+  else hipLaunchKernelGGL((concat_kernel<uint16_t>), grid, block, 0, handle->stream, g, (uint16_t *)Y, total);
+  DNNRT_CHECK_LAUNCH("dnnrtConcat");
+  return Y;
 }
 
 void *dnnrtTranspose(dnnrtHandle_t handle, const void *X, const int64_t *dimX, void *Y,

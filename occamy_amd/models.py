@@ -2,9 +2,12 @@
 export of these models gives (node vocabulary and order as in the reference's
 test/models/*/run.py flows), with seeded synthetic weights.
 
-Each builder returns ``(Graph, [input arrays])``.  BatchNorm is folded into
-the convolution bias, as onnx-mlir's ONNX-level rewrites leave it before the
-reference's own passes run.
+Each builder returns ``(Graph, [input arrays])``.  In ResNet-50, MobileNetV2
+and BERT BatchNorm is already folded into the convolution bias, as onnx-mlir's
+ONNX-level rewrites leave it before the reference's own passes run; AlexNet,
+YOLOv1 and the SRGAN generator (test/models/{alexnet,yolo,srgan}/run.py of the
+reference) keep the exporter's BatchNormalization / Dropout nodes, which the
+compiler folds or forwards itself.
 """
 import numpy as np
 
@@ -118,6 +121,129 @@ def mobilenet_v2(batch=1, dtype=np.float32, seed=3, image=224, classes=1000):
     bias = g.constant(np.zeros((classes,), dtype))
     y = g.node("Gemm", [x, w, bias], "logits", alpha=1.0, beta=1.0, transB=1)
     g.output(y)
+    return g, [x_np]
+
+
+def _batchnorm(g, init, x, c):
+    scale = g.constant(init.uniform((c,), 0.5, 1.5))
+    bias = g.constant(init.uniform((c,), -0.1, 0.1))
+    mean = g.constant(init.normal((c,), 0.1))
+    var = g.constant(init.uniform((c,), 0.5, 1.5))
+    return g.node("BatchNormalization", [x, scale, bias, mean, var], epsilon=1e-5, momentum=0.9)
+
+
+def _linear(g, init, x, nin, nout, name=None):
+    w = g.constant(init.he_normal((nout, nin)))
+    b = g.constant(init.uniform((nout,), -0.1, 0.1))
+    return g.node("Gemm", [x, w, b], name, alpha=1.0, beta=1.0, transB=1)
+
+
+def alexnet(batch=1, dtype=np.float32, seed=5, image=224, classes=1000, hidden=4096):
+    """torchvision AlexNet as torch.onnx.export writes it: the adaptive 6x6
+    average pool of a 224x224 image is an AveragePool with a 1x1 window, the
+    classifier's Dropout nodes are kept (inference: they forward their input)."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x_np = rng.normal(seed, 0, (batch, 3, image, image)).astype(dtype)
+    g.input("input", x_np.shape, dtype)
+    pool = dict(kernel_shape=[3, 3], pads=[0, 0, 0, 0], strides=[2, 2])
+    x = g.node("Relu", [_conv(g, init, "input", 3, 64, 11, 4, 2)])
+    x = g.node("MaxPool", [x], **pool)
+    x = g.node("Relu", [_conv(g, init, x, 64, 192, 5, 1, 2)])
+    x = g.node("MaxPool", [x], **pool)
+    x = g.node("Relu", [_conv(g, init, x, 192, 384, 3, 1, 1)])
+    x = g.node("Relu", [_conv(g, init, x, 384, 256, 3, 1, 1)])
+    x = g.node("Relu", [_conv(g, init, x, 256, 256, 3, 1, 1)])
+    x = g.node("MaxPool", [x], **pool)
+    side = (((image + 4 - 11) // 4 + 1 - 3) // 2 + 1 - 3) // 2 + 1
+    side = (side - 3) // 2 + 1
+    x = g.node("AveragePool", [x], kernel_shape=[1, 1], pads=[0, 0, 0, 0], strides=[1, 1])
+    x = g.node("Flatten", [x], axis=1)
+    x = g.node("Dropout", [x])
+    x = g.node("Relu", [_linear(g, init, x, 256 * side * side, hidden)])
+    x = g.node("Dropout", [x])
+    x = g.node("Relu", [_linear(g, init, x, hidden, hidden)])
+    y = _linear(g, init, x, hidden, classes, "logits")
+    g.output(y)
+    return g, [x_np]
+
+
+YOLO_V1_LAYERS = [(7, 64, 2, 3), "M", (3, 192, 1, 1), "M", (1, 128, 1, 0), (3, 256, 1, 1), (1, 256, 1, 0),
+                  (3, 512, 1, 1), "M", [(1, 256, 1, 0), (3, 512, 1, 1), 4], (1, 512, 1, 0), (3, 1024, 1, 1), "M",
+                  [(1, 512, 1, 0), (3, 1024, 1, 1), 2], (3, 1024, 1, 1), (3, 1024, 2, 1), (3, 1024, 1, 1),
+                  (3, 1024, 1, 1)]
+
+
+def yolo_v1(batch=2, dtype=np.float32, seed=6, image=448, width=1.0, boxes=2, classes=20, fc=496):
+    """YOLOv1 with BatchNorm (test/models/yolo/run.py of the reference):
+    bias-free Conv -> BatchNormalization -> LeakyRelu(0.1) blocks, 2x2 max
+    pools, Flatten, two Linear layers.  `image` must be a multiple of 64;
+    `width` scales the channel counts (tests use a narrow copy)."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x_np = rng.normal(seed, 0, (batch, 3, image, image)).astype(dtype)
+    g.input("input", x_np.shape, dtype)
+    x, cin = "input", 3
+
+    def block(x, cin, k, cout, stride, pad):
+        cout = max(8, int(cout * width))
+        c = _conv(g, init, x, cin, cout, k, stride, pad, bias=False)
+        return g.node("LeakyRelu", [_batchnorm(g, init, c, cout)], alpha=0.1), cout
+
+    for item in YOLO_V1_LAYERS:
+        if item == "M":
+            x = g.node("MaxPool", [x], kernel_shape=[2, 2], pads=[0, 0, 0, 0], strides=[2, 2])
+        elif isinstance(item, tuple):
+            x, cin = block(x, cin, *item)
+        else:
+            for _ in range(item[2]):
+                x, cin = block(x, cin, *item[0])
+                x, cin = block(x, cin, *item[1])
+    split = image // 64
+    x = g.node("Flatten", [x], axis=1)
+    x = g.node("LeakyRelu", [_linear(g, init, x, cin * split * split, fc)], alpha=0.1)
+    y = _linear(g, init, x, fc, split * split * (classes + boxes * 5), "cells")
+    g.output(y)
+    return g, [x_np]
+
+
+def srgan_generator(batch=1, dtype=np.float32, seed=7, height=24, width=24, feats=64, blocks=16):
+    """SRGAN generator, 4x upscaling (test/models/srgan/srgan_model.py of the
+    reference): 9x9 conv, residual blocks of conv-BN-PReLU-conv-BN, two
+    conv + PixelShuffle(2) + PReLU stages, 3x3 conv + Tanh.  One PReLU
+    parameter is shared by every activation, as nn.PReLU() gives.  PixelShuffle
+    is Reshape -> Transpose(0,1,4,2,5,3) -> Reshape.  Two results: the image
+    and the feature map before upsampling."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x_np = rng.normal(seed, 0, (batch, 3, height, width)).astype(dtype)
+    g.input("lr", x_np.shape, dtype)
+    slope = g.constant(np.full((1,), 0.25, dtype), "prelu_slope")
+
+    def conv(x, cin, cout, k):
+        w = g.constant(init.normal((cout, cin, k, k), 0.02))  # the reference's own initialisation (srgan/ops.py)
+        b = g.constant(init.uniform((cout,), -0.05, 0.05))
+        return g.node("Conv", [x, w, b], kernel_shape=[k, k], pads=[k // 2] * 4, strides=[1, 1], group=1)
+
+    x = g.node("PRelu", [conv("lr", 3, feats, 9), slope])
+    skip = x
+    for _ in range(blocks):
+        r = g.node("PRelu", [_batchnorm(g, init, conv(x, feats, feats, 3), feats), slope])
+        r = _batchnorm(g, init, conv(r, feats, feats, 3), feats)
+        x = g.node("Add", [r, x])
+    x = _batchnorm(g, init, conv(x, feats, feats, 3), feats)
+    feat = g.node("Add", [x, skip], "feat")
+    x, h, w = feat, height, width
+    for _ in range(2):
+        x = conv(x, feats, feats * 4, 3)
+        x = g.node("Reshape", [x, g.constant(np.array([batch, feats, 2, 2, h, w], np.int64))])
+        x = g.node("Transpose", [x], perm=[0, 1, 4, 2, 5, 3])
+        h, w = h * 2, w * 2
+        x = g.node("Reshape", [x, g.constant(np.array([batch, feats, h, w], np.int64))])
+        x = g.node("PRelu", [x, slope])
+    y = g.node("Tanh", [conv(x, feats, 3, 3)], "sr")
+    g.output(y)
+    g.output(feat)
     return g, [x_np]
 
 

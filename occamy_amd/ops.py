@@ -108,6 +108,16 @@ class Ops:
         return self._ret(self.lib.dnnrtClip(self.handle, X, Y, dims(dimY), lo, hi, len(dimY), dtype),
                          "dnnrtClip")
 
+    def leaky_relu(self, X, Y, dimY, alpha, dtype=_abi.F32):
+        return self._ret(self.lib.dnnrtLeakyRelu(self.handle, X, Y, dims(dimY), alpha, len(dimY), dtype),
+                         "dnnrtLeakyRelu")
+
+    def prelu(self, X, Y, dimY, slope, dimSlope, dtype=_abi.F32):
+        """dimSlope is right-aligned to dimY here (ONNX's unidirectional broadcast)."""
+        ds = [1] * (len(dimY) - len(dimSlope)) + list(dimSlope)
+        return self._ret(self.lib.dnnrtPRelu(self.handle, X, Y, dims(dimY), slope, dims(ds), len(dimY), dtype),
+                         "dnnrtPRelu")
+
     def _unary(self, name, X, Y, dim, dtype):
         fn = getattr(self.lib, name)
         return self._ret(fn(self.handle, X, Y, dims(dim), len(dim), dtype), name)
@@ -170,6 +180,23 @@ class Ops:
     def reshape(self, X, dimX, Y, dtype=_abi.F32):
         return self._ret(self.lib.dnnrtReshape(self.handle, X, dims(dimX), len(dimX), Y, dtype),
                          "dnnrtReshape")
+
+    def squeeze(self, X, dimX, Y, dimY, dtype=_abi.F32):
+        return self._ret(self.lib.dnnrtSqueeze(self.handle, X, dims(dimX), len(dimX), Y, dims(dimY), len(dimY),
+                                               dtype), "dnnrtSqueeze")
+
+    def unsqueeze(self, X, dimX, Y, dimY, dtype=_abi.F32):
+        return self._ret(self.lib.dnnrtUnsqueeze(self.handle, X, dims(dimX), len(dimX), Y, dims(dimY), len(dimY),
+                                                 dtype), "dnnrtUnsqueeze")
+
+    def concat(self, Xs, dimXs, Y, dimY, axis, dtype=_abi.F32):
+        """Xs: device pointers (ints), dimXs: one dim list per input."""
+        n = len(Xs)
+        ptrs = (C.c_void_p * n)(*Xs)
+        dim_arrays = [dims(d) for d in dimXs]  # kept alive until the call returns
+        dim_ptrs = (C.c_void_p * n)(*[C.cast(a, C.c_void_p) for a in dim_arrays])
+        return self._ret(self.lib.dnnrtConcat(self.handle, ptrs, dim_ptrs, Y, dims(dimY), axis, n, len(dimY),
+                                              dtype), "dnnrtConcat")
 
     def transpose(self, X, dimX, Y, perm, dtype=_abi.F32):
         dimY = [dimX[p] for p in perm]

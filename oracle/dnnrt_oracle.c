@@ -424,6 +424,48 @@ void *dnnrtClip(dnnrtHandle_t h, const void *X, void *Y, const int64_t *d, float
   return Y;
 }
 
+/* CUDALeakyReluFunc.cu:4-15: x < 0 ? alpha * x : x. */
+void *dnnrtLeakyRelu(dnnrtHandle_t h, const void *X, void *Y, const int64_t *d, float alpha,
+                     int64_t rank, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("leakyrelu: bad dtype");
+  const int64_t n = numel(d, rank);
+  float *tx, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t i = 0; i < n; i++) y[i] = x[i] < 0.f ? alpha * x[i] : x[i];
+  narrow(Y, ty, n, dtype); free(tx);
+  return Y;
+}
+
+/* CUDAPReluFunc.cu:4-15 applies slope[0] to the whole tensor; ONNX PRelu
+ * broadcasts the slope tensor to X (unidirectional, right-aligned), which is
+ * what is computed here: with a one-element slope the two agree. */
+void *dnnrtPRelu(dnnrtHandle_t h, const void *X, void *Y, const int64_t *d, const void *S,
+                 const int64_t *dS, int64_t rank, int32_t dtype) {
+  (void)h;
+  if (bad_dtype(dtype)) FAIL("prelu: bad dtype");
+  if (rank < 1 || rank > 8) FAIL("prelu: rank");
+  int64_t ss[8], acc = 1;
+  for (int i = (int)rank - 1; i >= 0; i--) {
+    if (dS[i] != d[i] && dS[i] != 1) FAIL("prelu: slope does not broadcast");
+    ss[i] = dS[i] == 1 ? 0 : acc;
+    acc *= dS[i];
+  }
+  const int64_t n = numel(d, rank), ns = numel(dS, rank);
+  float *tx, *ts, *ty;
+  const float *x = widen(X, n, dtype, &tx);
+  const float *sl = widen(S, ns, dtype, &ts);
+  float *y = outbuf(Y, n, dtype, &ty);
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, is = 0;
+    for (int k = (int)rank - 1; k >= 0; k--) { is += (rem % d[k]) * ss[k]; rem /= d[k]; }
+    y[i] = x[i] < 0.f ? sl[is] * x[i] : x[i];
+  }
+  narrow(Y, ty, n, dtype); free(tx); free(ts);
+  return Y;
+}
+
 /* CUDAPowFunc.cu:4-32: exponent from a 1-element tensor; exponent 2 is x*x. */
 void *dnnrtPow(dnnrtHandle_t h, const void *X, const void *E, void *Y,
                const int64_t *d, int64_t rank, int32_t dtype) {
@@ -696,6 +738,64 @@ void *dnnrtReshape(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t ra
   (void)h;
   if (!esize(dtype)) FAIL("reshape: bad dtype");
   memmove(Y, X, (size_t)(numel(dX, rank) * esize(dtype)));
+  return Y;
+}
+/* CUDASqueezeFloatFunc.cpp:25-31 / CUDAUnsqueezeFloatFunc.cpp: device-to-device copy. */
+static int same_but_ones(const int64_t *dX, int64_t rX, const int64_t *dY, int64_t rY) {
+  int64_t i = 0, j = 0;
+  for (;;) {
+    while (i < rX && dX[i] == 1) i++;
+    while (j < rY && dY[j] == 1) j++;
+    if (i == rX || j == rY) return i == rX && j == rY;
+    if (dX[i++] != dY[j++]) return 0;
+  }
+}
+void *dnnrtSqueeze(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rX, void *Y,
+                   const int64_t *dY, int64_t rY, int32_t dtype) {
+  (void)h;
+  if (!esize(dtype)) FAIL("squeeze: bad dtype");
+  if (!same_but_ones(dX, rX, dY, rY)) FAIL("squeeze: dims differ beyond size-1 axes");
+  memmove(Y, X, (size_t)(numel(dX, rX) * esize(dtype)));
+  return Y;
+}
+void *dnnrtUnsqueeze(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rX, void *Y,
+                     const int64_t *dY, int64_t rY, int32_t dtype) {
+  (void)h;
+  if (!esize(dtype)) FAIL("unsqueeze: bad dtype");
+  if (!same_but_ones(dX, rX, dY, rY)) FAIL("unsqueeze: dims differ beyond size-1 axes");
+  memmove(Y, X, (size_t)(numel(dX, rX) * esize(dtype)));
+  return Y;
+}
+/* CUDAConcatFloatFunc.cu:7-62, per output element: split the flat index into
+ * a multi-index, find the input whose span along the axis holds it, rebase
+ * that coordinate and gather from that input. */
+void *dnnrtConcat(dnnrtHandle_t h, const void *const *X, const int64_t *const *dX, void *Y,
+                  const int64_t *dY, int64_t axis, int64_t n_in, int32_t rank, int32_t dtype) {
+  (void)h;
+  const int64_t es = esize(dtype);
+  if (!es) FAIL("concat: bad dtype");
+  if (rank < 1 || rank > 8 || n_in < 1 || n_in > 16) FAIL("concat: rank or input count");
+  if (axis < 0) axis += rank;
+  if (axis < 0 || axis >= rank) FAIL("concat: axis");
+  int64_t acc[17];
+  acc[0] = 0;
+  for (int64_t k = 0; k < n_in; k++) {
+    for (int i = 0; i < rank; i++)
+      if (i != axis && dX[k][i] != dY[i]) FAIL("concat: input dims");
+    acc[k + 1] = acc[k] + dX[k][axis];
+  }
+  if (acc[n_in] != dY[axis]) FAIL("concat: axis dims do not add up");
+  const int64_t n = numel(dY, rank);
+  for (int64_t i = 0; i < n; i++) {
+    int64_t idx[8], rem = i;
+    for (int k = rank - 1; k >= 0; k--) { idx[k] = rem % dY[k]; rem /= dY[k]; }
+    int64_t src = 0;
+    while (!(idx[axis] >= acc[src] && idx[axis] < acc[src + 1])) src++;
+    idx[axis] -= acc[src];
+    int64_t off = 0;
+    for (int k = 0; k < rank; k++) off = off * dX[src][k] + idx[k];
+    memcpy((char *)Y + i * es, (const char *)X[src] + off * es, (size_t)es);
+  }
   return Y;
 }
 /* CUDATranspose4DFloatFunc.cu: Y[i_perm] = X[i]; dimY[j] = dimX[perm[j]]. */

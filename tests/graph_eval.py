@@ -78,6 +78,28 @@ def evaluate(graph, inputs):
             env[out] = F.layer_norm(x[0], (x[0].shape[-1],), x[1], x[2], at.get("epsilon", 1e-5))
         elif op == "Cast":
             env[out] = x[0].double()
+        elif op == "LeakyRelu":
+            env[out] = F.leaky_relu(x[0], at.get("alpha", 0.01))
+        elif op == "PRelu":
+            env[out] = torch.where(x[0] < 0, x[0] * x[1], x[0])
+        elif op == "Concat":
+            env[out] = torch.cat(x, at["axis"])
+        elif op == "Squeeze":
+            if "axes" in at or len(x) > 1:
+                axes = at["axes"] if "axes" in at else [int(v) for v in x[1]]
+                env[out] = x[0].reshape([d for i, d in enumerate(x[0].shape) if i not in [a % x[0].dim() for a in axes]])
+            else:
+                env[out] = x[0].squeeze()
+        elif op == "Unsqueeze":
+            axes = at["axes"] if "axes" in at else [int(v) for v in x[1]]
+            y = x[0]
+            for a in sorted(a % (x[0].dim() + len(axes)) for a in axes):
+                y = y.unsqueeze(a)
+            env[out] = y
+        elif op in ("Identity", "Dropout"):
+            env[out] = x[0]
+        elif op == "BatchNormalization":
+            env[out] = F.batch_norm(x[0], x[3], x[4], x[1], x[2], False, 0.0, at.get("epsilon", 1e-5))
         else:
             raise NotImplementedError(op)
     return [env[o].numpy() for o in graph.outputs]

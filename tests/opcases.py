@@ -175,3 +175,37 @@ def gather(be, x, idx, axis):
     be.ops.gather(be.ptr(X), x.shape, be.ptr(Y), out, be.ptr(I), idx.shape, axis, DT[x.dtype])
     be.sync()
     return be.get(Y)
+
+
+def leaky_relu(be, x, alpha):
+    X = be.put(x)
+    Y = be.empty(x.shape, x.dtype)
+    be.ops.leaky_relu(be.ptr(X), be.ptr(Y), x.shape, alpha, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def prelu(be, x, slope):
+    X, S = be.put(x), be.put(slope)
+    Y = be.empty(x.shape, x.dtype)
+    be.ops.prelu(be.ptr(X), be.ptr(Y), x.shape, be.ptr(S), slope.shape, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def concat(be, xs, axis):
+    out = list(xs[0].shape)
+    out[axis] = sum(x.shape[axis] for x in xs)
+    Xs = [be.put(x) for x in xs]
+    Y = be.empty(out, xs[0].dtype)
+    be.ops.concat([be.ptr(X) for X in Xs], [x.shape for x in xs], be.ptr(Y), out, axis, DT[xs[0].dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def squeeze(be, x, out, un=False):
+    X = be.put(x)
+    Y = be.empty(out, x.dtype)
+    (be.ops.unsqueeze if un else be.ops.squeeze)(be.ptr(X), x.shape, be.ptr(Y), out, DT[x.dtype])
+    be.sync()
+    return be.get(Y)

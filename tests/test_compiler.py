@@ -113,6 +113,25 @@ def test_lifetimes_bert(fused):
     check_lifetimes(lambda: models.bert_encoder(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100, fused=fused))
 
 
+@pytest.mark.parametrize("fusion", [False, True])
+def test_lifetimes_alexnet_yolo_srgan(fusion):
+    check_lifetimes(lambda: models.alexnet(image=96, classes=10, hidden=64), fusion=fusion)
+    check_lifetimes(lambda: models.yolo_v1(batch=1, image=64, width=0.0625, fc=32), fusion=fusion)
+    # the generator returns its feature map and goes on reading it
+    check_lifetimes(lambda: models.srgan_generator(height=8, width=6, feats=16, blocks=2), fusion=fusion)
+
+
+def test_batchnorm_folds_into_the_convolution_before_it():
+    g, _ = models.yolo_v1(batch=1, image=64, width=0.0625, fc=32)
+    n_conv = sum(1 for op, *_ in g.nodes if op == "Conv")
+    ops = [name for name, *_ in g.compile().compute_ops()]
+    # every block is conv, bias add (the folded shift), leaky relu: no Mul is left over
+    assert ops.count("dnn.convfwd") == n_conv == 24 and ops.count("dnn.add") == n_conv + 2 and "dnn.mul" not in ops
+    g, _ = models.yolo_v1(batch=1, image=64, width=0.0625, fc=32)
+    ops = [name for name, *_ in g.compile(fusion=True).compute_ops()]
+    assert ops.count("dnn.conv-bias-relufwd") == n_conv and "dnn.convfwd" not in ops
+
+
 def planned_vs_oracle(p):
     ev = p.events()
     off, peak = oracle_plan([(k, i, b) for k, i, b, _ in ev])

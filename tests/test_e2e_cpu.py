@@ -102,6 +102,76 @@ def test_every_emission_rule_once():
     assert out[0].shape == (2, 2, 2) and out[1].shape == (2, 6, 4, 4)
 
 
+ALEX = lambda: models.alexnet(image=96, classes=10, hidden=64)                    # noqa: E731
+YOLO = lambda: models.yolo_v1(batch=2, image=64, width=0.0625, fc=32)             # noqa: E731
+SRGAN = lambda: models.srgan_generator(height=8, width=6, feats=16, blocks=2)     # noqa: E731
+
+
+@pytest.mark.parametrize("builder", [ALEX, YOLO, SRGAN], ids=["alexnet", "yolo_v1", "srgan"])
+def test_reference_test_models_small(builder):
+    a = check(builder)
+    b = check(builder, fusion=True)
+    for x, y in zip(a, b):
+        np.testing.assert_allclose(x, y, rtol=1e-4, atol=1e-5 * max(1.0, float(np.abs(x).max())))
+    _, _, c = run_oracle(builder, mode=compiler.MODE_RESIDENT)
+    for x, y in zip(a, c):
+        np.testing.assert_array_equal(x, y)
+
+
+def test_returned_tensor_that_is_read_again_stays_alive():
+    # SRGAN returns the feature map and keeps reading it; freeing it at the
+    # copy to the host (what the reference's dealloc placement does) lets the
+    # pool hand its bytes to a later tensor.  Every flag combination must agree.
+    base = check(SRGAN)
+    for flags in [dict(dealloc_opt=False), dict(const_at_use=False), dict(pool_opt=True, dealloc_opt=True)]:
+        _, _, out = run_oracle(SRGAN, **flags)
+        for x, y in zip(base, out):
+            np.testing.assert_array_equal(x, y)
+
+
+def test_widened_operator_surface():
+    """LeakyRelu, PRelu (shared and per-channel slope), Concat, Squeeze,
+    Unsqueeze, Identity, Dropout, and BatchNormalization in its three shapes:
+    folded into the convolution before it, kept apart because the
+    convolution's result has a second reader, and on a non-convolution."""
+    def build():
+        r = np.random.default_rng(5)
+        g = compiler.Graph()
+        x = r.standard_normal((2, 4, 6, 6)).astype(np.float32)
+        g.input("x", x.shape)
+
+        def bn(v, c):
+            return g.node("BatchNormalization", [v] + [g.constant(a.astype(np.float32)) for a in (
+                r.uniform(0.5, 1.5, c), r.uniform(-0.2, 0.2, c), r.standard_normal(c) * 0.1, r.uniform(0.5, 1.5, c))],
+                epsilon=1e-3)
+
+        w1 = g.constant((r.standard_normal((8, 4, 3, 3)) * 0.2).astype(np.float32))
+        b1 = g.constant((r.standard_normal(8) * 0.1).astype(np.float32))
+        c1 = g.node("Conv", ["x", w1, b1], pads=[1, 1, 1, 1])
+        f1 = g.node("LeakyRelu", [bn(c1, 8)], alpha=0.2)                       # folds (bias present)
+        w2 = g.constant((r.standard_normal((8, 8, 1, 1)) * 0.3).astype(np.float32))
+        c2 = g.node("Conv", [f1, w2])
+        n2 = bn(c2, 8)                                                         # c2 has two readers: Mul + Add
+        cat = g.node("Concat", [n2, g.node("Identity", [c2]), f1], axis=1)     # 24 channels
+        pr = g.node("PRelu", [cat, g.constant(r.uniform(0.1, 0.4, (24, 1, 1)).astype(np.float32))])
+        pool = g.node("GlobalAveragePool", [pr])                               # [2,24,1,1]
+        sq = g.node("Squeeze", [pool, g.constant(np.array([2, 3], np.int64))])  # [2,24]
+        d = g.node("Dropout", [bn(sq, 24)])                                    # BN on a rank-2 tensor
+        un = g.node("Unsqueeze", [d], axes=[0, 3])                             # [1,2,24,1]
+        sh = g.node("PRelu", [un, g.constant(np.array([0.3], np.float32))])
+        g.output(g.node("Squeeze", [sh]))                                      # every 1 goes: [2,24]
+        g.output(g.node("Identity", [pr]))                                     # a returned Identity is a copy
+        g.output(g.node("Concat", [sq, sq], axis=-1))
+        return g, [x]
+    out = check(build)
+    assert out[0].shape == (2, 24) and out[1].shape == (2, 24, 6, 6) and out[2].shape == (2, 48)
+    g, _ = build()
+    text = g.compile().text
+    assert "BatchNormalization" not in text and text.count("dnn.convfwd") == 2
+    assert text.count("dnn.concat") == 2 and text.count("dnn.squeeze") == 2 and text.count("dnn.unsqueeze") == 1
+    assert text.count("dnn.prelu") == 2 and text.count("dnn.leakyrelu") == 1
+
+
 def test_executor_errors():
     g, inputs = models.single_conv()
     p = g.compile(pool_opt=False)

@@ -31,6 +31,10 @@ CONFIGS = {
     "resnet50": models.resnet50,
     "mobilenet_v2": models.mobilenet_v2,
     "bert_2_layers": lambda: models.bert_encoder(layers=2),
+    # the reference's other test models (test/models/{alexnet,yolo,srgan}/run.py) at their own sizes
+    "alexnet": models.alexnet,
+    "yolo_v1": lambda: models.yolo_v1(batch=1),
+    "srgan": lambda: models.srgan_generator(height=64, width=48),
 }
 
 
@@ -54,7 +58,7 @@ def test_fused_program_matches_oracle(name, oracle_outputs):
         close(o, r)
 
 
-@pytest.mark.parametrize("name", ["single_conv", "resnet50", "bert_2_layers"])
+@pytest.mark.parametrize("name", ["single_conv", "resnet50", "bert_2_layers", "srgan"])
 def test_resident_mode_and_graph_replay(name, oracle_outputs):
     import torch
     g, inputs = CONFIGS[name]()

@@ -269,6 +269,74 @@ def test_data_movement(gpu, cpu):
         oc.transpose(gpu, x, (0, 1, 1, 3))
 
 
+def test_leaky_relu_prelu(gpu, cpu):
+    r = rng(41)
+    for dtype in (np.float32, np.float16):
+        for shape in [(2, 24, 13, 13), (1, 64, 56, 56), (5,), (3, 7)]:
+            x = r.standard_normal(shape).astype(dtype)
+            np.testing.assert_array_equal(oc.leaky_relu(gpu, x, 0.1), oc.leaky_relu(cpu, x, 0.1))
+            np.testing.assert_array_equal(oc.prelu(gpu, x, np.array([0.25], dtype)), oc.prelu(cpu, x, np.array([0.25], dtype)))
+        x = r.standard_normal((2, 24, 13, 13)).astype(dtype)
+        for sshape in [(24, 1, 1), (1, 24, 1, 1), (13,), (2, 24, 13, 13), (1, 1, 13, 1)]:
+            sl = r.uniform(-0.5, 0.5, sshape).astype(dtype)
+            np.testing.assert_array_equal(oc.prelu(gpu, x, sl), oc.prelu(cpu, x, sl))
+    with pytest.raises(RuntimeError):
+        oc.prelu(gpu, x, np.ones((7, 1, 1), x.dtype))
+    # channels-last: the tensor is a dense [N,H,W,C] array, the slope runs along C
+    x = r.standard_normal((2, 24, 5, 7)).astype(np.float16)
+    sl = r.uniform(-0.5, 0.5, (24, 1, 1)).astype(np.float16)
+    gpu.ops.set_format(_abi.NHWC)
+    try:
+        X, S = gpu.put(np.ascontiguousarray(x.transpose(0, 2, 3, 1))), gpu.put(sl)
+        Y = gpu.empty((2, 5, 7, 24), np.float16)
+        gpu.ops.prelu(gpu.ptr(X), gpu.ptr(Y), x.shape, gpu.ptr(S), sl.shape, _abi.F16)
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    np.testing.assert_array_equal(gpu.get(Y).transpose(0, 3, 1, 2), oc.prelu(cpu, x, sl))
+
+
+def test_concat_squeeze_unsqueeze(gpu, cpu):
+    r = rng(42)
+    for dtype in (np.float32, np.float16, np.int64):
+        mk = (lambda s: r.integers(-99, 99, s).astype(np.int64)) if dtype == np.int64 else (lambda s: r.standard_normal(s).astype(dtype))
+        for axis in range(4):
+            for sizes in [(1, 3, 7), (4, 4), (8, 16, 8)]:         # element-wise and 16-byte paths
+                shapes = []
+                for k in sizes:
+                    sh = [2, 8, 4, 8]
+                    sh[axis] = k
+                    shapes.append(sh)
+                xs = [mk(s) for s in shapes]
+                got = oc.concat(gpu, xs, axis)
+                np.testing.assert_array_equal(got, np.concatenate(xs, axis))
+                np.testing.assert_array_equal(got, oc.concat(cpu, xs, axis))
+    many = [r.standard_normal((3, k + 1, 5)).astype(np.float32) for k in range(16)]
+    np.testing.assert_array_equal(oc.concat(gpu, many, 1), np.concatenate(many, 1))
+    big = [r.standard_normal((2, c, 52, 52)).astype(np.float32) for c in (128, 256)]  # a detection neck's concat
+    np.testing.assert_array_equal(oc.concat(gpu, big, 1), np.concatenate(big, 1))
+    with pytest.raises(RuntimeError):
+        oc.concat(gpu, many + [many[0]], 1)
+    with pytest.raises(RuntimeError):
+        oc.concat(gpu, [big[0], big[1][:, :, :50]], 1)
+    # channels-last: concatenating channels interleaves per pixel
+    xs = [r.standard_normal((2, c, 6, 5)).astype(np.float16) for c in (8, 24, 3)]
+    gpu.ops.set_format(_abi.NHWC)
+    try:
+        Xs = [gpu.put(np.ascontiguousarray(x.transpose(0, 2, 3, 1))) for x in xs]
+        Y = gpu.empty((2, 6, 5, 35), np.float16)
+        gpu.ops.concat([gpu.ptr(X) for X in Xs], [x.shape for x in xs], gpu.ptr(Y), (2, 35, 6, 5), 1, _abi.F16)
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    np.testing.assert_array_equal(gpu.get(Y).transpose(0, 3, 1, 2), np.concatenate(xs, 1))
+    s = r.standard_normal((2, 1, 4, 1)).astype(np.float32)
+    np.testing.assert_array_equal(oc.squeeze(gpu, s, (2, 4)), s.reshape(2, 4))
+    np.testing.assert_array_equal(oc.squeeze(gpu, s.reshape(2, 4), (1, 2, 1, 4), un=True), s.reshape(1, 2, 1, 4))
+    with pytest.raises(RuntimeError):
+        oc.squeeze(gpu, s, (4, 2))
+
+
 # ---- fp16, channels-last -----------------------------------------------------------------
 
 def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt, z=None):

@@ -19,6 +19,9 @@ SMALL = {
     "bert": lambda: models.bert_encoder(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100),
     "bert_fused": lambda: models.bert_encoder(layers=1, hidden=64, heads=4, ffn=128, seq=16, vocab=100, fused=True),
     "resnet50_fp16": lambda: models.resnet50(2, np.float16, image=32, classes=10),
+    "alexnet": lambda: models.alexnet(image=96, classes=10, hidden=64),
+    "yolo_v1": lambda: models.yolo_v1(batch=1, image=64, width=0.0625, fc=32),
+    "srgan": lambda: models.srgan_generator(height=8, width=6, feats=16, blocks=2),
 }
 
 # x: float[1,2] -> Relu -> y, by hand from onnx.proto3:
@@ -158,6 +161,39 @@ def test_what_the_reader_refuses():
     vi = ow.value_info("x", (1, 1, 4, 4), np.float32)
     with pytest.raises(RuntimeError, match="more than one output"):
         compiler.load_onnx(ow.f_bytes(7, ow.f_bytes(1, n) + ow.f_bytes(11, vi) + ow.f_bytes(12, ow.f_string(1, "y"))))
+
+
+def test_training_outputs_of_dropout_and_batchnorm_are_tolerated():
+    # exporters list Dropout's mask and BatchNormalization's running statistics as further outputs
+    r = np.random.default_rng(8)
+    c = 3
+    stats = [r.uniform(0.5, 1.5, c), r.uniform(-0.2, 0.2, c), r.standard_normal(c) * 0.1, r.uniform(0.5, 1.5, c)]
+    names = ["scale", "bias", "mean", "var"]
+    graph = b""
+    bn = ow.f_string(1, "x") + b"".join(ow.f_string(1, n) for n in names) + ow.f_string(2, "n") + ow.f_string(2, "run_mean") + \
+        ow.f_string(2, "run_var") + ow.f_string(4, "BatchNormalization") + ow.f_bytes(5, ow.attribute("epsilon", 1e-3))
+    dr = ow.f_string(1, "n") + ow.f_string(2, "d") + ow.f_string(2, "mask") + ow.f_string(4, "Dropout")
+    rl = ow.f_string(1, "d") + ow.f_string(2, "y") + ow.f_string(4, "Relu")
+    graph += ow.f_bytes(1, bn) + ow.f_bytes(1, dr) + ow.f_bytes(1, rl)
+    for n, a in zip(names, stats):
+        graph += ow.f_bytes(5, ow.tensor_proto(n, a.astype(np.float32)))
+    graph += ow.f_bytes(11, ow.value_info("x", (2, c, 4, 4), np.float32)) + ow.f_bytes(12, ow.f_string(1, "y"))
+    g = compiler.load_onnx(ow.f_varint(1, 8) + ow.f_bytes(7, graph))
+    p = g.compile()
+    assert [n for n, *_ in p.compute_ops()] == ["dnn.mul", "dnn.add", "dnn.activationfwd"]
+    x = r.standard_normal((2, c, 4, 4)).astype(np.float32)
+    s = p.session(runtime_library=ORACLE_PATH)
+    sc, bi, mu, va = (a.reshape(1, c, 1, 1) for a in stats)
+    want = np.maximum((x - mu) / np.sqrt(va + 1e-3) * sc + bi, 0)
+    np.testing.assert_allclose(s.run(x)[0], want, rtol=1e-5, atol=1e-6)
+    s.close()
+    # training mode is refused, and so is a reader of a training output
+    bad = bn + ow.f_bytes(5, ow.attribute("training_mode", 1))
+    with pytest.raises(RuntimeError, match="training mode"):
+        compiler.load_onnx(ow.f_varint(1, 8) + ow.f_bytes(7, graph.replace(ow.f_bytes(1, bn), ow.f_bytes(1, bad))))
+    rl2 = ow.f_string(1, "mask") + ow.f_string(2, "y") + ow.f_string(4, "Relu")
+    with pytest.raises(RuntimeError, match="not defined"):
+        compiler.load_onnx(ow.f_varint(1, 8) + ow.f_bytes(7, graph.replace(ow.f_bytes(1, rl), ow.f_bytes(1, rl2)))).compile()
 
 
 def test_unknown_fields_are_skipped():

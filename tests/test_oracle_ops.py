@@ -341,6 +341,57 @@ def test_data_movement(be):
         oc.gather(be, table, np.array([11]), 0)
 
 
+def test_leaky_relu_and_prelu(be):
+    # pinned by the defining formula on hand-picked values and by torch's operators
+    x = np.array([-2.0, -0.5, 0.0, 0.5, 3.0], np.float32)
+    np.testing.assert_array_equal(oc.leaky_relu(be, x, 0.25), np.array([-0.5, -0.125, 0.0, 0.5, 3.0], np.float32))
+    np.testing.assert_array_equal(oc.leaky_relu(be, x, 0.0), np.maximum(x, 0))      # alpha 0 is relu
+    np.testing.assert_array_equal(oc.leaky_relu(be, x, 1.0), x)                     # alpha 1 is the identity
+    r = rng(31)
+    t = r.standard_normal((2, 5, 3, 4)).astype(np.float32)
+    np.testing.assert_array_equal(oc.leaky_relu(be, t, 0.1), F.leaky_relu(torch.from_numpy(t), 0.1).numpy())
+    # one shared slope: what the reference kernel computes (it reads slope[0])
+    np.testing.assert_array_equal(oc.prelu(be, t, np.array([0.3], np.float32)),
+                                  F.prelu(torch.from_numpy(t), torch.tensor([0.3])).numpy())
+    # per-channel slope, ONNX shape [C,1,1]: a transposed broadcast (over W or N) fails here
+    sl = r.standard_normal((5, 1, 1)).astype(np.float32)
+    np.testing.assert_array_equal(oc.prelu(be, t, sl), F.prelu(torch.from_numpy(t), torch.from_numpy(sl.reshape(5))).numpy())
+    full = r.standard_normal(t.shape).astype(np.float32)
+    np.testing.assert_array_equal(oc.prelu(be, t, full), np.where(t < 0, full * t, t))
+    h = t.astype(np.float16)
+    np.testing.assert_array_equal(oc.leaky_relu(be, h, 0.1), np.where(h < 0, (np.float32(0.1) * h.astype(np.float32)), h).astype(np.float16))
+    with pytest.raises(RuntimeError):
+        oc.prelu(be, t, np.ones((4, 1, 1), np.float32))
+
+
+def test_concat_squeeze_unsqueeze(be):
+    r = rng(32)
+    a = r.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    for axis in range(4):
+        shapes = [list(a.shape) for _ in range(3)]
+        shapes[1][axis], shapes[2][axis] = 1, 7
+        xs = [r.standard_normal(s).astype(np.float32) for s in shapes]
+        np.testing.assert_array_equal(oc.concat(be, xs, axis), np.concatenate(xs, axis))
+    np.testing.assert_array_equal(oc.concat(be, [a], 1), a)
+    np.testing.assert_array_equal(oc.concat(be, [a, a], -1), np.concatenate([a, a], -1))
+    xi = [r.integers(-9, 9, (3, k)).astype(np.int64) for k in (1, 4, 2)]
+    np.testing.assert_array_equal(oc.concat(be, xi, 1), np.concatenate(xi, 1))
+    xh = [r.standard_normal((2, k, 3)).astype(np.float16) for k in (3, 5)]
+    np.testing.assert_array_equal(oc.concat(be, xh, 1), np.concatenate(xh, 1))
+    many = [r.standard_normal((1, 2)).astype(np.float32) for _ in range(16)]
+    np.testing.assert_array_equal(oc.concat(be, many, 0), np.concatenate(many, 0))
+    with pytest.raises(RuntimeError):
+        oc.concat(be, many + [many[0]], 0)                 # 17 inputs
+    with pytest.raises(RuntimeError):
+        oc.concat(be, [a, a[:, :, :3]], 1)                 # differ off the axis
+    s = r.standard_normal((2, 1, 4, 1)).astype(np.float32)
+    np.testing.assert_array_equal(oc.squeeze(be, s, (2, 4)), s.reshape(2, 4))
+    np.testing.assert_array_equal(oc.squeeze(be, s, (2, 4, 1)), s.reshape(2, 4, 1))
+    np.testing.assert_array_equal(oc.squeeze(be, s.reshape(2, 4), (1, 2, 1, 4), un=True), s.reshape(1, 2, 1, 4))
+    with pytest.raises(RuntimeError):
+        oc.squeeze(be, s, (4, 2))
+
+
 def test_layouts_the_oracle_lacks_are_refused(be):
     # The oracle restates the reference, which knows N,C,H,W tensors and
     # K,C,R,S filters only; asking it for anything else must fail, not drift.
