@@ -208,28 +208,50 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
 
   // ---- epilogue: accumulator register r of lane l is
   //      D[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 block --------------
+  // Bias and residual values are read in batches from clamped addresses and
+  // only the stores are predicated: a load inside a per-row branch would cost
+  // a memory round trip per row.
   float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
-  const float *__restrict__ Cg = a.Cin ? a.Cin + (int64_t)z * a.y_z_stride : nullptr;
-  const float *__restrict__ biasg = a.bias ? a.bias + (int64_t)z * a.bias_z_stride : nullptr;
   const int PQ = a.P * a.Q;
+  float bias_r[TM][16];
+  if (a.bias) {
+    const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) bias_r[i][r] = biasg[min(m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3), a.M - 1)];
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) bias_r[i][r] = 0.f;
+  }
 #pragma unroll
   for (int j = 0; j < TN; j++) {
     const int col = n0 + wn0 + j * 32 + lcol;
-    if (col >= a.Ncols) continue;
-    const int img = col / PQ, pq = col - img * PQ;
+    const bool col_ok = col < a.Ncols;
+    const int colc = col_ok ? col : 0;
+    const int img = colc / PQ, pq = colc - img * PQ;
     const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+      float res_r[16];
+      if (a.Cin) {
+        const float *__restrict__ Cg = a.Cin + (int64_t)z * a.y_z_stride;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          res_r[r] = Cg[ycol + (int64_t)min(m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3), a.M - 1) * a.y_row_stride];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) res_r[r] = 0.f;
+      }
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int m = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3);
-        if (m >= a.M) continue;
-        const int64_t off = ycol + (int64_t)m * a.y_row_stride;
-        float v = a.alpha * acc[i][j][r];
-        if (biasg) v += biasg[m];
-        if (Cg) v += a.beta * Cg[off];
+        float v = a.alpha * acc[i][j][r] + bias_r[i][r];
+        if (a.Cin) v += a.beta * res_r[r];
         if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
-        Yg[off] = v;
+        if (col_ok && m < a.M) Yg[ycol + (int64_t)m * a.y_row_stride] = v;
       }
     }
   }

@@ -60,7 +60,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
 
-#pragma unroll 2
+
   for (int k0 = kbeg; k0 < kend; k0 += 8) {
     const int ka = k0 + 4 * half;
     float av[4], bv[4];
@@ -126,22 +126,37 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
   }
 
   // ---- epilogue: register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] ----
-  if (!col_ok) return;
+  // Bias and residual values are read in one batch from clamped addresses and
+  // only the stores are predicated: a load inside a per-row branch would cost
+  // a memory round trip per row.
   float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
-  const float *__restrict__ Cg = a.Cin ? a.Cin + (int64_t)z * a.y_z_stride : nullptr;
-  const float *__restrict__ biasg = a.bias ? a.bias + (int64_t)z * a.bias_z_stride : nullptr;
-  const int img = col / PQ, pq = col - img * PQ;
+  const int colc = col_ok ? col : 0;
+  const int img = colc / PQ, pq = colc - img * PQ;
   const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
+  float bias_r[16], res_r[16];
+  if (a.bias) {
+    const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] = biasg[min(m0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1)];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] = 0.f;
+  }
+  if (a.Cin) {
+    const float *__restrict__ Cg = a.Cin + (int64_t)z * a.y_z_stride;
+#pragma unroll
+    for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(m0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1) * a.y_row_stride];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) res_r[r] = 0.f;
+  }
 #pragma unroll
   for (int r = 0; r < 16; r++) {
     const int mm = m0 + 8 * (r >> 2) + 4 * half + (r & 3);
-    if (mm >= a.M) continue;
-    const int64_t off = ycol + (int64_t)mm * a.y_row_stride;
-    float v = a.alpha * acc[r];
-    if (biasg) v += biasg[mm];
-    if (Cg) v += a.beta * Cg[off];
+    float v = a.alpha * acc[r] + bias_r[r];
+    if (a.Cin) v += a.beta * res_r[r];
     if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
-    Yg[off] = v;
+    if (col_ok && mm < a.M) Yg[ycol + (int64_t)mm * a.y_row_stride] = v;
   }
 }
 

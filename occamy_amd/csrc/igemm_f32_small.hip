@@ -25,6 +25,24 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float mask_f(float v, unsigned m) { return __uint_as_float(__float_as_uint(v) & m); }
 
+// The 16 accumulator registers of a lane hold rows m0 + 8 * (r >> 2) + 4 * half + (r & 3)
+// of output column n0 + l32.
+__device__ __forceinline__ int acc_row(int m0, int half, int r) { return m0 + 8 * (r >> 2) + 4 * half + (r & 3); }
+
+// Bias of the lane's 16 rows, requested at kernel start so that the values
+// are there when the epilogue wants them (a load per row at that point costs
+// a memory round trip each: the rows are handled under a divergent branch).
+__device__ __forceinline__ void prefetch_bias(const IgemmArgs &a, int z, int m0, int half, float (&bias_r)[16]) {
+  if (a.bias) {
+    const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] = biasg[min(acc_row(m0, half, r), a.M - 1)];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] = 0.f;
+  }
+}
+
 // Sum the KS partial tiles in LDS, then bias / residual / activation / store by wavefront 0.
 // The reduction may also be split over gridDim.y workgroups.  Each of them
 // leaves its partial tile in `partials` and bumps the tile's arrival counter;
@@ -33,8 +51,24 @@ __device__ __forceinline__ float mask_f(float v, unsigned m) { return __uint_as_
 // finishes the tile.  Nobody waits for anybody.  The last arriver puts the
 // counter back to zero for the next kernel on the stream.
 template <int KS>
-__device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, float (*red)[16][64], int wave, int lane,
-                                                 int m0, int col, bool col_ok, int z, unsigned tile, float *partials, unsigned *counters) {
+__device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, const float (&bias_r)[16], float (*red)[16][64],
+                                                 int wave, int lane, int m0, int col, bool col_ok, int z, unsigned tile,
+                                                 float *partials, unsigned *counters) {
+  const int half = lane >> 5, PQ = a.P * a.Q;
+  // the residual tensor's 16 values, requested before anything is waited for
+  const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
+  const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
+  float res_r[16];
+  if (a.Cin) {
+    if (wave == 0) {
+      const float *__restrict__ Cg = a.Cin + (int64_t)z * a.y_z_stride;
+#pragma unroll
+      for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(acc_row(m0, half, r), a.M - 1) * a.y_row_stride];
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) res_r[r] = 0.f;
+  }
   if (KS > 1) {
     if (wave > 0) {
 #pragma unroll
@@ -62,32 +96,32 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     if (lane == 0) arrived = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != (unsigned)splits - 1) return;
+    // splits is a power of two >= 2: two partial tiles are requested together
+    // and added in split order
     const float *all = partials + (size_t)tile * splits * 1024;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    for (int y = 0; y < splits; y++)
+    for (int y = 0; y < splits; y += 2) {
+      float p0[16], p1[16];
 #pragma unroll
-      for (int r = 0; r < 16; r++)
-        acc[r] += __hip_atomic_load(all + (size_t)y * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int r = 0; r < 16; r++) p0[r] = __hip_atomic_load(all + (size_t)y * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int r = 0; r < 16; r++) p1[r] = __hip_atomic_load(all + (size_t)(y + 1) * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] = (acc[r] + p0[r]) + p1[r];
+    }
     if (lane == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (!col_ok) return;
-  const int half = lane >> 5, PQ = a.P * a.Q;
   float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
-  const float *__restrict__ Cg = a.Cin ? a.Cin + (int64_t)z * a.y_z_stride : nullptr;
-  const float *__restrict__ biasg = a.bias ? a.bias + (int64_t)z * a.bias_z_stride : nullptr;
-  const int img = col / PQ, pq = col - img * PQ;
-  const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
 #pragma unroll
   for (int r = 0; r < 16; r++) {
-    const int mm = m0 + 8 * (r >> 2) + 4 * half + (r & 3);
+    const int mm = acc_row(m0, half, r);
     if (mm >= a.M) continue;
-    const int64_t off = ycol + (int64_t)mm * a.y_row_stride;
-    float v = a.alpha * acc[r];
-    if (biasg) v += biasg[mm];
-    if (Cg) v += a.beta * Cg[off];
+    float v = a.alpha * acc[r] + bias_r[r];
+    if (a.Cin) v += a.beta * res_r[r];
     if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
-    Yg[off] = v;
+    Yg[ycol + (int64_t)mm * a.y_row_stride] = v;
   }
 }
 
@@ -113,6 +147,8 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   const int col = n0 + l32;
   const bool col_ok = col < a.Ncols;
   const int PQ = a.P * a.Q, HW = a.H * a.W, C = a.Kdim / 9;
+  float bias_r[16];
+  prefetch_bias(a, z, m0, half, bias_r);
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int p = pq / a.Q, q = pq - p * a.Q;
   const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
@@ -130,7 +166,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   const int cbeg = ((int)blockIdx.y * KS + wave) * c_per_wave, cend = min(C, cbeg + c_per_wave);
   const int niter = c_per_wave >> 1;
 
-  constexpr int DEPTH = 2;
+  constexpr int DEPTH = 4;
   float ra[DEPTH][9], rb[DEPTH][9];
   unsigned cm[DEPTH];
   auto load_iter = [&](int i, float (&av)[9], float (&bv)[9], unsigned &cmask) {
@@ -167,7 +203,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
+  reduce_and_store<KS>(a, acc, bias_r, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // 1x1 geometry (convolution, possibly strided, or matrix product with A rows
@@ -194,6 +230,8 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   const int col = n0 + l32;
   const bool col_ok = col < a.Ncols;
   const int PQ = a.P * a.Q, HW = a.H * a.W;
+  float bias_r[16];
+  prefetch_bias(a, z, m0, half, bias_r);
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int p = pq / a.Q, q = pq - p * a.Q;
   const unsigned x_pix = (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
@@ -238,7 +276,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
+  reduce_and_store<KS>(a, acc, bias_r, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // Returns true if one of the specialised kernels took the problem.

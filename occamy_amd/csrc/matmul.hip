@@ -14,36 +14,41 @@
 namespace dnnrt {
 
 // Out[m, n] = alpha * dot(A[m, :], B[n, :]) + beta * C[m, n], M <= 8.
-// One wavefront per n; lanes stride over k; B is read exactly once.
-template <int MMAX>
-__global__ __launch_bounds__(256) void gemv_f32_kernel(const float *__restrict__ A,
-                                                       const float *__restrict__ B,
-                                                       const float *__restrict__ C,
-                                                       float *__restrict__ Out, int M, int N, int K,
-                                                       float alpha, float beta, bool vec4) {
+// WPO wavefronts share one n, each striding over its own slices of k; B is
+// read exactly once.  The partial sums of an n meet in LDS and are added in
+// wavefront order, so the result does not depend on timing.  WPO is picked on
+// the host so that a narrow N (a few hundred outputs over a long K) still puts
+// a few thousand wavefronts on the device.
+template <int MMAX, int WPO>
+__global__ __launch_bounds__(WPO > 4 ? 64 * WPO : 256) void gemv_f32_kernel(
+    const float *__restrict__ A, const float *__restrict__ B, const float *__restrict__ C,
+    float *__restrict__ Out, int M, int N, int K, float alpha, float beta, bool vec4) {
+  constexpr int WAVES = WPO > 4 ? WPO : 4, NPB = WAVES / WPO;
+  __shared__ float part[WAVES][MMAX];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = blockIdx.x * 4 + wave;
-  if (n >= N) return;
-  const float *b = B + (int64_t)n * K;
+  const int n = blockIdx.x * NPB + wave / WPO, slice = wave % WPO;
   float acc[MMAX];
 #pragma unroll
   for (int m = 0; m < MMAX; m++) acc[m] = 0.f;
-  if (vec4) {
-    for (int k = lane * 4; k < K; k += 256) {
-      const float4 bv = *reinterpret_cast<const float4 *>(b + k);
+  if (n < N) {
+    const float *b = B + (int64_t)n * K;
+    if (vec4) {
+      for (int k = (slice * 64 + lane) * 4; k < K; k += 256 * WPO) {
+        const float4 bv = *reinterpret_cast<const float4 *>(b + k);
 #pragma unroll
-      for (int m = 0; m < MMAX; m++)
-        if (m < M) {
-          const float4 av = *reinterpret_cast<const float4 *>(A + (int64_t)m * K + k);
-          acc[m] += av.x * bv.x + av.y * bv.y + av.z * bv.z + av.w * bv.w;
-        }
-    }
-  } else {
-    for (int k = lane; k < K; k += 64) {
-      const float bv = b[k];
+        for (int m = 0; m < MMAX; m++)
+          if (m < M) {
+            const float4 av = *reinterpret_cast<const float4 *>(A + (int64_t)m * K + k);
+            acc[m] += av.x * bv.x + av.y * bv.y + av.z * bv.z + av.w * bv.w;
+          }
+      }
+    } else {
+      for (int k = slice * 64 + lane; k < K; k += 64 * WPO) {
+        const float bv = b[k];
 #pragma unroll
-      for (int m = 0; m < MMAX; m++)
-        if (m < M) acc[m] += A[(int64_t)m * K + k] * bv;
+        for (int m = 0; m < MMAX; m++)
+          if (m < M) acc[m] += A[(int64_t)m * K + k] * bv;
+      }
     }
   }
 #pragma unroll
@@ -51,12 +56,25 @@ __global__ __launch_bounds__(256) void gemv_f32_kernel(const float *__restrict__
     float v = acc[m];
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    if (lane == 0 && m < M) {
-      float r = alpha * v;
-      if (C) r += beta * C[(int64_t)m * N + n];
-      Out[(int64_t)m * N + n] = r;
-    }
+    if (lane == 0) part[wave][m] = v;
   }
+  __syncthreads();
+  if (slice == 0 && n < N && lane < M) {
+    float v = part[wave][lane];
+#pragma unroll
+    for (int w = 1; w < WPO; w++) v += part[wave + w][lane];
+    float r = alpha * v;
+    if (C) r += beta * C[(int64_t)lane * N + n];
+    Out[(int64_t)lane * N + n] = r;
+  }
+}
+
+template <int WPO>
+static void launch_gemv(const dnnrtContext *ctx, const float *A, const float *B, const float *C, float *Out,
+                        int M, int N, int K, float alpha, float beta, bool vec4) {
+  constexpr int WAVES = WPO > 4 ? WPO : 4, NPB = WAVES / WPO;
+  hipLaunchKernelGGL((gemv_f32_kernel<8, WPO>), dim3((unsigned)ceil_div(N, NPB)), dim3(64 * WAVES), 0, ctx->stream,
+                     A, B, C, Out, M, N, K, alpha, beta, vec4);
 }
 
 static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, const float *C,
@@ -64,8 +82,12 @@ static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, co
                      bool transB, int Z, int64_t az, int64_t bz, int64_t yz) {
   if (Z == 1 && M <= 8 && transB && !transA) {
     const bool vec4 = (K % 4 == 0) && aligned16(A) && aligned16(B);
-    hipLaunchKernelGGL((gemv_f32_kernel<8>), dim3((unsigned)ceil_div(N, 4)), dim3(256), 0, ctx->stream,
-                       A, B, C, Out, M, N, K, alpha, beta, vec4);
+    // wavefronts per output: the fewest that give 2048 wavefronts, each keeping >= 512 elements of k
+    int wpo = 1;
+    while (wpo < 16 && (int64_t)N * wpo < 2048 && K / (wpo * 4) >= 512) wpo *= 4;
+    if (wpo == 1) launch_gemv<1>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4);
+    else if (wpo == 4) launch_gemv<4>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4);
+    else launch_gemv<16>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("gemv_f32: launch failed: %s", hipGetErrorString(e)); return false; }
     return true;

@@ -218,7 +218,9 @@ def test_pooling(gpu, cpu):
 
 def test_matmul2d(gpu, cpu):
     r = rng(14)
-    for M, K, N in [(1, 2048, 1000), (1, 1280, 1000), (5, 9, 7), (64, 64, 64), (130, 70, 33), (3, 2048, 10), (16, 250, 40)]:
+    # the few-row shapes take the dot-product kernel with 1, 4 or 16 wavefronts per output
+    for M, K, N in [(1, 2048, 1000), (1, 1280, 1000), (5, 9, 7), (64, 64, 64), (130, 70, 33), (3, 2048, 10), (16, 250, 40),
+                    (2, 50176, 496), (8, 8194, 33), (1, 9216, 4096), (7, 2049, 5)]:
         a = r.standard_normal((M, K)).astype(np.float32)
         b = (r.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
         c = r.standard_normal((M, N)).astype(np.float32)
