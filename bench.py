@@ -32,7 +32,7 @@ def build_workload(name):
     if name == "resnet50_fp16_bs64":
         return models.resnet50(64, np.float16, seed=5), dict(fusion=True, fuse_residual=True, channels_last=True), 64, "img/s", "f16"
     if name == "mobilenet_v2_fp32_bs1":
-        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True), 1, "img/s", "f32"
+        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
         return models.bert_encoder(), dict(), 1, "seq/s", "f32"
     if name == "single_conv_fp32":
@@ -40,9 +40,9 @@ def build_workload(name):
     if name == "alexnet_fp32_bs1":
         return models.alexnet(1, np.float32), dict(fusion=True), 1, "img/s", "f32"
     if name == "yolo_v1_fp32_bs2":
-        return models.yolo_v1(2, np.float32), dict(fusion=True), 2, "img/s", "f32"
+        return models.yolo_v1(2, np.float32), dict(fusion=True, fuse_activations=True), 2, "img/s", "f32"
     if name == "srgan_fp32_96x96":
-        return models.srgan_generator(1, np.float32, height=96, width=96), dict(fusion=True), 1, "img/s", "f32"
+        return models.srgan_generator(1, np.float32, height=96, width=96), dict(fusion=True, fuse_residual=True, fuse_activations=True), 1, "img/s", "f32"
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -117,7 +117,7 @@ def main():
         dt = time.perf_counter() - t0
         res = dict(name=name, batch=batch, unit=unit, dtype=dtype, ms_per_step=1e3 * dt / steps,
                    value=batch * steps / dt, pool_bytes=prog.pool_bytes, weights_bytes=sess.weights_bytes,
-                   kernels_per_step=prog.num_ops(compute_only=True))
+                   kernels_per_step=prog.num_ops(compute_only=True), flags=flags)
         if want_profile:
             # per-kernel device timestamps on the session's own stream, eager launches
             ops = prog.compute_ops()
@@ -138,7 +138,7 @@ def main():
         # the reference's per-inference semantics: pool alloc, all weights H2D, kernels, D2H, sync, pool free
         # (compiled with the reference's own flags: no residual fusion)
         (ref_graph, _), _, _, _, _ = build_workload(name)  # a graph compiles once; the builders are seeded
-        ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k != "fuse_residual"})
+        ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k not in ("fuse_residual", "fuse_activations")})
         res["pool_bytes_reference_flags"] = ref_prog.pool_bytes
         so = ref_prog.session(compiler.MODE_OCCAMY)
         so.run(*inputs)
@@ -200,7 +200,7 @@ def main():
         "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic",
         "config": {"workload": args.workload, "batch": main_res["batch"],
-                   "fusion": "conv+bias+relu, conv+bias+residual add+relu",
+                   "fusion": ", ".join(k for k, v in main_res["flags"].items() if v and k.startswith("fus")),
                    "mode": "weights and input resident in HBM, kernels replayed from a captured graph",
                    "kernels_per_step": main_res["kernels_per_step"]},
         "roofline": roof,

@@ -56,6 +56,8 @@ typedef struct {
   int32_t channels_last;  /* fp16 only: rank-4 activations are NHWC on the device */
   int32_t fuse_residual;  /* no reference flag: with `fusion`, conv+bias -> add -> relu
                              closing a residual block becomes one call (default 0) */
+  int32_t fuse_activations; /* no reference flag: with `fusion`, conv+bias -> Clip(0, c) /
+                             LeakyRelu / one-slope PRelu becomes one call (default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);

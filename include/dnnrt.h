@@ -64,7 +64,9 @@ enum { DNNRT_FILTER_KCRS = 0, DNNRT_FILTER_CRSK = 1 };
  * (src/Tools/dnn-wrapper/cudnn/CUDNNActiveFunc.cpp:8-91;
  *  fusedOp/CUDNNConvBiasReluFunc.cpp:65-68). */
 enum { DNNRT_ACT_SIGMOID = 0, DNNRT_ACT_RELU = 1, DNNRT_ACT_TANH = 2,
-       DNNRT_ACT_IDENTITY = 5 };
+       DNNRT_ACT_CLIPPED_RELU = 3, /* min(max(x, 0), coef): cuDNN's mode 3 */
+       DNNRT_ACT_IDENTITY = 5,
+       DNNRT_ACT_LEAKY_RELU = 6    /* x < 0 ? coef * x : x: no cuDNN mode */ };
 
 /* tensor-op modes: cudnnOpTensorOp_t values the reference emits
  * (src/Conversion/DNNToLLVM/Ops/cudnn/Add.cpp:148, Mul.cpp:144, Sqrt.cpp:112). */
@@ -96,6 +98,13 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format);
 /* New.  Physical layout of fp32 convolution filters for subsequent calls
  * (DNNRT_FILTER_KCRS is the default and the reference's). */
 int32_t dnnrtSetFilterLayout(dnnrtHandle_t handle, int32_t layout);
+/* The coefficient of the activation modes that take one: the ceiling of
+ * DNNRT_ACT_CLIPPED_RELU, the slope of DNNRT_ACT_LEAKY_RELU.  It stands where
+ * the `coef` of cudnnSetActivationDescriptor stands (the reference sets up one
+ * descriptor per call with coef 0, src/Tools/dnn-wrapper/cudnn/fusedOp/
+ * CUDNNConvBiasReluFunc.cpp); sticky per handle like the tensor format,
+ * default 0.  Read by dnnrtConvBiasActiv, dnnrtConvBiasAddActiv, dnnrtActive. */
+int32_t dnnrtSetActivationCoef(dnnrtHandle_t handle, float coef);
 /* New.  Blocks until all work on the handle's stream is done; the reference
  * returns to the host without waiting for its device-to-host copies
  * (src/Tools/dnn-wrapper/cuda/wrapDNNMemcpy.cpp:32). */
@@ -152,7 +161,9 @@ void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
 /* DNNAPISpecs.inc:121 "DNNConvBiasActivFunc"
  * (src/Tools/dnn-wrapper/cudnn/fusedOp/CUDNNConvBiasReluFunc.cpp:8-140).
  * Y = act(conv(X, W) + B), B holds K values (dimB is {1,K,1,1}),
- * activMode DNNRT_ACT_RELU or DNNRT_ACT_IDENTITY. */
+ * activMode DNNRT_ACT_RELU or DNNRT_ACT_IDENTITY (what the reference emits),
+ * or DNNRT_ACT_CLIPPED_RELU / DNNRT_ACT_LEAKY_RELU with the handle's
+ * activation coefficient. */
 void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X,
                          const int64_t *dimX, const void *W,
                          const int64_t *dimW, const void *B,

@@ -16,6 +16,8 @@ def main():
     ap.add_argument("model", help="ONNX model file (static shapes)")
     ap.add_argument("--dnn-kernel-fusion", dest="fusion", action="store_true")
     ap.add_argument("--fuse-residual", action="store_true", help="with fusion: conv+bias -> add -> relu as one call")
+    ap.add_argument("--fuse-activations", action="store_true",
+                    help="with fusion: conv+bias -> Clip(0, c) / LeakyRelu / one-slope PRelu as one call")
     ap.add_argument("--no-dnn-dealloc-opt", dest="dealloc_opt", action="store_false")
     ap.add_argument("--no-onnx-const-at-use", dest="const_at_use", action="store_false")
     ap.add_argument("--channels-last", action="store_true", help="fp16 graphs: NHWC on the device")
@@ -27,7 +29,7 @@ def main():
     args = ap.parse_args()
 
     graph = compiler.load_onnx(args.model)
-    prog = graph.compile(fusion=args.fusion, fuse_residual=args.fuse_residual, dealloc_opt=args.dealloc_opt,
+    prog = graph.compile(fusion=args.fusion, fuse_residual=args.fuse_residual, fuse_activations=args.fuse_activations, dealloc_opt=args.dealloc_opt,
                          const_at_use=args.const_at_use, channels_last=args.channels_last)
     print(f"inputs: {graph.input_shapes}")
     print(f"pool: {prog.pool_bytes} bytes (maxAllocByte); {prog.num_ops(compute_only=True)} runtime calls per inference")

@@ -23,6 +23,7 @@ SIGNATURES = {
     "dnnrtSetStream": (i32, [P, P]),
     "dnnrtSetTensorFormat": (i32, [P, i32]),
     "dnnrtSetFilterLayout": (i32, [P, i32]),
+    "dnnrtSetActivationCoef": (i32, [P, f32]),
     "dnnrtSync": (i32, [P]),
     "dnnrtGraphBegin": (i32, [P]),
     "dnnrtGraphEnd": (i32, [P, C.POINTER(P)]),
@@ -74,7 +75,7 @@ SIGNATURES = {
 F32, F16, I64 = 0, 1, 2
 NCHW, NHWC, NCHW_TO_NHWC = 0, 1, 2
 FILTER_KCRS, FILTER_CRSK = 0, 1
-ACT_SIGMOID, ACT_RELU, ACT_TANH, ACT_IDENTITY = 0, 1, 2, 5
+ACT_SIGMOID, ACT_RELU, ACT_TANH, ACT_CLIPPED_RELU, ACT_IDENTITY, ACT_LEAKY_RELU = 0, 1, 2, 3, 5, 6
 OP_ADD, OP_MUL, OP_SQRT = 0, 1, 4
 REDUCE_AVG = 5
 H2D, D2H, D2D = 1, 2, 3

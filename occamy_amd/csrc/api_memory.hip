@@ -46,6 +46,7 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
   c->stream = nullptr;
   c->format = DNNRT_NCHW;
   c->filter_layout = DNNRT_FILTER_KCRS;
+  c->act_coef = 0.f;
   c->device = dev;
   c->num_cu = prop.multiProcessorCount;
   c->splitk_partials = nullptr;
@@ -99,6 +100,13 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format) {
     return 1;
   }
   handle->format = format;
+  return 0;
+}
+
+int32_t dnnrtSetActivationCoef(dnnrtHandle_t handle, float coef) {
+  if (!handle) { dnnrt::set_error("dnnrtSetActivationCoef: null handle"); return 1; }
+  if (coef != coef) { dnnrt::set_error("dnnrtSetActivationCoef: NaN"); return 1; }
+  handle->act_coef = coef;
   return 0;
 }
 

@@ -14,6 +14,7 @@ struct dnnrtContext {
   hipStream_t stream;  // kernels of this handle are launched here
   int format;          // DNNRT_NCHW / DNNRT_NHWC / DNNRT_NCHW_TO_NHWC
   int filter_layout;   // DNNRT_FILTER_KCRS / DNNRT_FILTER_CRSK (fp32 convolutions)
+  float act_coef;      // ceiling of CLIPPED_RELU / slope of LEAKY_RELU
   int device;
   int num_cu;
   // Scratch for reductions split over workgroups: partial tiles and one
@@ -53,5 +54,17 @@ inline int64_t numel(const int64_t *d, int64_t rank) {
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool float_dtype(int32_t dt) { return dt == DNNRT_F32 || dt == DNNRT_F16; }
+
+// The activations a convolution epilogue can apply (sigmoid and tanh are
+// separate calls, as in the reference).
+__device__ __forceinline__ float apply_act(float v, int act, float coef) {
+  if (act == DNNRT_ACT_RELU) return v < 0.f ? 0.f : v;
+  if (act == DNNRT_ACT_CLIPPED_RELU) { v = v < 0.f ? 0.f : v; return v > coef ? coef : v; }
+  if (act == DNNRT_ACT_LEAKY_RELU) return v < 0.f ? coef * v : v;
+  return v;
+}
+__host__ __device__ inline bool fusable_act(int64_t act) {
+  return act == DNNRT_ACT_RELU || act == DNNRT_ACT_IDENTITY || act == DNNRT_ACT_CLIPPED_RELU || act == DNNRT_ACT_LEAKY_RELU;
+}
 
 }  // namespace dnnrt

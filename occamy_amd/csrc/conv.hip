@@ -19,7 +19,7 @@ template <int R, int S>
 __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
     const float *__restrict__ X, const float *__restrict__ Wt, const float *__restrict__ bias,
     const float *__restrict__ Zr, float *__restrict__ Y, int C, int H, int W, int K, int Kg, int P, int Q, int ph, int pw,
-    int sh, int sw, int rr, int ss, int act, int64_t total, int w_k_stride, int w_tap_stride) {
+    int sh, int sw, int rr, int ss, int act, float act_coef, int64_t total, int w_k_stride, int w_tap_stride) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
   const int q = (int)(i % Q);
@@ -34,11 +34,11 @@ __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
   const float *w = Wt + (int64_t)k * w_k_stride;  // tap (r, s) at w[(r * S + s) * w_tap_stride]
   const int ih0 = p * sh - ph, iw0 = q * sw - pw;
   float acc = 0.f;
-#pragma unroll
+#pragma unroll 3
   for (int r = 0; r < Rr; r++) {
     const int ih = ih0 + r;
     if ((unsigned)ih >= (unsigned)H) continue;
-#pragma unroll
+#pragma unroll 3
     for (int s = 0; s < Ss; s++) {
       const int iw = iw0 + s;
       if ((unsigned)iw < (unsigned)W) acc = fmaf(x[(int64_t)ih * W + iw], w[(r * Ss + s) * w_tap_stride], acc);
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
   }
   if (bias) acc += bias[k];
   if (Zr) acc += Zr[i];
-  if (act == DNNRT_ACT_RELU) acc = acc < 0.f ? 0.f : acc;
+  acc = apply_act(acc, act, act_coef);
   Y[i] = acc;
 }
 
@@ -100,17 +100,17 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
     const int w_k = crsk ? 1 : s.R * s.S, w_tap = crsk ? s.K : 1;
     if (s.R == 3 && s.S == 3)
       hipLaunchKernelGGL((dwconv_f32_nchw_kernel<3, 3>), grid, block, 0, ctx->stream, X, Wt, bias, Z, Y,
-                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, total, w_k, w_tap);
+                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, ctx->act_coef, total, w_k, w_tap);
     else
       hipLaunchKernelGGL((dwconv_f32_nchw_kernel<0, 0>), grid, block, 0, ctx->stream, X, Wt, bias, Z, Y,
-                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, total, w_k, w_tap);
+                         s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, ctx->act_coef, total, w_k, w_tap);
     DNNRT_CHECK_LAUNCH("conv(depthwise)");
     return Y;
   }
   IgemmArgs a{};
   const int Kg = s.K / s.group;
   a.A = Wt; a.X = X; a.Y = Y; a.bias = bias; a.Cin = Z;  // residual: (acc + bias) + Z
-  a.alpha = 1.f; a.beta = Z ? 1.f : 0.f; a.act = act;
+  a.alpha = 1.f; a.beta = Z ? 1.f : 0.f; a.act = act; a.act_coef = ctx->act_coef;
   a.M = Kg; a.Kdim = s.Cg * s.R * s.S; a.Ncols = s.N * s.P * s.Q;
   a.H = s.H; a.W = s.W; a.R = s.R; a.S = s.S; a.P = s.P; a.Q = s.Q;
   a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw;
@@ -149,7 +149,7 @@ static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, cons
     a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Z = (const __half *)Z; a.Y = (__half *)Y;
     a.N = s.N; a.C = s.C; a.H = s.H; a.W = s.W; a.K = s.K; a.Cg = s.Cg; a.R = s.R; a.S = s.S;
     a.P = s.P; a.Q = s.Q; a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw; a.group = s.group;
-    a.act = act; a.format = h->format;
+    a.act = act; a.act_coef = h->act_coef; a.format = h->format;
     if (!launch_conv_f16(h, a)) return nullptr;
     return Y;
   }
@@ -173,8 +173,8 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dim
                          int64_t workspaceBytes, int64_t algo, int64_t group, const int64_t *pads,
                          const int64_t *strides, int64_t activMode, void *Y, int32_t dtype) {
   (void)workspace; (void)workspaceBytes; (void)algo;
-  if (activMode != DNNRT_ACT_RELU && activMode != DNNRT_ACT_IDENTITY)
-    DNNRT_FAIL("dnnrtConvBiasActiv: activMode %ld (1 = ReLU, 5 = identity)", (long)activMode);
+  if (!dnnrt::fusable_act(activMode))
+    DNNRT_FAIL("dnnrtConvBiasActiv: activMode %ld (1 ReLU, 3 clipped ReLU, 5 identity, 6 leaky ReLU)", (long)activMode);
   if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
     DNNRT_FAIL("dnnrtConvBiasActiv: bias must hold K values");
   return dnnrt::conv_dispatch("dnnrtConvBiasActiv", handle, X, dimX, W, dimW, B, nullptr, group, pads,
@@ -187,8 +187,8 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X, const int64_t *
                             const int64_t *pads, const int64_t *strides, int64_t activMode, void *Y,
                             int32_t dtype) {
   (void)workspace; (void)workspaceBytes; (void)algo;
-  if (activMode != DNNRT_ACT_RELU && activMode != DNNRT_ACT_IDENTITY)
-    DNNRT_FAIL("dnnrtConvBiasAddActiv: activMode %ld (1 = ReLU, 5 = identity)", (long)activMode);
+  if (!dnnrt::fusable_act(activMode))
+    DNNRT_FAIL("dnnrtConvBiasAddActiv: activMode %ld (1 ReLU, 3 clipped ReLU, 5 identity, 6 leaky ReLU)", (long)activMode);
   if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
     DNNRT_FAIL("dnnrtConvBiasAddActiv: bias must hold K values");
   if (!Z) DNNRT_FAIL("dnnrtConvBiasAddActiv: null residual tensor");

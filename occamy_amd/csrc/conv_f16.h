@@ -9,7 +9,8 @@ struct ConvF16Args {
   const __half *Z;  // residual tensor laid out like Y, or null
   __half *Y;
   int N, C, H, W, K, Cg, R, S, P, Q, ph, pw, sh, sw, group;
-  int act;     // DNNRT_ACT_RELU / DNNRT_ACT_IDENTITY
+  int act;     // DNNRT_ACT_{IDENTITY, RELU, CLIPPED_RELU, LEAKY_RELU}
+  float act_coef;  // ceiling / slope of the last two
   int format;  // physical layout of X and Y (DNNRT_NCHW / NHWC / NCHW_TO_NHWC)
   unsigned magic_pq, magic_q;  // filled in by the launcher: ceil(2^32 / (P*Q)), ceil(2^32 / Q)
 };

@@ -339,7 +339,7 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
     __syncthreads();  // the output staging below reuses the same LDS
   }
   const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
-  const bool relu_now = a.act == DNNRT_ACT_RELU && !Zg;  // with a residual the activation comes after the sum
+  const int act_now = Zg ? DNNRT_ACT_IDENTITY : a.act;  // with a residual the activation comes after the sum
   _Float16 *Cs = smem;  // [BN pixels][CROW]
   // the residual chunks this thread will need, requested now (clamped
   // addresses) so that they arrive while the tile is staged through LDS
@@ -353,46 +353,56 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
       zpre[it] = *reinterpret_cast<const half8 *>(Zg + (int64_t)pix * a.K + k_out);
     }
   }
+  // The activation mode is the same for the whole launch: each loop below is
+  // instantiated per mode and picked once, so the per-element code is that of
+  // the one mode (ReLU: a single max).
+  auto per_mode = [&](int mode, auto &&body) {
+    switch (mode) {
+      case DNNRT_ACT_RELU: body(std::integral_constant<int, DNNRT_ACT_RELU>{}); break;
+      case DNNRT_ACT_CLIPPED_RELU: body(std::integral_constant<int, DNNRT_ACT_CLIPPED_RELU>{}); break;
+      case DNNRT_ACT_LEAKY_RELU: body(std::integral_constant<int, DNNRT_ACT_LEAKY_RELU>{}); break;
+      default: body(std::integral_constant<int, DNNRT_ACT_IDENTITY>{}); break;
+    }
+  };
   if (KG == 1 || kg == 0)
+    per_mode(act_now, [&](auto mode_c) {
+      constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+      for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int kl = wm0 + i * 32 + 8 * g + 4 * half;  // k_out within the tile
-        half4 o;
+          for (int g = 0; g < 4; g++) {
+            const int kl = wm0 + i * 32 + 8 * g + 4 * half;  // k_out within the tile
+            half4 o;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          float v = acc[i][j][4 * g + e] + (float)bias4[i][g][e];
-          if (relu_now) v = v < 0.f ? 0.f : v;
-          o[e] = (_Float16)v;
-        }
-        *reinterpret_cast<half4 *>(Cs + (wn0 + j * 32 + l32) * CROW + kl) = o;
-      }
+            for (int e = 0; e < 4; e++)
+              o[e] = (_Float16)apply_act(acc[i][j][4 * g + e] + (float)bias4[i][g][e], MODE, a.act_coef);
+            *reinterpret_cast<half4 *>(Cs + (wn0 + j * 32 + l32) * CROW + kl) = o;
+          }
+    });
   __syncthreads();
   _Float16 *__restrict__ Yg = reinterpret_cast<_Float16 *>(a.Y);
+  per_mode(Zg ? a.act : DNNRT_ACT_IDENTITY, [&](auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-  for (int it = 0; it < OUT_IT; it++) {
-    const int id = tid + it * NT;
-    const int row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
-    const int pix = n0 + row, k_out = m0 + ch * 8;
-    if (pix < NPQ && k_out < a.K) {
-      half8 o = *reinterpret_cast<const half8 *>(Cs + row * CROW + ch * 8);
-      if (Zg) {
-        // conv + bias was rounded to fp16 above, as a separate convolution
-        // would have stored it; the residual sum follows in fp32
-        const half8 zv = zpre[it];
+    for (int it = 0; it < OUT_IT; it++) {
+      const int id = tid + it * NT;
+      const int row = id / CH_PER_ROW, ch = id - row * CH_PER_ROW;
+      const int pix = n0 + row, k_out = m0 + ch * 8;
+      if (pix < NPQ && k_out < a.K) {
+        half8 o = *reinterpret_cast<const half8 *>(Cs + row * CROW + ch * 8);
+        if (Zg) {
+          // conv + bias was rounded to fp16 above, as a separate convolution
+          // would have stored it; the residual sum follows in fp32
+          const half8 zv = zpre[it];
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          float v = (float)o[e] + (float)zv[e];
-          if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
-          o[e] = (_Float16)v;
+          for (int e = 0; e < 8; e++) o[e] = (_Float16)apply_act((float)o[e] + (float)zv[e], MODE, a.act_coef);
         }
+        *reinterpret_cast<half8 *>(Yg + (int64_t)pix * a.K + k_out) = o;
       }
-      *reinterpret_cast<half8 *>(Yg + (int64_t)pix * a.K + k_out) = o;
     }
-  }
+  });
 }
 
 // ---- generic kernel ---------------------------------------------------------
@@ -472,7 +482,7 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
     if (biasg) v += (float)biasg[ko];
     const int64_t off = out_nhwc ? (int64_t)opix * a.K + ko : ((int64_t)on * a.K + ko) * PQ + opq;
     if (Zg) v = (float)(_Float16)v + (float)Zg[off];
-    if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+    v = apply_act(v, a.act, a.act_coef);
     Yg[off] = (_Float16)v;
   }
 }

@@ -183,7 +183,8 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched) {
   launched = false;
   if (a.format != DNNRT_NCHW_TO_NHWC || a.group != 1 || a.C != 3 || a.R != 7 || a.S != 7 || a.sh != 2 || a.sw != 2 ||
-      a.ph != 3 || a.pw != 3 || a.K != 64 || a.Z != nullptr || !aligned16(a.Y))
+      a.ph != 3 || a.pw != 3 || a.K != 64 || a.Z != nullptr || !aligned16(a.Y) ||
+      (a.act != DNNRT_ACT_RELU && a.act != DNNRT_ACT_IDENTITY))
     return true;
   if ((int64_t)3 * a.H * a.W >= (1ll << 31)) return true;
   const int tiles_p = (a.P + stem::TP - 1) / stem::TP, tiles_q = (a.Q + stem::TQ - 1) / stem::TQ;

@@ -130,6 +130,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   func_args_to_device(p);
   erase_dummy_constants(p);
   if (opt->fusion) fuse_conv_bias_activ(p);
+  if (opt->fusion && opt->fuse_activations) fuse_conv_activations(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {

@@ -32,7 +32,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
   if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
   LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
-  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
@@ -228,6 +228,10 @@ bool Session::issue(const Op *op, std::string &err) {
     if (lay != cur_filter_layout) {
       if (rt.dnnrtSetFilterLayout(handle, lay)) { err = rt_error("dnnrtSetFilterLayout"); return false; }
       cur_filter_layout = lay;
+    }
+    if ((op->mode == 3 || op->mode == 6) && op->kind != OP_CONVFWD && op->coef != cur_act_coef) {
+      if (rt.dnnrtSetActivationCoef(handle, op->coef)) { err = rt_error("dnnrtSetActivationCoef"); return false; }
+      cur_act_coef = op->coef;
     }
   }
   void *r = nullptr;

@@ -59,6 +59,7 @@ struct RuntimeApi {
   decltype(&::dnnrtReshape) dnnrtReshape = nullptr;
   decltype(&::dnnrtTranspose) dnnrtTranspose = nullptr;
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
+  decltype(&::dnnrtSetActivationCoef) dnnrtSetActivationCoef = nullptr;
   decltype(&::dnnrtLeakyRelu) dnnrtLeakyRelu = nullptr;
   decltype(&::dnnrtPRelu) dnnrtPRelu = nullptr;
   decltype(&::dnnrtConcat) dnnrtConcat = nullptr;
@@ -92,6 +93,7 @@ class Session {
   dnnrtStream_t stream = nullptr;
   bool host_backend = false;
   int cur_format = 0, cur_filter_layout = 0;
+  float cur_act_coef = 0.f;   // what the handle's activation coefficient was last set to
   std::map<std::string, bool> crsk_const;  // constants re-laid C,R,S,K on the host
   std::vector<char> filter_crsk;           // value id -> its device copy is C,R,S,K
   void *pool = nullptr, *weights = nullptr, *graph = nullptr;

@@ -177,6 +177,7 @@ std::string Program::to_text() const {
         print_shape(os, op->strides);
         os << ", group=" << op->group;
         if (op->kind != OP_CONVFWD) os << ", activMode=" << op->mode;
+        if (op->kind != OP_CONVFWD && (op->mode == 3 || op->mode == 6)) os << ", activCoef=" << op->coef;
         os << "}";
         break;
       case OP_ACTIVATION: os << " {mode=" << op->mode << "}"; break;

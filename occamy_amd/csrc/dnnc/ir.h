@@ -162,6 +162,7 @@ bool graph_from_onnx(const uint8_t *data, size_t nbytes, Graph &g, std::string &
 // passes.cpp
 void fuse_conv_bias_activ(Program &p);
 void fuse_residual_add(Program &p);
+void fuse_conv_activations(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);
 bool malloc_pool_opt(Program &p, std::string &err);

@@ -7,6 +7,8 @@
 #include "planner.h"
 
 #include <algorithm>
+#include <cmath>
+#include <cstring>
 
 namespace dnnc {
 
@@ -74,10 +76,11 @@ void fuse_conv_bias_activ(Program &p) {
   }
 }
 
-// conv+bias (identity) -> add(full-shape tensor Z) -> relu, each intermediate
-// read by nothing else, becomes one conv-bias-add-relu writing the ReLU's
-// buffer.  The reference has no such pattern; cuDNN's fused call has the z
-// operand for it (the reference passes it with weight 0,
+// conv+bias (identity) -> add(full-shape tensor Z) [-> relu], the convolution's
+// result read by nothing else (and the sum by nothing but the ReLU), becomes
+// one conv-bias-add-activation writing the last buffer of the chain.  The
+// reference has no such pattern; cuDNN's fused call has the z operand for it
+// (the reference passes it with weight 0,
 // src/Tools/dnn-wrapper/cudnn/fusedOp/CUDNNConvBiasReluFunc.cpp:94-112).
 void fuse_residual_add(Program &p) {
   std::vector<Op *> convs;
@@ -96,31 +99,101 @@ void fuse_residual_add(Program &p) {
     if (add->kind != OP_ADD || add->coef != 1.f || add->dimA != add->dimB) continue;
     Value *z = add->operands[0] == conv->result ? add->operands[1] : add->operands[0];
     if (z == conv->result || z->shape != conv->result->shape) continue;
-    if (add->result->uses.size() != 1) continue;
-    Op *relu = add->result->uses.front().first;
-    if (relu->kind != OP_ACTIVATION || relu->mode != 1 || relu->operands[0] != add->result) continue;
-
-    Value *out = relu->operands[1];
+    // a ReLU that is the sum's only reader joins in; else the fused call stops at the sum
+    Op *relu = nullptr;
+    if (add->result->uses.size() == 1) {
+      Op *u = add->result->uses.front().first;
+      if (u->kind == OP_ACTIVATION && u->mode == 1 && u->operands[0] == add->result) relu = u;
+    }
+    Value *out = relu ? relu->operands[1] : add->operands[2];
     Op *fused = p.new_op(OP_CONV_BIAS_ADD_ACTIV);
     fused->pads = conv->pads;
     fused->strides = conv->strides;
     fused->group = conv->group;
     fused->dimA = conv->dimA;
     fused->dimB = conv->dimB;
-    fused->mode = 1;
+    fused->mode = relu ? 1 : 5;
     fused->result = p.new_value(out->dtype, out->shape);
     fused->result->def = fused;
-    // where the ReLU stood: Z and the ReLU's buffer both exist by then
-    p.insert_after(fused, relu);
+    // where the last fused operation stood: Z and the output buffer both exist by then
+    p.insert_after(fused, relu ? relu : add);
     p.set_operands(fused, {conv->operands[0], conv->operands[1], conv->operands[2], conv->operands[3], z, out});
-    p.replace_all_uses(relu->result, fused->result);
+    p.replace_all_uses(relu ? relu->result : add->result, fused->result);
     Value *conv_buf = conv->operands[4], *add_buf = add->operands[2];
-    p.erase(relu);
+    if (relu) p.erase(relu);
     p.erase(add);
     p.erase(conv);
-    drop_buffer(conv_buf);
+    if (conv_buf != out) drop_buffer(conv_buf);
+    if (!relu) continue;
     if (add_buf != conv_buf) drop_buffer(add_buf);
   }
+}
+
+// conv+bias (identity) -> Clip(0, c) | LeakyRelu(alpha) | PRelu(one constant
+// slope), the convolution's result read by nothing else, becomes one fused
+// call with activation mode 3 (clipped ReLU, ceiling c) or 6 (leaky ReLU,
+// slope alpha) writing the activation's buffer; the convolution's own buffer
+// disappears.  The reference has no such pattern (cuDNN's fused call knows
+// ReLU and identity only, CUDNNConvBiasReluFunc.cpp:60-71); MobileNetV2's
+// ReLU6, YOLO's LeakyRelu and SRGAN's shared-slope PRelu are its cases.
+static bool constant_scalar(const Program &p, const Value *dev, float &out) {
+  if (!dev->def || dev->def->kind != OP_MALLOC) return false;
+  for (const auto &u : dev->uses) {
+    const Op *cp = u.first;
+    if (cp->kind != OP_MEMCPY || cp->mode != 1 || u.second != 0) continue;
+    const Op *hc = cp->operands[1]->def;
+    if (!hc || hc->kind != OP_HOST_CONST) return false;
+    const GTensor &t = p.graph->tensors.at(hc->const_name);
+    if (shape_numel(t.shape) != 1 || t.dtype == I64) return false;
+    if (t.dtype == F32) { std::memcpy(&out, t.data.data(), 4); return true; }
+    uint16_t h;
+    std::memcpy(&h, t.data.data(), 2);
+    const int s = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+    const float v = e == 0 ? std::ldexp((float)m, -24) : e == 31 ? (m ? NAN : INFINITY) : std::ldexp((float)(m + 1024), e - 25);
+    out = s ? -v : v;
+    return true;
+  }
+  return false;
+}
+
+void fuse_conv_activations(Program &p) {
+  std::vector<Op *> convs;
+  for (Op *op : p.ops)
+    if (op->kind == OP_CONV_BIAS_ACTIV && op->mode == 5) convs.push_back(op);
+  for (Op *conv : convs) {
+    if (conv->result->uses.size() != 1) continue;
+    Op *act = conv->result->uses.front().first;
+    if (act->operands[0] != conv->result) continue;
+    int64_t mode;
+    float coef;
+    if (act->kind == OP_CLIP && act->lo == 0.f && act->hi > 0.f && act->hi < INFINITY) { mode = 3; coef = act->hi; }
+    else if (act->kind == OP_LEAKYRELU) { mode = 6; coef = act->alpha; }
+    else if (act->kind == OP_PRELU && constant_scalar(p, act->operands[1], coef)) mode = 6;
+    else continue;
+    Value *out = act->operands.back();
+    Op *fused = p.new_op(OP_CONV_BIAS_ACTIV);
+    fused->pads = conv->pads;
+    fused->strides = conv->strides;
+    fused->group = conv->group;
+    fused->dimA = conv->dimA;
+    fused->dimB = conv->dimB;
+    fused->mode = mode;
+    fused->coef = coef;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    p.insert_after(fused, act);  // the activation's buffer exists by then
+    p.set_operands(fused, {conv->operands[0], conv->operands[1], conv->operands[2], conv->operands[3], out});
+    p.replace_all_uses(act->result, fused->result);
+    Value *conv_buf = conv->operands[4];
+    p.erase(act);
+    p.erase(conv);
+    std::vector<Op *> deallocs;
+    for (const auto &u : conv_buf->uses)
+      if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+    for (Op *d : deallocs) p.erase(d);
+    if (conv_buf->uses.empty() && conv_buf->def) p.erase(conv_buf->def);
+  }
+  erase_dummy_constants(p);  // a PRelu slope that nothing reads any more
 }
 
 // Each dealloc (visited in block order, i.e. creation order of the parked

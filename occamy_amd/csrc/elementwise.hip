@@ -237,7 +237,13 @@ void *dnnrtActive(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int3
     case DNNRT_ACT_RELU: return unary_entry("dnnrtActive", handle, X, Y, dimX, 4, dtype, FRelu{});
     case DNNRT_ACT_SIGMOID: return unary_entry("dnnrtActive", handle, X, Y, dimX, 4, dtype, FSigmoid{});
     case DNNRT_ACT_TANH: return unary_entry("dnnrtActive", handle, X, Y, dimX, 4, dtype, FTanh{});
-    default: DNNRT_FAIL("dnnrtActive: mode %d (0 sigmoid, 1 relu, 2 tanh)", mode);
+    case DNNRT_ACT_CLIPPED_RELU:
+      if (!handle) DNNRT_FAIL("dnnrtActive: null handle");
+      return unary_entry("dnnrtActive", handle, X, Y, dimX, 4, dtype, FClip{0.f, handle->act_coef});
+    case DNNRT_ACT_LEAKY_RELU:
+      if (!handle) DNNRT_FAIL("dnnrtActive: null handle");
+      return unary_entry("dnnrtActive", handle, X, Y, dimX, 4, dtype, FLeaky{handle->act_coef});
+    default: DNNRT_FAIL("dnnrtActive: mode %d (0 sigmoid, 1 relu, 2 tanh, 3 clipped relu, 6 leaky relu)", mode);
   }
 }
 

@@ -19,7 +19,8 @@ struct IgemmArgs {
   const float *bias;  // per row m, may be null
   const float *Cin;   // same indexing as Y, scaled by beta, may be null
   float alpha, beta;
-  int act;            // DNNRT_ACT_RELU or DNNRT_ACT_IDENTITY
+  int act;            // DNNRT_ACT_{IDENTITY, RELU, CLIPPED_RELU, LEAKY_RELU}
+  float act_coef;     // ceiling / slope of the last two
   int M, Kdim, Ncols;
   // geometry of B: column -> (img, p, q); k -> (c, r, s)
   int H, W, R, S, P, Q, ph, pw, sh, sw;

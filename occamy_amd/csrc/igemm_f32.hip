@@ -250,7 +250,7 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
         const int m = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3);
         float v = a.alpha * acc[i][j][r] + bias_r[i][r];
         if (a.Cin) v += a.beta * res_r[r];
-        if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+        v = apply_act(v, a.act, a.act_coef);
         if (col_ok && m < a.M) Yg[ycol + (int64_t)m * a.y_row_stride] = v;
       }
     }

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
     const int mm = m0 + 8 * (r >> 2) + 4 * half + (r & 3);
     float v = a.alpha * acc[r] + bias_r[r];
     if (a.Cin) v += a.beta * res_r[r];
-    if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+    v = apply_act(v, a.act, a.act_coef);
     if (col_ok && mm < a.M) Yg[ycol + (int64_t)mm * a.y_row_stride] = v;
   }
 }

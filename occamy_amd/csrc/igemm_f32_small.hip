@@ -120,7 +120,7 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     if (mm >= a.M) continue;
     float v = a.alpha * acc[r] + bias_r[r];
     if (a.Cin) v += a.beta * res_r[r];
-    if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+    v = apply_act(v, a.act, a.act_coef);
     Yg[ycol + (int64_t)mm * a.y_row_stride] = v;
   }
 }

@@ -48,6 +48,10 @@ class Ops:
     def set_format(self, fmt):
         self._check(self.lib.dnnrtSetTensorFormat(self.handle, fmt), "dnnrtSetTensorFormat")
 
+    def set_activation_coef(self, coef):
+        """Ceiling of ACT_CLIPPED_RELU / slope of ACT_LEAKY_RELU for the calls that follow."""
+        self._check(self.lib.dnnrtSetActivationCoef(self.handle, coef), "dnnrtSetActivationCoef")
+
     def set_filter_layout(self, layout):
         self._check(self.lib.dnnrtSetFilterLayout(self.handle, layout), "dnnrtSetFilterLayout")
 

@@ -129,7 +129,7 @@ static int bad_dtype(int32_t dtype) { return dtype != DNNRT_F32 && dtype != DNNR
 
 /* ---- handle / stream / memory: host stand-ins -------------------------- */
 
-struct dnnrtContext { int format; };
+struct dnnrtContext { int format; float act_coef; };
 
 int32_t dnnrtCreate(dnnrtHandle_t *h) {
   *h = (dnnrtHandle_t)calloc(1, sizeof(struct dnnrtContext));
@@ -153,6 +153,11 @@ int32_t dnnrtSetFilterLayout(dnnrtHandle_t h, int32_t layout) {
     snprintf(g_err, sizeof g_err, "oracle: only K,C,R,S filters are implemented");
     return 1;
   }
+  return 0;
+}
+int32_t dnnrtSetActivationCoef(dnnrtHandle_t h, float coef) {
+  if (!h || coef != coef) { snprintf(g_err, sizeof g_err, "setActivationCoef: bad argument"); return 1; }
+  h->act_coef = coef;
   return 0;
 }
 int32_t dnnrtSync(dnnrtHandle_t h) { (void)h; return 0; }
@@ -205,9 +210,11 @@ int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind, dnnrtStre
  *                            * W[k, c, r, s],        g = k / (K/group)
  * with out-of-range taps contributing 0.  CUDNNConvBiasReluFunc.cpp:8-140
  * adds B[k] and applies ReLU (mode 1) or identity (mode 5). */
-static float act_apply(float v, int64_t mode) {
+static float act_apply(float v, int64_t mode, float coef) {
   switch (mode) {
   case DNNRT_ACT_RELU: return v < 0.0f ? 0.0f : v; /* NaN passes through */
+  case DNNRT_ACT_CLIPPED_RELU: v = v < 0.0f ? 0.0f : v; return v > coef ? coef : v;
+  case DNNRT_ACT_LEAKY_RELU: return v < 0.0f ? coef * v : v;
   case DNNRT_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
   case DNNRT_ACT_TANH: return tanhf(v);
   default: return v;
@@ -249,7 +256,7 @@ static void conv_core(const float *X, const int64_t *dX, const float *Wt,
       }
       float *y = Y + (n * K + k) * P * Q;
       const double b = B ? (double)B[k] : 0.0;
-      for (int64_t i = 0; i < P * Q; i++) y[i] = act_apply((float)(acc[i] + b), act);
+      for (int64_t i = 0; i < P * Q; i++) y[i] = act_apply((float)(acc[i] + b), act, 0.0f);
       free(acc);
     }
 }
@@ -290,10 +297,20 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
                          int64_t algo, int64_t group, const int64_t *pads,
                          const int64_t *strides, int64_t act, void *Y,
                          int32_t dtype) {
-  (void)h; (void)ws; (void)wsBytes; (void)algo;
+  (void)ws; (void)wsBytes; (void)algo;
+  if (numel(dB, 4) != dW[0]) FAIL("convBiasActiv: bias must hold K values");
+  if (act == DNNRT_ACT_CLIPPED_RELU || act == DNNRT_ACT_LEAKY_RELU) {
+    /* the reference has no such fused call: it runs conv+bias (identity) and
+     * then CUDAClipFunc.cu / CUDALeakyReluFunc.cu on the stored tensor */
+    if (!conv_entry(X, dX, W, dW, B, group, pads, strides, DNNRT_ACT_IDENTITY, Y, dtype)) return NULL;
+    const int64_t P = (dX[2] + 2 * pads[0] - dW[2]) / strides[0] + 1,
+                  Q = (dX[3] + 2 * pads[1] - dW[3]) / strides[1] + 1;
+    const int64_t dY[4] = {dX[0], dW[0], P, Q};
+    return act == DNNRT_ACT_CLIPPED_RELU ? dnnrtClip(h, Y, Y, dY, 0.f, h->act_coef, 4, dtype)
+                                         : dnnrtLeakyRelu(h, Y, Y, dY, h->act_coef, 4, dtype);
+  }
   if (act != DNNRT_ACT_RELU && act != DNNRT_ACT_IDENTITY)
     FAIL("convBiasActiv: activMode %ld", (long)act);
-  if (numel(dB, 4) != dW[0]) FAIL("convBiasActiv: bias must hold K values");
   return conv_entry(X, dX, W, dW, B, group, pads, strides, act, Y, dtype);
 }
 /* No reference wrapper of its own: the reference runs this as three calls,
@@ -306,8 +323,8 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
                             int64_t wsBytes, int64_t algo, int64_t group,
                             const int64_t *pads, const int64_t *strides,
                             int64_t act, void *Y, int32_t dtype) {
-  (void)h; (void)ws; (void)wsBytes; (void)algo;
-  if (act != DNNRT_ACT_RELU && act != DNNRT_ACT_IDENTITY)
+  (void)ws; (void)wsBytes; (void)algo;
+  if (act != DNNRT_ACT_RELU && act != DNNRT_ACT_IDENTITY && act != DNNRT_ACT_CLIPPED_RELU && act != DNNRT_ACT_LEAKY_RELU)
     FAIL("convBiasAddActiv: activMode %ld", (long)act);
   if (numel(dB, 4) != dW[0]) FAIL("convBiasAddActiv: bias must hold K values");
   if (!Z) FAIL("convBiasAddActiv: null residual tensor");
@@ -322,7 +339,7 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
   float *o = outbuf(Y, ny, dtype, &to);
   /* rounding to the tensor's type commutes with ReLU, so one narrow() at the
    * end stands for the add's and the activation's stores */
-  for (int64_t i = 0; i < ny; i++) o[i] = act_apply(y[i] + z[i], act);
+  for (int64_t i = 0; i < ny; i++) o[i] = act_apply(y[i] + z[i], act, h->act_coef);
   narrow(Y, to, ny, dtype);
   free(ty); free(tz);
   return Y;
@@ -333,15 +350,15 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
 /* CUDNNActiveFunc.cpp:8-91: cudnnActivationForward, alpha 1 beta 0. */
 void *dnnrtActive(dnnrtHandle_t h, const void *X, const int64_t *dX, int32_t mode,
                   void *Y, int32_t dtype) {
-  (void)h;
   if (bad_dtype(dtype)) FAIL("active: bad dtype");
-  if (mode != DNNRT_ACT_RELU && mode != DNNRT_ACT_SIGMOID && mode != DNNRT_ACT_TANH)
+  if (mode != DNNRT_ACT_RELU && mode != DNNRT_ACT_SIGMOID && mode != DNNRT_ACT_TANH &&
+      mode != DNNRT_ACT_CLIPPED_RELU && mode != DNNRT_ACT_LEAKY_RELU)
     FAIL("active: mode %d", mode);
   const int64_t n = numel(dX, 4);
   float *tx, *ty;
   const float *x = widen(X, n, dtype, &tx);
   float *y = outbuf(Y, n, dtype, &ty);
-  for (int64_t i = 0; i < n; i++) y[i] = act_apply(x[i], mode);
+  for (int64_t i = 0; i < n; i++) y[i] = act_apply(x[i], mode, h->act_coef);
   narrow(Y, ty, n, dtype); free(tx);
   return Y;
 }

@@ -12,9 +12,10 @@ def conv_out_hw(H, W, R, S, pads, strides):
     return (H + 2 * pads[0] - R) // strides[0] + 1, (W + 2 * pads[1] - S) // strides[1] + 1
 
 
-def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crsk=False, z=None):
+def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crsk=False, z=None, coef=None):
     """crsk: hand the filter over stored C,R,S,K (the dims stay logical K,C,R,S).
-    z: residual tensor shaped like the result (needs b): act((conv + b) + z)."""
+    z: residual tensor shaped like the result (needs b): act((conv + b) + z).
+    coef: the handle's activation coefficient (ceiling of ACT_CLIPPED_RELU, slope of ACT_LEAKY_RELU)."""
     N, C, H, W = x.shape
     K, Cg, R, S = w.shape
     P, Q = conv_out_hw(H, W, R, S, pads, strides)
@@ -24,6 +25,8 @@ def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crs
     Y = be.empty((N, K, max(P, 1), max(Q, 1)), x.dtype)  # the call rejects empty outputs itself
     if crsk:
         be.ops.set_filter_layout(_abi.FILTER_CRSK)
+    if coef is not None:
+        be.ops.set_activation_coef(coef)
     try:
         if b is None:
             assert activ is None

@@ -132,6 +132,25 @@ def test_batchnorm_folds_into_the_convolution_before_it():
     assert ops.count("dnn.conv-bias-relufwd") == n_conv and "dnn.convfwd" not in ops
 
 
+def test_activation_fusion_flag():
+    count = lambda p: {n: [m for m, *_ in p.compute_ops()].count(n) for n in  # noqa: E731
+                       ("dnn.clip", "dnn.leakyrelu", "dnn.prelu", "dnn.add", "dnn.conv-bias-relufwd", "dnn.conv-bias-add-relufwd")}
+    flags = dict(fusion=True, fuse_activations=True, fuse_residual=True)
+    g, _ = models.mobilenet_v2(**SMALL)
+    c = count(check_lifetimes(lambda: models.mobilenet_v2(**SMALL), **flags))
+    # every ReLU6 and every residual sum is gone; the one add left is the classifier's bias
+    assert c["dnn.clip"] == 0 and c["dnn.add"] == 1 and c["dnn.conv-bias-add-relufwd"] == 10 and c["dnn.conv-bias-relufwd"] == 42
+    p = g.compile(**flags)
+    assert "activMode=3, activCoef=6" in p.text
+    c = count(check_lifetimes(lambda: models.yolo_v1(batch=1, image=64, width=0.0625, fc=32), **flags))
+    assert c["dnn.leakyrelu"] == 1 and c["dnn.conv-bias-relufwd"] == 24            # the one left follows a Gemm
+    c = count(check_lifetimes(lambda: models.srgan_generator(height=8, width=6, feats=16, blocks=2), **flags))
+    assert c["dnn.prelu"] == 2 and c["dnn.add"] == 0 and c["dnn.conv-bias-add-relufwd"] == 3   # two PRelu follow a pixel shuffle
+    # without `fusion` the flag does nothing
+    g, _ = models.mobilenet_v2(**SMALL)
+    assert count(g.compile(fuse_activations=True))["dnn.clip"] == 35
+
+
 def planned_vs_oracle(p):
     ev = p.events()
     off, peak = oracle_plan([(k, i, b) for k, i, b, _ in ev])

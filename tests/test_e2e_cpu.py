@@ -172,6 +172,22 @@ def test_widened_operator_surface():
     assert text.count("dnn.prelu") == 2 and text.count("dnn.leakyrelu") == 1
 
 
+@pytest.mark.parametrize("builder", [lambda: models.mobilenet_v2(image=32, classes=10), YOLO, SRGAN,
+                                     lambda: models.resnet50(image=32, classes=10)],
+                         ids=["mobilenet_v2", "yolo_v1", "srgan", "resnet50"])
+def test_activation_fusion_matches_unfused_chain(builder):
+    # The oracle runs a fused conv + clipped / leaky ReLU as the reference's
+    # separate calls, so the flags must not change a single bit on the CPU.
+    _, _, a = run_oracle(builder, fusion=True)
+    _, _, b = run_oracle(builder, fusion=True, fuse_activations=True, fuse_residual=True)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+    check(builder, fusion=True, fuse_activations=True, fuse_residual=True)
+    _, _, c = run_oracle(builder, mode=compiler.MODE_RESIDENT, fusion=True, fuse_activations=True, fuse_residual=True)
+    for x, y in zip(a, c):
+        np.testing.assert_array_equal(x, y)
+
+
 def test_executor_errors():
     g, inputs = models.single_conv()
     p = g.compile(pool_opt=False)

@@ -158,6 +158,16 @@ def test_residual_fusion_fp16_channels_last():
                                atol=2e-2 * float(np.abs(chain[0].astype(np.float32)).max()))
 
 
+@pytest.mark.parametrize("name", ["mobilenet_v2", "yolo_v1", "srgan"])
+def test_activation_fusion_fp32(name, oracle_outputs):
+    out, _ = run(CONFIGS[name], fusion=True, fuse_residual=True, fuse_activations=True)
+    for o, r in zip(out, oracle_outputs[name]):
+        close(o, r)
+    out, _ = run(CONFIGS[name], mode=compiler.MODE_RESIDENT, fusion=True, fuse_residual=True, fuse_activations=True)
+    for o, r in zip(out, oracle_outputs[name]):
+        close(o, r)
+
+
 def test_model_from_an_onnx_file_runs_like_the_built_graph(tmp_path):
     """ResNet-50 through a file: ONNX bytes -> reader -> compiler -> gfx950."""
     import onnx_writer

@@ -271,6 +271,37 @@ def test_data_movement(gpu, cpu):
         oc.transpose(gpu, x, (0, 1, 1, 3))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_conv_clipped_and_leaky_relu(gpu, cpu, dtype):
+    r = rng(43)
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == np.float32 else dict(rtol=2e-2, atol=2e-3)
+    # dense 3x3 and 1x1 (the MFMA kernels), a depthwise 3x3, and a product large enough for the LDS-tiled kernel
+    for (N, C, H, K, R, st, pd, grp) in [(1, 64, 14, 64, 3, 1, 1, 1), (2, 32, 9, 48, 1, 1, 0, 1), (1, 32, 12, 32, 3, 2, 1, 32),
+                                          (4, 64, 28, 128, 3, 1, 1, 1)]:
+        if dtype == np.float16 and grp != 1:
+            continue
+        x = r.standard_normal((N, C, H, H)).astype(dtype)
+        w = (r.standard_normal((K, C // grp, R, R)) * (0.5 / np.sqrt(C // grp * R * R))).astype(dtype)
+        b = r.standard_normal(K).astype(dtype)
+        P = (H + 2 * pd - R) // st + 1
+        z = r.standard_normal((N, K, P, P)).astype(dtype)
+        for activ, coef in [(_abi.ACT_CLIPPED_RELU, 0.75), (_abi.ACT_LEAKY_RELU, 0.1)]:
+            for zz in (None, z):
+                got = oc.conv(gpu, x, w, b, (pd, pd), (st, st), grp, activ, z=zz, coef=coef)
+                ref = oc.conv(cpu, x, w, b, (pd, pd), (st, st), grp, activ, z=zz, coef=coef)
+                np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), **tol)
+                if activ == _abi.ACT_CLIPPED_RELU:
+                    assert got.max() <= 0.75 and got.min() >= 0
+    x = r.standard_normal((3, 5, 7, 2)).astype(dtype)
+    X, Y = gpu.put(x), gpu.empty(x.shape, x.dtype)
+    gpu.ops.set_activation_coef(0.25)
+    gpu.ops.active(gpu.ptr(X), x.shape, _abi.ACT_LEAKY_RELU, gpu.ptr(Y), oc.DT[np.dtype(dtype)])
+    gpu.sync()
+    np.testing.assert_array_equal(gpu.get(Y), oc.leaky_relu(cpu, x, 0.25))
+    with pytest.raises(RuntimeError):
+        oc.conv(gpu, x, np.zeros((4, 5, 1, 1), dtype), np.zeros(4, dtype), activ=4)
+
+
 def test_leaky_relu_prelu(gpu, cpu):
     r = rng(41)
     for dtype in (np.float32, np.float16):

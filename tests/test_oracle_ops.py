@@ -341,6 +341,36 @@ def test_data_movement(be):
         oc.gather(be, table, np.array([11]), 0)
 
 
+def test_conv_with_clipped_and_leaky_relu(be):
+    # modes 3 and 6 of the fused call against torch's operators applied to torch's convolution
+    r = rng(33)
+    x = r.standard_normal((2, 6, 9, 9)).astype(np.float32)
+    w = (r.standard_normal((8, 6, 3, 3)) * 0.5).astype(np.float32)
+    b = r.standard_normal(8).astype(np.float32)
+    z = r.standard_normal((2, 8, 9, 9)).astype(np.float32)
+    y = F.conv2d(t64(x), t64(w), t64(b), padding=1)
+    got = oc.conv(be, x, w, b, pads=(1, 1), activ=_abi.ACT_CLIPPED_RELU, coef=1.5)
+    np.testing.assert_allclose(got, torch.clamp(y, 0, 1.5).numpy(), rtol=1e-5, atol=1e-5)
+    assert got.max() == 1.5 and got.min() == 0.0            # both bounds bite on this input
+    got = oc.conv(be, x, w, b, pads=(1, 1), activ=_abi.ACT_LEAKY_RELU, coef=0.1)
+    np.testing.assert_allclose(got, F.leaky_relu(y, 0.1).numpy(), rtol=1e-5, atol=1e-5)
+    got = oc.conv(be, x, w, b, pads=(1, 1), activ=_abi.ACT_LEAKY_RELU, coef=0.1, z=z)
+    np.testing.assert_allclose(got, F.leaky_relu(y + t64(z), 0.1).numpy(), rtol=1e-5, atol=1e-5)
+    got = oc.conv(be, x, w, b, pads=(1, 1), activ=_abi.ACT_CLIPPED_RELU, coef=6.0, z=z)
+    np.testing.assert_allclose(got, torch.clamp(y + t64(z), 0, 6).numpy(), rtol=1e-5, atol=1e-5)
+    # the coefficient is sticky and does not touch ReLU
+    np.testing.assert_allclose(oc.conv(be, x, w, b, pads=(1, 1), activ=_abi.ACT_RELU), F.relu(y).numpy(), rtol=1e-5, atol=1e-5)
+    # the same through the stand-alone activation call
+    X, Y = be.put(x), be.empty(x.shape, x.dtype)
+    be.ops.set_activation_coef(0.25)
+    be.ops.active(be.ptr(X), x.shape, _abi.ACT_LEAKY_RELU, be.ptr(Y), _abi.F32)
+    np.testing.assert_array_equal(be.get(Y), np.where(x < 0, np.float32(0.25) * x, x))
+    be.ops.active(be.ptr(X), x.shape, _abi.ACT_CLIPPED_RELU, be.ptr(Y), _abi.F32)
+    np.testing.assert_array_equal(be.get(Y), np.clip(x, 0, 0.25))
+    with pytest.raises(RuntimeError):
+        oc.conv(be, x, w, b, pads=(1, 1), activ=4)             # ELU: not a mode of this runtime
+
+
 def test_leaky_relu_and_prelu(be):
     # pinned by the defining formula on hand-picked values and by torch's operators
     x = np.array([-2.0, -0.5, 0.0, 0.5, 3.0], np.float32)
