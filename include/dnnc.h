@@ -58,6 +58,10 @@ typedef struct {
                              closing a residual block becomes one call (default 0) */
   int32_t fuse_activations; /* no reference flag: with `fusion`, conv+bias -> Clip(0, c) /
                              LeakyRelu / one-slope PRelu becomes one call (default 0) */
+  int32_t recompose;      /* no reference flag: LayerNormalization and Gelu written out in
+                             primitive operators become one call each (default 0) */
+  int32_t fuse_matmul_bias; /* no reference flag: with `fusion`, MatMul -> Add(bias row)
+                             becomes one call (default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);

@@ -295,6 +295,14 @@ void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
                     int32_t rankA, const void *B, const int64_t *dimB,
                     int32_t rankB, void *Y, const int64_t *dimY, int32_t rankY,
                     int32_t dtype);
+/* The same with one row of N values added to every row of every product:
+ * Y = A B + bias.  No reference wrapper: the reference runs CUDAMatmulNdFunc
+ * and then cudnnAddTensor with the bias broadcast (Ops/cudnn/Add.cpp), which
+ * is what a transformer's Linear layers lower to.  fp32 only. */
+void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
+                        int32_t rankA, const void *B, const int64_t *dimB,
+                        int32_t rankB, const void *bias, void *Y,
+                        const int64_t *dimY, int32_t rankY, int32_t dtype);
 
 /* ---- data movement --------------------------------------------------- */
 

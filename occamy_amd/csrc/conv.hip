@@ -124,6 +124,7 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
   a.a_ld = s.K;
   a.x_z_stride = (int64_t)s.Cg * s.H * s.W;
   a.y_z_stride = (int64_t)Kg * s.P * s.Q;
+  a.c_row_stride = a.y_row_stride; a.c_z_stride = a.y_z_stride;  // the residual is laid out like Y
   a.bias_z_stride = Kg;
   a.b_kcontig = false; a.a_mcontig = crsk;
   a.a_vec4 = !crsk && (a.Kdim % 4 == 0) && aligned16(Wt);

@@ -121,7 +121,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (!g || !opt) { g_err = "dnncCompile: bad arguments"; return nullptr; }
   if (g->compiled) { g_err = "dnncCompile: a graph can be compiled once"; return nullptr; }
   std::string err;
-  if (!infer_shapes(g->g, err)) { g_err = err; return nullptr; }
+  if (!infer_shapes(g->g, opt->recompose != 0, err)) { g_err = err; return nullptr; }
   if (opt->const_at_use) constant_at_use(g->g);
   g->compiled = true;
   dnncProgram *pp = new dnncProgram();
@@ -131,6 +131,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   erase_dummy_constants(p);
   if (opt->fusion) fuse_conv_bias_activ(p);
   if (opt->fusion && opt->fuse_activations) fuse_conv_activations(p);
+  if (opt->fusion && opt->fuse_matmul_bias) fuse_matmul_bias(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {

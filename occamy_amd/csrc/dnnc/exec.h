@@ -60,6 +60,7 @@ struct RuntimeApi {
   decltype(&::dnnrtTranspose) dnnrtTranspose = nullptr;
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
   decltype(&::dnnrtSetActivationCoef) dnnrtSetActivationCoef = nullptr;
+  decltype(&::dnnrtMatmulNdBias) dnnrtMatmulNdBias = nullptr;
   decltype(&::dnnrtLeakyRelu) dnnrtLeakyRelu = nullptr;
   decltype(&::dnnrtPRelu) dnnrtPRelu = nullptr;
   decltype(&::dnnrtConcat) dnnrtConcat = nullptr;

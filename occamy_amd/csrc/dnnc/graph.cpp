@@ -198,6 +198,185 @@ static bool rewrite_batchnorm(Graph &g, size_t at, std::string &err) {
   return true;
 }
 
+// ---- recomposition of LayerNormalization and Gelu from the primitive
+// operators exporters write them as (what onnx-mlir's recompose patterns do
+// at the ONNX level; the DNN dialect of the reference never sees the fused
+// forms, so this runs only when asked for).  Shapes are known.
+namespace {
+struct Matcher {
+  Graph &g;
+  std::map<std::string, size_t> producer;
+  explicit Matcher(Graph &g_) : g(g_) {
+    for (size_t i = 0; i < g.nodes.size(); i++) producer[g.nodes[i].output] = i;
+  }
+  const GNode *def(const std::string &name, const char *op) const {
+    auto it = producer.find(name);
+    if (it == producer.end() || g.nodes[it->second].op_type != op) return nullptr;
+    return &g.nodes[it->second];
+  }
+  bool scalar(const std::string &name, double &v) const {
+    auto it = g.tensors.find(name);
+    if (it == g.tensors.end() || !it->second.is_const || it->second.dtype == I64 || shape_numel(it->second.shape) != 1) return false;
+    v = load_elem(it->second, 0);
+    return true;
+  }
+  bool single_use(const std::string &name) const { return count_uses(g, name) == 1; }
+  // n is a binary node with one operand produced by `op` and the other anything: returns the pair
+  bool split(const GNode &n, const char *op, const GNode *&inner, std::string &other) const {
+    if (n.inputs.size() != 2) return false;
+    for (int k = 0; k < 2; k++)
+      if ((inner = def(n.inputs[(size_t)k], op)) != nullptr) { other = n.inputs[(size_t)(1 - k)]; return true; }
+    return false;
+  }
+  bool last_axis_mean(const GNode &n) const {
+    auto ax = n.ints.find("axes");
+    auto kd = n.ints.find("keepdims");
+    if (ax == n.ints.end() || ax->second.size() != 1 || n.inputs.empty()) return false;
+    if (kd != n.ints.end() && !kd->second.empty() && kd->second[0] != 1) return false;
+    const int64_t rank = (int64_t)g.tensors.at(n.inputs[0]).shape.size();
+    return ax->second[0] == -1 || ax->second[0] == rank - 1;
+  }
+};
+}  // namespace
+
+// out = Add(Mul(Div(d, Sqrt(Add(ReduceMean(Pow(d, 2)), eps))), gamma), beta), d = Sub(x, ReduceMean(x))
+static bool match_layernorm(const Matcher &m, const GNode &root, GNode &fused, std::vector<std::string> &dead) {
+  if (root.op_type != "Add") return false;
+  const GNode *mul, *div, *sub, *sqrt_, *add_eps, *mean2, *pow_, *mean1;
+  std::string beta, gamma, eps_name, two_name;
+  if (!m.split(root, "Mul", mul, beta) || !m.split(*mul, "Div", div, gamma)) return false;
+  if (div->inputs.size() != 2 || !(sub = m.def(div->inputs[0], "Sub")) || !(sqrt_ = m.def(div->inputs[1], "Sqrt"))) return false;
+  if (!(add_eps = m.def(sqrt_->inputs[0], "Add")) || !m.split(*add_eps, "ReduceMean", mean2, eps_name)) return false;
+  if (!(pow_ = m.def(mean2->inputs[0], "Pow")) || pow_->inputs.size() != 2 || pow_->inputs[0] != sub->output) return false;
+  two_name = pow_->inputs[1];
+  if (sub->inputs.size() != 2 || !(mean1 = m.def(sub->inputs[1], "ReduceMean")) || mean1->inputs[0] != sub->inputs[0]) return false;
+  double eps, two;
+  if (!m.scalar(eps_name, eps) || !m.scalar(two_name, two) || two != 2.0 || !(eps > 0.0)) return false;
+  if (!m.last_axis_mean(*mean1) || !m.last_axis_mean(*mean2)) return false;
+  const GTensor &x = m.g.tensors.at(sub->inputs[0]);
+  auto vec_const = [&](const std::string &n) {
+    auto it = m.g.tensors.find(n);
+    return it != m.g.tensors.end() && it->second.is_const && it->second.dtype == x.dtype &&
+           shape_numel(it->second.shape) == x.shape.back() && !it->second.shape.empty() && it->second.shape.back() == x.shape.back();
+  };
+  if (x.shape.empty() || !vec_const(gamma) || !vec_const(beta)) return false;
+  // nothing else may read the intermediates
+  if (!m.single_use(mean1->output) || m.g.tensors.count(sub->output) == 0 || count_uses(m.g, sub->output) != 2) return false;
+  for (const GNode *n : {pow_, mean2, add_eps, sqrt_, div, mul})
+    if (!m.single_use(n->output)) return false;
+  fused = GNode();
+  fused.op_type = "LayerNormalization";
+  fused.inputs = {sub->inputs[0], gamma, beta};
+  fused.output = root.output;
+  fused.ints["axis"] = {-1};
+  fused.floats["epsilon"] = eps;
+  dead = {mean1->output, sub->output, pow_->output, mean2->output, add_eps->output, sqrt_->output, div->output, mul->output};
+  return true;
+}
+
+// out = Mul(Mul(x, Add(Erf(Div(x, sqrt 2)), 1)), 0.5)
+static bool match_gelu(const Matcher &m, const GNode &root, GNode &fused, std::vector<std::string> &dead) {
+  if (root.op_type != "Mul") return false;
+  const GNode *inner, *add1, *erf, *div;
+  std::string half_name, x, one_name;
+  double half, one, c;
+  if (!m.split(root, "Mul", inner, half_name) || !m.scalar(half_name, half) || half != 0.5) return false;
+  if (inner->inputs.size() != 2) return false;
+  bool ok = false;
+  for (int k = 0; k < 2 && !ok; k++) {  // x itself may come from an Add: try both operand orders
+    x = inner->inputs[(size_t)(1 - k)];
+    if (!(add1 = m.def(inner->inputs[(size_t)k], "Add"))) continue;
+    if (!m.split(*add1, "Erf", erf, one_name) || !m.scalar(one_name, one) || one != 1.0) continue;
+    if (!(div = m.def(erf->inputs[0], "Div")) || div->inputs.size() != 2 || div->inputs[0] != x) continue;
+    if (!m.scalar(div->inputs[1], c) || std::fabs(c - 1.4142135623730951) > 1e-3) continue;
+    ok = true;
+  }
+  if (!ok) return false;
+  for (const GNode *n : {div, erf, add1, inner})
+    if (!m.single_use(n->output)) return false;
+  fused = GNode();
+  fused.op_type = "Gelu";
+  fused.inputs = {x};
+  fused.output = root.output;
+  dead = {div->output, erf->output, add1->output, inner->output};
+  return true;
+}
+
+// Div(x, c) with a one-element constant c becomes Mul(x, 1/c): the reference
+// lowers Div to reciprocal + mul (Ops/cudnn/Div.cpp), so only the reciprocal
+// moves from run time to compile time (1.0f / c in the tensor's type, as the
+// device computes it).
+static bool fold_constant_divisors(Graph &g) {
+  bool any = false;
+  for (size_t i = 0; i < g.nodes.size(); i++) {
+    GNode &n = g.nodes[i];
+    if (n.op_type != "Div" || n.inputs.size() != 2) continue;
+    auto it = g.tensors.find(n.inputs[1]);
+    if (it == g.tensors.end() || !it->second.is_const || it->second.dtype == I64 || shape_numel(it->second.shape) != 1) continue;
+    const std::string name = n.output + "_recip", old = n.inputs[1];
+    if (g.tensors.count(name)) continue;
+    GTensor r = it->second;
+    r.name = name;
+    store_elem(r, 0, (double)(1.0f / (float)load_elem(it->second, 0)));
+    g.tensors[name] = r;
+    n.op_type = "Mul";
+    n.inputs[1] = name;
+    GNode cn;
+    cn.op_type = "Constant";
+    cn.output = name;
+    g.nodes.insert(g.nodes.begin() + (long)i, cn);
+    i++;
+    if (count_uses(g, old) == 0) {
+      for (size_t j = 0; j < g.nodes.size(); j++)
+        if (g.nodes[j].op_type == "Constant" && g.nodes[j].output == old) {
+          g.nodes.erase(g.nodes.begin() + (long)j);
+          if (j < i) i--;
+          break;
+        }
+      g.tensors.erase(old);
+    }
+    any = true;
+  }
+  return any;
+}
+
+static bool recompose(Graph &g) {
+  bool any = false;
+  for (size_t i = 0; i < g.nodes.size(); i++) {
+    Matcher m(g);
+    GNode fused;
+    std::vector<std::string> dead;
+    if (!match_layernorm(m, g.nodes[i], fused, dead) && !match_gelu(m, g.nodes[i], fused, dead)) continue;
+    // constants read by the matched nodes only go with them
+    std::vector<std::string> consts;
+    for (const std::string &d : dead)
+      for (const std::string &in : g.nodes[m.producer.at(d)].inputs) {
+        auto t = g.tensors.find(in);
+        if (t != g.tensors.end() && t->second.is_const) consts.push_back(in);
+      }
+    for (const std::string &in : g.nodes[i].inputs) {
+      auto t = g.tensors.find(in);
+      if (t != g.tensors.end() && t->second.is_const) consts.push_back(in);
+    }
+    g.nodes[i] = fused;
+    std::vector<GNode> kept;
+    for (GNode &n : g.nodes)
+      if (std::find(dead.begin(), dead.end(), n.output) == dead.end()) kept.push_back(n);
+    g.nodes.swap(kept);
+    for (const std::string &d : dead) g.tensors.erase(d);
+    for (const std::string &c : consts) {
+      if (!g.tensors.count(c) || count_uses(g, c) != 0) continue;
+      for (size_t j = 0; j < g.nodes.size(); j++)
+        if (g.nodes[j].op_type == "Constant" && g.nodes[j].output == c) { g.nodes.erase(g.nodes.begin() + (long)j); break; }
+      g.tensors.erase(c);
+    }
+    any = true;
+    i = (size_t)-1;  // positions moved: rescan
+  }
+  // after the matchers: Gelu's own Div by sqrt(2) must still be there for them
+  return fold_constant_divisors(g) || any;
+}
+
 static bool infer_pass(Graph &g, std::string &err) {
   for (GNode &n : g.nodes) {
     if (n.op_type == "Constant") continue;
@@ -392,10 +571,10 @@ static bool infer_pass(Graph &g, std::string &err) {
   return true;
 }
 
-bool infer_shapes(Graph &g, std::string &err) {
+bool infer_shapes(Graph &g, bool recompose_norms, std::string &err) {
   forward_aliases(g);
   if (!infer_pass(g, err)) return false;
-  bool rewritten = false;
+  bool rewritten = recompose_norms && recompose(g);
   for (size_t i = 0; i < g.nodes.size();) {
     if (g.nodes[i].op_type != "BatchNormalization") { i++; continue; }
     if (!rewrite_batchnorm(g, i, err)) return false;

@@ -45,6 +45,7 @@ const char *op_name(OpKind k) {
     case OP_LAYERNORM: return "dnn.layernorm";
     case OP_GELU: return "dnn.gelu";
     case OP_CONV_BIAS_ADD_ACTIV: return "dnn.conv-bias-add-relufwd";
+    case OP_MATMUL_BIAS: return "dnn.matmulnd-bias";
     case OP_RETURN: return "return";
   }
   return "?";

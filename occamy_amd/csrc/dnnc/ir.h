@@ -65,6 +65,7 @@ enum OpKind {
   // fused operators that have no counterpart in DNN.td
   OP_LAYERNORM, OP_GELU,
   OP_CONV_BIAS_ADD_ACTIV,  // conv + bias + residual tensor + activation (cuDNN's z operand)
+  OP_MATMUL_BIAS,          // batched matrix product + one row added to every row
   OP_RETURN
 };
 const char *op_name(OpKind k);
@@ -148,7 +149,7 @@ struct CompileOptions {
 };
 
 // graph.cpp
-bool infer_shapes(Graph &g, std::string &err);
+bool infer_shapes(Graph &g, bool recompose_norms, std::string &err);
 void constant_at_use(Graph &g);
 // emit.cpp
 bool emit_program(const Graph &g, Program &p, std::string &err);
@@ -163,6 +164,7 @@ bool graph_from_onnx(const uint8_t *data, size_t nbytes, Graph &g, std::string &
 void fuse_conv_bias_activ(Program &p);
 void fuse_residual_add(Program &p);
 void fuse_conv_activations(Program &p);
+void fuse_matmul_bias(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);
 bool malloc_pool_opt(Program &p, std::string &err);

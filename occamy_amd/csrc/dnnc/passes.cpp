@@ -196,6 +196,43 @@ void fuse_conv_activations(Program &p) {
   erase_dummy_constants(p);  // a PRelu slope that nothing reads any more
 }
 
+// matmulnd -> add(one row of N values), the product read by nothing else,
+// becomes one matmulnd-bias writing the sum's buffer: the Linear layers of a
+// transformer as exporters write them (MatMul, then Add of the bias).  No
+// counterpart in the reference.
+void fuse_matmul_bias(Program &p) {
+  std::vector<Op *> mms;
+  for (Op *op : p.ops)
+    if (op->kind == OP_MATMULND) mms.push_back(op);
+  for (Op *mm : mms) {
+    if (mm->result->dtype != F32 || mm->result->uses.size() != 1) continue;
+    Op *add = mm->result->uses.front().first;
+    if (add->kind != OP_ADD || add->coef != 1.f || add->operands[0] != mm->result) continue;
+    bool row = !add->dimB.empty() && add->dimB.back() == mm->dimOut.back();
+    for (size_t i = 0; i + 1 < add->dimB.size(); i++) row = row && add->dimB[i] == 1;
+    if (!row) continue;
+    Value *out = add->operands[2], *buf = mm->operands[2];
+    Op *fused = p.new_op(OP_MATMUL_BIAS);
+    fused->dimA = mm->dimA;
+    fused->dimB = mm->dimB;
+    fused->dimOut = mm->dimOut;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    p.insert_after(fused, add);
+    p.set_operands(fused, {mm->operands[0], mm->operands[1], add->operands[1], out});
+    p.replace_all_uses(add->result, fused->result);
+    p.erase(add);
+    p.erase(mm);
+    if (buf != out) {
+      std::vector<Op *> deallocs;
+      for (const auto &u : buf->uses)
+        if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+      for (Op *d : deallocs) p.erase(d);
+      if (buf->uses.empty() && buf->def) p.erase(buf->def);
+    }
+  }
+}
+
 // Each dealloc (visited in block order, i.e. creation order of the parked
 // deallocs) is moved to just after its tensor's last use.  If the last direct
 // user writes the tensor (the malloc is that op's last operand), the tensor

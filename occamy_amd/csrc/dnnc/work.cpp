@@ -12,7 +12,8 @@ const char *op_class(const Op *op) {
     case OP_CONV_BIAS_ACTIV:
     case OP_CONV_BIAS_ADD_ACTIV: return (op->dimB[1] == 1 && op->group > 1) ? "conv_depthwise" : "conv_dense";
     case OP_MATMUL2D: return "gemm";
-    case OP_MATMULND: return "matmul";
+    case OP_MATMULND:
+    case OP_MATMUL_BIAS: return "matmul";
     case OP_SOFTMAX: return "softmax";
     case OP_LAYERNORM: return "layernorm";
     case OP_REDUCE: return "reduce";
@@ -53,9 +54,10 @@ void op_work(const Op *op, double &flops, double &bytes) {
       bytes = (n_in(0) + n_in(1) + n_out) * es;
       break;
     }
-    case OP_MATMULND: {
+    case OP_MATMULND:
+    case OP_MATMUL_BIAS: {
       flops = 2.0 * n_out * (double)op->dimA.back();
-      bytes = (n_in(0) + n_in(1) + n_out) * es;
+      bytes = (n_in(0) + n_in(1) + n_out + (op->kind == OP_MATMUL_BIAS ? n_in(2) : 0.0)) * es;
       break;
     }
     case OP_ADD:

@@ -27,6 +27,8 @@ struct IgemmArgs {
   int64_t x_img_stride;   // elements between images of X (C*H*W)
   int64_t y_img_stride;   // elements between images of Y (K*P*Q)
   int64_t y_row_stride;   // elements between rows m of Y (P*Q, or ldc)
+  int64_t c_row_stride;   // the same for Cin (0: one row added to every row of D)
+  int64_t c_z_stride;     // elements between the Cin of consecutive z
   // blockIdx.z: group of a grouped convolution or batch of a batched matmul
   int Z;
   int64_t a_z_stride, x_z_stride, y_z_stride, bias_z_stride;

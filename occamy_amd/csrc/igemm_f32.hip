@@ -237,10 +237,10 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
     for (int i = 0; i < TM; i++) {
       float res_r[16];
       if (a.Cin) {
-        const float *__restrict__ Cg = a.Cin + (int64_t)z * a.y_z_stride;
+        const float *__restrict__ Cg = a.Cin + (int64_t)z * a.c_z_stride;
 #pragma unroll
         for (int r = 0; r < 16; r++)
-          res_r[r] = Cg[ycol + (int64_t)min(m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3), a.M - 1) * a.y_row_stride];
+          res_r[r] = Cg[ycol + (int64_t)min(m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3), a.M - 1) * a.c_row_stride];
       } else {
 #pragma unroll
         for (int r = 0; r < 16; r++) res_r[r] = 0.f;

@@ -143,9 +143,9 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
     for (int r = 0; r < 16; r++) bias_r[r] = 0.f;
   }
   if (a.Cin) {
-    const float *__restrict__ Cg = a.Cin + (int64_t)z * a.y_z_stride;
+    const float *__restrict__ Cg = a.Cin + (int64_t)z * a.c_z_stride;
 #pragma unroll
-    for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(m0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1) * a.y_row_stride];
+    for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(m0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1) * a.c_row_stride];
   } else {
 #pragma unroll
     for (int r = 0; r < 16; r++) res_r[r] = 0.f;

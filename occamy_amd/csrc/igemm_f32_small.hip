@@ -19,6 +19,8 @@
 // kernels when every operand is below 2^31 elements.
 #include "igemm_f32.h"
 
+#include <type_traits>
+
 namespace dnnrt {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -61,9 +63,9 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
   float res_r[16];
   if (a.Cin) {
     if (wave == 0) {
-      const float *__restrict__ Cg = a.Cin + (int64_t)z * a.y_z_stride;
+      const float *__restrict__ Cg = a.Cin + (int64_t)z * a.c_z_stride;
 #pragma unroll
-      for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(acc_row(m0, half, r), a.M - 1) * a.y_row_stride];
+      for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(acc_row(m0, half, r), a.M - 1) * a.c_row_stride];
     }
   } else {
 #pragma unroll
@@ -114,14 +116,23 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
   }
   if (!col_ok) return;
   float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
+  // one copy of the store loop per activation mode, picked once (the mode is the same for every lane)
+  auto store = [&](auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-  for (int r = 0; r < 16; r++) {
-    const int mm = acc_row(m0, half, r);
-    if (mm >= a.M) continue;
-    float v = a.alpha * acc[r] + bias_r[r];
-    if (a.Cin) v += a.beta * res_r[r];
-    v = apply_act(v, a.act, a.act_coef);
-    Yg[ycol + (int64_t)mm * a.y_row_stride] = v;
+    for (int r = 0; r < 16; r++) {
+      const int mm = acc_row(m0, half, r);
+      if (mm >= a.M) continue;
+      float v = a.alpha * acc[r] + bias_r[r];
+      if (a.Cin) v += a.beta * res_r[r];
+      Yg[ycol + (int64_t)mm * a.y_row_stride] = apply_act(v, MODE, a.act_coef);
+    }
+  };
+  switch (a.act) {
+    case DNNRT_ACT_RELU: store(std::integral_constant<int, DNNRT_ACT_RELU>{}); break;
+    case DNNRT_ACT_CLIPPED_RELU: store(std::integral_constant<int, DNNRT_ACT_CLIPPED_RELU>{}); break;
+    case DNNRT_ACT_LEAKY_RELU: store(std::integral_constant<int, DNNRT_ACT_LEAKY_RELU>{}); break;
+    default: store(std::integral_constant<int, DNNRT_ACT_IDENTITY>{}); break;
   }
 }
 

@@ -22,7 +22,7 @@ namespace dnnrt {
 template <int MMAX, int WPO>
 __global__ __launch_bounds__(WPO > 4 ? 64 * WPO : 256) void gemv_f32_kernel(
     const float *__restrict__ A, const float *__restrict__ B, const float *__restrict__ C,
-    float *__restrict__ Out, int M, int N, int K, float alpha, float beta, bool vec4) {
+    float *__restrict__ Out, int M, int N, int K, float alpha, float beta, bool vec4, int64_t c_ld) {
   constexpr int WAVES = WPO > 4 ? WPO : 4, NPB = WAVES / WPO;
   __shared__ float part[WAVES][MMAX];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -64,30 +64,31 @@ __global__ __launch_bounds__(WPO > 4 ? 64 * WPO : 256) void gemv_f32_kernel(
 #pragma unroll
     for (int w = 1; w < WPO; w++) v += part[wave + w][lane];
     float r = alpha * v;
-    if (C) r += beta * C[(int64_t)lane * N + n];
+    if (C) r += beta * C[(int64_t)lane * c_ld + n];
     Out[(int64_t)lane * N + n] = r;
   }
 }
 
 template <int WPO>
 static void launch_gemv(const dnnrtContext *ctx, const float *A, const float *B, const float *C, float *Out,
-                        int M, int N, int K, float alpha, float beta, bool vec4) {
+                        int M, int N, int K, float alpha, float beta, bool vec4, int64_t c_ld) {
   constexpr int WAVES = WPO > 4 ? WPO : 4, NPB = WAVES / WPO;
   hipLaunchKernelGGL((gemv_f32_kernel<8, WPO>), dim3((unsigned)ceil_div(N, NPB)), dim3(64 * WAVES), 0, ctx->stream,
-                     A, B, C, Out, M, N, K, alpha, beta, vec4);
+                     A, B, C, Out, M, N, K, alpha, beta, vec4, c_ld);
 }
 
 static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, const float *C,
                      float *Out, int M, int N, int K, float alpha, float beta, bool transA,
-                     bool transB, int Z, int64_t az, int64_t bz, int64_t yz) {
+                     bool transB, int Z, int64_t az, int64_t bz, int64_t yz, bool c_is_row = false) {
+  // c_is_row: C holds one row of N values that is added to every row of every product
   if (Z == 1 && M <= 8 && transB && !transA) {
     const bool vec4 = (K % 4 == 0) && aligned16(A) && aligned16(B);
     // wavefronts per output: the fewest that give 2048 wavefronts, each keeping >= 512 elements of k
     int wpo = 1;
     while (wpo < 16 && (int64_t)N * wpo < 2048 && K / (wpo * 4) >= 512) wpo *= 4;
-    if (wpo == 1) launch_gemv<1>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4);
-    else if (wpo == 4) launch_gemv<4>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4);
-    else launch_gemv<16>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4);
+    if (wpo == 1) launch_gemv<1>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4, c_is_row ? 0 : N);
+    else if (wpo == 4) launch_gemv<4>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4, c_is_row ? 0 : N);
+    else launch_gemv<16>(ctx, A, B, C, Out, M, N, K, alpha, beta, vec4, c_is_row ? 0 : N);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("gemv_f32: launch failed: %s", hipGetErrorString(e)); return false; }
     return true;
@@ -99,6 +100,7 @@ static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, co
   a.H = 1; a.W = N; a.R = 1; a.S = 1; a.P = 1; a.Q = N; a.ph = 0; a.pw = 0; a.sh = 1; a.sw = 1;
   a.x_img_stride = 0; a.y_img_stride = 0; a.y_row_stride = N;
   a.Z = Z; a.a_z_stride = az; a.x_z_stride = bz; a.y_z_stride = yz; a.bias_z_stride = 0;
+  a.c_row_stride = c_is_row ? 0 : N; a.c_z_stride = c_is_row ? 0 : yz;
   a.b_kcontig = transB; a.a_mcontig = transA; a.a_ld = M;
   a.a_vec4 = !transA && (K % 4 == 0) && aligned16(A) && (az % 4 == 0);
   a.b_vec4 = transB && (K % 4 == 0) && aligned16(B) && (bz % 4 == 0);
@@ -141,9 +143,9 @@ void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A, const int
   DNNRT_FAIL("dnnrtMatmul2d: dtype %d", dtype);
 }
 
-void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
-                    const void *B, const int64_t *dimB, int32_t rankB, void *Y, const int64_t *dimY,
-                    int32_t rankY, int32_t dtype) {
+static void *matmul_nd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
+                       const void *B, const int64_t *dimB, int32_t rankB, const void *bias, void *Y,
+                       const int64_t *dimY, int32_t rankY, int32_t dtype) {
   if (!handle) DNNRT_FAIL("dnnrtMatmulNd: null handle");
   if (!A || !B || !Y || !dimA || !dimB || !dimY) DNNRT_FAIL("dnnrtMatmulNd: null argument");
   if (rankA < 2 || rankB < 2 || rankA > 4 || rankB > 4 || rankY != (rankA > rankB ? rankA : rankB))
@@ -175,11 +177,12 @@ void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, in
   if (bz == 0 && Z > 1 && az != 0) { Mz = M * batchY; Z = 1; azz = 0; yz = 0; }
   if (Mz > INT32_MAX) DNNRT_FAIL("dnnrtMatmulNd: dims exceed 32 bits");
   if (dtype == DNNRT_F32) {
-    if (!gemm_f32(handle, (const float *)A, (const float *)B, nullptr, (float *)Y, (int)Mz, (int)N, (int)K,
-                  1.f, 0.f, false, false, Z, azz, bz, yz))
+    if (!gemm_f32(handle, (const float *)A, (const float *)B, (const float *)bias, (float *)Y, (int)Mz, (int)N, (int)K,
+                  1.f, bias ? 1.f : 0.f, false, false, Z, azz, bz, yz, bias != nullptr))
       return nullptr;
     return Y;
   }
+  if (dtype == DNNRT_F16 && bias) DNNRT_FAIL("dnnrtMatmulNdBias: fp16 is not built");
   if (dtype == DNNRT_F16) {
     if (!gemm_f16(handle, (const __half *)A, (const __half *)B, nullptr, (__half *)Y, (int)Mz, (int)N,
                   (int)K, 1.f, 0.f, false, false, Z, azz, bz, yz))
@@ -187,6 +190,19 @@ void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, in
     return Y;
   }
   DNNRT_FAIL("dnnrtMatmulNd: dtype %d", dtype);
+}
+
+void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
+                    const void *B, const int64_t *dimB, int32_t rankB, void *Y, const int64_t *dimY,
+                    int32_t rankY, int32_t dtype) {
+  return matmul_nd(handle, A, dimA, rankA, B, dimB, rankB, nullptr, Y, dimY, rankY, dtype);
+}
+
+void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
+                        const void *B, const int64_t *dimB, int32_t rankB, const void *bias, void *Y,
+                        const int64_t *dimY, int32_t rankY, int32_t dtype) {
+  if (!bias) DNNRT_FAIL("dnnrtMatmulNdBias: null bias");
+  return matmul_nd(handle, A, dimA, rankA, B, dimB, rankB, bias, Y, dimY, rankY, dtype);
 }
 
 }  // extern "C"

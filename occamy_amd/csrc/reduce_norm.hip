@@ -103,6 +103,92 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T *__restrict__ x,
     st_f(yr + i, (ld_f(xr + i) - mu) * inv * ld_f(g + i) + ld_f(b + i));
 }
 
+// The same for rows of up to 64 * 4 * V elements (L % 4 == 0): a lane keeps
+// its V groups of four in registers, so the row, gamma and beta are read once
+// and all of it is requested before anything is waited for.  WAVES rows per
+// workgroup: 1 when there are few rows, so that they spread over the CUs.
+__device__ __forceinline__ float as_f(float v) { return v; }
+__device__ __forceinline__ float as_f(__half v) { return __half2float(v); }
+template <typename T> __device__ __forceinline__ T as_t(float v);
+template <> __device__ __forceinline__ float as_t<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half as_t<__half>(float v) { return __float2half_rn(v); }
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float4 type; };
+template <> struct Vec4<__half> { struct alignas(8) type { __half x, y, z, w; }; };
+template <typename T, int V, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void layernorm_reg_kernel(const T *__restrict__ x, const T *__restrict__ g,
+                                                                   const T *__restrict__ b, T *__restrict__ y,
+                                                                   int64_t rows, int L, float eps) {
+  typedef typename Vec4<T>::type V4;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * WAVES + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int n4 = L >> 2;
+  const V4 *xr = reinterpret_cast<const V4 *>(x + row * L);
+  const V4 *g4 = reinterpret_cast<const V4 *>(g), *b4 = reinterpret_cast<const V4 *>(b);
+  V4 xv[V], gv[V], bv[V];
+#pragma unroll
+  for (int v = 0; v < V; v++) {
+    const int j = min(v * 64 + lane, n4 - 1);  // clamped: the duplicates are left out of the sums below
+    xv[v] = xr[j]; gv[v] = g4[j]; bv[v] = b4[j];
+  }
+  float f[V][4];
+  float s = 0.f;
+#pragma unroll
+  for (int v = 0; v < V; v++) {
+    f[v][0] = as_f(xv[v].x); f[v][1] = as_f(xv[v].y); f[v][2] = as_f(xv[v].z); f[v][3] = as_f(xv[v].w);
+    if (v * 64 + lane < n4) s += (f[v][0] + f[v][1]) + (f[v][2] + f[v][3]);
+  }
+  const float mu = wave_sum(s) / (float)L;
+  float q = 0.f;
+#pragma unroll
+  for (int v = 0; v < V; v++) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) f[v][e] -= mu;
+    if (v * 64 + lane < n4) q += (f[v][0] * f[v][0] + f[v][1] * f[v][1]) + (f[v][2] * f[v][2] + f[v][3] * f[v][3]);
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(q) / (float)L + eps);
+  V4 *yr = reinterpret_cast<V4 *>(y + row * L);
+#pragma unroll
+  for (int v = 0; v < V; v++) {
+    const int j = v * 64 + lane;
+    if (j >= n4) continue;
+    V4 o;
+    o.x = as_t<T>(f[v][0] * inv * as_f(gv[v].x) + as_f(bv[v].x));
+    o.y = as_t<T>(f[v][1] * inv * as_f(gv[v].y) + as_f(bv[v].y));
+    o.z = as_t<T>(f[v][2] * inv * as_f(gv[v].z) + as_f(bv[v].z));
+    o.w = as_t<T>(f[v][3] * inv * as_f(gv[v].w) + as_f(bv[v].w));
+    yr[j] = o;
+  }
+}
+
+template <typename T, int V>
+static void launch_layernorm_reg(const dnnrtContext *ctx, const void *X, const void *g, const void *b, void *Y,
+                                 int64_t rows, int L, float eps) {
+  if (rows <= 4 * (int64_t)ctx->num_cu)
+    hipLaunchKernelGGL((layernorm_reg_kernel<T, V, 1>), dim3((unsigned)rows), dim3(64), 0, ctx->stream, (const T *)X,
+                       (const T *)g, (const T *)b, (T *)Y, rows, L, eps);
+  else
+    hipLaunchKernelGGL((layernorm_reg_kernel<T, V, 4>), dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, ctx->stream,
+                       (const T *)X, (const T *)g, (const T *)b, (T *)Y, rows, L, eps);
+}
+template <typename T>
+static bool layernorm_in_registers(const dnnrtContext *ctx, const void *X, const void *g, const void *b, void *Y,
+                                   int64_t rows, int64_t L, float eps) {
+  const uintptr_t align = 4 * sizeof(T) - 1;
+  if (L % 4 || L > 2048 || ((uintptr_t)X & align) || ((uintptr_t)Y & align) || ((uintptr_t)g & align) || ((uintptr_t)b & align))
+    return false;
+  switch ((int)ceil_div(L, 256)) {
+    case 1: launch_layernorm_reg<T, 1>(ctx, X, g, b, Y, rows, (int)L, eps); break;
+    case 2: launch_layernorm_reg<T, 2>(ctx, X, g, b, Y, rows, (int)L, eps); break;
+    case 3: launch_layernorm_reg<T, 3>(ctx, X, g, b, Y, rows, (int)L, eps); break;
+    case 4: launch_layernorm_reg<T, 4>(ctx, X, g, b, Y, rows, (int)L, eps); break;
+    case 5: case 6: launch_layernorm_reg<T, 6>(ctx, X, g, b, Y, rows, (int)L, eps); break;
+    default: launch_layernorm_reg<T, 8>(ctx, X, g, b, Y, rows, (int)L, eps); break;
+  }
+  return true;
+}
+
 template <typename T>
 static bool run_reduce(const dnnrtContext *ctx, const void *X, void *Y, int64_t outer, int64_t red,
                        int64_t inner) {
@@ -209,7 +295,9 @@ void *dnnrtLayerNorm(dnnrtHandle_t handle, const void *X, const int64_t *dimX, i
   if (L <= 0 || L > INT32_MAX || rows <= 0) DNNRT_FAIL("dnnrtLayerNorm: bad dims");
   const int64_t blocks = ceil_div(rows, 4);
   if (blocks > INT32_MAX) DNNRT_FAIL("dnnrtLayerNorm: too many rows");
-  if (dtype == DNNRT_F32)
+  if (dtype == DNNRT_F32 && layernorm_in_registers<float>(handle, X, gamma, beta, Y, rows, L, eps)) {
+  } else if (dtype == DNNRT_F16 && layernorm_in_registers<__half>(handle, X, gamma, beta, Y, rows, L, eps)) {
+  } else if (dtype == DNNRT_F32)
     hipLaunchKernelGGL((layernorm_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, handle->stream,
                        (const float *)X, (const float *)gamma, (const float *)beta, (float *)Y, rows,
                        (int)L, eps);

@@ -177,6 +177,11 @@ class Ops:
                                                 len(dimB), Y, dims(dimY), len(dimY), dtype),
                          "dnnrtMatmulNd")
 
+    def matmul_nd_bias(self, A, dimA, B, dimB, bias, Y, dimY, dtype=_abi.F32):
+        return self._ret(self.lib.dnnrtMatmulNdBias(self.handle, A, dims(dimA), len(dimA), B, dims(dimB),
+                                                    len(dimB), bias, Y, dims(dimY), len(dimY), dtype),
+                         "dnnrtMatmulNdBias")
+
     def flatten(self, X, dimX, Y, dimY, axis, dtype=_abi.F32):
         return self._ret(self.lib.dnnrtFlatten(self.handle, X, dims(dimX), Y, dims(dimY), axis,
                                                len(dimX), dtype), "dnnrtFlatten")

@@ -736,6 +736,18 @@ void *dnnrtMatmulNd(dnnrtHandle_t h, const void *A, const int64_t *dA, int32_t r
   narrow(Y, ty, ny, dtype); free(ta); free(tb);
   return Y;
 }
+/* No reference wrapper of its own: CUDAMatmulNdFunc.cu, then the broadcast
+ * add of CUDNNTensorOpFunc.cpp on the stored product -- restated as that chain. */
+void *dnnrtMatmulNdBias(dnnrtHandle_t h, const void *A, const int64_t *dA, int32_t rA,
+                        const void *B, const int64_t *dB, int32_t rB, const void *bias,
+                        void *Y, const int64_t *dY, int32_t rY, int32_t dtype) {
+  if (!bias) FAIL("matmulNdBias: null bias");
+  if (!dnnrtMatmulNd(h, A, dA, rA, B, dB, rB, Y, dY, rY, dtype)) return NULL;
+  int64_t db[8];
+  for (int i = 0; i < rY; i++) db[i] = 1;
+  db[rY - 1] = dY[rY - 1];
+  return dnnrtTensorOp(h, DNNRT_OP_ADD, Y, dY, rY, bias, db, rY, Y, dY, rY, 1.0f, dtype);
+}
 
 /* ---- data movement -------------------------------------------------------- */
 

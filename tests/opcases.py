@@ -212,3 +212,12 @@ def squeeze(be, x, out, un=False):
     (be.ops.unsqueeze if un else be.ops.squeeze)(be.ptr(X), x.shape, be.ptr(Y), out, DT[x.dtype])
     be.sync()
     return be.get(Y)
+
+
+def matmul_nd_bias(be, a, b, bias):
+    y_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2]) + (a.shape[-2], b.shape[-1])
+    A, B, Bi = be.put(a), be.put(b), be.put(bias)
+    Y = be.empty(y_shape, a.dtype)
+    be.ops.matmul_nd_bias(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Bi), be.ptr(Y), y_shape, DT[a.dtype])
+    be.sync()
+    return be.get(Y)

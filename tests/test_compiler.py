@@ -151,6 +151,48 @@ def test_activation_fusion_flag():
     assert count(g.compile(fuse_activations=True))["dnn.clip"] == 35
 
 
+def test_recompose_flag():
+    small = dict(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100)
+    names = lambda p: [n for n, *_ in p.compute_ops()]  # noqa: E731
+    g, _ = models.bert_encoder(**small)
+    plain = names(g.compile())
+    assert "dnn.layernorm" not in plain and "dnn.gelu" not in plain and plain.count("dnn.reciprocal") == 9
+    p = check_lifetimes(lambda: models.bert_encoder(**small), recompose=True)
+    got = names(p)
+    # 1 + 2 per layer LayerNorms, one Gelu per layer, no reciprocal of a constant left at run time
+    assert got.count("dnn.layernorm") == 5 and got.count("dnn.gelu") == 2 and "dnn.reciprocal" not in got
+    assert not {"dnn.pow", "dnn.sqrt", "dnn.erf", "dnn.reduce", "dnn.negative"} & set(got)
+    # what the builder's own fused graph compiles to, but for the folded divisors
+    g, _ = models.bert_encoder(fused=True, **small)
+    ref = names(g.compile())
+    assert [n for n in ref if n != "dnn.reciprocal"] == got
+    p = check_lifetimes(lambda: models.bert_encoder(**small), recompose=True, fusion=True, fuse_matmul_bias=True)
+    got = names(p)
+    assert got.count("dnn.matmulnd-bias") == 12 and got.count("dnn.matmulnd") == 4 and got.count("dnn.add") == 6
+
+
+def test_recompose_leaves_near_misses_alone():
+    def ln_graph(eps_node="eps", power=2.0, extra_reader=False, axes=(-1,)):
+        g = compiler.Graph()
+        x = g.input("x", (2, 5, 8))
+        c = lambda v, n: g.constant(np.array(v, np.float32), n)  # noqa: E731
+        mu = g.node("ReduceMean", [x], "mu", axes=list(axes), keepdims=1)
+        d = g.node("Sub", [x, mu], "d")
+        var = g.node("ReduceMean", [g.node("Pow", [d, c(power, "two")], "sq")], "var", axes=list(axes), keepdims=1)
+        sd = g.node("Sqrt", [g.node("Add", [var, c(1e-5, eps_node)], "ve")], "sd")
+        y = g.node("Add", [g.node("Mul", [g.node("Div", [d, sd], "n"), g.constant(np.ones(8, np.float32), "gamma")], "sc"),
+                           g.constant(np.zeros(8, np.float32), "beta")], "y")
+        g.output(y)
+        if extra_reader:
+            g.output(g.node("Relu", ["sd"], "also"))
+        return g
+    count = lambda g: [n for n, *_ in g.compile(recompose=True).compute_ops()].count("dnn.layernorm")  # noqa: E731
+    assert count(ln_graph()) == 1
+    assert count(ln_graph(power=3.0)) == 0            # not a variance
+    assert count(ln_graph(extra_reader=True)) == 0    # the standard deviation is read elsewhere
+    assert count(ln_graph(axes=(1,))) == 0            # not the last axis
+
+
 def planned_vs_oracle(p):
     ev = p.events()
     off, peak = oracle_plan([(k, i, b) for k, i, b, _ in ev])

@@ -188,6 +188,16 @@ def test_activation_fusion_matches_unfused_chain(builder):
         np.testing.assert_array_equal(x, y)
 
 
+def test_recomposed_bert_matches_torch_and_the_decomposed_program():
+    small = dict(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100)
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True)
+    a = check(lambda: models.bert_encoder(**small), rtol=1e-4, atol=1e-4)
+    b = check(lambda: models.bert_encoder(**small), rtol=1e-4, atol=1e-4, **flags)
+    np.testing.assert_allclose(a[0], b[0], rtol=1e-4, atol=1e-4)
+    _, _, c = run_oracle(lambda: models.bert_encoder(**small), mode=compiler.MODE_RESIDENT, **flags)
+    np.testing.assert_array_equal(b[0], c[0])
+
+
 def test_executor_errors():
     g, inputs = models.single_conv()
     p = g.compile(pool_opt=False)

@@ -168,6 +168,14 @@ def test_activation_fusion_fp32(name, oracle_outputs):
         close(o, r)
 
 
+def test_bert_recomposed_with_fused_linear_layers(oracle_outputs):
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True)
+    out, _ = run(CONFIGS["bert_2_layers"], **flags)
+    close(out[0], oracle_outputs["bert_2_layers"][0], 1e-4, 1e-4)
+    out, _ = run(CONFIGS["bert_2_layers"], mode=compiler.MODE_RESIDENT, **flags)
+    close(out[0], oracle_outputs["bert_2_layers"][0], 1e-4, 1e-4)
+
+
 def test_model_from_an_onnx_file_runs_like_the_built_graph(tmp_path):
     """ResNet-50 through a file: ONNX bytes -> reader -> compiler -> gfx950."""
     import onnx_writer

@@ -190,12 +190,20 @@ def test_softmax(gpu, cpu):
 
 def test_layernorm(gpu, cpu):
     r = rng(12)
-    for shape in [(1, 128, 768), (2, 7, 48), (5, 1000), (3, 1)]:
+    # rows held in registers (L % 4 == 0, up to 2048: one to eight groups of four per lane, few and
+    # many rows) and the general kernel (odd L, long rows)
+    for shape in [(1, 128, 768), (2, 7, 48), (5, 1000), (3, 1), (3, 4), (2, 300), (1, 2048), (1300, 256), (2, 1540), (2, 4096), (4, 1026)]:
         L = shape[-1]
         x = (r.standard_normal(shape) * 3 + 1).astype(np.float32)
         g = r.standard_normal(L).astype(np.float32)
         b = r.standard_normal(L).astype(np.float32)
         close(oc.layernorm(gpu, x, g, b, 1e-12 if L > 1 else 1e-5), oc.layernorm(cpu, x, g, b, 1e-12 if L > 1 else 1e-5), 1e-4, 1e-4)
+    for shape in [(16, 768), (3, 64), (2, 2052)]:
+        L = shape[-1]
+        x = (r.standard_normal(shape) * 3 + 1).astype(np.float16)
+        g, b = r.standard_normal(L).astype(np.float16), r.standard_normal(L).astype(np.float16)
+        np.testing.assert_allclose(oc.layernorm(gpu, x, g, b, 1e-5).astype(np.float32), oc.layernorm(cpu, x, g, b, 1e-5).astype(np.float32),
+                                   rtol=2e-2, atol=2e-2)
 
 
 # ---- pooling ---------------------------------------------------------------------------
@@ -244,6 +252,19 @@ def test_matmul_nd(gpu, cpu):
         a = r.standard_normal(sa).astype(np.float32)
         b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float32)
         close(oc.matmul_nd(gpu, a, b), oc.matmul_nd(cpu, a, b))
+
+
+def test_matmul_nd_bias(gpu, cpu):
+    r = rng(44)
+    # transformer Linear layers (one tall product, the dot-product kernel for few rows) and batched products
+    for sa, sb in [((1, 128, 768), (768, 768)), ((1, 128, 768), (768, 3072)), ((1, 128, 3072), (3072, 768)), ((5, 7), (7, 3)),
+                   ((3, 6, 5), (3, 5, 4)), ((2, 12, 40, 64), (2, 12, 64, 40)), ((1, 3, 33), (33, 130))]:
+        a = r.standard_normal(sa).astype(np.float32)
+        b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float32)
+        bias = r.standard_normal(sb[-1]).astype(np.float32)
+        close(oc.matmul_nd_bias(gpu, a, b, bias), oc.matmul_nd_bias(cpu, a, b, bias))
+    with pytest.raises(RuntimeError):
+        oc.matmul_nd_bias(gpu, a.astype(np.float16), b.astype(np.float16), bias.astype(np.float16))  # not built: loud
 
 
 # ---- data movement -------------------------------------------------------------------------

@@ -319,6 +319,16 @@ def test_matmul_nd(be):
         np.testing.assert_allclose(oc.matmul_nd(be, a, b), np.matmul(a.astype(np.float64), b.astype(np.float64)), rtol=1e-6, atol=1e-6)
 
 
+def test_matmul_nd_bias(be):
+    r = rng(34)
+    for sa, sb in [((5, 7), (7, 3)), ((2, 4, 6, 5), (5, 8)), ((3, 6, 5), (3, 5, 4))]:
+        a = r.standard_normal(sa).astype(np.float32)
+        b = r.standard_normal(sb).astype(np.float32)
+        bias = r.standard_normal(sb[-1]).astype(np.float32)
+        ref = np.matmul(a.astype(np.float64), b.astype(np.float64)) + bias
+        np.testing.assert_allclose(oc.matmul_nd_bias(be, a, b, bias), ref, rtol=1e-5, atol=1e-5)
+
+
 # ---- data movement --------------------------------------------------------------------------------
 
 def test_data_movement(be):
