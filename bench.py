@@ -34,7 +34,7 @@ def build_workload(name):
     if name == "mobilenet_v2_fp32_bs1":
         return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
-        return models.bert_encoder(), dict(recompose=True, fusion=True, fuse_matmul_bias=True), 1, "seq/s", "f32"
+        return models.bert_encoder(), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True), 1, "seq/s", "f32"
     if name == "single_conv_fp32":
         return models.single_conv(), dict(fusion=True), 1, "img/s", "f32"
     if name == "alexnet_fp32_bs1":
@@ -138,7 +138,7 @@ def main():
         # the reference's per-inference semantics: pool alloc, all weights H2D, kernels, D2H, sync, pool free
         # (compiled with the reference's own flags: no residual fusion)
         (ref_graph, _), _, _, _, _ = build_workload(name)  # a graph compiles once; the builders are seeded
-        ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k not in ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias")})
+        ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k not in ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention")})
         res["pool_bytes_reference_flags"] = ref_prog.pool_bytes
         so = ref_prog.session(compiler.MODE_OCCAMY)
         so.run(*inputs)

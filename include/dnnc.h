@@ -62,6 +62,8 @@ typedef struct {
                              primitive operators become one call each (default 0) */
   int32_t fuse_matmul_bias; /* no reference flag: with `fusion`, MatMul -> Add(bias row)
                              becomes one call (default 0) */
+  int32_t fuse_attention; /* no reference flag: the head split, QK^T, scaling, Softmax, PV and
+                             head merge of an exported attention block become one call (default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);
@@ -84,7 +86,7 @@ int32_t dnncProgramOutputInfo(const dnncProgram *p, int32_t i, int32_t *dtype, i
 int64_t dnncProgramNumOps(const dnncProgram *p, int32_t compute_only);
 /* i-th compute operation in program order: its mnemonic, its work class
  * (conv_dense, conv_depthwise, gemm, matmul, softmax, layernorm, reduce, pool,
- * move, elementwise) and its algorithmic FLOPs and bytes (each tensor read or
+ * attention, move, elementwise) and its algorithmic FLOPs and bytes (each tensor read or
  * written counted once at its dense size) */
 int32_t dnncProgramComputeOp(const dnncProgram *p, int64_t i, const char **name, const char **work_class, double *flops, double *bytes);
 

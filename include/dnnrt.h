@@ -303,6 +303,17 @@ void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA
                         int32_t rankA, const void *B, const int64_t *dimB,
                         int32_t rankB, const void *bias, void *Y,
                         const int64_t *dimY, int32_t rankY, int32_t dtype);
+/* Multi-head attention core, Y = softmax(scale * Q K^T) V per head, with Q
+ * [batch, seqQ, heads*headDim], K and V [batch, seqK, heads*headDim] and Y like
+ * Q.  No reference wrapper: it stands for the chain the reference runs call
+ * by call for an exported transformer (CUDAReshapeFunc + CUDATranspose4DFloatFunc
+ * per operand, CUDAMatmulNdFunc, the scaling Mul, CUDASoftmaxFunc,
+ * CUDAMatmulNdFunc, Transpose + Reshape back).  fp32, headDim 32 / 64 / 128,
+ * 16-byte aligned operands, Y distinct from the inputs. */
+void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void *K,
+                     const void *V, void *Y, int64_t batch, int64_t seqQ,
+                     int64_t seqK, int64_t heads, int64_t headDim, float scale,
+                     int32_t dtype);
 
 /* ---- data movement --------------------------------------------------- */
 

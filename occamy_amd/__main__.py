@@ -17,6 +17,7 @@ def main():
     ap.add_argument("--dnn-kernel-fusion", dest="fusion", action="store_true")
     ap.add_argument("--fuse-residual", action="store_true", help="with fusion: conv+bias -> add -> relu as one call")
     ap.add_argument("--recompose", action="store_true", help="LayerNormalization / Gelu written in primitive operators become one call each")
+    ap.add_argument("--fuse-attention", action="store_true", help="head split, QK^T, Softmax, PV, head merge as one call")
     ap.add_argument("--fuse-matmul-bias", action="store_true", help="with fusion: MatMul -> Add(bias row) as one call")
     ap.add_argument("--fuse-activations", action="store_true",
                     help="with fusion: conv+bias -> Clip(0, c) / LeakyRelu / one-slope PRelu as one call")
@@ -31,7 +32,7 @@ def main():
     args = ap.parse_args()
 
     graph = compiler.load_onnx(args.model)
-    prog = graph.compile(fusion=args.fusion, fuse_residual=args.fuse_residual, fuse_activations=args.fuse_activations, recompose=args.recompose, fuse_matmul_bias=args.fuse_matmul_bias, dealloc_opt=args.dealloc_opt,
+    prog = graph.compile(fusion=args.fusion, fuse_residual=args.fuse_residual, fuse_activations=args.fuse_activations, recompose=args.recompose, fuse_matmul_bias=args.fuse_matmul_bias, fuse_attention=args.fuse_attention, dealloc_opt=args.dealloc_opt,
                          const_at_use=args.const_at_use, channels_last=args.channels_last)
     print(f"inputs: {graph.input_shapes}")
     print(f"pool: {prog.pool_bytes} bytes (maxAllocByte); {prog.num_ops(compute_only=True)} runtime calls per inference")

@@ -121,7 +121,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (!g || !opt) { g_err = "dnncCompile: bad arguments"; return nullptr; }
   if (g->compiled) { g_err = "dnncCompile: a graph can be compiled once"; return nullptr; }
   std::string err;
-  if (!infer_shapes(g->g, opt->recompose != 0, err)) { g_err = err; return nullptr; }
+  if (!infer_shapes(g->g, opt->recompose != 0, opt->fuse_attention != 0, err)) { g_err = err; return nullptr; }
   if (opt->const_at_use) constant_at_use(g->g);
   g->compiled = true;
   dnncProgram *pp = new dnncProgram();

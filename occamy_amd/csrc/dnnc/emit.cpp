@@ -361,6 +361,17 @@ struct Emitter {
         result = a->result;
       }
       park_dealloc(out_buf);
+    } else if (t == "FusedAttention") {
+      Value *k = in(1), *v = in(2);
+      if (!k || !v) { err = "FusedAttention: K or V not available"; return false; }
+      out_buf = malloc_(ot.dtype, ot.shape);
+      Op *o = compute(OP_ATTENTION, {x, k, v, out_buf});
+      o->dimA = x->shape;
+      o->dimB = k->shape;
+      o->group = int1("heads", 1);
+      o->alpha = (float)flt("scale", 1.0);
+      result = o->result;
+      park_dealloc(out_buf);
     } else if (t == "LayerNormalization") {
       Value *gm = in(1), *bt = in(2);
       if (!gm || !bt) { err = "LayerNormalization: scale and bias are required"; return false; }

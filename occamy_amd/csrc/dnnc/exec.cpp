@@ -32,7 +32,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
   if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
   LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
-  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
@@ -346,6 +346,10 @@ bool Session::issue(const Op *op, std::string &err) {
     case OP_MATMULND:
       r = rt.dnnrtMatmulNd(handle, P(0), op->dimA.data(), (int32_t)op->dimA.size(), P(1), op->dimB.data(),
                            (int32_t)op->dimB.size(), out, op->dimOut.data(), (int32_t)op->dimOut.size(), dt);
+      break;
+    case OP_ATTENTION:  // operands: q, k, v, out
+      r = rt.dnnrtAttention(handle, P(0), P(1), P(2), out, op->dimA[0], op->dimA[1], op->dimB[1], op->group,
+                            op->dimA[2] / op->group, op->alpha, dt);
       break;
     case OP_MATMUL_BIAS:  // operands: a, b, bias, out
       r = rt.dnnrtMatmulNdBias(handle, P(0), op->dimA.data(), (int32_t)op->dimA.size(), P(1), op->dimB.data(),

@@ -61,6 +61,7 @@ struct RuntimeApi {
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
   decltype(&::dnnrtSetActivationCoef) dnnrtSetActivationCoef = nullptr;
   decltype(&::dnnrtMatmulNdBias) dnnrtMatmulNdBias = nullptr;
+  decltype(&::dnnrtAttention) dnnrtAttention = nullptr;
   decltype(&::dnnrtLeakyRelu) dnnrtLeakyRelu = nullptr;
   decltype(&::dnnrtPRelu) dnnrtPRelu = nullptr;
   decltype(&::dnnrtConcat) dnnrtConcat = nullptr;

@@ -340,13 +340,71 @@ static bool fold_constant_divisors(Graph &g) {
   return any;
 }
 
-static bool recompose(Graph &g) {
+// out = Reshape(Transpose(MatMul(Softmax(scale * MatMul(q, k)), v), [0,2,1,3]), [B, S, H*D]) with
+// q, v = Transpose(Reshape(Q | V, [B, S, H, D]), [0,2,1,3]) and k = Transpose(Reshape(K, [B, S, H, D]), [0,2,3,1]):
+// the attention core of an exported transformer encoder, heads split and merged by data movement.
+static bool match_attention(const Matcher &m, const GNode &root, GNode &fused, std::vector<std::string> &dead) {
+  if (root.op_type != "Reshape" || root.inputs.empty()) return false;
+  auto perm_is = [](const GNode *n, std::initializer_list<int64_t> want) {
+    auto it = n->ints.find("perm");
+    return it != n->ints.end() && it->second == std::vector<int64_t>(want);
+  };
+  const GNode *merge, *mm2, *soft, *mm1, *scl = nullptr, *t[3], *r[3];
+  if (!(merge = m.def(root.inputs[0], "Transpose")) || !perm_is(merge, {0, 2, 1, 3})) return false;
+  if (!(mm2 = m.def(merge->inputs[0], "MatMul")) || mm2->inputs.size() != 2) return false;
+  if (!(soft = m.def(mm2->inputs[0], "Softmax"))) return false;
+  auto ax = soft->ints.find("axis");
+  const int64_t axis = ax == soft->ints.end() || ax->second.empty() ? -1 : ax->second[0];
+  if (axis != -1 && axis != 3) return false;
+  double scale = 1.0, c;
+  std::string other;
+  if ((mm1 = m.def(soft->inputs[0], "MatMul")) == nullptr) {
+    if ((scl = m.def(soft->inputs[0], "Div")) != nullptr) {
+      if (scl->inputs.size() != 2 || !(mm1 = m.def(scl->inputs[0], "MatMul")) || !m.scalar(scl->inputs[1], c) || c == 0.0) return false;
+      scale = (double)(1.0f / (float)c);
+    } else if ((scl = m.def(soft->inputs[0], "Mul")) != nullptr) {
+      if (!m.split(*scl, "MatMul", mm1, other) || !m.scalar(other, c)) return false;
+      scale = c;
+    } else {
+      return false;
+    }
+  }
+  if (mm1->inputs.size() != 2) return false;
+  const std::string tn[3] = {mm1->inputs[0], mm1->inputs[1], mm2->inputs[1]};
+  for (int i = 0; i < 3; i++) {
+    if (!(t[i] = m.def(tn[i], "Transpose")) || !(r[i] = m.def(t[i]->inputs[0], "Reshape"))) return false;
+    if (i == 1 ? !perm_is(t[i], {0, 2, 3, 1}) : !perm_is(t[i], {0, 2, 1, 3})) return false;
+  }
+  const GTensor &q = m.g.tensors.at(r[0]->inputs[0]), &k = m.g.tensors.at(r[1]->inputs[0]), &v = m.g.tensors.at(r[2]->inputs[0]);
+  const Shape &qs = m.g.tensors.at(r[0]->output).shape, &ks = m.g.tensors.at(r[1]->output).shape, &vs = m.g.tensors.at(r[2]->output).shape;
+  if (q.dtype != F32 || q.shape.size() != 3 || k.shape.size() != 3 || v.shape != k.shape || qs.size() != 4 || ks.size() != 4 || vs != ks) return false;
+  const int64_t B = qs[0], Sq = qs[1], H = qs[2], D = qs[3], Sk = ks[1];
+  if (ks[0] != B || ks[2] != H || ks[3] != D || (D != 32 && D != 64 && D != 128)) return false;
+  if (q.shape != Shape{B, Sq, H * D} || k.shape != Shape{B, Sk, H * D} || m.g.tensors.at(root.output).shape != q.shape) return false;
+  std::vector<const GNode *> inner{merge, mm2, soft, mm1, t[0], t[1], t[2], r[0], r[1], r[2]};
+  if (scl) inner.push_back(scl);
+  for (const GNode *n : inner)
+    if (!m.single_use(n->output)) return false;
+  fused = GNode();
+  fused.op_type = "FusedAttention";
+  fused.inputs = {r[0]->inputs[0], r[1]->inputs[0], r[2]->inputs[0]};
+  fused.output = root.output;
+  fused.ints["heads"] = {H};
+  fused.floats["scale"] = scale;
+  dead.clear();
+  for (const GNode *n : inner) dead.push_back(n->output);
+  return true;
+}
+
+static bool recompose(Graph &g, bool norms, bool attention) {
   bool any = false;
   for (size_t i = 0; i < g.nodes.size(); i++) {
     Matcher m(g);
     GNode fused;
     std::vector<std::string> dead;
-    if (!match_layernorm(m, g.nodes[i], fused, dead) && !match_gelu(m, g.nodes[i], fused, dead)) continue;
+    const bool hit = (attention && match_attention(m, g.nodes[i], fused, dead)) ||
+                     (norms && (match_layernorm(m, g.nodes[i], fused, dead) || match_gelu(m, g.nodes[i], fused, dead)));
+    if (!hit) continue;
     // constants read by the matched nodes only go with them
     std::vector<std::string> consts;
     for (const std::string &d : dead)
@@ -374,7 +432,7 @@ static bool recompose(Graph &g) {
     i = (size_t)-1;  // positions moved: rescan
   }
   // after the matchers: Gelu's own Div by sqrt(2) must still be there for them
-  return fold_constant_divisors(g) || any;
+  return (norms && fold_constant_divisors(g)) || any;
 }
 
 static bool infer_pass(Graph &g, std::string &err) {
@@ -425,6 +483,9 @@ static bool infer_pass(Graph &g, std::string &err) {
     } else if (t == "Relu" || t == "Sigmoid" || t == "Tanh" || t == "Sqrt" || t == "Erf" || t == "Clip" ||
                t == "Gelu" || t == "Pow" || t == "Softmax" || t == "LayerNormalization" || t == "LeakyRelu" ||
                t == "Identity" || t == "BatchNormalization") {
+      out.shape = x;
+    } else if (t == "FusedAttention") {  // produced by the recomposition only
+      if (in.size() != 3 || !in[1] || !in[2] || x.size() != 3) return fail("needs Q, K and V of rank 3");
       out.shape = x;
     } else if (t == "PRelu") {
       if (in.size() < 2 || !in[1]) return fail("needs a slope");
@@ -571,10 +632,10 @@ static bool infer_pass(Graph &g, std::string &err) {
   return true;
 }
 
-bool infer_shapes(Graph &g, bool recompose_norms, std::string &err) {
+bool infer_shapes(Graph &g, bool recompose_norms, bool fuse_attention, std::string &err) {
   forward_aliases(g);
   if (!infer_pass(g, err)) return false;
-  bool rewritten = recompose_norms && recompose(g);
+  bool rewritten = (recompose_norms || fuse_attention) && recompose(g, recompose_norms, fuse_attention);
   for (size_t i = 0; i < g.nodes.size();) {
     if (g.nodes[i].op_type != "BatchNormalization") { i++; continue; }
     if (!rewrite_batchnorm(g, i, err)) return false;

@@ -46,6 +46,7 @@ const char *op_name(OpKind k) {
     case OP_GELU: return "dnn.gelu";
     case OP_CONV_BIAS_ADD_ACTIV: return "dnn.conv-bias-add-relufwd";
     case OP_MATMUL_BIAS: return "dnn.matmulnd-bias";
+    case OP_ATTENTION: return "dnn.attention";
     case OP_RETURN: return "return";
   }
   return "?";
@@ -200,6 +201,7 @@ std::string Program::to_text() const {
       case OP_CONCAT:
       case OP_GATHER: os << " {axis=" << op->axis << "}"; break;
       case OP_LEAKYRELU: os << " {alpha=" << op->alpha << "}"; break;
+      case OP_ATTENTION: os << " {heads=" << op->group << ", scale=" << op->alpha << "}"; break;
       case OP_SQUEEZE:
       case OP_UNSQUEEZE: os << " {axes="; print_shape(os, op->perm); os << "}"; break;
       case OP_TRANSPOSE: os << " {perm="; print_shape(os, op->perm); os << "}"; break;

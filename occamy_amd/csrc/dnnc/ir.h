@@ -66,6 +66,7 @@ enum OpKind {
   OP_LAYERNORM, OP_GELU,
   OP_CONV_BIAS_ADD_ACTIV,  // conv + bias + residual tensor + activation (cuDNN's z operand)
   OP_MATMUL_BIAS,          // batched matrix product + one row added to every row
+  OP_ATTENTION,            // softmax(scale * Q K^T) V per head on [batch, seq, heads * dim] tensors
   OP_RETURN
 };
 const char *op_name(OpKind k);
@@ -149,7 +150,7 @@ struct CompileOptions {
 };
 
 // graph.cpp
-bool infer_shapes(Graph &g, bool recompose_norms, std::string &err);
+bool infer_shapes(Graph &g, bool recompose_norms, bool fuse_attention, std::string &err);
 void constant_at_use(Graph &g);
 // emit.cpp
 bool emit_program(const Graph &g, Program &p, std::string &err);

@@ -15,6 +15,7 @@ const char *op_class(const Op *op) {
     case OP_MATMULND:
     case OP_MATMUL_BIAS: return "matmul";
     case OP_SOFTMAX: return "softmax";
+    case OP_ATTENTION: return "attention";
     case OP_LAYERNORM: return "layernorm";
     case OP_REDUCE: return "reduce";
     case OP_MAXPOOL:
@@ -60,6 +61,10 @@ void op_work(const Op *op, double &flops, double &bytes) {
       bytes = (n_in(0) + n_in(1) + n_out + (op->kind == OP_MATMUL_BIAS ? n_in(2) : 0.0)) * es;
       break;
     }
+    case OP_ATTENTION:  // two products of 2 * B * H * Sq * Sk * D each
+      flops = 4.0 * n_in(0) * (double)op->dimB[1];
+      bytes = (n_in(0) + n_in(1) + n_in(2) + n_out) * es;
+      break;
     case OP_ADD:
     case OP_MUL:
       flops = n_out;

@@ -182,6 +182,11 @@ class Ops:
                                                     len(dimB), bias, Y, dims(dimY), len(dimY), dtype),
                          "dnnrtMatmulNdBias")
 
+    def attention(self, Q, K, V, Y, batch, seq_q, seq_k, heads, head_dim, scale, dtype=_abi.F32):
+        """Q [batch, seq_q, heads*head_dim], K and V [batch, seq_k, heads*head_dim], Y like Q."""
+        return self._ret(self.lib.dnnrtAttention(self.handle, Q, K, V, Y, batch, seq_q, seq_k, heads, head_dim,
+                                                 scale, dtype), "dnnrtAttention")
+
     def flatten(self, X, dimX, Y, dimY, axis, dtype=_abi.F32):
         return self._ret(self.lib.dnnrtFlatten(self.handle, X, dims(dimX), Y, dims(dimY), axis,
                                                len(dimX), dtype), "dnnrtFlatten")

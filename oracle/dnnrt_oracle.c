@@ -748,6 +748,47 @@ void *dnnrtMatmulNdBias(dnnrtHandle_t h, const void *A, const int64_t *dA, int32
   db[rY - 1] = dY[rY - 1];
   return dnnrtTensorOp(h, DNNRT_OP_ADD, Y, dY, rY, bias, db, rY, Y, dY, rY, 1.0f, dtype);
 }
+/* No reference wrapper of its own: per head, the reference's chain of
+ * CUDAMatmulNdFunc.cu (scores), the scaling multiply, CUDASoftmaxFunc.cu (over
+ * the keys, maximum subtracted) and CUDAMatmulNdFunc.cu again; the Reshape /
+ * Transpose calls around them only move data.  Each stage is stored in fp32
+ * as the chain would store it. */
+void *dnnrtAttention(dnnrtHandle_t h, const void *Q, const void *K, const void *V, void *Y,
+                     int64_t B, int64_t Sq, int64_t Sk, int64_t H, int64_t D, float scale,
+                     int32_t dtype) {
+  (void)h;
+  if (dtype != DNNRT_F32) FAIL("attention: fp32 only");
+  if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0 || D <= 0) FAIL("attention: bad dims");
+  const float *q = (const float *)Q, *k = (const float *)K, *v = (const float *)V;
+  float *y = (float *)Y;
+  const int64_t ld = H * D;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t b = 0; b < B; b++)
+    for (int64_t hd = 0; hd < H; hd++) {
+      float *p = (float *)malloc((size_t)Sk * sizeof(float));
+      for (int64_t i = 0; i < Sq; i++) {
+        const float *qi = q + (b * Sq + i) * ld + hd * D;
+        float mx = -INFINITY;
+        for (int64_t j = 0; j < Sk; j++) {
+          const float *kj = k + (b * Sk + j) * ld + hd * D;
+          double acc = 0.0;
+          for (int64_t d = 0; d < D; d++) acc += (double)qi[d] * (double)kj[d];
+          p[j] = (float)acc * scale;
+          mx = p[j] > mx ? p[j] : mx;
+        }
+        double sum = 0.0;
+        for (int64_t j = 0; j < Sk; j++) { p[j] = expf(p[j] - mx); sum += p[j]; }
+        for (int64_t j = 0; j < Sk; j++) p[j] = (float)(p[j] / sum);
+        for (int64_t d = 0; d < D; d++) {
+          double acc = 0.0;
+          for (int64_t j = 0; j < Sk; j++) acc += (double)p[j] * (double)v[(b * Sk + j) * ld + hd * D + d];
+          y[(b * Sq + i) * ld + hd * D + d] = (float)acc;
+        }
+      }
+      free(p);
+    }
+  return Y;
+}
 
 /* ---- data movement -------------------------------------------------------- */
 

@@ -221,3 +221,13 @@ def matmul_nd_bias(be, a, b, bias):
     be.ops.matmul_nd_bias(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Bi), be.ptr(Y), y_shape, DT[a.dtype])
     be.sync()
     return be.get(Y)
+
+
+def attention(be, q, k, v, heads, scale):
+    """q [B, Sq, heads*D], k and v [B, Sk, heads*D]."""
+    B, Sq, hidden = q.shape
+    Q, K, V = be.put(q), be.put(k), be.put(v)
+    Y = be.empty(q.shape, q.dtype)
+    be.ops.attention(be.ptr(Q), be.ptr(K), be.ptr(V), be.ptr(Y), B, Sq, k.shape[1], heads, hidden // heads, scale, DT[q.dtype])
+    be.sync()
+    return be.get(Y)

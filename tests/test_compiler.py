@@ -171,6 +171,19 @@ def test_recompose_flag():
     assert got.count("dnn.matmulnd-bias") == 12 and got.count("dnn.matmulnd") == 4 and got.count("dnn.add") == 6
 
 
+def test_attention_fusion_flag():
+    small = dict(layers=2, hidden=64, heads=2, ffn=128, seq=16, vocab=100)
+    names = lambda p: [n for n, *_ in p.compute_ops()]  # noqa: E731
+    p = check_lifetimes(lambda: models.bert_encoder(**small), fuse_attention=True)
+    got = names(p)
+    # per layer: 3 head splits (Reshape + Transpose), two MatMuls, the scaling, Softmax and the head merge go
+    assert got.count("dnn.attention") == 2 and "dnn.softmax" not in got and "dnn.transpose" not in got and "dnn.reshape" not in got
+    assert "heads=2, scale=0.176777" in p.text
+    # head size 16 has no kernel: the graph is left as it is
+    g, _ = models.bert_encoder(layers=1, hidden=64, heads=4, ffn=128, seq=16, vocab=100)
+    assert "dnn.attention" not in names(g.compile(fuse_attention=True))
+
+
 def test_recompose_leaves_near_misses_alone():
     def ln_graph(eps_node="eps", power=2.0, extra_reader=False, axes=(-1,)):
         g = compiler.Graph()

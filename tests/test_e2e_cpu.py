@@ -190,7 +190,7 @@ def test_activation_fusion_matches_unfused_chain(builder):
 
 def test_recomposed_bert_matches_torch_and_the_decomposed_program():
     small = dict(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100)
-    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True)
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)
     a = check(lambda: models.bert_encoder(**small), rtol=1e-4, atol=1e-4)
     b = check(lambda: models.bert_encoder(**small), rtol=1e-4, atol=1e-4, **flags)
     np.testing.assert_allclose(a[0], b[0], rtol=1e-4, atol=1e-4)

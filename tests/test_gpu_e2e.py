@@ -169,7 +169,7 @@ def test_activation_fusion_fp32(name, oracle_outputs):
 
 
 def test_bert_recomposed_with_fused_linear_layers(oracle_outputs):
-    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True)
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)
     out, _ = run(CONFIGS["bert_2_layers"], **flags)
     close(out[0], oracle_outputs["bert_2_layers"][0], 1e-4, 1e-4)
     out, _ = run(CONFIGS["bert_2_layers"], mode=compiler.MODE_RESIDENT, **flags)

@@ -267,6 +267,18 @@ def test_matmul_nd_bias(gpu, cpu):
         oc.matmul_nd_bias(gpu, a.astype(np.float16), b.astype(np.float16), bias.astype(np.float16))  # not built: loud
 
 
+def test_attention(gpu, cpu):
+    r = rng(45)
+    # BERT-base's shape; key counts around the 32-key wavefront slice and the 128-key block; every head size
+    for B, Sq, Sk, H, D in [(1, 128, 128, 12, 64), (2, 50, 77, 3, 32), (1, 300, 300, 2, 128), (1, 1, 5, 1, 64), (1, 33, 129, 4, 64),
+                            (3, 64, 31, 2, 64), (1, 40, 512, 2, 64)]:
+        q, k, v = (r.standard_normal((B, S, H * D)).astype(np.float32) for S in (Sq, Sk, Sk))
+        q *= 2.0                                              # sharper soft-max: the running maximum moves between blocks
+        close(oc.attention(gpu, q, k, v, H, 1.0 / np.sqrt(D)), oc.attention(cpu, q, k, v, H, 1.0 / np.sqrt(D)), 1e-4, 1e-5)
+    with pytest.raises(RuntimeError):
+        oc.attention(gpu, q[:, :, :96], k[:, :, :96], v[:, :, :96], 2, 1.0)   # head size 48
+
+
 # ---- data movement -------------------------------------------------------------------------
 
 def test_data_movement(gpu, cpu):

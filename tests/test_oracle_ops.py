@@ -329,6 +329,33 @@ def test_matmul_nd_bias(be):
         np.testing.assert_allclose(oc.matmul_nd_bias(be, a, b, bias), ref, rtol=1e-5, atol=1e-5)
 
 
+def attention_ref(q, k, v, heads, scale):
+    B, Sq, hidden = q.shape
+    D = hidden // heads
+    qh = t64(q).reshape(B, Sq, heads, D).permute(0, 2, 1, 3)
+    kh = t64(k).reshape(B, -1, heads, D).permute(0, 2, 1, 3)
+    vh = t64(v).reshape(B, -1, heads, D).permute(0, 2, 1, 3)
+    p = torch.softmax(qh @ kh.transpose(-1, -2) * scale, -1)
+    return (p @ vh).permute(0, 2, 1, 3).reshape(B, Sq, hidden).numpy()
+
+
+def test_attention(be):
+    r = rng(35)
+    for B, Sq, Sk, H, D in [(1, 16, 16, 4, 64), (2, 5, 9, 3, 32), (1, 7, 1, 2, 128)]:
+        q, k, v = (r.standard_normal((B, S, H * D)).astype(np.float32) for S in (Sq, Sk, Sk))
+        got = oc.attention(be, q, k, v, H, 1.0 / math.sqrt(D))
+        np.testing.assert_allclose(got, attention_ref(q, k, v, H, 1.0 / math.sqrt(D)), rtol=1e-5, atol=1e-6)
+    # one key: the soft-max is 1 and the output is that key's value row, whatever the scores
+    np.testing.assert_allclose(got, np.broadcast_to(v, got.shape), rtol=1e-6, atol=1e-6)
+    # heads do not mix: changing head 1's keys leaves head 0's output alone
+    q, k, v = (r.standard_normal((1, 6, 128)).astype(np.float32) for _ in range(3))
+    a = oc.attention(be, q, k, v, 2, 0.125)
+    k2 = k.copy(); k2[:, :, 64:] *= 2.0
+    b = oc.attention(be, q, k2, v, 2, 0.125)
+    np.testing.assert_array_equal(a[:, :, :64], b[:, :, :64])
+    assert np.abs(a[:, :, 64:] - b[:, :, 64:]).max() > 1e-3
+
+
 # ---- data movement --------------------------------------------------------------------------------
 
 def test_data_movement(be):
