@@ -295,25 +295,32 @@ void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
                     int32_t rankA, const void *B, const int64_t *dimB,
                     int32_t rankB, void *Y, const int64_t *dimY, int32_t rankY,
                     int32_t dtype);
-/* The same with one row of N values added to every row of every product:
- * Y = A B + bias.  No reference wrapper: the reference runs CUDAMatmulNdFunc
- * and then cudnnAddTensor with the bias broadcast (Ops/cudnn/Add.cpp), which
- * is what a transformer's Linear layers lower to.  fp32 only. */
+/* The same with a Linear layer's epilogue: Y = act((A B + bias) + Z), bias one
+ * row of N values added to every row of every product, Z an optional residual
+ * tensor shaped like Y (NULL: none), act = Gelu if `gelu` != 0 else identity.
+ * No reference wrapper: the reference runs CUDAMatmulNdFunc and then the
+ * broadcast add of the bias (Ops/cudnn/Add.cpp), the residual add, and Gelu
+ * operator by operator (Div, Erf, Add, Mul, Mul).  fp32 only. */
 void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
                         int32_t rankA, const void *B, const int64_t *dimB,
-                        int32_t rankB, const void *bias, void *Y,
-                        const int64_t *dimY, int32_t rankY, int32_t dtype);
+                        int32_t rankB, const void *bias, const void *Z,
+                        int32_t gelu, void *Y, const int64_t *dimY,
+                        int32_t rankY, int32_t dtype);
 /* Multi-head attention core, Y = softmax(scale * Q K^T) V per head, with Q
  * [batch, seqQ, heads*headDim], K and V [batch, seqK, heads*headDim] and Y like
  * Q.  No reference wrapper: it stands for the chain the reference runs call
  * by call for an exported transformer (CUDAReshapeFunc + CUDATranspose4DFloatFunc
  * per operand, CUDAMatmulNdFunc, the scaling Mul, CUDASoftmaxFunc,
- * CUDAMatmulNdFunc, Transpose + Reshape back).  fp32, headDim 32 / 64 / 128,
+ * CUDAMatmulNdFunc, Transpose + Reshape back).  ldIn is the row stride of Q, K
+ * and V in elements (0: heads*headDim); with the three projections computed
+ * by one product into a [batch, seq, 3*heads*headDim] tensor, Q, K and V are
+ * that tensor's base plus 0, 1 and 2 times heads*headDim and ldIn is its row
+ * length.  Y's rows are heads*headDim long.  fp32, headDim 32 / 64 / 128,
  * 16-byte aligned operands, Y distinct from the inputs. */
 void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void *K,
                      const void *V, void *Y, int64_t batch, int64_t seqQ,
-                     int64_t seqK, int64_t heads, int64_t headDim, float scale,
-                     int32_t dtype);
+                     int64_t seqK, int64_t heads, int64_t headDim, int64_t ldIn,
+                     float scale, int32_t dtype);
 
 /* ---- data movement --------------------------------------------------- */
 

@@ -63,8 +63,8 @@ SIGNATURES = {
     "dnnrtAveragePool": (P, [P, P, I64P, P, I64P, I64P, I64P, I64P, i32]),
     "dnnrtMatmul2d": (P, [P, i64, P, I64P, P, I64P, P, I64P, P, I64P, f32, f32, i64, i64, i32]),
     "dnnrtMatmulNd": (P, [P, P, I64P, i32, P, I64P, i32, P, I64P, i32, i32]),
-    "dnnrtMatmulNdBias": (P, [P, P, I64P, i32, P, I64P, i32, P, P, I64P, i32, i32]),
-    "dnnrtAttention": (P, [P, P, P, P, P, i64, i64, i64, i64, i64, f32, i32]),
+    "dnnrtMatmulNdBias": (P, [P, P, I64P, i32, P, I64P, i32, P, P, i32, P, I64P, i32, i32]),
+    "dnnrtAttention": (P, [P, P, P, P, P, i64, i64, i64, i64, i64, i64, f32, i32]),
     "dnnrtFlatten": (P, [P, P, I64P, P, I64P, i32, i64, i32]),
     "dnnrtReshape": (P, [P, P, I64P, i64, P, i32]),
     "dnnrtSqueeze": (P, [P, P, I64P, i64, P, I64P, i64, i32]),

@@ -24,7 +24,7 @@ constexpr int ATT_QB = 32, ATT_KB = 128;
 template <int DH>
 __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restrict__ Q, const float *__restrict__ K,
                                                             const float *__restrict__ V, float *__restrict__ Y, int Sq,
-                                                            int Sk, int ld, float scale) {
+                                                            int Sk, int ld_in, int ld, float scale) {
   constexpr int ROW = DH + 4;       // LDS row stride in floats: 16-byte aligned rows, 16-byte reads spread over the banks
   constexpr int TD = DH / 32;       // 32-wide tiles of the head dimension
   extern __shared__ float smem[];
@@ -35,15 +35,15 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
   float *sm = mx + 4 * 32;          // [4][32] final sums per wavefront
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
   const int q0 = blockIdx.x * ATT_QB, head = blockIdx.y, b = blockIdx.z;
-  const float *Qg = Q + (int64_t)b * Sq * ld + head * DH;
-  const float *Kg = K + (int64_t)b * Sk * ld + head * DH;
-  const float *Vg = V + (int64_t)b * Sk * ld + head * DH;
+  const float *Qg = Q + (int64_t)b * Sq * ld_in + head * DH;
+  const float *Kg = K + (int64_t)b * Sk * ld_in + head * DH;
+  const float *Vg = V + (int64_t)b * Sk * ld_in + head * DH;
 
   // the query tile (rows past the end repeat the last query; they are not stored)
   for (int i = tid; i < ATT_QB * (DH / 4); i += 256) {
     const int r = i / (DH / 4), c4 = i - r * (DH / 4);
     *reinterpret_cast<float4 *>(Qs + r * ROW + c4 * 4) =
-        *reinterpret_cast<const float4 *>(Qg + (int64_t)min(q0 + r, Sq - 1) * ld + c4 * 4);
+        *reinterpret_cast<const float4 *>(Qg + (int64_t)min(q0 + r, Sq - 1) * ld_in + c4 * 4);
   }
 
   floatx16 o[TD];
@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
     __syncthreads();  // everyone is done with the previous block's K and V
     for (int i = tid; i < ATT_KB * (DH / 4); i += 256) {
       const int r = i / (DH / 4), c4 = i - r * (DH / 4);
-      const int64_t row = (int64_t)min(kb + r, Sk - 1) * ld + c4 * 4;
+      const int64_t row = (int64_t)min(kb + r, Sk - 1) * ld_in + c4 * 4;
       *reinterpret_cast<float4 *>(Ks + r * ROW + c4 * 4) = *reinterpret_cast<const float4 *>(Kg + row);
       *reinterpret_cast<float4 *>(Vs + r * ROW + c4 * 4) = *reinterpret_cast<const float4 *>(Vg + row);
     }
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
 
 template <int DH>
 static void launch_attention(const dnnrtContext *ctx, const float *Q, const float *K, const float *V, float *Y, int B,
-                             int Sq, int Sk, int H, float scale) {
+                             int Sq, int Sk, int H, int ld_in, float scale) {
   constexpr int ROW = DH + 4;
   const size_t lds = (size_t)((ATT_QB + 2 * ATT_KB) * ROW + 8 * 32) * sizeof(float);
   static bool raised = false;  // per instantiation: more than 64 KiB of dynamic LDS must be asked for once
@@ -153,7 +153,7 @@ static void launch_attention(const dnnrtContext *ctx, const float *Q, const floa
     raised = true;
   }
   hipLaunchKernelGGL((attention_f32_kernel<DH>), dim3((unsigned)ceil_div(Sq, ATT_QB), (unsigned)H, (unsigned)B), dim3(256),
-                     lds, ctx->stream, Q, K, V, Y, Sq, Sk, H * DH, scale);
+                     lds, ctx->stream, Q, K, V, Y, Sq, Sk, ld_in, H * DH, scale);
 }
 
 }  // namespace dnnrt
@@ -162,7 +162,7 @@ using namespace dnnrt;
 
 extern "C" void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void *K, const void *V, void *Y,
                                 int64_t batch, int64_t seqQ, int64_t seqK, int64_t heads, int64_t headDim,
-                                float scale, int32_t dtype) {
+                                int64_t ldIn, float scale, int32_t dtype) {
   if (!handle) DNNRT_FAIL("dnnrtAttention: null handle");
   if (!Q || !K || !V || !Y) DNNRT_FAIL("dnnrtAttention: null argument");
   if (dtype != DNNRT_F32) DNNRT_FAIL("dnnrtAttention: dtype %d (fp32 only)", dtype);
@@ -171,10 +171,12 @@ extern "C" void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void 
   if (headDim != 32 && headDim != 64 && headDim != 128) DNNRT_FAIL("dnnrtAttention: head dim %ld (32, 64, 128)", (long)headDim);
   if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(Y)) DNNRT_FAIL("dnnrtAttention: operands must be 16-byte aligned");
   if (Y == Q || Y == K || Y == V) DNNRT_FAIL("dnnrtAttention: Y must not alias an input");
+  if (ldIn == 0) ldIn = heads * headDim;
+  if (ldIn < heads * headDim || ldIn % 4 || ldIn > INT32_MAX) DNNRT_FAIL("dnnrtAttention: ldIn %ld (>= heads * headDim, multiple of 4)", (long)ldIn);
   const float *q = (const float *)Q, *k = (const float *)K, *v = (const float *)V;
-  if (headDim == 32) launch_attention<32>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, scale);
-  else if (headDim == 64) launch_attention<64>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, scale);
-  else launch_attention<128>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, scale);
+  if (headDim == 32) launch_attention<32>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
+  else if (headDim == 64) launch_attention<64>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
+  else launch_attention<128>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
   DNNRT_CHECK_LAUNCH("dnnrtAttention");
   return Y;
 }

@@ -55,12 +55,16 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline bool float_dtype(int32_t dt) { return dt == DNNRT_F32 || dt == DNNRT_F16; }
 
+// Gelu as an epilogue of the matrix products only (not an activMode of the convolution calls).
+constexpr int ACT_GELU = 7;
+
 // The activations a convolution epilogue can apply (sigmoid and tanh are
 // separate calls, as in the reference).
 __device__ __forceinline__ float apply_act(float v, int act, float coef) {
   if (act == DNNRT_ACT_RELU) return v < 0.f ? 0.f : v;
   if (act == DNNRT_ACT_CLIPPED_RELU) { v = v < 0.f ? 0.f : v; return v > coef ? coef : v; }
   if (act == DNNRT_ACT_LEAKY_RELU) return v < 0.f ? coef * v : v;
+  if (act == ACT_GELU) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
   return v;
 }
 __host__ __device__ inline bool fusable_act(int64_t act) {

@@ -366,8 +366,9 @@ struct Emitter {
       if (!k || !v) { err = "FusedAttention: K or V not available"; return false; }
       out_buf = malloc_(ot.dtype, ot.shape);
       Op *o = compute(OP_ATTENTION, {x, k, v, out_buf});
-      o->dimA = x->shape;
-      o->dimB = k->shape;
+      o->axis = int1("packed", 0);  // 1: the three operands are one [B, S, 3*hidden] tensor
+      o->dimA = ot.shape;
+      o->dimB = o->axis ? ot.shape : k->shape;
       o->group = int1("heads", 1);
       o->alpha = (float)flt("scale", 1.0);
       result = o->result;

@@ -348,12 +348,20 @@ bool Session::issue(const Op *op, std::string &err) {
                            (int32_t)op->dimB.size(), out, op->dimOut.data(), (int32_t)op->dimOut.size(), dt);
       break;
     case OP_ATTENTION:  // operands: q, k, v, out
-      r = rt.dnnrtAttention(handle, P(0), P(1), P(2), out, op->dimA[0], op->dimA[1], op->dimB[1], op->group,
-                            op->dimA[2] / op->group, op->alpha, dt);
+      if (op->axis) {  // one tensor holds [Q | K | V] per row
+        const int64_t hidden = op->dimA[2];
+        char *base = (char *)P(0);
+        r = rt.dnnrtAttention(handle, base, base + hidden * 4, base + 2 * hidden * 4, out, op->dimA[0], op->dimA[1], op->dimB[1],
+                              op->group, hidden / op->group, 3 * hidden, op->alpha, dt);
+      } else {
+        r = rt.dnnrtAttention(handle, P(0), P(1), P(2), out, op->dimA[0], op->dimA[1], op->dimB[1], op->group,
+                              op->dimA[2] / op->group, 0, op->alpha, dt);
+      }
       break;
-    case OP_MATMUL_BIAS:  // operands: a, b, bias, out
+    case OP_MATMUL_BIAS:  // operands: a, b, bias, [residual,] out
       r = rt.dnnrtMatmulNdBias(handle, P(0), op->dimA.data(), (int32_t)op->dimA.size(), P(1), op->dimB.data(),
-                               (int32_t)op->dimB.size(), P(2), out, op->dimOut.data(), (int32_t)op->dimOut.size(), dt);
+                               (int32_t)op->dimB.size(), P(2), op->operands.size() == 5 ? P(3) : nullptr, op->mode == 7,
+                               out, op->dimOut.data(), (int32_t)op->dimOut.size(), dt);
       break;
     default: err = std::string("executor: unexpected op ") + op_name(op->kind); return false;
   }

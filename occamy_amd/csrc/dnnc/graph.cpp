@@ -396,14 +396,63 @@ static bool match_attention(const Matcher &m, const GNode &root, GNode &fused, s
   return true;
 }
 
+// Q, K and V of a matched attention block that are three Linear layers of the
+// same input, Add(bias, MatMul(x, W)) with constant W [in, hidden] and bias
+// [hidden], read by nothing else: one product with the three weight matrices
+// side by side gives a [B, S, 3*hidden] tensor whose rows hold Q | K | V, and
+// the attention call reads its operands out of that tensor.
+static void pack_qkv(const Matcher &m, GNode &fused, std::vector<std::string> &dead, std::vector<GNode> &pre) {
+  Graph &g = m.g;
+  const GNode *add[3], *mm[3];
+  std::string bias[3];
+  for (int i = 0; i < 3; i++) {
+    if (!(add[i] = m.def(fused.inputs[(size_t)i], "Add")) || !m.split(*add[i], "MatMul", mm[i], bias[i])) return;
+    if (!m.single_use(add[i]->output) || !m.single_use(mm[i]->output) || mm[i]->inputs.size() != 2) return;
+    if (mm[i]->inputs[0] != mm[0]->inputs[0]) return;
+  }
+  const GTensor *w[3], *b[3];
+  for (int i = 0; i < 3; i++) {
+    auto wi = g.tensors.find(mm[i]->inputs[1]), bi = g.tensors.find(bias[i]);
+    if (wi == g.tensors.end() || bi == g.tensors.end() || !wi->second.is_const || !bi->second.is_const) return;
+    w[i] = &wi->second; b[i] = &bi->second;
+    if (w[i]->dtype != F32 || b[i]->dtype != F32 || w[i]->shape.size() != 2 || w[i]->shape != w[0]->shape ||
+        b[i]->shape != Shape{w[i]->shape[1]})
+      return;
+  }
+  const int64_t in = w[0]->shape[0], hid = w[0]->shape[1];
+  const std::string base = fused.output + "_qkv", wn = base + "_w", bn = base + "_b", mn = base + "_mm";
+  if (g.tensors.count(base) || g.tensors.count(wn) || g.tensors.count(bn) || g.tensors.count(mn)) return;
+  GTensor wt, bt;
+  wt.name = wn; wt.dtype = F32; wt.shape = {in, 3 * hid}; wt.is_const = true; wt.data.resize((size_t)(in * 3 * hid * 4));
+  bt.name = bn; bt.dtype = F32; bt.shape = {3 * hid}; bt.is_const = true; bt.data.resize((size_t)(3 * hid * 4));
+  for (int i = 0; i < 3; i++) {
+    for (int64_t r = 0; r < in; r++)
+      std::memcpy(wt.data.data() + ((r * 3 + i) * hid) * 4, w[i]->data.data() + r * hid * 4, (size_t)hid * 4);
+    std::memcpy(bt.data.data() + (int64_t)i * hid * 4, b[i]->data.data(), (size_t)hid * 4);
+  }
+  g.tensors[wn] = std::move(wt);
+  g.tensors[bn] = std::move(bt);
+  GNode cw, cb, nm, na;
+  cw.op_type = "Constant"; cw.output = wn;
+  cb.op_type = "Constant"; cb.output = bn;
+  nm.op_type = "MatMul"; nm.inputs = {mm[0]->inputs[0], wn}; nm.output = mn;
+  na.op_type = "Add"; na.inputs = {bn, mn}; na.output = base;  // bias first, as exporters write it
+  pre = {cw, cb, nm, na};
+  for (int i = 0; i < 3; i++) { dead.push_back(add[i]->output); dead.push_back(mm[i]->output); }
+  fused.inputs = {base, base, base};
+  fused.ints["packed"] = {1};
+}
+
 static bool recompose(Graph &g, bool norms, bool attention) {
   bool any = false;
   for (size_t i = 0; i < g.nodes.size(); i++) {
     Matcher m(g);
     GNode fused;
     std::vector<std::string> dead;
-    const bool hit = (attention && match_attention(m, g.nodes[i], fused, dead)) ||
-                     (norms && (match_layernorm(m, g.nodes[i], fused, dead) || match_gelu(m, g.nodes[i], fused, dead)));
+    std::vector<GNode> pre;  // nodes to put in front of the fused one
+    bool hit = attention && match_attention(m, g.nodes[i], fused, dead);
+    if (hit) pack_qkv(m, fused, dead, pre);
+    else hit = norms && (match_layernorm(m, g.nodes[i], fused, dead) || match_gelu(m, g.nodes[i], fused, dead));
     if (!hit) continue;
     // constants read by the matched nodes only go with them
     std::vector<std::string> consts;
@@ -417,6 +466,7 @@ static bool recompose(Graph &g, bool norms, bool attention) {
       if (t != g.tensors.end() && t->second.is_const) consts.push_back(in);
     }
     g.nodes[i] = fused;
+    g.nodes.insert(g.nodes.begin() + (long)i, pre.begin(), pre.end());
     std::vector<GNode> kept;
     for (GNode &n : g.nodes)
       if (std::find(dead.begin(), dead.end(), n.output) == dead.end()) kept.push_back(n);
@@ -487,6 +537,7 @@ static bool infer_pass(Graph &g, std::string &err) {
     } else if (t == "FusedAttention") {  // produced by the recomposition only
       if (in.size() != 3 || !in[1] || !in[2] || x.size() != 3) return fail("needs Q, K and V of rank 3");
       out.shape = x;
+      if (get_int(n, "packed", 0)) out.shape[2] = x[2] / 3;
     } else if (t == "PRelu") {
       if (in.size() < 2 || !in[1]) return fail("needs a slope");
       Shape b;

@@ -201,7 +201,8 @@ std::string Program::to_text() const {
       case OP_CONCAT:
       case OP_GATHER: os << " {axis=" << op->axis << "}"; break;
       case OP_LEAKYRELU: os << " {alpha=" << op->alpha << "}"; break;
-      case OP_ATTENTION: os << " {heads=" << op->group << ", scale=" << op->alpha << "}"; break;
+      case OP_MATMUL_BIAS: if (op->mode == 7) os << " {gelu}"; break;
+      case OP_ATTENTION: os << " {heads=" << op->group << ", scale=" << op->alpha << (op->axis ? ", packed" : "") << "}"; break;
       case OP_SQUEEZE:
       case OP_UNSQUEEZE: os << " {axes="; print_shape(os, op->perm); os << "}"; break;
       case OP_TRANSPOSE: os << " {perm="; print_shape(os, op->perm); os << "}"; break;

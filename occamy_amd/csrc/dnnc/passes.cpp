@@ -216,6 +216,7 @@ void fuse_matmul_bias(Program &p) {
     fused->dimA = mm->dimA;
     fused->dimB = mm->dimB;
     fused->dimOut = mm->dimOut;
+    fused->mode = 5;
     fused->result = p.new_value(out->dtype, out->shape);
     fused->result->def = fused;
     p.insert_after(fused, add);
@@ -223,6 +224,45 @@ void fuse_matmul_bias(Program &p) {
     p.replace_all_uses(add->result, fused->result);
     p.erase(add);
     p.erase(mm);
+    if (buf != out) {
+      std::vector<Op *> deallocs;
+      for (const auto &u : buf->uses)
+        if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+      for (Op *d : deallocs) p.erase(d);
+      if (buf->uses.empty() && buf->def) p.erase(buf->def);
+    }
+  }
+  // second step: the Linear layer's consumer joins in when it is the only
+  // reader -- Gelu (mode 7), or the sum with a residual tensor of the same shape
+  std::vector<Op *> linears;
+  for (Op *op : p.ops)
+    if (op->kind == OP_MATMUL_BIAS && op->operands.size() == 4 && op->mode != 7) linears.push_back(op);
+  for (Op *lin : linears) {
+    if (lin->result->uses.size() != 1) continue;
+    Op *next = lin->result->uses.front().first;
+    Value *z = nullptr;
+    if (next->kind == OP_GELU && next->operands[0] == lin->result) {
+    } else if (next->kind == OP_ADD && next->coef == 1.f && next->dimA == next->dimB &&
+               (next->operands[0] == lin->result) != (next->operands[1] == lin->result)) {
+      z = next->operands[0] == lin->result ? next->operands[1] : next->operands[0];
+      if (z->shape != lin->result->shape) continue;
+    } else {
+      continue;
+    }
+    Value *out = next->operands.back(), *buf = lin->operands[3];
+    Op *fused = p.new_op(OP_MATMUL_BIAS);
+    fused->dimA = lin->dimA;
+    fused->dimB = lin->dimB;
+    fused->dimOut = lin->dimOut;
+    fused->mode = z ? 5 : 7;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    p.insert_after(fused, next);
+    if (z) p.set_operands(fused, {lin->operands[0], lin->operands[1], lin->operands[2], z, out});
+    else p.set_operands(fused, {lin->operands[0], lin->operands[1], lin->operands[2], out});
+    p.replace_all_uses(next->result, fused->result);
+    p.erase(next);
+    p.erase(lin);
     if (buf != out) {
       std::vector<Op *> deallocs;
       for (const auto &u : buf->uses)

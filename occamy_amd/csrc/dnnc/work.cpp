@@ -58,12 +58,13 @@ void op_work(const Op *op, double &flops, double &bytes) {
     case OP_MATMULND:
     case OP_MATMUL_BIAS: {
       flops = 2.0 * n_out * (double)op->dimA.back();
-      bytes = (n_in(0) + n_in(1) + n_out + (op->kind == OP_MATMUL_BIAS ? n_in(2) : 0.0)) * es;
+      bytes = (n_in(0) + n_in(1) + n_out + (op->kind == OP_MATMUL_BIAS ? n_in(2) : 0.0) +
+               (op->kind == OP_MATMUL_BIAS && op->operands.size() == 5 ? n_out : 0.0)) * es;
       break;
     }
     case OP_ATTENTION:  // two products of 2 * B * H * Sq * Sk * D each
-      flops = 4.0 * n_in(0) * (double)op->dimB[1];
-      bytes = (n_in(0) + n_in(1) + n_in(2) + n_out) * es;
+      flops = 4.0 * n_out * (double)op->dimB[1];
+      bytes = (op->axis ? 4.0 * n_out : n_in(0) + n_in(1) + n_in(2) + n_out) * es;
       break;
     case OP_ADD:
     case OP_MUL:

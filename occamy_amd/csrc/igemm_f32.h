@@ -1,7 +1,7 @@
 // fp32 implicit-GEMM on gfx950 MFMA: one kernel family serves dense
 // convolution (NCHW), 2-D GEMM and batched matmul.
 //
-//   D[m, col] = act(alpha * sum_k A[m, k] * B[k, col] + bias[m] + beta * Cin[m, col])
+//   D[m, col] = act(alpha * sum_k A[m, k] * B[k, col] + bias[m] + bias_col[col] + beta * Cin[m, col])
 //
 // A is the weight / left matrix, B the im2col view of the input / right
 // matrix.  Columns are output pixels (n, p, q) flattened; for a plain matrix
@@ -17,6 +17,7 @@ struct IgemmArgs {
   const float *X;     // conv input / right matrix
   float *Y;
   const float *bias;  // per row m, may be null
+  const float *bias_col;  // per column (shared by every z), may be null
   const float *Cin;   // same indexing as Y, scaled by beta, may be null
   float alpha, beta;
   int act;            // DNNRT_ACT_{IDENTITY, RELU, CLIPPED_RELU, LEAKY_RELU}
@@ -44,6 +45,8 @@ bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a);
 // The variant for problems too small to fill the chip with LDS-staged tiles
 // (igemm_f32_direct.hip); rsmode / layout as computed by launch_igemm_f32.
 bool launch_igemm_f32_direct(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout);
+// Row-major products with a few hundred rows (gemm_f32_rows.hip); `launched` says whether it applied.
+bool launch_gemm_f32_rows(const dnnrtContext *ctx, const IgemmArgs &a, bool &launched);
 // 3x3 / 1x1 specialisations of the above (igemm_f32_small.hip); `launched` says whether one applied.
 bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout, bool &launched);
 

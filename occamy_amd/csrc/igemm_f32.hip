@@ -233,6 +233,7 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
     const int colc = col_ok ? col : 0;
     const int img = colc / PQ, pq = colc - img * PQ;
     const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
+    const float bias_c = a.bias_col ? a.bias_col[colc] : 0.f;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       float res_r[16];
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int m = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * lrow + (r & 3);
-        float v = a.alpha * acc[i][j][r] + bias_r[i][r];
+        float v = a.alpha * acc[i][j][r] + bias_r[i][r] + bias_c;
         if (a.Cin) v += a.beta * res_r[r];
         v = apply_act(v, a.act, a.act_coef);
         if (col_ok && m < a.M) Yg[ycol + (int64_t)m * a.y_row_stride] = v;

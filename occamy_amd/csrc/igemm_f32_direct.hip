@@ -134,6 +134,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
   const int img = colc / PQ, pq = colc - img * PQ;
   const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
   float bias_r[16], res_r[16];
+  const float bias_c = a.bias_col ? a.bias_col[colc] : 0.f;
   if (a.bias) {
     const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
 #pragma unroll
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
 #pragma unroll
   for (int r = 0; r < 16; r++) {
     const int mm = m0 + 8 * (r >> 2) + 4 * half + (r & 3);
-    float v = a.alpha * acc[r] + bias_r[r];
+    float v = a.alpha * acc[r] + bias_r[r] + bias_c;
     if (a.Cin) v += a.beta * res_r[r];
     v = apply_act(v, a.act, a.act_coef);
     if (col_ok && mm < a.M) Yg[ycol + (int64_t)mm * a.y_row_stride] = v;

@@ -60,6 +60,7 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
   // the residual tensor's 16 values, requested before anything is waited for
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
+  const float bias_c = a.bias_col ? a.bias_col[col_ok ? col : 0] : 0.f;
   float res_r[16];
   if (a.Cin) {
     if (wave == 0) {
@@ -123,7 +124,7 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     for (int r = 0; r < 16; r++) {
       const int mm = acc_row(m0, half, r);
       if (mm >= a.M) continue;
-      float v = a.alpha * acc[r] + bias_r[r];
+      float v = a.alpha * acc[r] + bias_r[r] + bias_c;
       if (a.Cin) v += a.beta * res_r[r];
       Yg[ycol + (int64_t)mm * a.y_row_stride] = apply_act(v, MODE, a.act_coef);
     }
@@ -132,6 +133,7 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     case DNNRT_ACT_RELU: store(std::integral_constant<int, DNNRT_ACT_RELU>{}); break;
     case DNNRT_ACT_CLIPPED_RELU: store(std::integral_constant<int, DNNRT_ACT_CLIPPED_RELU>{}); break;
     case DNNRT_ACT_LEAKY_RELU: store(std::integral_constant<int, DNNRT_ACT_LEAKY_RELU>{}); break;
+    case ACT_GELU: store(std::integral_constant<int, ACT_GELU>{}); break;
     default: store(std::integral_constant<int, DNNRT_ACT_IDENTITY>{}); break;
   }
 }

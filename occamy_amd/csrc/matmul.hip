@@ -79,9 +79,11 @@ static void launch_gemv(const dnnrtContext *ctx, const float *A, const float *B,
 
 static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, const float *C,
                      float *Out, int M, int N, int K, float alpha, float beta, bool transA,
-                     bool transB, int Z, int64_t az, int64_t bz, int64_t yz, bool c_is_row = false) {
+                     bool transB, int Z, int64_t az, int64_t bz, int64_t yz, bool c_is_row = false,
+                     const float *bias_col = nullptr, int act = DNNRT_ACT_IDENTITY) {
   // c_is_row: C holds one row of N values that is added to every row of every product
-  if (Z == 1 && M <= 8 && transB && !transA) {
+  // bias_col, act: Out = act(alpha * A B + bias_col[n] + beta * C)
+  if (Z == 1 && M <= 8 && transB && !transA && !bias_col && act == DNNRT_ACT_IDENTITY) {
     const bool vec4 = (K % 4 == 0) && aligned16(A) && aligned16(B);
     // wavefronts per output: the fewest that give 2048 wavefronts, each keeping >= 512 elements of k
     int wpo = 1;
@@ -95,7 +97,7 @@ static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, co
   }
   IgemmArgs a{};
   a.A = A; a.X = B; a.Y = Out; a.bias = nullptr; a.Cin = C;
-  a.alpha = alpha; a.beta = beta; a.act = DNNRT_ACT_IDENTITY;
+  a.alpha = alpha; a.beta = beta; a.act = act; a.bias_col = bias_col;
   a.M = M; a.Kdim = K; a.Ncols = N;
   a.H = 1; a.W = N; a.R = 1; a.S = 1; a.P = 1; a.Q = N; a.ph = 0; a.pw = 0; a.sh = 1; a.sw = 1;
   a.x_img_stride = 0; a.y_img_stride = 0; a.y_row_stride = N;
@@ -104,6 +106,9 @@ static bool gemm_f32(const dnnrtContext *ctx, const float *A, const float *B, co
   a.b_kcontig = transB; a.a_mcontig = transA; a.a_ld = M;
   a.a_vec4 = !transA && (K % 4 == 0) && aligned16(A) && (az % 4 == 0);
   a.b_vec4 = transB && (K % 4 == 0) && aligned16(B) && (bz % 4 == 0);
+  bool launched = false;
+  if (!launch_gemm_f32_rows(ctx, a, launched)) return false;
+  if (launched) return true;
   return launch_igemm_f32(ctx, a);
 }
 
@@ -144,8 +149,8 @@ void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A, const int
 }
 
 static void *matmul_nd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
-                       const void *B, const int64_t *dimB, int32_t rankB, const void *bias, void *Y,
-                       const int64_t *dimY, int32_t rankY, int32_t dtype) {
+                       const void *B, const int64_t *dimB, int32_t rankB, const void *bias, const void *Zr, int act,
+                       void *Y, const int64_t *dimY, int32_t rankY, int32_t dtype) {
   if (!handle) DNNRT_FAIL("dnnrtMatmulNd: null handle");
   if (!A || !B || !Y || !dimA || !dimB || !dimY) DNNRT_FAIL("dnnrtMatmulNd: null argument");
   if (rankA < 2 || rankB < 2 || rankA > 4 || rankB > 4 || rankY != (rankA > rankB ? rankA : rankB))
@@ -177,12 +182,13 @@ static void *matmul_nd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
   if (bz == 0 && Z > 1 && az != 0) { Mz = M * batchY; Z = 1; azz = 0; yz = 0; }
   if (Mz > INT32_MAX) DNNRT_FAIL("dnnrtMatmulNd: dims exceed 32 bits");
   if (dtype == DNNRT_F32) {
-    if (!gemm_f32(handle, (const float *)A, (const float *)B, (const float *)bias, (float *)Y, (int)Mz, (int)N, (int)K,
-                  1.f, bias ? 1.f : 0.f, false, false, Z, azz, bz, yz, bias != nullptr))
+    // the residual is laid out like Y: one tall product (yz == 0) or one product per batch
+    if (!gemm_f32(handle, (const float *)A, (const float *)B, (const float *)Zr, (float *)Y, (int)Mz, (int)N, (int)K,
+                  1.f, Zr ? 1.f : 0.f, false, false, Z, azz, bz, yz, false, (const float *)bias, act))
       return nullptr;
     return Y;
   }
-  if (dtype == DNNRT_F16 && bias) DNNRT_FAIL("dnnrtMatmulNdBias: fp16 is not built");
+  if (dtype == DNNRT_F16 && (bias || Zr || act != DNNRT_ACT_IDENTITY)) DNNRT_FAIL("dnnrtMatmulNdBias: fp16 is not built");
   if (dtype == DNNRT_F16) {
     if (!gemm_f16(handle, (const __half *)A, (const __half *)B, nullptr, (__half *)Y, (int)Mz, (int)N,
                   (int)K, 1.f, 0.f, false, false, Z, azz, bz, yz))
@@ -195,14 +201,15 @@ static void *matmul_nd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
 void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
                     const void *B, const int64_t *dimB, int32_t rankB, void *Y, const int64_t *dimY,
                     int32_t rankY, int32_t dtype) {
-  return matmul_nd(handle, A, dimA, rankA, B, dimB, rankB, nullptr, Y, dimY, rankY, dtype);
+  return matmul_nd(handle, A, dimA, rankA, B, dimB, rankB, nullptr, nullptr, DNNRT_ACT_IDENTITY, Y, dimY, rankY, dtype);
 }
 
 void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA, int32_t rankA,
-                        const void *B, const int64_t *dimB, int32_t rankB, const void *bias, void *Y,
-                        const int64_t *dimY, int32_t rankY, int32_t dtype) {
+                        const void *B, const int64_t *dimB, int32_t rankB, const void *bias, const void *Z,
+                        int32_t gelu, void *Y, const int64_t *dimY, int32_t rankY, int32_t dtype) {
   if (!bias) DNNRT_FAIL("dnnrtMatmulNdBias: null bias");
-  return matmul_nd(handle, A, dimA, rankA, B, dimB, rankB, bias, Y, dimY, rankY, dtype);
+  if (Z && Z == Y) DNNRT_FAIL("dnnrtMatmulNdBias: the residual must not be the output buffer");
+  return matmul_nd(handle, A, dimA, rankA, B, dimB, rankB, bias, Z, gelu ? ACT_GELU : DNNRT_ACT_IDENTITY, Y, dimY, rankY, dtype);
 }
 
 }  // extern "C"

@@ -177,15 +177,17 @@ class Ops:
                                                 len(dimB), Y, dims(dimY), len(dimY), dtype),
                          "dnnrtMatmulNd")
 
-    def matmul_nd_bias(self, A, dimA, B, dimB, bias, Y, dimY, dtype=_abi.F32):
+    def matmul_nd_bias(self, A, dimA, B, dimB, bias, Y, dimY, dtype=_abi.F32, Z=None, gelu=False):
+        """Y = act((A B + bias) + Z); Z: optional residual shaped like Y; act: Gelu or identity."""
         return self._ret(self.lib.dnnrtMatmulNdBias(self.handle, A, dims(dimA), len(dimA), B, dims(dimB),
-                                                    len(dimB), bias, Y, dims(dimY), len(dimY), dtype),
+                                                    len(dimB), bias, Z, int(gelu), Y, dims(dimY), len(dimY), dtype),
                          "dnnrtMatmulNdBias")
 
-    def attention(self, Q, K, V, Y, batch, seq_q, seq_k, heads, head_dim, scale, dtype=_abi.F32):
-        """Q [batch, seq_q, heads*head_dim], K and V [batch, seq_k, heads*head_dim], Y like Q."""
+    def attention(self, Q, K, V, Y, batch, seq_q, seq_k, heads, head_dim, scale, dtype=_abi.F32, ld_in=0):
+        """Q [batch, seq_q, heads*head_dim], K and V [batch, seq_k, heads*head_dim], Y like Q;
+        ld_in: row stride of Q, K, V in elements when they are slices of a wider tensor."""
         return self._ret(self.lib.dnnrtAttention(self.handle, Q, K, V, Y, batch, seq_q, seq_k, heads, head_dim,
-                                                 scale, dtype), "dnnrtAttention")
+                                                 ld_in, scale, dtype), "dnnrtAttention")
 
     def flatten(self, X, dimX, Y, dimY, axis, dtype=_abi.F32):
         return self._ret(self.lib.dnnrtFlatten(self.handle, X, dims(dimX), Y, dims(dimY), axis,

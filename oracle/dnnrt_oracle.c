@@ -737,16 +737,21 @@ void *dnnrtMatmulNd(dnnrtHandle_t h, const void *A, const int64_t *dA, int32_t r
   return Y;
 }
 /* No reference wrapper of its own: CUDAMatmulNdFunc.cu, then the broadcast
- * add of CUDNNTensorOpFunc.cpp on the stored product -- restated as that chain. */
+ * add of CUDNNTensorOpFunc.cpp on the stored product, then the residual add
+ * and Gelu (CUDAErfFunc.cu and friends) -- restated as that chain. */
 void *dnnrtMatmulNdBias(dnnrtHandle_t h, const void *A, const int64_t *dA, int32_t rA,
                         const void *B, const int64_t *dB, int32_t rB, const void *bias,
-                        void *Y, const int64_t *dY, int32_t rY, int32_t dtype) {
+                        const void *Z, int32_t gelu, void *Y, const int64_t *dY, int32_t rY,
+                        int32_t dtype) {
   if (!bias) FAIL("matmulNdBias: null bias");
   if (!dnnrtMatmulNd(h, A, dA, rA, B, dB, rB, Y, dY, rY, dtype)) return NULL;
   int64_t db[8];
   for (int i = 0; i < rY; i++) db[i] = 1;
   db[rY - 1] = dY[rY - 1];
-  return dnnrtTensorOp(h, DNNRT_OP_ADD, Y, dY, rY, bias, db, rY, Y, dY, rY, 1.0f, dtype);
+  if (!dnnrtTensorOp(h, DNNRT_OP_ADD, Y, dY, rY, bias, db, rY, Y, dY, rY, 1.0f, dtype)) return NULL;
+  if (Z && !dnnrtTensorOp(h, DNNRT_OP_ADD, Y, dY, rY, Z, dY, rY, Y, dY, rY, 1.0f, dtype)) return NULL;
+  if (gelu && !dnnrtGelu(h, Y, Y, dY, rY, dtype)) return NULL;
+  return Y;
 }
 /* No reference wrapper of its own: per head, the reference's chain of
  * CUDAMatmulNdFunc.cu (scores), the scaling multiply, CUDASoftmaxFunc.cu (over
@@ -754,14 +759,15 @@ void *dnnrtMatmulNdBias(dnnrtHandle_t h, const void *A, const int64_t *dA, int32
  * Transpose calls around them only move data.  Each stage is stored in fp32
  * as the chain would store it. */
 void *dnnrtAttention(dnnrtHandle_t h, const void *Q, const void *K, const void *V, void *Y,
-                     int64_t B, int64_t Sq, int64_t Sk, int64_t H, int64_t D, float scale,
+                     int64_t B, int64_t Sq, int64_t Sk, int64_t H, int64_t D, int64_t ldIn, float scale,
                      int32_t dtype) {
   (void)h;
   if (dtype != DNNRT_F32) FAIL("attention: fp32 only");
   if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0 || D <= 0) FAIL("attention: bad dims");
   const float *q = (const float *)Q, *k = (const float *)K, *v = (const float *)V;
   float *y = (float *)Y;
-  const int64_t ld = H * D;
+  const int64_t ldy = H * D, ld = ldIn ? ldIn : ldy;
+  if (ld < ldy) FAIL("attention: ldIn");
 #pragma omp parallel for collapse(2) schedule(static)
   for (int64_t b = 0; b < B; b++)
     for (int64_t hd = 0; hd < H; hd++) {
@@ -782,7 +788,7 @@ void *dnnrtAttention(dnnrtHandle_t h, const void *Q, const void *K, const void *
         for (int64_t d = 0; d < D; d++) {
           double acc = 0.0;
           for (int64_t j = 0; j < Sk; j++) acc += (double)p[j] * (double)v[(b * Sk + j) * ld + hd * D + d];
-          y[(b * Sq + i) * ld + hd * D + d] = (float)acc;
+          y[(b * Sq + i) * ldy + hd * D + d] = (float)acc;
         }
       }
       free(p);

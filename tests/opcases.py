@@ -214,11 +214,13 @@ def squeeze(be, x, out, un=False):
     return be.get(Y)
 
 
-def matmul_nd_bias(be, a, b, bias):
+def matmul_nd_bias(be, a, b, bias, z=None, gelu=False):
     y_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2]) + (a.shape[-2], b.shape[-1])
     A, B, Bi = be.put(a), be.put(b), be.put(bias)
+    Z = be.put(z) if z is not None else None
     Y = be.empty(y_shape, a.dtype)
-    be.ops.matmul_nd_bias(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Bi), be.ptr(Y), y_shape, DT[a.dtype])
+    be.ops.matmul_nd_bias(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Bi), be.ptr(Y), y_shape, DT[a.dtype],
+                          Z=be.ptr(Z) if Z is not None else None, gelu=gelu)
     be.sync()
     return be.get(Y)
 
@@ -229,5 +231,19 @@ def attention(be, q, k, v, heads, scale):
     Q, K, V = be.put(q), be.put(k), be.put(v)
     Y = be.empty(q.shape, q.dtype)
     be.ops.attention(be.ptr(Q), be.ptr(K), be.ptr(V), be.ptr(Y), B, Sq, k.shape[1], heads, hidden // heads, scale, DT[q.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def attention_packed(be, qkv, heads, scale):
+    """qkv [B, S, 3*hidden]: every row holds Q | K | V."""
+    B, S, three = qkv.shape
+    hidden = three // 3
+    X = be.put(qkv)
+    Y = be.empty((B, S, hidden), qkv.dtype)
+    es = qkv.dtype.itemsize
+    p = be.ptr(X)
+    be.ops.attention(p, p + hidden * es, p + 2 * hidden * es, be.ptr(Y), B, S, S, heads, hidden // heads, scale,
+                     DT[qkv.dtype], ld_in=three)
     be.sync()
     return be.get(Y)

@@ -168,7 +168,13 @@ def test_recompose_flag():
     assert [n for n in ref if n != "dnn.reciprocal"] == got
     p = check_lifetimes(lambda: models.bert_encoder(**small), recompose=True, fusion=True, fuse_matmul_bias=True)
     got = names(p)
-    assert got.count("dnn.matmulnd-bias") == 12 and got.count("dnn.matmulnd") == 4 and got.count("dnn.add") == 6
+    # the residual sums and the Gelu of every layer ride on their Linear layer: what is left are the
+    # two embedding sums
+    assert got.count("dnn.matmulnd-bias") == 12 and got.count("dnn.matmulnd") == 4 and got.count("dnn.add") == 2
+    two_heads = dict(small, heads=2)   # head size 32: the attention kernel takes it
+    p = check_lifetimes(lambda: models.bert_encoder(**two_heads), recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)
+    assert len(names(p)) == 2 * 7 + 4   # per layer: qkv, attention, projection, LayerNorm, two feed-forward layers, LayerNorm
+    assert "dnn.gelu" not in got and p.text.count("{gelu}") == 2
 
 
 def test_attention_fusion_flag():
@@ -178,7 +184,8 @@ def test_attention_fusion_flag():
     got = names(p)
     # per layer: 3 head splits (Reshape + Transpose), two MatMuls, the scaling, Softmax and the head merge go
     assert got.count("dnn.attention") == 2 and "dnn.softmax" not in got and "dnn.transpose" not in got and "dnn.reshape" not in got
-    assert "heads=2, scale=0.176777" in p.text
+    assert "heads=2, scale=0.176777, packed" in p.text          # Q, K, V come out of one product
+    assert got.count("dnn.matmulnd") == 2 * 4                    # qkv, output projection, two feed-forward layers
     # head size 16 has no kernel: the graph is left as it is
     g, _ = models.bert_encoder(layers=1, hidden=64, heads=4, ffn=128, seq=16, vocab=100)
     assert "dnn.attention" not in names(g.compile(fuse_attention=True))

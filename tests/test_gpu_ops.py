@@ -247,11 +247,17 @@ def test_matmul_nd(gpu, cpu):
     r = rng(15)
     cases = [((1, 128, 768), (768, 768)), ((1, 12, 128, 64), (1, 12, 64, 128)), ((1, 12, 128, 128), (1, 12, 128, 64)),
              ((1, 128, 768), (768, 3072)), ((1, 128, 3072), (3072, 768)),
-             ((4, 6), (6, 3)), ((2, 4, 6), (6, 3)), ((2, 3, 4, 6), (2, 3, 6, 5)), ((2, 4, 6), (2, 6, 3)), ((4, 6), (3, 6, 2))]
+             ((4, 6), (6, 3)), ((2, 4, 6), (6, 3)), ((2, 3, 4, 6), (2, 3, 6, 5)), ((2, 4, 6), (2, 6, 3)), ((4, 6), (3, 6, 2)),
+             # the LDS-staged row-major kernel: ragged rows and columns, 1 to 11 reduction splits (odd counts too)
+             # (it takes products of 1.5e8 multiply-adds and more)
+             ((1, 100, 1056), (1056, 1540)), ((1, 33, 3072), (3072, 1604)), ((200, 2048), (2048, 388)), ((300, 1024), (1024, 512)),
+             ((2, 77, 1024), (1024, 1028)), ((1024, 256), (256, 1024)), ((1, 128, 768), (768, 2304))]
     for sa, sb in cases:
         a = r.standard_normal(sa).astype(np.float32)
         b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float32)
-        close(oc.matmul_nd(gpu, a, b), oc.matmul_nd(cpu, a, b))
+        ref = oc.matmul_nd(cpu, a, b)
+        close(oc.matmul_nd(gpu, a, b), ref)
+        close(oc.matmul_nd(gpu, a, b), ref)   # again: the split-reduction counters must be back at zero
 
 
 def test_matmul_nd_bias(gpu, cpu):
@@ -263,6 +269,9 @@ def test_matmul_nd_bias(gpu, cpu):
         b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float32)
         bias = r.standard_normal(sb[-1]).astype(np.float32)
         close(oc.matmul_nd_bias(gpu, a, b, bias), oc.matmul_nd_bias(cpu, a, b, bias))
+        z = r.standard_normal(np.broadcast_shapes(sa[:-2], sb[:-2]) + (sa[-2], sb[-1])).astype(np.float32)
+        close(oc.matmul_nd_bias(gpu, a, b, bias, z=z), oc.matmul_nd_bias(cpu, a, b, bias, z=z))
+        close(oc.matmul_nd_bias(gpu, a, b, bias, gelu=True), oc.matmul_nd_bias(cpu, a, b, bias, gelu=True))
     with pytest.raises(RuntimeError):
         oc.matmul_nd_bias(gpu, a.astype(np.float16), b.astype(np.float16), bias.astype(np.float16))  # not built: loud
 
@@ -275,6 +284,8 @@ def test_attention(gpu, cpu):
         q, k, v = (r.standard_normal((B, S, H * D)).astype(np.float32) for S in (Sq, Sk, Sk))
         q *= 2.0                                              # sharper soft-max: the running maximum moves between blocks
         close(oc.attention(gpu, q, k, v, H, 1.0 / np.sqrt(D)), oc.attention(cpu, q, k, v, H, 1.0 / np.sqrt(D)), 1e-4, 1e-5)
+    qkv = r.standard_normal((2, 130, 3 * 256)).astype(np.float32)          # Q | K | V per row
+    close(oc.attention_packed(gpu, qkv, 4, 0.125), oc.attention_packed(cpu, qkv, 4, 0.125), 1e-4, 1e-5)
     with pytest.raises(RuntimeError):
         oc.attention(gpu, q[:, :, :96], k[:, :, :96], v[:, :, :96], 2, 1.0)   # head size 48
 

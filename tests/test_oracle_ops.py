@@ -327,6 +327,11 @@ def test_matmul_nd_bias(be):
         bias = r.standard_normal(sb[-1]).astype(np.float32)
         ref = np.matmul(a.astype(np.float64), b.astype(np.float64)) + bias
         np.testing.assert_allclose(oc.matmul_nd_bias(be, a, b, bias), ref, rtol=1e-5, atol=1e-5)
+        z = r.standard_normal(ref.shape).astype(np.float32)
+        np.testing.assert_allclose(oc.matmul_nd_bias(be, a, b, bias, z=z), ref + z, rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(oc.matmul_nd_bias(be, a, b, bias, gelu=True), F.gelu(torch.from_numpy(ref)).numpy(), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(oc.matmul_nd_bias(be, a, b, bias, z=z, gelu=True), F.gelu(torch.from_numpy(ref + z)).numpy(),
+                                   rtol=1e-5, atol=1e-5)
 
 
 def attention_ref(q, k, v, heads, scale):
@@ -347,6 +352,10 @@ def test_attention(be):
         np.testing.assert_allclose(got, attention_ref(q, k, v, H, 1.0 / math.sqrt(D)), rtol=1e-5, atol=1e-6)
     # one key: the soft-max is 1 and the output is that key's value row, whatever the scores
     np.testing.assert_allclose(got, np.broadcast_to(v, got.shape), rtol=1e-6, atol=1e-6)
+    # Q, K, V as column blocks of one wider tensor
+    qkv = r.standard_normal((2, 9, 3 * 96)).astype(np.float32)
+    np.testing.assert_allclose(oc.attention_packed(be, qkv, 3, 0.2),
+                               attention_ref(qkv[:, :, :96], qkv[:, :, 96:192], qkv[:, :, 192:], 3, 0.2), rtol=1e-5, atol=1e-6)
     # heads do not mix: changing head 1's keys leaves head 0's output alone
     q, k, v = (r.standard_normal((1, 6, 128)).astype(np.float32) for _ in range(3))
     a = oc.attention(be, q, k, v, 2, 0.125)
