@@ -86,6 +86,103 @@ static bool parse_conv(const char *who, const int64_t *dX, const int64_t *dW, in
   return true;
 }
 
+// Dense convolution with at most four output channels (an image-producing
+// last layer: 64 -> 3).  A 32-wide MFMA tile would idle 29 of its 32 rows, so
+// this is plain FMA code: one thread per output pixel computes all K outputs.
+// A workgroup owns a 16 x 16 patch of pixels, so the rows a tap above or
+// below reads are rows the same workgroup reads anyway (L1 hits; with a
+// workgroup per image row segment every input row came from L2 three times).
+// The filter is copied to LDS once per workgroup as [c][tap][KMAX] (zeros
+// for k >= K): every lane reads the same address, one broadcast 16-byte LDS
+// read per tap instead of K scalar loads.
+// Weight element (k, c, r, s) sits at w[k * w_k + ((c * R + r) * S + s) * w_tap].
+template <int KMAX, int R, int S>
+__global__ __launch_bounds__(256) void conv_f32_narrow_kernel(
+    const float *__restrict__ X, const float *__restrict__ Wt, const float *__restrict__ bias,
+    const float *__restrict__ Zr, float *__restrict__ Y, int C, int H, int W, int K, int P, int Q, int ph, int pw,
+    int sh, int sw, int act, float act_coef, int w_k, int w_tap) {
+  extern __shared__ float wl[];
+  static_assert(KMAX == 4, "one float4 of filter values per tap");
+  for (int i = threadIdx.x; i < C * R * S * KMAX; i += 256) {
+    const int k = i % KMAX, ct = i / KMAX;  // ct = c * R * S + tap
+    wl[i] = k < K ? Wt[(int64_t)k * w_k + (int64_t)ct * w_tap] : 0.f;
+  }
+  __syncthreads();
+  const int tiles_q = (Q + 15) >> 4, tiles_p = (P + 15) >> 4;
+  const int tq = (int)(blockIdx.x % tiles_q), tp = (int)((blockIdx.x / tiles_q) % tiles_p), n = (int)(blockIdx.x / (tiles_q * tiles_p));
+  const int p_raw = tp * 16 + (threadIdx.x >> 4), q_raw = tq * 16 + (threadIdx.x & 15);
+  const bool live = p_raw < P && q_raw < Q;
+  const int p = min(p_raw, P - 1), q = min(q_raw, Q - 1);
+  const int ih0 = p * sh - ph, iw0 = q * sw - pw;
+  // clamped tap offsets and masks, once
+  int off[R][S];
+  unsigned msk[R][S];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int s = 0; s < S; s++) {
+      const int ih = ih0 + r, iw = iw0 + s;
+      const bool ok = (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+      off[r][s] = ok ? ih * W + iw : 0;
+      msk[r][s] = ok ? 0xffffffffu : 0u;
+    }
+  float acc[KMAX];
+#pragma unroll
+  for (int k = 0; k < KMAX; k++) acc[k] = 0.f;
+  const int HW = H * W;
+  const float *x = X + (int64_t)n * C * HW;
+  // The reads of one channel are a page apart from the next channel's and
+  // come back after about a microsecond; four channels' taps are kept in
+  // flight in four named register sets (loads of channels past the end
+  // re-read the last one and are not used).
+  struct Taps { float v[R][S]; };
+  auto fetch = [&](int c) {
+    Taps t;
+    const float *xc = x + (int64_t)min(c, C - 1) * HW;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int s = 0; s < S; s++) t.v[r][s] = xc[off[r][s]];
+    return t;
+  };
+  auto use = [&](const Taps &t, int c) {
+    const float4 *w = reinterpret_cast<const float4 *>(wl) + c * R * S;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (int s = 0; s < S; s++) {
+        const float v = __uint_as_float(__float_as_uint(t.v[r][s]) & msk[r][s]);
+        const float4 f = w[r * S + s];
+        acc[0] = fmaf(v, f.x, acc[0]);
+        acc[1] = fmaf(v, f.y, acc[1]);
+        acc[2] = fmaf(v, f.z, acc[2]);
+        acc[3] = fmaf(v, f.w, acc[3]);
+      }
+  };
+  Taps t0 = fetch(0), t1 = fetch(1), t2 = fetch(2), t3 = fetch(3);
+  for (int c = 0; c < C; c += 4) {
+    use(t0, c);
+    t0 = fetch(c + 4);
+    if (c + 1 < C) use(t1, c + 1);
+    t1 = fetch(c + 5);
+    if (c + 2 < C) use(t2, c + 2);
+    t2 = fetch(c + 6);
+    if (c + 3 < C) use(t3, c + 3);
+    t3 = fetch(c + 7);
+  }
+  if (!live) return;
+  const int64_t PQ = (int64_t)P * Q, pix = (int64_t)p * Q + q;
+#pragma unroll
+  for (int k = 0; k < KMAX; k++)
+    if (k < K) {
+      const int64_t o = ((int64_t)n * K + k) * PQ + pix;
+      float r = acc[k];
+      if (bias) r += bias[k];
+      if (Zr) r += Zr[o];
+      Y[o] = apply_act(r, act, act_coef);
+    }
+}
+
 static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const float *X,
                            const float *Wt, const float *bias, const float *Z, int act, float *Y) {
   // Filter storage: K,C,R,S (the reference's) or C,R,S,K (k_out contiguous),
@@ -105,6 +202,22 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
       hipLaunchKernelGGL((dwconv_f32_nchw_kernel<0, 0>), grid, block, 0, ctx->stream, X, Wt, bias, Z, Y,
                          s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, s.R, s.S, act, ctx->act_coef, total, w_k, w_tap);
     DNNRT_CHECK_LAUNCH("conv(depthwise)");
+    return Y;
+  }
+  if (s.group == 1 && s.K <= 4 && ((s.R == 3 && s.S == 3) || (s.R == 1 && s.S == 1)) && (int64_t)s.C * s.H * s.W < (1ll << 31) &&
+      (int64_t)s.C * s.R * s.S * 16 <= 48 * 1024) {  // the filter copy fits the default LDS limit
+    const int64_t blocks = (int64_t)s.N * ceil_div(s.P, 16) * ceil_div(s.Q, 16);
+    if (blocks > INT32_MAX) DNNRT_FAIL("conv: output too large");
+    dim3 grid((unsigned)blocks), block(256);
+    const size_t lds = (size_t)s.C * s.R * s.S * 4 * sizeof(float);
+    const int w_k = crsk ? 1 : s.C * s.R * s.S, w_tap = crsk ? s.K : 1;
+    if (s.R == 3)
+      hipLaunchKernelGGL((conv_f32_narrow_kernel<4, 3, 3>), grid, block, lds, ctx->stream, X, Wt, bias, Z, Y, s.C, s.H, s.W, s.K,
+                         s.P, s.Q, s.ph, s.pw, s.sh, s.sw, act, ctx->act_coef, w_k, w_tap);
+    else
+      hipLaunchKernelGGL((conv_f32_narrow_kernel<4, 1, 1>), grid, block, lds, ctx->stream, X, Wt, bias, Z, Y, s.C, s.H, s.W, s.K,
+                         s.P, s.Q, s.ph, s.pw, s.sh, s.sw, act, ctx->act_coef, w_k, w_tap);
+    DNNRT_CHECK_LAUNCH("conv(narrow)");
     return Y;
   }
   IgemmArgs a{};

@@ -51,6 +51,9 @@ CONV_CASES = [
     (1, 96, 112, 112, 96, 3, 3, 2, 1, 96),  # depthwise stride 2
     (2, 6, 7, 7, 12, 3, 3, 1, 1, 6),        # depthwise with channel multiplier 2
     (1, 1, 5, 5, 1, 3, 3, 1, 1, 1),         # smallest
+    (1, 64, 96, 80, 3, 3, 3, 1, 1, 1),      # image-producing last layer: three output channels
+    (2, 16, 21, 17, 4, 3, 3, 2, 1, 1),      # four output channels, stride 2
+    (2, 24, 9, 9, 2, 1, 1, 1, 0, 1),        # two output channels, 1x1
 ]
 
 
