@@ -341,6 +341,25 @@ void *dnnrtSqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
 void *dnnrtUnsqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
                      int64_t rankX, void *Y, const int64_t *dimY,
                      int64_t rankY, int32_t dtype);
+/* DNNAPISpecs.inc:32-35 "CUDAExpandInt64Func"
+ * (cuda/CUDAExpandInt64Func.cu:5-19), for every dtype.  The reference copies
+ * prod(dimX) elements and leaves the rest of Y unwritten, which is ONNX Expand
+ * only when dimY equals dimX; this entry point broadcasts (dimX aligned with
+ * the trailing dims of dimY, size-1 dims repeated) and so agrees with the
+ * reference wherever the reference's result is defined.  The reference's
+ * `shape` operand is not taken: dimY already is its value.  rankY <= 8. */
+void *dnnrtExpand(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                  int64_t rankX, void *Y, const int64_t *dimY, int64_t rankY,
+                  int32_t dtype);
+/* DNNAPISpecs.inc:52-55 "CUDANonZero{Int64,Float}Func"
+ * (cuda/CUDANonZeroFloatFunc.cu:4-34): the flat indices of the elements of X
+ * that are not zero, ascending, converted to X's own element type, written to
+ * the front of Y; the rest of Y keeps its contents.  Indices beyond
+ * prod(dimY) entries are dropped (the reference writes past the end); the
+ * reference passes one rank, the input's, for both dim arrays. */
+void *dnnrtNonZero(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
+                   int64_t rankX, void *Y, const int64_t *dimY, int64_t rankY,
+                   int32_t dtype);
 /* DNNAPISpecs.inc:15-18 "CUDAConcat{Int64,Float}Func"
  * (cuda/CUDAConcatFloatFunc.cu:64-99): Y = concatenation of numInputs tensors
  * along `axis`.  X and dimX are HOST arrays (of device pointers / of host dim

@@ -70,6 +70,8 @@ SIGNATURES = {
     "dnnrtSqueeze": (P, [P, P, I64P, i64, P, I64P, i64, i32]),
     "dnnrtUnsqueeze": (P, [P, P, I64P, i64, P, I64P, i64, i32]),
     "dnnrtConcat": (P, [P, P, P, P, I64P, i64, i64, i32, i32]),
+    "dnnrtExpand": (P, [P, P, I64P, i64, P, I64P, i64, i32]),
+    "dnnrtNonZero": (P, [P, P, I64P, i64, P, I64P, i64, i32]),
     "dnnrtTranspose": (P, [P, P, I64P, P, I64P, I64P, i64, i32]),
     "dnnrtGather": (P, [P, P, I64P, i64, P, I64P, i64, P, I64P, i64, i64, i32]),
 }

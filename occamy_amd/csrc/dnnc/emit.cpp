@@ -266,6 +266,21 @@ struct Emitter {
       o->perm = ints("axes", {});
       result = o->result;
       park_dealloc(out_buf);
+    } else if (t == "Expand") {
+      // Ops/cuda/Expand.cpp:40-47.  The shape constant stays a device tensor
+      // and an operand, as there; the output buffer is kept as the LAST
+      // operand (the reference puts the shape last), because the dealloc
+      // placement takes an op's last operand for the buffer its result lives
+      // in: with the reference's order the output would be released right
+      // after the call and the shape constant kept alive in its place.
+      Value *sh = in(1);
+      if (!sh) { err = "Expand: shape not available"; return false; }
+      out_buf = malloc_(ot.dtype, ot.shape);
+      Op *o = compute(OP_EXPAND, {x, sh, out_buf});
+      o->dimA = x->shape;
+      o->dimOut = ot.shape;
+      result = o->result;
+      park_dealloc(out_buf);
     } else if (t == "Cast") {
       if (x->dtype != I64 || ot.dtype == I64) { err = "Cast: only int64 -> float is covered"; return false; }
       out_buf = malloc_(ot.dtype, ot.shape);

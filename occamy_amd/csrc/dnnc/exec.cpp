@@ -42,7 +42,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   LOAD(dnnrtGelu); LOAD(dnnrtReduce); LOAD(dnnrtSoftmax); LOAD(dnnrtLayerNorm); LOAD(dnnrtMaxPool);
   LOAD(dnnrtAveragePool); LOAD(dnnrtMatmul2d); LOAD(dnnrtMatmulNd); LOAD(dnnrtFlatten);
   LOAD(dnnrtReshape); LOAD(dnnrtTranspose); LOAD(dnnrtGather);
-  LOAD(dnnrtLeakyRelu); LOAD(dnnrtPRelu); LOAD(dnnrtConcat); LOAD(dnnrtSqueeze); LOAD(dnnrtUnsqueeze);
+  LOAD(dnnrtLeakyRelu); LOAD(dnnrtPRelu); LOAD(dnnrtConcat); LOAD(dnnrtSqueeze); LOAD(dnnrtUnsqueeze); LOAD(dnnrtExpand);
   return true;
 }
 #undef LOAD
@@ -303,6 +303,10 @@ bool Session::issue(const Op *op, std::string &err) {
     case OP_UNSQUEEZE:
       r = rt.dnnrtUnsqueeze(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), out, op->dimOut.data(),
                             (int64_t)op->dimOut.size(), dt);
+      break;
+    case OP_EXPAND:  // operands: input, shape (device copy, not read), output
+      r = rt.dnnrtExpand(handle, P(0), op->dimA.data(), (int64_t)op->dimA.size(), out, op->dimOut.data(),
+                         (int64_t)op->dimOut.size(), dt);
       break;
     case OP_CAST:
       r = rt.dnnrtCastI64toFloat(handle, (const int64_t *)P(0), out, op->dimA.data(), (int64_t)op->dimA.size(), dt);

@@ -67,6 +67,7 @@ struct RuntimeApi {
   decltype(&::dnnrtConcat) dnnrtConcat = nullptr;
   decltype(&::dnnrtSqueeze) dnnrtSqueeze = nullptr;
   decltype(&::dnnrtUnsqueeze) dnnrtUnsqueeze = nullptr;
+  decltype(&::dnnrtExpand) dnnrtExpand = nullptr;
 };
 
 bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err);

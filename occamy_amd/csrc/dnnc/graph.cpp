@@ -89,7 +89,16 @@ static void forward_aliases(Graph &g) {
       auto it = alias.find(i);
       if (it != alias.end()) i = it->second;
     }
-    const bool fwd = (n.op_type == "Identity" || n.op_type == "Dropout") && !n.inputs.empty() && !n.inputs[0].empty();
+    bool fwd = (n.op_type == "Identity" || n.op_type == "Dropout") && !n.inputs.empty() && !n.inputs[0].empty();
+    if (n.op_type == "Pad" && n.inputs.size() >= 2 && !n.inputs[0].empty()) {
+      // Ops/cuda/Pad.cpp:33-55: a Pad whose constant pads are zero is its input; any other Pad is refused
+      auto it = g.tensors.find(n.inputs[1]);
+      if (it != g.tensors.end() && it->second.is_const && it->second.dtype == I64) {
+        const int64_t *p = reinterpret_cast<const int64_t *>(it->second.data.data());
+        fwd = true;
+        for (size_t k = 0; k < it->second.data.size() / 8; k++) fwd = fwd && p[k] == 0;
+      }
+    }
     if (fwd && std::find(g.outputs.begin(), g.outputs.end(), n.output) == g.outputs.end()) {
       alias[n.output] = n.inputs[0];
       continue;
@@ -643,6 +652,12 @@ static bool infer_pass(Graph &g, std::string &err) {
       out.shape.assign(x.begin(), x.begin() + axis);
       out.shape.insert(out.shape.end(), in[1]->shape.begin(), in[1]->shape.end());
       out.shape.insert(out.shape.end(), x.begin() + axis + 1, x.end());
+    } else if (t == "Expand") {
+      if (in.size() < 2 || !in[1] || !in[1]->is_const || in[1]->dtype != I64) return fail("shape must be an int64 constant");
+      const int64_t *s = reinterpret_cast<const int64_t *>(in[1]->data.data());
+      const Shape want(s, s + in[1]->data.size() / 8);
+      if (!broadcast_shape(x, want, out.shape)) return fail("input does not broadcast to shape");
+      if (out.shape.size() > 8) return fail("rank above 8");
     } else if (t == "Reshape") {
       if (in.size() < 2 || !in[1] || !in[1]->is_const || in[1]->dtype != I64) return fail("shape must be an int64 constant");
       const int64_t *s = reinterpret_cast<const int64_t *>(in[1]->data.data());

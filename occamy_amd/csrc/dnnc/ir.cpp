@@ -42,6 +42,7 @@ const char *op_name(OpKind k) {
     case OP_CONCAT: return "dnn.concat";
     case OP_SQUEEZE: return "dnn.squeeze";
     case OP_UNSQUEEZE: return "dnn.unsqueeze";
+    case OP_EXPAND: return "dnn.expand";
     case OP_LAYERNORM: return "dnn.layernorm";
     case OP_GELU: return "dnn.gelu";
     case OP_CONV_BIAS_ADD_ACTIV: return "dnn.conv-bias-add-relufwd";

@@ -61,7 +61,7 @@ enum OpKind {
   OP_CONVFWD, OP_CONV_BIAS_ACTIV, OP_ACTIVATION, OP_ADD, OP_MUL, OP_SQRT, OP_NEGATIVE,
   OP_RECIPROCAL, OP_REDUCE, OP_MAXPOOL, OP_AVGPOOL, OP_SOFTMAX, OP_FLATTEN, OP_RESHAPE,
   OP_TRANSPOSE, OP_GATHER, OP_MATMUL2D, OP_MATMULND, OP_POW, OP_ERF, OP_CAST, OP_CLIP,
-  OP_LEAKYRELU, OP_PRELU, OP_CONCAT, OP_SQUEEZE, OP_UNSQUEEZE,
+  OP_LEAKYRELU, OP_PRELU, OP_CONCAT, OP_SQUEEZE, OP_UNSQUEEZE, OP_EXPAND,
   // fused operators that have no counterpart in DNN.td
   OP_LAYERNORM, OP_GELU,
   OP_CONV_BIAS_ADD_ACTIV,  // conv + bias + residual tensor + activation (cuDNN's z operand)

@@ -26,6 +26,7 @@ const char *op_class(const Op *op) {
     case OP_CONCAT:
     case OP_SQUEEZE:
     case OP_UNSQUEEZE:
+    case OP_EXPAND:
     case OP_GATHER: return "move";
     default: return "elementwise";
   }

@@ -233,6 +233,66 @@ __global__ __launch_bounds__(256) void concat_kernel(ConcatGeom g, U *__restrict
   y[i] = static_cast<const U *>(g.x[s])[o * len + (j - g.begin[s])];
 }
 
+
+// Expand: output element i reads the input element whose index along every
+// broadcast axis is 0 (input stride 0 there).  U is the element as an
+// unsigned integer of the same width: the values are only moved.
+constexpr int EXPAND_MAX_RANK = 8;
+struct ExpandGeom {
+  int64_t out_dim[EXPAND_MAX_RANK], in_stride[EXPAND_MAX_RANK];
+  int rank;
+};
+template <typename U>
+__global__ __launch_bounds__(256) void expand_kernel(ExpandGeom g, const U *__restrict__ x, U *__restrict__ y, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  int64_t rest = i, src = 0;
+#pragma unroll 1
+  for (int d = g.rank - 1; d >= 0; d--) {
+    const int64_t q = rest / g.out_dim[d];
+    src += (rest - q * g.out_dim[d]) * g.in_stride[d];
+    rest = q;
+  }
+  y[i] = x[src];
+}
+
+// NonZero, in the reference's sense: the flat indices of the elements that are
+// not zero, in ascending order, converted to the tensor's own element type and
+// written to the front of Y; the rest of Y is left as it is.  One workgroup
+// walks the tensor 1024 elements at a time: a ballot gives every wavefront its
+// count and every lane its rank inside the wavefront, the 16 wavefront counts
+// are summed in LDS, and the running total stays in a register.
+template <typename T> __device__ __forceinline__ bool is_nonzero(T v) { return v != T(0); }
+template <> __device__ __forceinline__ bool is_nonzero<__half>(__half v) { return __half2float(v) != 0.f; }
+template <typename T> __device__ __forceinline__ T from_index(int64_t j) { return (T)j; }
+template <> __device__ __forceinline__ __half from_index<__half>(int64_t j) { return __float2half((float)j); }
+template <typename T>
+__global__ __launch_bounds__(1024) void nonzero_kernel(const T *__restrict__ x, T *__restrict__ y, int64_t n, int64_t cap) {
+  __shared__ int wave_count[2][16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int64_t base = 0;
+  int flip = 0;
+  for (int64_t start = 0; start < n; start += 1024, flip ^= 1) {
+    const int64_t j = start + threadIdx.x;
+    const bool hit = j < n && is_nonzero<T>(x[j]);
+    const unsigned long long votes = __ballot(hit);
+    if (lane == 0) wave_count[flip][wave] = __popcll(votes);
+    __syncthreads();  // the other half of wave_count is what the previous chunk used
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++) {
+      const int c = wave_count[flip][w];
+      before += w < wave ? c : 0;
+      all += c;
+    }
+    if (hit) {
+      const int64_t slot = base + before + __popcll(votes & ((1ull << lane) - 1ull));
+      if (slot < cap) y[slot] = from_index<T>(j);
+    }
+    base += all;
+  }
+}
+
 }  // namespace dnnrt
 
 using namespace dnnrt;
@@ -285,6 +345,53 @@ void *dnnrtSqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int
 void *dnnrtUnsqueeze(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
                      const int64_t *dimY, int64_t rankY, int32_t dtype) {
   return same_order_copy("dnnrtUnsqueeze", handle, X, dimX, rankX, Y, dimY, rankY, dtype);
+}
+
+void *dnnrtExpand(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
+                  const int64_t *dimY, int64_t rankY, int32_t dtype) {
+  if (!handle) DNNRT_FAIL("dnnrtExpand: null handle");
+  if (!X || !Y || !dimX || !dimY) DNNRT_FAIL("dnnrtExpand: null argument");
+  if (rankY < 1 || rankY > EXPAND_MAX_RANK || rankX < 0 || rankX > rankY)
+    DNNRT_FAIL("dnnrtExpand: ranks %ld -> %ld (input rank <= output rank <= %d)", (long)rankX, (long)rankY, EXPAND_MAX_RANK);
+  const int64_t es = esize(dtype);
+  if (!es) DNNRT_FAIL("dnnrtExpand: dtype %d", dtype);
+  if (handle->format != DNNRT_NCHW && (rankX == 4 || rankY == 4)) DNNRT_FAIL("dnnrtExpand: channels-last tensors are not supported");
+  ExpandGeom g{};
+  g.rank = (int)rankY;
+  int64_t stride = 1;
+  for (int64_t d = rankY - 1; d >= 0; d--) {
+    const int64_t dx = d - (rankY - rankX);  // dimX is aligned with the trailing dims of dimY
+    const int64_t in = dx >= 0 ? dimX[dx] : 1;
+    if (dimY[d] < 0 || in < 0) DNNRT_FAIL("dnnrtExpand: negative dim");
+    if (in != dimY[d] && in != 1) DNNRT_FAIL("dnnrtExpand: input dim %ld cannot be broadcast to %ld", (long)in, (long)dimY[d]);
+    g.out_dim[d] = dimY[d];
+    g.in_stride[d] = in == 1 ? 0 : stride;
+    stride *= in;
+  }
+  const int64_t total = numel(dimY, rankY);
+  if (total == 0) return Y;
+  if (ceil_div(total, 256) > INT32_MAX) DNNRT_FAIL("dnnrtExpand: tensor too large");
+  const dim3 grid((unsigned)ceil_div(total, 256)), block(256);
+  if (es == 8) hipLaunchKernelGGL(expand_kernel<uint64_t>, grid, block, 0, handle->stream, g, (const uint64_t *)X, (uint64_t *)Y, total);
+  else if (es == 4) hipLaunchKernelGGL(expand_kernel<uint32_t>, grid, block, 0, handle->stream, g, (const uint32_t *)X, (uint32_t *)Y, total);
+  else hipLaunchKernelGGL(expand_kernel<uint16_t>, grid, block, 0, handle->stream, g, (const uint16_t *)X, (uint16_t *)Y, total);
+  DNNRT_CHECK_LAUNCH("dnnrtExpand");
+  return Y;
+}
+
+void *dnnrtNonZero(dnnrtHandle_t handle, const void *X, const int64_t *dimX, int64_t rankX, void *Y,
+                   const int64_t *dimY, int64_t rankY, int32_t dtype) {
+  if (!handle) DNNRT_FAIL("dnnrtNonZero: null handle");
+  if (!X || !Y || !dimX || !dimY || rankX < 0 || rankY < 0) DNNRT_FAIL("dnnrtNonZero: null argument");
+  if (handle->format != DNNRT_NCHW && rankX == 4) DNNRT_FAIL("dnnrtNonZero: channels-last tensors are not supported");
+  const int64_t n = numel(dimX, rankX), cap = numel(dimY, rankY);
+  if (n == 0) return Y;
+  if (dtype == DNNRT_F32) hipLaunchKernelGGL(nonzero_kernel<float>, dim3(1), dim3(1024), 0, handle->stream, (const float *)X, (float *)Y, n, cap);
+  else if (dtype == DNNRT_F16) hipLaunchKernelGGL(nonzero_kernel<__half>, dim3(1), dim3(1024), 0, handle->stream, (const __half *)X, (__half *)Y, n, cap);
+  else if (dtype == DNNRT_I64) hipLaunchKernelGGL(nonzero_kernel<int64_t>, dim3(1), dim3(1024), 0, handle->stream, (const int64_t *)X, (int64_t *)Y, n, cap);
+  else DNNRT_FAIL("dnnrtNonZero: dtype %d", dtype);
+  DNNRT_CHECK_LAUNCH("dnnrtNonZero");
+  return Y;
 }
 
 void *dnnrtConcat(dnnrtHandle_t handle, const void *const *X, const int64_t *const *dimX, void *Y,

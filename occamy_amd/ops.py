@@ -205,6 +205,15 @@ class Ops:
         return self._ret(self.lib.dnnrtUnsqueeze(self.handle, X, dims(dimX), len(dimX), Y, dims(dimY), len(dimY),
                                                  dtype), "dnnrtUnsqueeze")
 
+    def expand(self, X, dimX, Y, dimY, dtype=_abi.I64):
+        return self._ret(self.lib.dnnrtExpand(self.handle, X, dims(dimX), len(dimX), Y, dims(dimY), len(dimY),
+                                              dtype), "dnnrtExpand")
+
+    def nonzero(self, X, dimX, Y, dimY, dtype=_abi.F32):
+        """Flat indices of the non-zero elements, in X's element type, at the front of Y."""
+        return self._ret(self.lib.dnnrtNonZero(self.handle, X, dims(dimX), len(dimX), Y, dims(dimY), len(dimY),
+                                               dtype), "dnnrtNonZero")
+
     def concat(self, Xs, dimXs, Y, dimY, axis, dtype=_abi.F32):
         """Xs: device pointers (ints), dimXs: one dim list per input."""
         n = len(Xs)

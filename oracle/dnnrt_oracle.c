@@ -842,6 +842,57 @@ void *dnnrtUnsqueeze(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t 
   memmove(Y, X, (size_t)(numel(dX, rX) * esize(dtype)));
   return Y;
 }
+/* CUDAExpandInt64Func.cu:10-15 copies prod(dimX) elements, which is the whole
+ * answer only when dimY == dimX.  Restated as the ONNX operator the lowering
+ * stands for (Ops/cuda/Expand.cpp:30-47: output sized by the broadcast shape):
+ * per output element, the multi-index with every broadcast coordinate set to
+ * 0 addresses the input.  With dimY == dimX this is the reference's copy. */
+void *dnnrtExpand(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rX, void *Y,
+                  const int64_t *dY, int64_t rY, int32_t dtype) {
+  (void)h;
+  const int64_t es = esize(dtype);
+  if (!es) FAIL("expand: bad dtype");
+  if (rY < 1 || rY > 8 || rX < 0 || rX > rY) FAIL("expand: ranks");
+  int64_t in_dim[8];
+  for (int64_t d = 0; d < rY; d++) {
+    const int64_t dx = d - (rY - rX);
+    in_dim[d] = dx >= 0 ? dX[dx] : 1;
+    if (in_dim[d] != dY[d] && in_dim[d] != 1) FAIL("expand: dims cannot be broadcast");
+  }
+  const int64_t total = numel(dY, rY);
+  for (int64_t i = 0; i < total; i++) {
+    int64_t idx[8], rest = i, src = 0;
+    for (int64_t d = rY - 1; d >= 0; d--) { idx[d] = rest % dY[d]; rest /= dY[d]; }
+    for (int64_t d = 0; d < rY; d++) src = src * in_dim[d] + (in_dim[d] == 1 ? 0 : idx[d]);
+    memcpy((char *)Y + i * es, (const char *)X + src * es, (size_t)es);
+  }
+  return Y;
+}
+/* CUDANonZeroFloatFunc.cu:4-17 / CUDANonZeroInt64Func.cu: one sequential walk;
+ * the index of every element != 0 goes to the next output slot, converted to
+ * the element type.  Slots past prod(dimY) are not written (the reference
+ * does not check). */
+void *dnnrtNonZero(dnnrtHandle_t h, const void *X, const int64_t *dX, int64_t rX, void *Y,
+                   const int64_t *dY, int64_t rY, int32_t dtype) {
+  (void)h;
+  if (!esize(dtype)) FAIL("nonzero: bad dtype");
+  const int64_t n = numel(dX, rX), cap = numel(dY, rY);
+  int64_t cur = 0;
+  for (int64_t j = 0; j < n; j++) {
+    int hit;
+    if (dtype == DNNRT_F32) hit = ((const float *)X)[j] != 0.f;
+    else if (dtype == DNNRT_F16) hit = h2f(((const uint16_t *)X)[j]) != 0.f;
+    else hit = ((const int64_t *)X)[j] != 0;
+    if (!hit) continue;
+    if (cur < cap) {
+      if (dtype == DNNRT_F32) ((float *)Y)[cur] = (float)j;
+      else if (dtype == DNNRT_F16) ((uint16_t *)Y)[cur] = f2h((float)j);
+      else ((int64_t *)Y)[cur] = j;
+    }
+    cur++;
+  }
+  return Y;
+}
 /* CUDAConcatFloatFunc.cu:7-62, per output element: split the flat index into
  * a multi-index, find the input whose span along the axis holds it, rebase
  * that coordinate and gather from that input. */

@@ -98,6 +98,12 @@ def evaluate(graph, inputs):
             env[out] = y
         elif op in ("Identity", "Dropout"):
             env[out] = x[0]
+        elif op == "Expand":
+            shape = torch.broadcast_shapes(tuple(x[0].shape), tuple(int(v) for v in x[1]))
+            env[out] = x[0].expand(shape).contiguous()
+        elif op == "Pad":
+            assert all(int(v) == 0 for v in x[1]), "only the all-zero Pad is in the dialect's reach"
+            env[out] = x[0]
         elif op == "BatchNormalization":
             env[out] = F.batch_norm(x[0], x[3], x[4], x[1], x[2], False, 0.0, at.get("epsilon", 1e-5))
         else:

@@ -214,6 +214,23 @@ def squeeze(be, x, out, un=False):
     return be.get(Y)
 
 
+def expand(be, x, out):
+    X = be.put(x)
+    Y = be.empty(out, x.dtype)
+    be.ops.expand(be.ptr(X), x.shape, be.ptr(Y), out, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
+def nonzero(be, x, out, fill):
+    """Y starts as `fill` everywhere: the call writes only the front."""
+    X = be.put(x)
+    Y = be.put(np.full(out, fill, x.dtype))
+    be.ops.nonzero(be.ptr(X), x.shape, be.ptr(Y), out, DT[x.dtype])
+    be.sync()
+    return be.get(Y)
+
+
 def matmul_nd_bias(be, a, b, bias, z=None, gelu=False):
     y_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2]) + (a.shape[-2], b.shape[-1])
     A, B, Bi = be.put(a), be.put(b), be.put(bias)

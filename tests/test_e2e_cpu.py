@@ -172,6 +172,42 @@ def test_widened_operator_surface():
     assert text.count("dnn.prelu") == 2 and text.count("dnn.leakyrelu") == 1
 
 
+def expand_pad_graph():
+    r = np.random.default_rng(6)
+    g = compiler.Graph()
+    x = r.standard_normal((2, 1, 5)).astype(np.float32)
+    g.input("x", x.shape)
+    p = g.node("Pad", ["x", g.constant(np.zeros(6, np.int64))])                     # zero pads: the input itself
+    e = g.node("Expand", [p, g.constant(np.array([3, 2, 4, 5], np.int64))])         # [3,2,4,5]
+    m = g.node("Mul", [e, g.constant(r.standard_normal((4, 1)).astype(np.float32))])
+    g.output(g.node("Relu", [m]))
+    g.output(g.node("Expand", ["x", g.constant(np.array([1, 1, 1], np.int64))]))    # shape of ones: a copy
+    return g, [x]
+
+
+def test_expand_and_zero_pad():
+    """Expand broadcasts (the shape constant stays a device operand, as in
+    Ops/cuda/Expand.cpp:40-47); a Pad with zero pads is its input
+    (Ops/cuda/Pad.cpp:48-52) and any other Pad is refused."""
+    out = check(expand_pad_graph)
+    assert out[0].shape == (3, 2, 4, 5) and out[1].shape == (2, 1, 5)
+    g, _ = expand_pad_graph()
+    text = g.compile().text
+    assert text.count("dnn.expand") == 2 and "Pad" not in text
+    # the expanded tensor outlives the call: its buffer is released after the Mul that reads it
+    lines = expand_pad_graph()[0].compile(pool_opt=False).text.splitlines()
+    first = next(i for i, l in enumerate(lines) if "dnn.expand" in l)
+    mul = next(i for i, l in enumerate(lines) if "dnn.mul" in l)
+    buf = lines[first].split("dnn.expand")[1].split(" :")[0].split(",")[-1].strip()
+    freed = next(i for i, l in enumerate(lines) if "dnn.dealloc" in l and l.split("dnn.dealloc")[1].split()[0] == buf)
+    assert freed > mul
+    g = compiler.Graph()
+    g.input("x", (1, 3, 4, 4))
+    g.output(g.node("Pad", ["x", g.constant(np.array([0, 0, 1, 1, 0, 0, 1, 1], np.int64))]))
+    with pytest.raises(RuntimeError, match="Pad"):
+        g.compile()
+
+
 @pytest.mark.parametrize("builder", [lambda: models.mobilenet_v2(image=32, classes=10), YOLO, SRGAN,
                                      lambda: models.resnet50(image=32, classes=10)],
                          ids=["mobilenet_v2", "yolo_v1", "srgan", "resnet50"])

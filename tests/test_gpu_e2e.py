@@ -7,6 +7,7 @@ import pytest
 
 from helpers import ORACLE_PATH
 from occamy_amd import compiler, models
+from test_e2e_cpu import expand_pad_graph
 
 pytestmark = pytest.mark.gpu
 
@@ -35,6 +36,7 @@ CONFIGS = {
     "alexnet": models.alexnet,
     "yolo_v1": lambda: models.yolo_v1(batch=1),
     "srgan": lambda: models.srgan_generator(height=64, width=48),
+    "expand_pad": expand_pad_graph,
 }
 
 

@@ -314,6 +314,9 @@ def test_data_movement(gpu, cpu):
     idx = r.integers(0, 30522, (1, 128))
     np.testing.assert_array_equal(oc.gather(gpu, table, idx, 0), np.take(table, idx, 0))
     np.testing.assert_array_equal(oc.gather(gpu, x, np.array([2, -1]), 2), np.take(x, [2, -1], 2))
+    ti = r.integers(-1000, 1000, (70, 3, 20)).astype(np.int64)
+    np.testing.assert_array_equal(oc.gather(gpu, ti, np.array([[6, 0], [3, -2]]), 0), np.take(ti, [[6, 0], [3, -2]], 0))
+    np.testing.assert_array_equal(oc.gather(gpu, ti, np.array([19, 1]), 2), oc.gather(cpu, ti, np.array([19, 1]), 2))
     with pytest.raises(RuntimeError):
         oc.transpose(gpu, x, (0, 1, 1, 3))
 
@@ -415,6 +418,35 @@ def test_concat_squeeze_unsqueeze(gpu, cpu):
     np.testing.assert_array_equal(oc.squeeze(gpu, s.reshape(2, 4), (1, 2, 1, 4), un=True), s.reshape(1, 2, 1, 4))
     with pytest.raises(RuntimeError):
         oc.squeeze(gpu, s, (4, 2))
+
+
+def test_expand_and_nonzero(gpu, cpu):
+    r = rng(43)
+    for shape, out in [((3, 1, 5), (3, 1, 5)), ((3, 1, 5), (2, 3, 4, 5)), ((1,), (1000,)), ((64, 1), (64, 300)),
+                       ((1, 1, 1), (2, 3, 4)), ((2, 1, 3, 1, 2), (2, 4, 3, 5, 2)), ((1, 1, 128, 128), (2, 12, 128, 128))]:
+        for dtype in (np.int64, np.float32, np.float16):
+            x = r.integers(-99, 99, shape).astype(dtype)
+            got = oc.expand(gpu, x, out)
+            np.testing.assert_array_equal(got, np.broadcast_to(x, out))
+            np.testing.assert_array_equal(got, oc.expand(cpu, x, out))
+    with pytest.raises(RuntimeError):
+        oc.expand(gpu, np.zeros((3, 1, 5), np.int64), (3, 4, 6))
+    # sizes around the 1024-element chunk and the 64-lane wavefront, sparse and dense
+    for n, density in [(1, 1.0), (63, 0.5), (64, 1.0), (65, 0.3), (1023, 0.9), (1024, 1.0), (1025, 0.01), (5000, 0.5),
+                       (100_003, 0.1), (4096, 0.0)]:
+        for dtype in (np.float32, np.int64, np.float16):
+            x = (r.integers(1, 5, (n,)) * (r.random((n,)) < density)).astype(dtype)
+            got = oc.nonzero(gpu, x, (n,), -3)
+            want = np.flatnonzero(x)
+            np.testing.assert_array_equal(got, oc.nonzero(cpu, x, (n,), -3))
+            if dtype != np.float16:  # fp16 cannot hold indices above 2048 exactly: the oracle comparison covers it
+                np.testing.assert_array_equal(got[: want.size], want.astype(dtype))
+            np.testing.assert_array_equal(got[want.size:], np.full(n - want.size, -3, dtype))
+    x = (r.random((7, 9, 11)) < 0.5).astype(np.float32)
+    cut = oc.nonzero(gpu, x, (2, 10), -1.0)          # output rank differs from the input's; capacity 20
+    np.testing.assert_array_equal(cut.reshape(-1), np.flatnonzero(x.reshape(-1))[:20].astype(np.float32))
+    z = np.array([0.0, -0.0, np.nan, 1e-45, 0.0], np.float32)
+    np.testing.assert_array_equal(oc.nonzero(gpu, z, (5,), -1.0), np.array([2, 3, -1, -1, -1], np.float32))
 
 
 # ---- fp16, channels-last -----------------------------------------------------------------

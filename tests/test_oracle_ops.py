@@ -383,6 +383,9 @@ def test_data_movement(be):
     np.testing.assert_array_equal(oc.gather(be, table, idx, 0), np.take(table, idx, 0))
     np.testing.assert_array_equal(oc.gather(be, table, np.array([-1, 0]), 0), np.take(table, [-1, 0], 0))
     np.testing.assert_array_equal(oc.gather(be, x, np.array([2, 0]), 2), np.take(x, [2, 0], 2))
+    ti = r.integers(-1000, 1000, (7, 3, 2)).astype(np.int64)     # CUDAGatherInt64Func: same walk on 8-byte elements
+    np.testing.assert_array_equal(oc.gather(be, ti, np.array([[6, 0], [3, -2]]), 0), np.take(ti, [[6, 0], [3, -2]], 0))
+    np.testing.assert_array_equal(oc.gather(be, ti, np.array([1]), 2), np.take(ti, [1], 2))
     with pytest.raises(RuntimeError):
         oc.gather(be, table, np.array([11]), 0)
 
@@ -466,6 +469,39 @@ def test_concat_squeeze_unsqueeze(be):
     np.testing.assert_array_equal(oc.squeeze(be, s.reshape(2, 4), (1, 2, 1, 4), un=True), s.reshape(1, 2, 1, 4))
     with pytest.raises(RuntimeError):
         oc.squeeze(be, s, (4, 2))
+
+
+def test_expand_broadcasts_like_numpy(be):
+    # the reference's copy (CUDAExpandInt64Func.cu:10-15) is the case out == in
+    r = rng(33)
+    xi = r.integers(-9, 9, (3, 1, 5)).astype(np.int64)
+    np.testing.assert_array_equal(oc.expand(be, xi, (3, 1, 5)), xi)
+    for shape, out in [((3, 1, 5), (3, 4, 5)), ((3, 1, 5), (2, 3, 4, 5)), ((1,), (7,)), ((4, 1), (4, 6)),
+                       ((1, 1, 1), (2, 3, 4)), ((5,), (2, 5)), ((2, 1, 3, 1, 2), (2, 4, 3, 5, 2))]:
+        for dtype in (np.int64, np.float32, np.float16):
+            x = (r.integers(-99, 99, shape).astype(dtype))
+            np.testing.assert_array_equal(oc.expand(be, x, out), np.broadcast_to(x, out))
+    with pytest.raises(RuntimeError):
+        oc.expand(be, xi, (3, 4, 6))          # 5 does not broadcast to 6
+    with pytest.raises(RuntimeError):
+        oc.expand(be, xi, (4, 5))             # output rank below the input's
+
+
+def test_nonzero_lists_flat_indices_in_order(be):
+    # CUDANonZeroFloatFunc.cu:4-17: indices as values of the input's type, front of the output only
+    r = rng(34)
+    for dtype in (np.float32, np.int64, np.float16):
+        x = (r.integers(-2, 3, (3, 5, 7)) * (r.random((3, 5, 7)) < 0.4)).astype(dtype)
+        want = np.flatnonzero(x.reshape(-1))
+        out = oc.nonzero(be, x, (1, x.size), -7)
+        np.testing.assert_array_equal(out.reshape(-1)[: want.size], want.astype(dtype))
+        np.testing.assert_array_equal(out.reshape(-1)[want.size:], np.full(x.size - want.size, -7, dtype))
+        # an output smaller than the count holds the first indices only
+        small = oc.nonzero(be, x, (3,), -7)
+        np.testing.assert_array_equal(small, want[:3].astype(dtype))
+    z = np.array([0.0, -0.0, np.nan, 1e-45, 0.0], np.float32)   # -0 is zero, NaN and denormals are not
+    np.testing.assert_array_equal(oc.nonzero(be, z, (5,), -1.0), np.array([2, 3, -1, -1, -1], np.float32))
+    np.testing.assert_array_equal(oc.nonzero(be, np.zeros((4, 4), np.float32), (16,), 5.0), np.full(16, 5.0, np.float32))
 
 
 def test_layouts_the_oracle_lacks_are_refused(be):
