@@ -521,13 +521,16 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     // 128x128 when there are enough tiles for more than one workgroup per CU;
     // with about one per CU or fewer, the eight-wavefront variants (128x128,
     // then 128x64), which keep two wavefronts on every SIMD; 128x64 for very
-    // short reductions; 64x64 when K_out <= 64.
+    // short reductions; 64x64 when K_out <= 64 (64x128 for its 3x3 layers;
+    // walking an XCD's run of tiles pixel tiles first instead of k_out tiles
+    // first, so that an XCD touches a slice of a large filter only, changed
+    // nothing on the 7x7 layers).
     const int tile_sel = ctx->f16_tile;  // 0 = automatic; otherwise forced (tuning and tests)
     int sel = tile_sel;
     if (sel == 0) {
       const int nk = a.R * a.S * (a.C / BKF);
       const int64_t t128 = tiles_of(128, 128), cus = ctx->num_cu;
-      if (a.K <= 64) sel = 4;
+      if (a.K <= 64) sel = nk >= 9 ? 15 : 4;
       else if (nk <= 2) sel = 7;
       else if (4 * t128 >= 5 * cus) sel = 3;
       else if (5 * t128 >= 3 * cus) sel = 12;
@@ -538,6 +541,7 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1); break;
       case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2); break;
       case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2); break;
+      case 15: LAUNCH_FAST(64, 128, 2, 2, 2, 2, 1); break;
       default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1); break;
     }
 #undef LAUNCH_FAST
