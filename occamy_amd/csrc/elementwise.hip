@@ -79,6 +79,41 @@ __global__ __launch_bounds__(256) void bcast_kernel(const T *__restrict__ a, con
   o[i] = from_f<T>(f(to_f(a[i]), to_f(b[ib])));
 }
 
+// The same below 2^31 elements when the innermost run is a multiple of 16
+// bytes and everything is 16-byte aligned: a thread owns 16 bytes of a, which
+// lie inside one innermost run, so b is either one value for all of them
+// (INNER_BC: the innermost run is a broadcast one) or 16 consecutive bytes.
+struct BcastDims32 {
+  unsigned d[4];
+  unsigned sb[4];
+};
+template <typename T, bool INNER_BC, typename F>
+__global__ __launch_bounds__(256) void bcast_vec_kernel(const T *__restrict__ a, const T *__restrict__ b,
+                                                        T *__restrict__ o, unsigned n, BcastDims32 g, F f) {
+  constexpr int V = Pack<T>::N;
+  const unsigned i = (blockIdx.x * 256u + threadIdx.x) * (unsigned)V;
+  if (i >= n) return;
+  unsigned rem = i, ib = 0;
+#pragma unroll
+  for (int k = 3; k >= 0; k--) {
+    if (g.d[k] == 1u) continue;  // the same for every thread
+    const unsigned q = rem / g.d[k];
+    ib += (rem - q * g.d[k]) * g.sb[k];
+    rem = q;
+  }
+  Pack<T> pa = *reinterpret_cast<const Pack<T> *>(a + i);
+  if (INNER_BC) {
+    const float bv = to_f(b[ib]);
+#pragma unroll
+    for (int j = 0; j < V; j++) pa.v[j] = from_f<T>(f(to_f(pa.v[j]), bv));
+  } else {
+    const Pack<T> pb = *reinterpret_cast<const Pack<T> *>(b + ib);
+#pragma unroll
+    for (int j = 0; j < V; j++) pa.v[j] = from_f<T>(f(to_f(pa.v[j]), to_f(pb.v[j])));
+  }
+  *reinterpret_cast<Pack<T> *>(o + i) = pa;
+}
+
 template <typename T, typename F>
 static bool run_unary(const dnnrtContext *ctx, const void *x, void *y, int64_t n, F f) {
   if (n == 0) return true;
@@ -195,8 +230,24 @@ static bool run_binary(const dnnrtContext *ctx, const void *A, const void *B, vo
     for (int k = 0; k < nc; k++) { g.d[4 - nc + k] = cd[k]; g.sb[4 - nc + k] = cs[k]; }
     const int64_t blocks = ceil_div(n, 256);
     if (blocks > INT32_MAX) { set_error("tensorOp: tensor too large"); return false; }
-    hipLaunchKernelGGL((bcast_kernel<T, F>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
-                       (const T *)A, (const T *)B, (T *)O, n, g, f);
+    constexpr int V = Pack<T>::N;
+    const bool inner_bc = g.sb[3] == 0;
+    if (n < (1ll << 31) && nc >= 1 && g.d[3] % V == 0 && (inner_bc || g.sb[3] == 1) && aligned16(A) && aligned16(O) &&
+        (inner_bc || aligned16(B))) {
+      // b's strides for the outer runs are multiples of its innermost run's length, itself a multiple of V
+      BcastDims32 h;
+      for (int k = 0; k < 4; k++) { h.d[k] = (unsigned)g.d[k]; h.sb[k] = (unsigned)g.sb[k]; }
+      const unsigned vblocks = (unsigned)ceil_div(n / V, 256);
+      if (inner_bc)
+        hipLaunchKernelGGL((bcast_vec_kernel<T, true, F>), dim3(vblocks), dim3(256), 0, ctx->stream,
+                           (const T *)A, (const T *)B, (T *)O, (unsigned)n, h, f);
+      else
+        hipLaunchKernelGGL((bcast_vec_kernel<T, false, F>), dim3(vblocks), dim3(256), 0, ctx->stream,
+                           (const T *)A, (const T *)B, (T *)O, (unsigned)n, h, f);
+    } else {
+      hipLaunchKernelGGL((bcast_kernel<T, F>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                         (const T *)A, (const T *)B, (T *)O, n, g, f);
+    }
   }
   e = hipGetLastError();
   if (e != hipSuccess) { set_error("tensorOp: launch failed: %s", hipGetErrorString(e)); return false; }

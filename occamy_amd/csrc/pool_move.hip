@@ -158,6 +158,39 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T *__restrict__ x,
   y[i] = x[ix];
 }
 
+// The same for tensors below 2^31 elements, V consecutive output elements
+// per thread (V divides the last output dim): 32-bit index arithmetic, one
+// V-element store, and one V-element load too when the last output dim is
+// the input's last dim as well (CONTIG).  Dims arrive merged where a run of
+// output dims is a run of input dims, and without size-1 dims.
+struct PermGeom32 {
+  unsigned dy[6];  // output dims, the last one divided by V
+  unsigned sx[6];  // input strides in elements
+};
+template <typename U, int V> struct alignas(sizeof(U) * V) VecOf { U v[V]; };
+template <typename U, int V, bool CONTIG>
+__global__ __launch_bounds__(256) void transpose_vec_kernel(const U *__restrict__ x, U *__restrict__ y,
+                                                            PermGeom32 g, int rank, unsigned units) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= units) return;
+  unsigned rem = i, ix = 0;
+#pragma unroll 1
+  for (int d = rank - 1; d >= 0; d--) {
+    const unsigned q = rem / g.dy[d];
+    ix += (rem - q * g.dy[d]) * g.sx[d] * (d == rank - 1 ? (unsigned)V : 1u);
+    rem = q;
+  }
+  VecOf<U, V> out;
+  if (CONTIG) {
+    out = *reinterpret_cast<const VecOf<U, V> *>(x + ix);
+  } else {
+    const unsigned step = g.sx[rank - 1];
+#pragma unroll
+    for (int j = 0; j < V; j++) out.v[j] = x[ix + (unsigned)j * step];
+  }
+  reinterpret_cast<VecOf<U, V> *>(y)[i] = out;
+}
+
 // Y[o, j, in] = X[o, idx[j], in]; out-of-range indices produce zeros.
 template <typename T>
 __global__ __launch_bounds__(256) void gather_kernel(const T *__restrict__ x, const int64_t *__restrict__ idx,
@@ -461,6 +494,44 @@ void *dnnrtTranspose(dnnrtHandle_t handle, const void *X, const int64_t *dimX, v
     if (dimY[i] != dimX[perm[i]] || dimY[i] <= 0) DNNRT_FAIL("dnnrtTranspose: dimY[%d] != dimX[perm[%d]]", i, i);
     g.dy[i] = dimY[i];
     g.sx[i] = sx[perm[i]];
+  }
+  const int64_t es = esize(dtype);
+  if (!es) DNNRT_FAIL("dnnrtTranspose: dtype %d", dtype);
+  if (s > 0 && s < (1ll << 31)) {
+    // size-1 dims dropped, runs of dims that stay together merged
+    int64_t my[6], ms[6];
+    int n = 0;
+    for (int i = 0; i < rank; i++) {
+      if (g.dy[i] == 1) continue;
+      if (n > 0 && ms[n - 1] == g.sx[i] * g.dy[i]) { my[n - 1] *= g.dy[i]; ms[n - 1] = g.sx[i]; }
+      else { my[n] = g.dy[i]; ms[n] = g.sx[i]; n++; }
+    }
+    if (n == 0) { my[0] = 1; ms[0] = 1; n = 1; }
+    const bool contig = ms[n - 1] == 1;
+    int v = (int)(16 / es);
+    auto fits = [&](int w) {
+      if (my[n - 1] % w || (reinterpret_cast<uintptr_t>(Y) % (uintptr_t)(w * es))) return false;
+      if (!contig) return true;
+      if (reinterpret_cast<uintptr_t>(X) % (uintptr_t)(w * es)) return false;
+      for (int i = 0; i < n - 1; i++) if (ms[i] % w) return false;
+      return true;
+    };
+    while (v > 1 && !fits(v)) v >>= 1;
+    PermGeom32 h{};
+    for (int i = 0; i < n; i++) { h.dy[i] = (unsigned)my[i]; h.sx[i] = (unsigned)ms[i]; }
+    h.dy[n - 1] = (unsigned)(my[n - 1] / v);
+    const unsigned units = (unsigned)(s / v), blocks32 = (units + 255u) / 256u;
+#define LAUNCH_T(U, V_)                                                                                          \
+  do {                                                                                                           \
+    if (contig) hipLaunchKernelGGL((transpose_vec_kernel<U, V_, true>), dim3(blocks32), dim3(256), 0, handle->stream, (const U *)X, (U *)Y, h, n, units); \
+    else hipLaunchKernelGGL((transpose_vec_kernel<U, V_, false>), dim3(blocks32), dim3(256), 0, handle->stream, (const U *)X, (U *)Y, h, n, units);      \
+  } while (0)
+    if (es == 4) { if (v == 4) LAUNCH_T(uint32_t, 4); else if (v == 2) LAUNCH_T(uint32_t, 2); else LAUNCH_T(uint32_t, 1); }
+    else if (es == 2) { if (v == 8) LAUNCH_T(uint16_t, 8); else if (v == 4) LAUNCH_T(uint16_t, 4); else if (v == 2) LAUNCH_T(uint16_t, 2); else LAUNCH_T(uint16_t, 1); }
+    else { if (v == 2) LAUNCH_T(uint64_t, 2); else LAUNCH_T(uint64_t, 1); }
+#undef LAUNCH_T
+    DNNRT_CHECK_LAUNCH("dnnrtTranspose");
+    return Y;
   }
   const int64_t total = s, blocks = ceil_div(total, 256);
   if (blocks > INT32_MAX) DNNRT_FAIL("dnnrtTranspose: tensor too large");

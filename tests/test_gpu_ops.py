@@ -164,6 +164,17 @@ def test_tensor_op(gpu, cpu):
     a = r.standard_normal((2, 3, 4, 8)).astype(np.float16)
     b = r.standard_normal((1, 3, 1, 1)).astype(np.float16)
     np.testing.assert_array_equal(oc.tensor_op(gpu, _abi.OP_ADD, a, b), oc.tensor_op(cpu, _abi.OP_ADD, a, b))
+    # 16-byte broadcast path (innermost run a multiple of 16 bytes) next to the element-wise one, both dtypes
+    for dtype in (np.float32, np.float16):
+        for sa, sb in [((2, 6, 4, 8), (1, 6, 1, 1)), ((2, 6, 4, 8), (2, 1, 4, 8)), ((2, 6, 4, 8), (2, 6, 1, 1)),
+                       ((2, 6, 4, 8), (1, 1, 1, 8)), ((2, 6, 4, 8), (1, 6, 1, 8)), ((2, 6, 4, 8), (1, 1, 4, 1)),
+                       ((3, 5, 16), (3, 1, 16)), ((3, 5, 16), (1, 5, 1)), ((4, 24), (1, 1)), ((4, 24), (4, 1)),
+                       ((2, 6, 3, 6), (1, 6, 1, 1)), ((1, 64, 96, 96), (1, 1, 1, 1)), ((2, 64, 28, 28), (1, 64, 1, 1))]:
+            a = r.standard_normal(sa).astype(dtype)
+            b = r.standard_normal(sb).astype(dtype)
+            want = (a.astype(np.float32) + b.astype(np.float32)).astype(dtype)
+            np.testing.assert_array_equal(oc.tensor_op(gpu, _abi.OP_ADD, a, b), want)
+            np.testing.assert_array_equal(oc.tensor_op(gpu, _abi.OP_MUL, a, b), oc.tensor_op(cpu, _abi.OP_MUL, a, b))
 
 
 # ---- reductions --------------------------------------------------------------------
@@ -317,6 +328,18 @@ def test_data_movement(gpu, cpu):
     ti = r.integers(-1000, 1000, (70, 3, 20)).astype(np.int64)
     np.testing.assert_array_equal(oc.gather(gpu, ti, np.array([[6, 0], [3, -2]]), 0), np.take(ti, [[6, 0], [3, -2]], 0))
     np.testing.assert_array_equal(oc.gather(gpu, ti, np.array([19, 1]), 2), oc.gather(cpu, ti, np.array([19, 1]), 2))
+    # every permutation of a rank-4 tensor whose dims allow 1-, 2-, 4- and 8-element units, each dtype,
+    # plus shapes with size-1 dims and runs of dims that stay together
+    import itertools
+    for dtype in (np.float32, np.float16, np.int64):
+        t = r.integers(-999, 999, (4, 6, 8, 16)).astype(dtype)
+        for perm in itertools.permutations(range(4)):
+            np.testing.assert_array_equal(oc.transpose(gpu, t, perm), t.transpose(perm))
+        for shape, perm in [((2, 1, 8, 4), (2, 1, 0, 3)), ((1, 64, 2, 2, 12, 12), (0, 1, 4, 2, 5, 3)), ((3, 5, 7), (2, 0, 1)),
+                            ((2, 3, 4, 5, 6), (0, 3, 4, 1, 2)), ((1, 1, 1), (2, 1, 0)), ((6, 8), (0, 1))]:
+            t = r.integers(-999, 999, shape).astype(dtype)
+            np.testing.assert_array_equal(oc.transpose(gpu, t, perm), t.transpose(perm))
+            np.testing.assert_array_equal(oc.transpose(gpu, t, perm), oc.transpose(cpu, t, perm))
     with pytest.raises(RuntimeError):
         oc.transpose(gpu, x, (0, 1, 1, 3))
 
