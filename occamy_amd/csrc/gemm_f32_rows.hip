@@ -147,7 +147,7 @@ __global__ __launch_bounds__(512) void gemm_f32_rows_kernel(const IgemmArgs a, c
   const int col = n0 + wn0 + l32;
   const bool col_ok = col < a.Ncols;
   const int colc = col_ok ? col : 0;
-  const float bias_c = a.bias_col ? a.bias_col[colc] : 0.f;
+  const float bias_c = load_bias_col(a, colc);
   float res_r[16];
   if (a.Cin) {
 #pragma unroll

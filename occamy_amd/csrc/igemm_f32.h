@@ -39,6 +39,17 @@ struct IgemmArgs {
   bool b_vec4;        // (b_kcontig) B rows may be read as aligned float4
 };
 
+// The per-column bias of a lane's column, or 0 without one.  The load is
+// unconditional (with no bias_col it reads A[0], which always exists, and the
+// value is dropped): a load under a branch makes the compiler wait for every
+// outstanding load where it is first used, which cost the small kernels over
+// a microsecond.
+__device__ __forceinline__ float load_bias_col(const IgemmArgs &a, int col) {
+  const float *at = a.bias_col ? a.bias_col + col : a.A;
+  const float v = *at;
+  return a.bias_col ? v : 0.f;
+}
+
 // Launches the kernel on `stream`; returns false (with the error text set) if
 // the shape cannot be handled.
 bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a);

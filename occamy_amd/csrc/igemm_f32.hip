@@ -233,7 +233,7 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
     const int colc = col_ok ? col : 0;
     const int img = colc / PQ, pq = colc - img * PQ;
     const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
-    const float bias_c = a.bias_col ? a.bias_col[colc] : 0.f;
+    const float bias_c = load_bias_col(a, colc);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       float res_r[16];

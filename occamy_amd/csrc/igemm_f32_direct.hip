@@ -134,7 +134,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
   const int img = colc / PQ, pq = colc - img * PQ;
   const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
   float bias_r[16], res_r[16];
-  const float bias_c = a.bias_col ? a.bias_col[colc] : 0.f;
+  const float bias_c = load_bias_col(a, colc);
   if (a.bias) {
     const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
 #pragma unroll

@@ -53,14 +53,13 @@ __device__ __forceinline__ void prefetch_bias(const IgemmArgs &a, int z, int m0,
 // finishes the tile.  Nobody waits for anybody.  The last arriver puts the
 // counter back to zero for the next kernel on the stream.
 template <int KS>
-__device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, const float (&bias_r)[16], float (*red)[16][64],
+__device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, const float (&bias_r)[16], float bias_c, float (*red)[16][64],
                                                  int wave, int lane, int m0, int col, bool col_ok, int z, unsigned tile,
                                                  float *partials, unsigned *counters) {
   const int half = lane >> 5, PQ = a.P * a.Q;
   // the residual tensor's 16 values, requested before anything is waited for
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
-  const float bias_c = a.bias_col ? a.bias_col[col_ok ? col : 0] : 0.f;
   float res_r[16];
   if (a.Cin) {
     if (wave == 0) {
@@ -162,6 +161,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   const int PQ = a.P * a.Q, HW = a.H * a.W, C = a.Kdim / 9;
   float bias_r[16];
   prefetch_bias(a, z, m0, half, bias_r);
+  const float bias_c = 0.f;  // a per-column bias belongs to matrix products, which are never 3x3
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int p = pq / a.Q, q = pq - p * a.Q;
   const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, bias_r, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
+  reduce_and_store<KS>(a, acc, bias_r, bias_c, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // 1x1 geometry (convolution, possibly strided, or matrix product with A rows
@@ -245,6 +245,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   const int PQ = a.P * a.Q, HW = a.H * a.W;
   float bias_r[16];
   prefetch_bias(a, z, m0, half, bias_r);
+  const float bias_c = load_bias_col(a, col_ok ? col : 0);  // requested up front as well
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int p = pq / a.Q, q = pq - p * a.Q;
   const unsigned x_pix = (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, bias_r, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
+  reduce_and_store<KS>(a, acc, bias_r, bias_c, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // Returns true if one of the specialised kernels took the problem.
@@ -301,7 +302,7 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
   const int64_t a_elems = amc ? (int64_t)a.Kdim * a.a_ld : (int64_t)a.M * a.Kdim;
   const int64_t x_elems = (int64_t)((a.Ncols + a.P * a.Q - 1) / (a.P * a.Q)) * a.x_img_stride + (int64_t)a.Kdim * a.H * a.W;
   if (a_elems >= (1ll << 31) || x_elems >= (1ll << 31)) return true;
-  const bool is3x3 = rsmode == 3 && a.Kdim % 9 == 0;
+  const bool is3x3 = rsmode == 3 && a.Kdim % 9 == 0 && !a.bias_col;
   const bool is1x1 = rsmode == 1 && (amc || a.a_vec4) && a.Kdim % 4 == 0 && a.Kdim >= 4;
   if (!is3x3 && !is1x1) return true;
 
