@@ -30,6 +30,9 @@ __device__ __forceinline__ float mask_f(float v, unsigned m) { return __uint_as_
 // The 16 accumulator registers of a lane hold rows m0 + 8 * (r >> 2) + 4 * half + (r & 3)
 // of output column n0 + l32.
 __device__ __forceinline__ int acc_row(int m0, int half, int r) { return m0 + 8 * (r >> 2) + 4 * half + (r & 3); }
+// ... that is, row m0 + 4 * half (the only part that differs between lanes) plus row_k(r), known at compile time:
+// address arithmetic per row is then a uniform offset (scalar unit) added to one per-lane base.
+__device__ __forceinline__ constexpr int row_k(int r) { return 8 * (r >> 2) + (r & 3); }
 
 // Bias of the lane's 16 rows, requested at kernel start so that the values
 // are there when the epilogue wants them (a load per row at that point costs
@@ -37,8 +40,17 @@ __device__ __forceinline__ int acc_row(int m0, int half, int r) { return m0 + 8 
 __device__ __forceinline__ void prefetch_bias(const IgemmArgs &a, int z, int m0, int half, float (&bias_r)[16]) {
   if (a.bias) {
     const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
+    if (m0 + 32 <= a.M && (reinterpret_cast<uintptr_t>(biasg) & 15u) == 0) {
+      // whole tile inside the matrix: the lane's rows are four runs of four, one 16-byte load each
 #pragma unroll
-    for (int r = 0; r < 16; r++) bias_r[r] = biasg[min(acc_row(m0, half, r), a.M - 1)];
+      for (int g = 0; g < 4; g++) {
+        const float4 v = *reinterpret_cast<const float4 *>(biasg + m0 + 8 * g + 4 * half);
+        bias_r[4 * g] = v.x; bias_r[4 * g + 1] = v.y; bias_r[4 * g + 2] = v.z; bias_r[4 * g + 3] = v.w;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; r++) bias_r[r] = biasg[min(acc_row(m0, half, r), a.M - 1)];
+    }
   } else {
 #pragma unroll
     for (int r = 0; r < 16; r++) bias_r[r] = 0.f;
@@ -52,20 +64,26 @@ __device__ __forceinline__ void prefetch_bias(const IgemmArgs &a, int z, int m0,
 // arrival does not matter, so the result is the same bits on every run -- and
 // finishes the tile.  Nobody waits for anybody.  The last arriver puts the
 // counter back to zero for the next kernel on the stream.
-template <int KS>
+template <int KS, bool WIDE_FIXUP>
 __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 acc, const float (&bias_r)[16], float bias_c, float (*red)[16][64],
-                                                 int wave, int lane, int m0, int col, bool col_ok, int z, unsigned tile,
+                                                 int wave, int lane, int m0, int img, int pq, bool col_ok, int z, unsigned tile,
                                                  float *partials, unsigned *counters) {
-  const int half = lane >> 5, PQ = a.P * a.Q;
+  const int half = lane >> 5;
+  const bool full = m0 + 32 <= a.M;  // the whole tile lies inside the matrix (same for every lane)
   // the residual tensor's 16 values, requested before anything is waited for
-  const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
   float res_r[16];
   if (a.Cin) {
     if (wave == 0) {
       const float *__restrict__ Cg = a.Cin + (int64_t)z * a.c_z_stride;
+      if (full) {
+        const float *__restrict__ c0 = Cg + ycol + (int64_t)(m0 + 4 * half) * a.c_row_stride;
 #pragma unroll
-      for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(acc_row(m0, half, r), a.M - 1) * a.c_row_stride];
+        for (int r = 0; r < 16; r++) res_r[r] = c0[(int64_t)row_k(r) * a.c_row_stride];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(acc_row(m0, half, r), a.M - 1) * a.c_row_stride];
+      }
     }
   } else {
 #pragma unroll
@@ -98,35 +116,57 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     if (lane == 0) arrived = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != (unsigned)splits - 1) return;
-    // splits is a power of two >= 2: two partial tiles are requested together
-    // and added in split order
-    const float *all = partials + (size_t)tile * splits * 1024;
+    // splits is a power of two >= 2: the partial tiles are requested four
+    // (WIDE_FIXUP: eight) at a time, a memory round trip each time, and added in split order
+    const float *all = partials + (size_t)tile * splits * 1024 + lane;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    for (int y = 0; y < splits; y += 2) {
+    auto part = [&](int y, float (&p)[16]) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) p[r] = __hip_atomic_load(all + (size_t)y * 1024 + r * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    if (splits == 2) {
       float p0[16], p1[16];
-#pragma unroll
-      for (int r = 0; r < 16; r++) p0[r] = __hip_atomic_load(all + (size_t)y * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int r = 0; r < 16; r++) p1[r] = __hip_atomic_load(all + (size_t)(y + 1) * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      part(0, p0); part(1, p1);
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[r] = (acc[r] + p0[r]) + p1[r];
+    } else if (splits == 4 || !WIDE_FIXUP) {
+      for (int y = 0; y < splits; y += 4) {
+        float p0[16], p1[16], p2[16], p3[16];
+        part(y, p0); part(y + 1, p1); part(y + 2, p2); part(y + 3, p3);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = (((acc[r] + p0[r]) + p1[r]) + p2[r]) + p3[r];
+      }
+    } else {  // the 3x3 kernel has the registers for it anyway
+      for (int y = 0; y < splits; y += 8) {
+        float p0[16], p1[16], p2[16], p3[16], p4[16], p5[16], p6[16], p7[16];
+        part(y, p0); part(y + 1, p1); part(y + 2, p2); part(y + 3, p3);
+        part(y + 4, p4); part(y + 5, p5); part(y + 6, p6); part(y + 7, p7);
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          acc[r] = (((((((acc[r] + p0[r]) + p1[r]) + p2[r]) + p3[r]) + p4[r]) + p5[r]) + p6[r]) + p7[r];
+      }
     }
     if (lane == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (!col_ok) return;
-  float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
-  // one copy of the store loop per activation mode, picked once (the mode is the same for every lane)
-  auto store = [&](auto mode_c) {
+  float *__restrict__ y0 = a.Y + (int64_t)z * a.y_z_stride + ycol + (int64_t)(m0 + 4 * half) * a.y_row_stride;
+  // one copy of the store loop per activation mode, picked once (the mode is the same for every lane);
+  // only a tile that sticks out of the matrix checks its rows
+  auto store_rows = [&](auto mode_c, auto full_c) {
     constexpr int MODE = decltype(mode_c)::value;
+    constexpr bool FULL = decltype(full_c)::value;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-      const int mm = acc_row(m0, half, r);
-      if (mm >= a.M) continue;
+      if (!FULL && acc_row(m0, half, r) >= a.M) continue;
       float v = a.alpha * acc[r] + bias_r[r] + bias_c;
       if (a.Cin) v += a.beta * res_r[r];
-      Yg[ycol + (int64_t)mm * a.y_row_stride] = apply_act(v, MODE, a.act_coef);
+      y0[(int64_t)row_k(r) * a.y_row_stride] = apply_act(v, MODE, a.act_coef);
     }
+  };
+  auto store = [&](auto mode_c) {
+    if (full) store_rows(mode_c, std::true_type{});
+    else store_rows(mode_c, std::false_type{});
   };
   switch (a.act) {
     case DNNRT_ACT_RELU: store(std::integral_constant<int, DNNRT_ACT_RELU>{}); break;
@@ -216,7 +256,7 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, bias_r, bias_c, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
+  reduce_and_store<KS, true>(a, acc, bias_r, bias_c, red, wave, lane, m0, img, pq, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // 1x1 geometry (convolution, possibly strided, or matrix product with A rows
@@ -290,7 +330,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
       }
     }
   }
-  reduce_and_store<KS>(a, acc, bias_r, bias_c, red, wave, lane, m0, col, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
+  reduce_and_store<KS, false>(a, acc, bias_r, bias_c, red, wave, lane, m0, img, pq, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
 // Returns true if one of the specialised kernels took the problem.
