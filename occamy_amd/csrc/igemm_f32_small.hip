@@ -245,17 +245,35 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
 #pragma unroll
   for (int d = 0; d < DEPTH; d++) load_iter(d, ra[d], rb[d], cm[d]);
-  for (int i0 = 0; i0 < niter; i0 += DEPTH) {
+  auto mfma_iter = [&](int u) {
+#pragma unroll
+    for (int j = 0; j < 9; j++)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u][j], mask_f(rb[u][j], tap_mask[j] & cm[u]), acc, 0, 0, 0);
+  };
+  // Iteration i lives in slot i % DEPTH and is refilled with iteration
+  // i + DEPTH.  Whole groups that need every refill run without a branch; the
+  // last DEPTH iterations refill nothing, and the group in between asks per
+  // slot.  Most batch-1 layers have exactly DEPTH iterations per wavefront:
+  // everything is requested by the prologue and nothing is loaded in vain.
+  int i0 = 0;
+  for (; i0 + 2 * DEPTH <= niter; i0 += DEPTH) {
 #pragma unroll
     for (int u = 0; u < DEPTH; u++) {
-      if (i0 + u < niter) {
-#pragma unroll
-        for (int j = 0; j < 9; j++)
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u][j], mask_f(rb[u][j], tap_mask[j] & cm[u]), acc, 0, 0, 0);
-        load_iter(i0 + u + DEPTH, ra[u], rb[u], cm[u]);
-      }
+      mfma_iter(u);
+      load_iter(i0 + u + DEPTH, ra[u], rb[u], cm[u]);
     }
   }
+#pragma unroll
+  for (int u = 0; u < DEPTH; u++) {
+    if (i0 + u < niter) {
+      mfma_iter(u);
+      if (i0 + u + DEPTH < niter) load_iter(i0 + u + DEPTH, ra[u], rb[u], cm[u]);
+    }
+  }
+  i0 += DEPTH;
+#pragma unroll
+  for (int u = 0; u < DEPTH; u++)
+    if (i0 + u < niter) mfma_iter(u);
   reduce_and_store<KS, true>(a, acc, bias_r, bias_c, red, wave, lane, m0, img, pq, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
@@ -318,18 +336,32 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
 #pragma unroll
   for (int d = 0; d < DEPTH; d++) load_iter(d, ra[d], rb[d], km[d]);
-  for (int i0 = 0; i0 < niter; i0 += DEPTH) {
+  auto mfma_iter = [&](int u) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].x, mask_f(rb[u][0], km[u]), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].y, mask_f(rb[u][1], km[u]), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].z, mask_f(rb[u][2], km[u]), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].w, mask_f(rb[u][3], km[u]), acc, 0, 0, 0);
+  };
+  // refills as in the 3x3 kernel: branch-free groups, then one group that asks per slot, then none
+  int i0 = 0;
+  for (; i0 + 2 * DEPTH <= niter; i0 += DEPTH) {
 #pragma unroll
     for (int u = 0; u < DEPTH; u++) {
-      if (i0 + u < niter) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].x, mask_f(rb[u][0], km[u]), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].y, mask_f(rb[u][1], km[u]), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].z, mask_f(rb[u][2], km[u]), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ra[u].w, mask_f(rb[u][3], km[u]), acc, 0, 0, 0);
-        load_iter(i0 + u + DEPTH, ra[u], rb[u], km[u]);
-      }
+      mfma_iter(u);
+      load_iter(i0 + u + DEPTH, ra[u], rb[u], km[u]);
     }
   }
+#pragma unroll
+  for (int u = 0; u < DEPTH; u++) {
+    if (i0 + u < niter) {
+      mfma_iter(u);
+      if (i0 + u + DEPTH < niter) load_iter(i0 + u + DEPTH, ra[u], rb[u], km[u]);
+    }
+  }
+  i0 += DEPTH;
+#pragma unroll
+  for (int u = 0; u < DEPTH; u++)
+    if (i0 + u < niter) mfma_iter(u);
   reduce_and_store<KS, false>(a, acc, bias_r, bias_c, red, wave, lane, m0, img, pq, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
