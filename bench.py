@@ -28,19 +28,19 @@ PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
 def build_workload(name):
     from occamy_amd import models
     if name == "resnet50_fp32_bs1":
-        return models.resnet50(1, np.float32), dict(fusion=True, fuse_residual=True), 1, "img/s", "f32"
+        return models.resnet50(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
         return models.resnet50(64, np.float16, seed=5), dict(fusion=True, fuse_residual=True, channels_last=True), 64, "img/s", "f16"
     if name == "mobilenet_v2_fp32_bs1":
-        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True), 1, "img/s", "f32"
+        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
         return models.bert_encoder(), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True), 1, "seq/s", "f32"
     if name == "single_conv_fp32":
         return models.single_conv(), dict(fusion=True), 1, "img/s", "f32"
     if name == "alexnet_fp32_bs1":
-        return models.alexnet(1, np.float32), dict(fusion=True), 1, "img/s", "f32"
+        return models.alexnet(1, np.float32), dict(fusion=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "yolo_v1_fp32_bs2":
-        return models.yolo_v1(2, np.float32), dict(fusion=True, fuse_activations=True), 2, "img/s", "f32"
+        return models.yolo_v1(2, np.float32), dict(fusion=True, fuse_activations=True, fuse_matmul_bias=True), 2, "img/s", "f32"
     if name == "srgan_fp32_96x96":
         return models.srgan_generator(1, np.float32, height=96, width=96), dict(fusion=True, fuse_residual=True, fuse_activations=True), 1, "img/s", "f32"
     raise SystemExit(f"unknown workload {name}")

@@ -344,8 +344,12 @@ bool Session::issue(const Op *op, std::string &err) {
                          op->axis, dt);
       break;
     case OP_MATMUL2D:
-      r = rt.dnnrtMatmul2d(handle, 2, P(0), op->dimA.data(), P(1), op->dimB.data(), out, op->dimOut.data(), out,
-                           op->dimOut.data(), op->alpha, op->beta, op->trans_a, op->trans_b, dt);
+      if (op->operands.size() == 4)  // a, b, c, out: C folded in by the matmul + bias fusion
+        r = rt.dnnrtMatmul2d(handle, 2, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), op->kernel.data(), out,
+                             op->dimOut.data(), op->alpha, op->beta, op->trans_a, op->trans_b, dt);
+      else
+        r = rt.dnnrtMatmul2d(handle, 2, P(0), op->dimA.data(), P(1), op->dimB.data(), out, op->dimOut.data(), out,
+                             op->dimOut.data(), op->alpha, op->beta, op->trans_a, op->trans_b, dt);
       break;
     case OP_MATMULND:
       r = rt.dnnrtMatmulNd(handle, P(0), op->dimA.data(), (int32_t)op->dimA.size(), P(1), op->dimB.data(),

@@ -209,7 +209,9 @@ std::string Program::to_text() const {
       case OP_TRANSPOSE: os << " {perm="; print_shape(os, op->perm); os << "}"; break;
       case OP_MATMUL2D:
         os << " {alpha=" << op->alpha << ", beta=" << op->beta << ", transA=" << op->trans_a
-           << ", transB=" << op->trans_b << "}";
+           << ", transB=" << op->trans_b;
+        if (op->operands.size() == 4) { os << ", dimC="; print_shape(os, op->kernel); }
+        os << "}";
         break;
       case OP_CLIP: os << " {min=" << op->lo << ", max=" << op->hi << "}"; break;
       case OP_LAYERNORM: os << " {eps=" << op->eps << "}"; break;

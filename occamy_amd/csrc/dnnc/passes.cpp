@@ -232,6 +232,43 @@ void fuse_matmul_bias(Program &p) {
       if (buf->uses.empty() && buf->def) p.erase(buf->def);
     }
   }
+  // Gemm (Ops/cublas/Gemm.cpp:60-81: a product with beta 0, then C added onto
+  // the same buffer): C becomes the product's own C operand with beta 1.
+  std::vector<Op *> gemms;
+  for (Op *op : p.ops)
+    if (op->kind == OP_MATMUL2D && op->operands.size() == 3 && op->beta == 0.f) gemms.push_back(op);
+  for (Op *mm : gemms) {
+    // the add works on the product's BUFFER (first operand and output), not on the product's result value
+    Value *buf = mm->operands[2];
+    if (mm->result->dtype != F32 || !mm->result->uses.empty()) continue;
+    Op *add = nullptr;
+    for (const auto &u : buf->uses) {
+      Op *o = u.first;
+      if (o == mm || p.order(o) < p.order(mm)) continue;
+      if (!add || p.order(o) < p.order(add)) add = o;  // the buffer's next user
+    }
+    if (!add || add->kind != OP_ADD || add->coef != 1.f || add->operands[0] != buf || add->operands[2] != buf ||
+        add->operands[1] == buf)
+      continue;
+    if (add->dimB.size() != 2 || add->dimB[1] != mm->dimOut[1] || (add->dimB[0] != 1 && add->dimB[0] != mm->dimOut[0])) continue;
+    Value *out = buf;
+    Op *fused = p.new_op(OP_MATMUL2D);
+    fused->dimA = mm->dimA;
+    fused->dimB = mm->dimB;
+    fused->dimOut = mm->dimOut;
+    fused->kernel = add->dimB;  // dims of C
+    fused->alpha = mm->alpha;
+    fused->beta = 1.f;
+    fused->trans_a = mm->trans_a;
+    fused->trans_b = mm->trans_b;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    p.insert_after(fused, add);
+    p.set_operands(fused, {mm->operands[0], mm->operands[1], add->operands[1], out});
+    p.replace_all_uses(add->result, fused->result);
+    p.erase(add);
+    p.erase(mm);
+  }
   // second step: the Linear layer's consumer joins in when it is the only
   // reader -- Gelu (mode 7), or the sum with a residual tensor of the same shape
   std::vector<Op *> linears;

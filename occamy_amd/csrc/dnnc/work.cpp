@@ -53,7 +53,7 @@ void op_work(const Op *op, double &flops, double &bytes) {
     case OP_MATMUL2D: {
       const double k = (double)(op->trans_a ? op->dimA[0] : op->dimA[1]);
       flops = 2.0 * n_out * k;
-      bytes = (n_in(0) + n_in(1) + n_out) * es;
+      bytes = (n_in(0) + n_in(1) + n_out + (op->operands.size() == 4 ? n_in(2) : 0.0)) * es;
       break;
     }
     case OP_MATMULND:

@@ -122,7 +122,7 @@ void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A, const int
                     const void *B, const int64_t *dimB, const void *C, const int64_t *dimC,
                     void *Out, const int64_t *dimOut, float alpha, float beta, int64_t transA,
                     int64_t transB, int32_t dtype) {
-  (void)rank; (void)dimC;
+  (void)rank;
   if (!handle) DNNRT_FAIL("dnnrtMatmul2d: null handle");
   if (!A || !B || !Out || !dimA || !dimB || !dimOut) DNNRT_FAIL("dnnrtMatmul2d: null argument");
   const int64_t M = transA ? dimA[1] : dimA[0], K = transA ? dimA[0] : dimA[1];
@@ -133,12 +133,17 @@ void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A, const int
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) DNNRT_FAIL("dnnrtMatmul2d: dims exceed 32 bits");
   if (beta != 0.f && !C) DNNRT_FAIL("dnnrtMatmul2d: beta != 0 needs C");
   const void *Cin = beta != 0.f ? C : nullptr;
+  // C is [M, N], or one row [1, N] added to every row of the product
+  const bool c_is_row = Cin && dimC && dimC[0] == 1 && dimC[1] == N && M > 1;
+  if (Cin && dimC && !c_is_row && (dimC[0] != M || dimC[1] != N))
+    DNNRT_FAIL("dnnrtMatmul2d: C is [%ld,%ld], neither [M,N] nor [1,N]", (long)dimC[0], (long)dimC[1]);
   if (dtype == DNNRT_F32) {
     if (!gemm_f32(handle, (const float *)A, (const float *)B, (const float *)Cin, (float *)Out, (int)M,
-                  (int)N, (int)K, alpha, beta, transA != 0, transB != 0, 1, 0, 0, 0))
+                  (int)N, (int)K, alpha, beta, transA != 0, transB != 0, 1, 0, 0, 0, c_is_row))
       return nullptr;
     return Out;
   }
+  if (dtype == DNNRT_F16 && c_is_row) DNNRT_FAIL("dnnrtMatmul2d: a one-row C is not built for fp16");
   if (dtype == DNNRT_F16) {
     if (!gemm_f16(handle, (const __half *)A, (const __half *)B, (const __half *)Cin, (__half *)Out,
                   (int)M, (int)N, (int)K, alpha, beta, transA != 0, transB != 0, 1, 0, 0, 0))

@@ -167,10 +167,11 @@ class Ops:
                          "dnnrtAveragePool")
 
     def matmul2d(self, A, dimA, B, dimB, Out, dimOut, alpha=1.0, beta=0.0, transA=0, transB=0, C_=None,
-                 dtype=_abi.F32):
+                 dtype=_abi.F32, dimC=None):
+        """dimC: [M, N] (default) or [1, N] for one row added to every row of the product."""
         return self._ret(self.lib.dnnrtMatmul2d(self.handle, 2, A, dims(dimA), B, dims(dimB), C_,
-                                                dims(dimOut), Out, dims(dimOut), alpha, beta, transA,
-                                                transB, dtype), "dnnrtMatmul2d")
+                                                dims(dimC if dimC is not None else dimOut), Out, dims(dimOut), alpha,
+                                                beta, transA, transB, dtype), "dnnrtMatmul2d")
 
     def matmul_nd(self, A, dimA, B, dimB, Y, dimY, dtype=_abi.F32):
         return self._ret(self.lib.dnnrtMatmulNd(self.handle, A, dims(dimA), len(dimA), B, dims(dimB),

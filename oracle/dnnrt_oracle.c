@@ -674,7 +674,7 @@ void *dnnrtMatmul2d(dnnrtHandle_t h, int64_t rank, const void *A, const int64_t 
                     const void *B, const int64_t *dB, const void *C,
                     const int64_t *dC, void *Out, const int64_t *dO, float alpha,
                     float beta, int64_t transA, int64_t transB, int32_t dtype) {
-  (void)h; (void)rank; (void)dC;
+  (void)h; (void)rank;
   if (bad_dtype(dtype)) FAIL("matmul2d: bad dtype");
   const int64_t M = transA ? dA[1] : dA[0], K = transA ? dA[0] : dA[1];
   const int64_t Kb = transB ? dB[1] : dB[0], N = transB ? dB[0] : dB[1];
@@ -683,15 +683,24 @@ void *dnnrtMatmul2d(dnnrtHandle_t h, int64_t rank, const void *A, const int64_t 
   float *ta, *tb, *tc = NULL, *to;
   const float *a = widen(A, M * K, dtype, &ta);
   const float *b = widen(B, K * N, dtype, &tb);
-  const float *c = (beta != 0.0f) ? widen(C, M * N, dtype, &tc) : NULL;
+  /* C: [M,N] (CUBLASMatmul2dFunc.cu:32 sizes it by dimOutput) or one row [1,N] for every row of the product */
+  const int c_row = beta != 0.0f && dC && dC[0] == 1 && dC[1] == N; /* also when M == 1: the chain's two roundings */
+  if (beta != 0.0f && dC && !c_row && (dC[0] != M || dC[1] != N)) FAIL("matmul2d: C dims");
+  const float *c = (beta != 0.0f) ? widen(C, c_row ? N : M * N, dtype, &tc) : NULL;
   float *o = outbuf(Out, M * N, dtype, &to);
   float *cc = NULL;
   if (c) { /* C may alias Out */
-    cc = (float *)malloc(sizeof(float) * (size_t)(M * N));
-    memcpy(cc, c, sizeof(float) * (size_t)(M * N));
+    cc = (float *)malloc(sizeof(float) * (size_t)(c_row ? N : M * N));
+    memcpy(cc, c, sizeof(float) * (size_t)(c_row ? N : M * N));
   }
   gemm_core(a, transA ? 1 : K, transA ? M : 1, b, transB ? 1 : N, transB ? K : 1,
-            cc, o, M, N, K, alpha, beta);
+            c_row ? NULL : cc, o, M, N, K, alpha, c_row ? 0.0f : beta);
+  if (c_row) /* the row case is the reference's Gemm chain (Ops/cublas/Gemm.cpp:60-81): product, then the broadcast add */
+    for (int64_t m = 0; m < M; m++)
+      for (int64_t n = 0; n < N; n++) {
+        const float t = beta * cc[n];
+        o[m * N + n] = o[m * N + n] + t;
+      }
   free(cc);
   narrow(Out, to, M * N, dtype); free(ta); free(tb); free(tc);
   return Out;

@@ -137,6 +137,17 @@ def matmul2d(be, a, b, c=None, alpha=1.0, beta=0.0, transA=0, transB=0):
     return be.get(Out)
 
 
+def matmul2d_row(be, a, b, row, alpha=1.0, beta=1.0, transB=0):
+    """Out = alpha a b + beta row, the row [N] added to every row of the product."""
+    M, N = a.shape[0], (b.shape[0] if transB else b.shape[1])
+    A, B, C_ = be.put(a), be.put(b), be.put(row.reshape(1, N))
+    Out = be.empty((M, N), a.dtype)
+    be.ops.matmul2d(be.ptr(A), a.shape, be.ptr(B), b.shape, be.ptr(Out), (M, N), alpha, beta, 0, transB,
+                    be.ptr(C_), DT[a.dtype], dimC=(1, N))
+    be.sync()
+    return be.get(Out)
+
+
 def matmul_nd(be, a, b):
     y_shape = np.matmul(np.zeros(a.shape, np.float32), np.zeros(b.shape, np.float32)).shape
     A, B = be.put(a), be.put(b)

@@ -224,6 +224,23 @@ def test_activation_fusion_matches_unfused_chain(builder):
         np.testing.assert_array_equal(x, y)
 
 
+@pytest.mark.parametrize("builder", [lambda: models.resnet50(image=32, classes=10), ALEX,
+                                     lambda: models.mobilenet_v2(image=32, classes=10)],
+                         ids=["resnet50", "alexnet", "mobilenet_v2"])
+def test_gemm_bias_fusion_matches_unfused_chain(builder):
+    # Gemm is a product and an in-place bias add in the reference (Ops/cublas/Gemm.cpp:60-81); folded
+    # into one call the oracle still runs the chain, so not a bit may change and one launch per Gemm goes
+    _, _, a = run_oracle(builder, fusion=True)
+    _, _, b = run_oracle(builder, fusion=True, fuse_matmul_bias=True)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+    ta, tb = builder()[0].compile(fusion=True).text, builder()[0].compile(fusion=True, fuse_matmul_bias=True).text
+    gemms = ta.count("dnn.matmul2d")
+    assert gemms >= 1 and tb.count("dnn.matmul2d") == gemms
+    assert ta.count("dnn.add") - tb.count("dnn.add") == gemms and "dimC=[1," in tb
+    check(builder, fusion=True, fuse_matmul_bias=True)
+
+
 def test_recomposed_bert_matches_torch_and_the_decomposed_program():
     small = dict(layers=2, hidden=64, heads=4, ffn=128, seq=16, vocab=100)
     flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)

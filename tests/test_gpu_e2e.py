@@ -170,6 +170,14 @@ def test_activation_fusion_fp32(name, oracle_outputs):
         close(o, r)
 
 
+@pytest.mark.parametrize("name", ["resnet50", "alexnet", "mobilenet_v2"])
+def test_gemm_bias_folded_into_the_product(name, oracle_outputs):
+    for mode in (compiler.MODE_OCCAMY, compiler.MODE_RESIDENT):
+        out, _ = run(CONFIGS[name], mode=mode, fusion=True, fuse_matmul_bias=True)
+        for o, r in zip(out, oracle_outputs[name]):
+            close(o, r)
+
+
 def test_bert_recomposed_with_fused_linear_layers(oracle_outputs):
     flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)
     out, _ = run(CONFIGS["bert_2_layers"], **flags)

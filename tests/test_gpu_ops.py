@@ -253,6 +253,12 @@ def test_matmul2d(gpu, cpu):
         close(oc.matmul2d(gpu, a.T.copy(), b.T.copy(), transA=1, transB=1), ref)
         close(oc.matmul2d(gpu, a, b.T.copy(), c.copy(), alpha=0.5, beta=-2.0, transB=1),
               oc.matmul2d(cpu, a, b.T.copy(), c.copy(), alpha=0.5, beta=-2.0, transB=1))
+        # C as one row (a Gemm's bias folded into the product): equal to product-then-add on the GPU, bit for bit
+        row = c[0].copy()
+        for tb, bb in ((0, b), (1, b.T.copy())):
+            fused = oc.matmul2d_row(gpu, a, bb, row, transB=tb)
+            close(fused, oc.matmul2d_row(cpu, a, bb, row, transB=tb))
+            np.testing.assert_array_equal(fused, oc.tensor_op(gpu, _abi.OP_ADD, oc.matmul2d(gpu, a, bb, transB=tb), row.reshape(1, -1)))
     with pytest.raises(RuntimeError):
         oc.matmul2d(gpu, np.zeros((5, 9), np.float32), np.zeros((9, 7), np.float32), transB=1)
 

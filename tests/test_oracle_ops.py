@@ -302,6 +302,11 @@ def test_matmul2d(be):
     np.testing.assert_allclose(oc.matmul2d(be, a, b.T.copy(), transB=1), A @ B, rtol=1e-6, atol=1e-6)
     np.testing.assert_allclose(oc.matmul2d(be, a.T.copy(), b.T.copy(), transA=1, transB=1), A @ B, rtol=1e-6, atol=1e-6)
     np.testing.assert_allclose(oc.matmul2d(be, a, b, c.copy(), alpha=0.5, beta=-2.0), 0.5 * (A @ B) - 2.0 * c, rtol=1e-6, atol=1e-6)
+    # C as one row: the Gemm bias.  With alpha = beta = 1 it is the product followed by the bias add, bit for bit
+    row = c[0].copy()
+    np.testing.assert_allclose(oc.matmul2d_row(be, a, b, row, alpha=0.5, beta=-2.0), 0.5 * (A @ B) - 2.0 * row, rtol=1e-6, atol=1e-6)
+    np.testing.assert_array_equal(oc.matmul2d_row(be, a, b, row), oc.tensor_op(be, _abi.OP_ADD, oc.matmul2d(be, a, b), row.reshape(1, -1)))
+    np.testing.assert_array_equal(oc.matmul2d_row(be, a[:1], b, row), oc.matmul2d(be, a[:1], b, row.reshape(1, -1).copy(), beta=1.0))
     # permutation matrix: rows of b reordered exactly
     perm = np.eye(9, dtype=np.float32)[r.permutation(9)]
     np.testing.assert_array_equal(oc.matmul2d(be, perm, b), perm @ b)
