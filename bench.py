@@ -119,13 +119,15 @@ def main():
                    value=batch * steps / dt, pool_bytes=prog.pool_bytes, weights_bytes=sess.weights_bytes,
                    kernels_per_step=prog.num_ops(compute_only=True), flags=flags)
         if want_profile:
-            # per-kernel device timestamps on the session's own stream, eager launches
+            # device timestamps on the session's own stream, eager launches: one pair per operation
+            # class around that class's launches issued back to back (a timestamp between two kernels
+            # of a few microseconds costs about as much as the kernels themselves)
             ops = prog.compute_ops()
             acc = np.zeros(len(ops))
             reps = 20
-            sess.profile(ip, on_device=True)
+            sess.profile(ip, on_device=True, by_class=True)
             for _ in range(reps):
-                acc += np.array(sess.profile(ip, on_device=True))
+                acc += np.array(sess.profile(ip, on_device=True, by_class=True))
             acc /= reps
             by_class = {}
             for (mn, cls, fl, by), ms in zip(ops, acc):

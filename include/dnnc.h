@@ -109,7 +109,11 @@ int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *o
 int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
 int32_t dnncSessionSync(dnncSession *s);
 /* resident mode: one eager pass with device timestamps around every compute
- * operation; ms[i] belongs to dnncProgramComputeOp(i).  Returns the count. */
+ * operation; ms[i] belongs to dnncProgramComputeOp(i).  Returns the count.
+ * on_device bit 0: the inputs are device buffers; bit 1: one pair of
+ * timestamps per operation class around that class's launches issued back to
+ * back, ms[i] = the class average (a timestamp between kernels of a few
+ * microseconds costs about as much as the kernels). */
 int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on_device, float *ms, int64_t cap);
 int64_t dnncSessionWeightsBytes(const dnncSession *s);
 /* bytes the last occamy-mode run requested from dnnrtMemPoolInit (-1 before any run) */

@@ -298,7 +298,7 @@ class Session:
         if lib().dnncSessionRunResident(self._s, ip, op, 1, int(use_graph)):
             raise RuntimeError("run_device: " + _err())
 
-    def profile(self, in_ptrs_or_arrays, on_device=False):
+    def profile(self, in_ptrs_or_arrays, on_device=False, by_class=False):
         """Resident mode: milliseconds per compute op (device timestamps), program order."""
         if on_device:
             ip = (C.c_void_p * max(len(in_ptrs_or_arrays), 1))(*in_ptrs_or_arrays)
@@ -307,7 +307,7 @@ class Session:
             ip = (C.c_void_p * max(len(keep), 1))(*[a.ctypes.data for a in keep])
         n = self.program.num_ops(compute_only=True)
         ms = (C.c_float * max(n, 1))()
-        if lib().dnncSessionProfile(self._s, ip, int(on_device), ms, n) < 0:
+        if lib().dnncSessionProfile(self._s, ip, int(on_device) | (2 if by_class else 0), ms, n) < 0:
             raise RuntimeError("profile: " + _err())
         return list(ms[:n])
 

@@ -284,7 +284,7 @@ int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on
   if (!s || !inputs) { fail("dnncSessionProfile: bad arguments"); return -1; }
   std::vector<float> t;
   std::string err;
-  if (!s->s.profile_resident(inputs, on_device, t, err)) { fail(err); return -1; }
+  if (!s->s.profile_resident(inputs, on_device & 1, (on_device & 2) != 0, t, err)) { fail(err); return -1; }
   for (size_t i = 0; i < t.size() && (int64_t)i < cap && ms; i++) ms[i] = t[i];
   return (int64_t)t.size();
 }

@@ -505,11 +505,12 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
   return true;
 }
 
-bool Session::profile_resident(const void *const *inputs, int on_device, std::vector<float> &ms, std::string &err) {
+bool Session::profile_resident(const void *const *inputs, int on_device, bool by_class, std::vector<float> &ms, std::string &err) {
   if (mode != MODE_RESIDENT) { err = "profiling needs a resident session"; return false; }
   std::vector<const Op *> compute;
   for (const Op *op : prog->ops)
     if (is_compute(op->kind)) compute.push_back(op);
+  if (by_class) return profile_classes(inputs, on_device, compute, ms, err);
   std::vector<void *> ev(compute.size() + 1, nullptr);
   bool ok = true;
   for (void *&e : ev)
@@ -535,6 +536,50 @@ bool Session::profile_resident(const void *const *inputs, int on_device, std::ve
   for (size_t i = 0; ok && i < compute.size(); i++)
     if (rt.dnnrtEventElapsedMs(ev[i], ev[i + 1], &ms[i])) { err = rt_error("dnnrtEventElapsedMs"); ok = false; }
   for (void *e : ev) rt.dnnrtEventDestroy(e);
+  return ok;
+}
+
+// One pair of timestamps per operation class, around all of the class's
+// launches issued back to back (in program order, on whatever the buffers
+// hold: only the durations matter).  A timestamp between two kernels of a few
+// microseconds costs about as much as the kernels; this way the class average
+// is the kernels' own duration plus the gap between consecutive dispatches.
+bool Session::profile_classes(const void *const *inputs, int on_device, const std::vector<const Op *> &compute,
+                              std::vector<float> &ms, std::string &err) {
+  std::vector<std::string> classes;
+  for (const Op *op : compute) {
+    const std::string c = op_class(op);
+    if (std::find(classes.begin(), classes.end(), c) == classes.end()) classes.push_back(c);
+  }
+  bool ok = true;
+  for (const Op *op : prog->ops) {  // inputs into their pool slots
+    if (op->kind != OP_MEMCPY || op->mode != 1 || op->operands[1]->arg_index < 0) continue;
+    const size_t ai = (size_t)op->operands[1]->arg_index;
+    const void *from = inputs[ai];
+    if (!on_device) { std::memcpy(host_in[ai], inputs[ai], (size_t)op->bytes); from = host_in[ai]; }
+    if (rt.dnnrtMemcpy(ptr[(size_t)op->operands[0]->id], const_cast<void *>(from), op->bytes, on_device ? 3 : 1, stream)) {
+      err = rt_error("dnnrtMemcpy(input)"); return false;
+    }
+  }
+  void *e0 = nullptr, *e1 = nullptr;
+  if (rt.dnnrtEventCreate(&e0) || rt.dnnrtEventCreate(&e1)) { err = rt_error("dnnrtEventCreate"); return false; }
+  ms.assign(compute.size(), 0.f);
+  for (size_t i = 0; ok && i < compute.size(); i++) ok = issue(compute[i], err);  // one whole pass first: real values everywhere
+  for (const std::string &c : classes) {
+    if (!ok) break;
+    size_t n = 0;
+    if (rt.dnnrtEventRecord(e0, stream)) { err = rt_error("dnnrtEventRecord"); ok = false; break; }
+    for (size_t i = 0; ok && i < compute.size(); i++)
+      if (c == op_class(compute[i])) { ok = issue(compute[i], err); n++; }
+    if (ok && rt.dnnrtEventRecord(e1, stream)) { err = rt_error("dnnrtEventRecord"); ok = false; }
+    if (ok && rt.dnnrtSync(handle)) { err = rt_error("dnnrtSync"); ok = false; }
+    float total = 0.f;
+    if (ok && rt.dnnrtEventElapsedMs(e0, e1, &total)) { err = rt_error("dnnrtEventElapsedMs"); ok = false; }
+    for (size_t i = 0; ok && i < compute.size(); i++)
+      if (c == op_class(compute[i])) ms[i] = total / (float)n;
+  }
+  rt.dnnrtEventDestroy(e0);
+  rt.dnnrtEventDestroy(e1);
   return ok;
 }
 

@@ -83,7 +83,11 @@ class Session {
   bool sync(std::string &err);
   // Resident mode: one eager pass with a device timestamp around every compute
   // operation; ms[i] is the time of the i-th compute op in program order.
-  bool profile_resident(const void *const *inputs, int on_device, std::vector<float> &ms, std::string &err);
+  // by_class: timestamps only around each operation class's launches issued
+  // back to back; ms[i] is then the class average.
+  bool profile_resident(const void *const *inputs, int on_device, bool by_class, std::vector<float> &ms, std::string &err);
+  bool profile_classes(const void *const *inputs, int on_device, const std::vector<const Op *> &compute,
+                       std::vector<float> &ms, std::string &err);
 
   const Program *prog = nullptr;
   int mode = MODE_OCCAMY;

@@ -70,9 +70,9 @@ __global__ __launch_bounds__(512) void gemm_f32_rows_kernel(const IgemmArgs a, c
   // One step: chunk c (ring slot r, LDS buffer `buf`) to LDS, refill the slot,
   // barrier, MFMAs.  The barrier of step c also separates the MFMAs of step
   // c - 1 from the store of step c + 1 into the same LDS buffer.
-  auto step = [&](int c, int buf, Chunk &r) {
+  auto step = [&](int c, int buf, Chunk &r, bool refill) {
     store_chunk(buf, r);
-    load_chunk(c + DEPTH, r);
+    if (refill) load_chunk(c + DEPTH, r);
     __syncthreads();
     const float *ap = &As[buf][kg * (BKC / 2) + half][wm0 + l32], *bp = &Bs[buf][kg * (BKC / 2) + half][wn0 + l32];
 #pragma unroll
@@ -84,16 +84,25 @@ __global__ __launch_bounds__(512) void gemm_f32_rows_kernel(const IgemmArgs a, c
     load_chunk(c_beg + 1, r1);
     load_chunk(c_beg + 2, r2);
     load_chunk(c_beg + 3, r3);
+    // Whole groups of DEPTH steps that need every refill run without a
+    // branch around the loads; the last DEPTH chunks refill nothing (a split
+    // holds about six chunks: refills past its end were most of the loads),
+    // and the group in between asks per slot.
     int c = c_beg;
-    for (; c + DEPTH <= c_end; c += DEPTH) {
-      step(c, 0, r0);
-      step(c + 1, 1, r1);
-      step(c + 2, 0, r2);
-      step(c + 3, 1, r3);
+    for (; c + 2 * DEPTH <= c_end; c += DEPTH) {
+      step(c, 0, r0, true);
+      step(c + 1, 1, r1, true);
+      step(c + 2, 0, r2, true);
+      step(c + 3, 1, r3, true);
     }
-    if (c < c_end) step(c, 0, r0);
-    if (c + 1 < c_end) step(c + 1, 1, r1);
-    if (c + 2 < c_end) step(c + 2, 0, r2);
+    if (c < c_end) step(c, 0, r0, c + DEPTH < c_end);
+    if (c + 1 < c_end) step(c + 1, 1, r1, c + 1 + DEPTH < c_end);
+    if (c + 2 < c_end) step(c + 2, 0, r2, c + 2 + DEPTH < c_end);
+    if (c + 3 < c_end) step(c + 3, 1, r3, c + 3 + DEPTH < c_end);
+    c += DEPTH;
+    if (c < c_end) step(c, 0, r0, false);
+    if (c + 1 < c_end) step(c + 1, 1, r1, false);
+    if (c + 2 < c_end) step(c + 2, 0, r2, false);
   }
 
   // the second k group hands its sums to the first through LDS (the tiles are free now)
