@@ -17,6 +17,8 @@
 // the epilogue and puts the counter back to zero.  Nobody waits for anybody.
 #include "igemm_f32.h"
 
+#include <type_traits>
+
 namespace dnnrt {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -105,7 +107,23 @@ __global__ __launch_bounds__(512) void gemm_f32_rows_kernel(const IgemmArgs a, c
     if (c + 2 < c_end) step(c + 2, 0, r2, false);
   }
 
-  // the second k group hands its sums to the first through LDS (the tiles are free now)
+  // what the epilogue adds, requested now: the values are there long before they are used
+  const int col = n0 + wn0 + l32;
+  const bool col_ok = col < a.Ncols;
+  const int colc = col_ok ? col : 0;
+  const float bias_c = load_bias_col(a, colc);
+  const int mrow0 = m0 + wm0 + 4 * half;  // the lane's rows are mrow0 + row_k(r)
+  auto row_k = [](int r) { return 8 * (r >> 2) + (r & 3); };
+  float res_r[16];
+  if (a.Cin && kg == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) res_r[r] = a.Cin[(int64_t)min(mrow0 + row_k(r), a.M - 1) * a.c_row_stride + colc];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) res_r[r] = 0.f;
+  }
+
+  // the second k group hands its sums to the first through LDS (the tiles are free after this barrier)
   __syncthreads();
   float *xch = &As[0][0][0];  // 4 wavefronts x 16 registers x 64 lanes = 16 KiB <= the 17 KiB of As
   if (kg == 1) {
@@ -132,47 +150,60 @@ __global__ __launch_bounds__(512) void gemm_f32_rows_kernel(const IgemmArgs a, c
     if (lane == 0) arrived = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != (unsigned)splits - 1) return;
-    const float *all = partials + (size_t)slot * splits * 1024;
+    // the partial tiles are requested four at a time (a memory round trip each time) and added in split order
+    const float *all = partials + (size_t)slot * splits * 1024 + lane;
+    auto part = [&](int y, float (&p)[16]) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) p[r] = __hip_atomic_load(all + (size_t)y * 1024 + r * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
     int y = 0;
-    for (; y + 2 <= splits; y += 2) {  // two partial tiles requested together, added in split order
-      float p0[16], p1[16];
+    for (; y + 4 <= splits; y += 4) {
+      float p0[16], p1[16], p2[16], p3[16];
+      part(y, p0); part(y + 1, p1); part(y + 2, p2); part(y + 3, p3);
 #pragma unroll
-      for (int r = 0; r < 16; r++) p0[r] = __hip_atomic_load(all + (size_t)y * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int r = 0; r < 16; r++) p1[r] = __hip_atomic_load(all + (size_t)(y + 1) * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[r] = (acc[r] + p0[r]) + p1[r];
+      for (int r = 0; r < 16; r++) acc[r] = (((acc[r] + p0[r]) + p1[r]) + p2[r]) + p3[r];
     }
-    if (y < splits) {
+    if (y < splits) {  // one to three left: requested together as well (an absent one re-reads the last and is not added)
+      float p0[16], p1[16], p2[16];
+      part(y, p0); part(min(y + 1, splits - 1), p1); part(min(y + 2, splits - 1), p2);
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[r] += __hip_atomic_load(all + (size_t)y * 1024 + r * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int r = 0; r < 16; r++) {
+        acc[r] += p0[r];
+        if (y + 1 < splits) acc[r] += p1[r];
+        if (y + 2 < splits) acc[r] += p2[r];
+      }
     }
     if (lane == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  // ---- epilogue: loads from clamped addresses in one batch, predicated stores
-  const int col = n0 + wn0 + l32;
-  const bool col_ok = col < a.Ncols;
-  const int colc = col_ok ? col : 0;
-  const float bias_c = load_bias_col(a, colc);
-  float res_r[16];
-  if (a.Cin) {
+  // ---- epilogue: one copy of the store loop per activation mode; a row is one per-lane base plus a uniform offset
+  if (!col_ok) return;
+  float *__restrict__ y0 = a.Y + (int64_t)mrow0 * a.y_row_stride + col;
+  auto store = [&](auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-    for (int r = 0; r < 16; r++)
-      res_r[r] = a.Cin[(int64_t)min(m0 + wm0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1) * a.c_row_stride + colc];
-  } else {
+    for (int r = 0; r < 16; r++) {
+      if (mrow0 + row_k(r) >= a.M) continue;
+      float v = a.alpha * acc[r] + bias_c;
+      if (a.Cin) v += a.beta * res_r[r];
+      y0[(int64_t)row_k(r) * a.y_row_stride] = apply_act(v, MODE, a.act_coef);
+    }
+  };
+  switch (a.act) {
+    case DNNRT_ACT_RELU: store(std::integral_constant<int, DNNRT_ACT_RELU>{}); break;
+    case ACT_GELU: store(std::integral_constant<int, ACT_GELU>{}); break;
+    case DNNRT_ACT_IDENTITY: store(std::integral_constant<int, DNNRT_ACT_IDENTITY>{}); break;
+    default: {  // the remaining modes through the run-time switch
 #pragma unroll
-    for (int r = 0; r < 16; r++) res_r[r] = 0.f;
-  }
-#pragma unroll
-  for (int r = 0; r < 16; r++) {
-    const int m = m0 + wm0 + 8 * (r >> 2) + 4 * half + (r & 3);
-    float v = a.alpha * acc[r] + bias_c;
-    if (a.Cin) v += a.beta * res_r[r];
-    v = apply_act(v, a.act, a.act_coef);
-    if (col_ok && m < a.M) a.Y[(int64_t)m * a.y_row_stride + col] = v;
+      for (int r = 0; r < 16; r++) {
+        if (mrow0 + row_k(r) >= a.M) continue;
+        float v = a.alpha * acc[r] + bias_c;
+        if (a.Cin) v += a.beta * res_r[r];
+        y0[(int64_t)row_k(r) * a.y_row_stride] = apply_act(v, a.act, a.act_coef);
+      }
+    }
   }
 }
 
@@ -189,7 +220,10 @@ bool launch_gemm_f32_rows(const dnnrtContext *ctx, const IgemmArgs &a, bool &lau
   // a problem that fills the chip with unsplit tiles several times over is better off with the big-tile kernel
   if (tiles >= 4 * (int64_t)ctx->num_cu) return true;
   const int nchunks = a.Kdim / BKC;
-  int64_t splits = tiles >= ctx->num_cu ? 1 : ceil_div(ctx->num_cu, tiles);
+  // about 1.75 workgroups per CU: two workgroups on a CU run out of step, so one's MFMAs overlap the
+  // other's LDS and memory phases (measured on the 128-row BERT products: 5-6 splits beat both 3 and 8)
+  const int64_t want = 7 * (int64_t)ctx->num_cu / 4;
+  int64_t splits = tiles >= want ? 1 : (want + tiles / 2) / tiles;
   splits = splits > 16 ? 16 : splits;
   splits = splits > nchunks ? nchunks : splits;
   while (splits > 1 && (tiles * 4 * splits * 4096 > SPLITK_PARTIAL_BYTES || tiles * 4 > SPLITK_MAX_TILES)) splits--;
