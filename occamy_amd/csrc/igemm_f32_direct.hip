@@ -20,7 +20,8 @@ namespace dnnrt {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int RSMODE, int LAYOUT, int KS>
+// VEC: k-contiguous operands (A unless transposed, B when transposed) are read as aligned float4.
+template <int RSMODE, int LAYOUT, int KS, bool VEC>
 __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmArgs a, const int k_per_wave) {
   constexpr bool B_KC = (LAYOUT & 1) != 0, A_MC = (LAYOUT & 2) != 0;
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
@@ -53,62 +54,120 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
 
   const int kbeg = wave * k_per_wave;
   const int kend = min(a.Kdim, kbeg + k_per_wave);
-  const float *__restrict__ arow = Ag + (int64_t)(m_ok ? m : 0) * a.Kdim;
+  const int mc = m_ok ? m : 0;
+  const float *__restrict__ arow = Ag + (int64_t)mc * a.Kdim;
   const float *__restrict__ brow = Xg + (int64_t)(col_ok ? col : 0) * a.Kdim;  // B_KC only
+
+  // Bias of the lane's 16 rows and of its column, requested before the
+  // reduction starts: the values are there when the epilogue wants them.
+  // Register r holds row m0 + 4 * half + row_k(r).
+  auto row_k = [](int r) { return 8 * (r >> 2) + (r & 3); };
+  const int mrow0 = m0 + 4 * half;
+  const int colc = col_ok ? col : 0;
+  const float bias_c = load_bias_col(a, colc);
+  float bias_r[16];
+  if (a.bias) {
+    const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] = biasg[min(mrow0 + row_k(r), a.M - 1)];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] = 0.f;
+  }
+
+  // One iteration = eight k: per lane four values of A and four of B.  Every
+  // load is unconditional, from an address clamped into the tensor; what must
+  // not contribute (k past the wavefront's slice, padding, columns past the
+  // end) is zeroed on the B side when it is used.  Rows past the end of A are
+  // read from row 0 and never stored.  With no load under a branch the
+  // compiler counts the outstanding loads exactly, and a ring of DEPTH
+  // iterations keeps several memory round trips in flight.
+  constexpr int DEPTH = 4;
+  struct It { float av[4], bv[4]; unsigned bm[4]; };
+  auto load_it = [&](int k0, It &t) {
+    const int ka = k0 + 4 * half;
+    // ---- A ----
+    if (!A_MC && VEC) {  // Kdim is a multiple of 4 then
+      const float4 v = *reinterpret_cast<const float4 *>(arow + min(ka, a.Kdim - 4));
+      t.av[0] = v.x; t.av[1] = v.y; t.av[2] = v.z; t.av[3] = v.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int kc = min(ka + j, a.Kdim - 1);
+        t.av[j] = A_MC ? Ag[(int64_t)kc * a.a_ld + mc] : arow[kc];
+      }
+    }
+    // ---- B ----
+    if (B_KC && VEC) {
+      const float4 v = *reinterpret_cast<const float4 *>(brow + min(ka, a.Kdim - 4));
+      t.bv[0] = v.x; t.bv[1] = v.y; t.bv[2] = v.z; t.bv[3] = v.w;
+#pragma unroll
+      for (int j = 0; j < 4; j++) t.bm[j] = (col_ok && ka + j < kend) ? 0xffffffffu : 0u;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int k = ka + j, kc = min(k, a.Kdim - 1);
+        bool ok = col_ok && k < kend;
+        if (B_KC) {
+          t.bv[j] = brow[kc];
+        } else if (RSMODE == 1) {
+          t.bv[j] = Xg[pix_off + (int64_t)kc * HW];
+        } else {
+          int c, r, s;
+          if (RSMODE == 3) { c = kc / 9; const int rs = kc - c * 9; r = rs / 3; s = rs - r * 3; }
+          else if (RSMODE == 7) { c = kc / 49; const int rs = kc - c * 49; r = rs / 7; s = rs - r * 7; }
+          else { const int RS = a.R * a.S; c = kc / RS; const int rs = kc - c * RS; r = rs / a.S; s = rs - r * a.S; }
+          const int ih = ih0 + r, iw = iw0 + s;
+          ok = ok && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+          const int64_t off = ok ? ((int64_t)c * a.H + ih) * a.W + iw : 0;
+          t.bv[j] = Xg[pix_off + off];
+        }
+        t.bm[j] = ok ? 0xffffffffu : 0u;
+      }
+    }
+  };
 
   floatx16 acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  auto mfma_it = [&](const It &t) {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(t.av[j], __uint_as_float(__float_as_uint(t.bv[j]) & t.bm[j]), acc, 0, 0, 0);
+  };
+  const int niter = kend > kbeg ? (kend - kbeg + 7) >> 3 : 0;
+  It t0, t1, t2, t3;  // named, not an array: they must stay in registers
+  load_it(kbeg, t0); load_it(kbeg + 8, t1); load_it(kbeg + 16, t2); load_it(kbeg + 24, t3);
+  // Iteration i lives in slot i % DEPTH and is refilled with iteration
+  // i + DEPTH: whole groups that need every refill run without a branch, the
+  // last DEPTH iterations refill nothing, the group in between asks per slot.
+  int i0 = 0;
+  for (; i0 + 2 * DEPTH <= niter; i0 += DEPTH) {
+    mfma_it(t0); load_it(kbeg + 8 * (i0 + DEPTH), t0);
+    mfma_it(t1); load_it(kbeg + 8 * (i0 + 1 + DEPTH), t1);
+    mfma_it(t2); load_it(kbeg + 8 * (i0 + 2 + DEPTH), t2);
+    mfma_it(t3); load_it(kbeg + 8 * (i0 + 3 + DEPTH), t3);
+  }
+  if (i0 < niter) { mfma_it(t0); if (i0 + DEPTH < niter) load_it(kbeg + 8 * (i0 + DEPTH), t0); }
+  if (i0 + 1 < niter) { mfma_it(t1); if (i0 + 1 + DEPTH < niter) load_it(kbeg + 8 * (i0 + 1 + DEPTH), t1); }
+  if (i0 + 2 < niter) { mfma_it(t2); if (i0 + 2 + DEPTH < niter) load_it(kbeg + 8 * (i0 + 2 + DEPTH), t2); }
+  if (i0 + 3 < niter) { mfma_it(t3); if (i0 + 3 + DEPTH < niter) load_it(kbeg + 8 * (i0 + 3 + DEPTH), t3); }
+  i0 += DEPTH;
+  if (i0 < niter) mfma_it(t0);
+  if (i0 + 1 < niter) mfma_it(t1);
+  if (i0 + 2 < niter) mfma_it(t2);
 
-
-  for (int k0 = kbeg; k0 < kend; k0 += 8) {
-    const int ka = k0 + 4 * half;
-    float av[4], bv[4];
-    // ---- A ----
-    if (!A_MC) {
-      if (a.a_vec4) {
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (m_ok && ka < kend) v = *reinterpret_cast<const float4 *>(arow + ka);
-        av[0] = v.x; av[1] = v.y; av[2] = v.z; av[3] = v.w;
-      } else {
+  // the residual tensor's 16 values, requested before the partial tiles meet
+  const int img = colc / PQ, pq = colc - img * PQ;
+  const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
+  float res_r[16];
+  if (a.Cin && wave == 0) {
+    const float *__restrict__ Cg = a.Cin + (int64_t)z * a.c_z_stride;
 #pragma unroll
-        for (int j = 0; j < 4; j++) av[j] = (m_ok && ka + j < kend) ? arow[ka + j] : 0.f;
-      }
-    } else {
+    for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(mrow0 + row_k(r), a.M - 1) * a.c_row_stride];
+  } else {
 #pragma unroll
-      for (int j = 0; j < 4; j++) av[j] = (m_ok && ka + j < kend) ? Ag[(int64_t)(ka + j) * a.a_ld + m] : 0.f;
-    }
-    // ---- B ----
-    if (B_KC) {
-      if (a.b_vec4) {
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (col_ok && ka < kend) v = *reinterpret_cast<const float4 *>(brow + ka);
-        bv[0] = v.x; bv[1] = v.y; bv[2] = v.z; bv[3] = v.w;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; j++) bv[j] = (col_ok && ka + j < kend) ? brow[ka + j] : 0.f;
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int k = ka + j;
-        float v = 0.f;
-        if (RSMODE == 1) {
-          if (col_ok && k < kend) v = Xg[pix_off + (int64_t)k * HW];
-        } else {
-          int c, r, s;
-          if (RSMODE == 3) { c = k / 9; const int rs = k - c * 9; r = rs / 3; s = rs - r * 3; }
-          else if (RSMODE == 7) { c = k / 49; const int rs = k - c * 49; r = rs / 7; s = rs - r * 7; }
-          else { const int RS = a.R * a.S; c = k / RS; const int rs = k - c * RS; r = rs / a.S; s = rs - r * a.S; }
-          const int ih = ih0 + r, iw = iw0 + s;
-          if (col_ok && k < kend && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W)
-            v = Xg[pix_off + ((int64_t)c * a.H + ih) * a.W + iw];
-        }
-        bv[j] = v;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[j], acc, 0, 0, 0);
+    for (int r = 0; r < 16; r++) res_r[r] = 0.f;
   }
 
   // ---- combine the KS partial tiles ----
@@ -125,39 +184,16 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
       for (int r = 0; r < 16; r++) acc[r] += red[w][r][lane];
   }
 
-  // ---- epilogue: register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32] ----
-  // Bias and residual values are read in one batch from clamped addresses and
-  // only the stores are predicated: a load inside a per-row branch would cost
-  // a memory round trip per row.
-  float *__restrict__ Yg = a.Y + (int64_t)z * a.y_z_stride;
-  const int colc = col_ok ? col : 0;
-  const int img = colc / PQ, pq = colc - img * PQ;
-  const int64_t ycol = (int64_t)img * a.y_img_stride + pq;
-  float bias_r[16], res_r[16];
-  const float bias_c = load_bias_col(a, colc);
-  if (a.bias) {
-    const float *__restrict__ biasg = a.bias + (int64_t)z * a.bias_z_stride;
-#pragma unroll
-    for (int r = 0; r < 16; r++) bias_r[r] = biasg[min(m0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1)];
-  } else {
-#pragma unroll
-    for (int r = 0; r < 16; r++) bias_r[r] = 0.f;
-  }
-  if (a.Cin) {
-    const float *__restrict__ Cg = a.Cin + (int64_t)z * a.c_z_stride;
-#pragma unroll
-    for (int r = 0; r < 16; r++) res_r[r] = Cg[ycol + (int64_t)min(m0 + 8 * (r >> 2) + 4 * half + (r & 3), a.M - 1) * a.c_row_stride];
-  } else {
-#pragma unroll
-    for (int r = 0; r < 16; r++) res_r[r] = 0.f;
-  }
+  // ---- epilogue: register r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l%32];
+  // a row's address is one per-lane base plus a uniform offset ----
+  if (!col_ok) return;
+  float *__restrict__ y0 = a.Y + (int64_t)z * a.y_z_stride + ycol + (int64_t)mrow0 * a.y_row_stride;
 #pragma unroll
   for (int r = 0; r < 16; r++) {
-    const int mm = m0 + 8 * (r >> 2) + 4 * half + (r & 3);
+    if (mrow0 + row_k(r) >= a.M) continue;
     float v = a.alpha * acc[r] + bias_r[r] + bias_c;
     if (a.Cin) v += a.beta * res_r[r];
-    v = apply_act(v, a.act, a.act_coef);
-    if (col_ok && mm < a.M) Yg[ycol + (int64_t)mm * a.y_row_stride] = v;
+    y0[(int64_t)row_k(r) * a.y_row_stride] = apply_act(v, a.act, a.act_coef);
   }
 }
 
@@ -165,8 +201,13 @@ template <int KS>
 static void launch_ks(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout, int tiles) {
   const int k_per_wave = (int)(ceil_div(ceil_div(a.Kdim, KS), 8) * 8);
   dim3 grid(tiles, 1, a.Z), block(64 * KS);
+  // float4 reads only if every k-contiguous operand allows them
+  const bool vec = (((layout & 2) != 0) || a.a_vec4) && (((layout & 1) == 0) || a.b_vec4) && (layout != 2);
 #define LAUNCH(RS, LAY)                                                                         \
-  hipLaunchKernelGGL((igemm_f32_direct_kernel<RS, LAY, KS>), grid, block, 0, ctx->stream, a, k_per_wave)
+  do {                                                                                          \
+    if (vec) hipLaunchKernelGGL((igemm_f32_direct_kernel<RS, LAY, KS, true>), grid, block, 0, ctx->stream, a, k_per_wave);  \
+    else hipLaunchKernelGGL((igemm_f32_direct_kernel<RS, LAY, KS, false>), grid, block, 0, ctx->stream, a, k_per_wave);     \
+  } while (0)
   if (layout == 0) {
     switch (rsmode) {
       case 1: LAUNCH(1, 0); break;
