@@ -27,6 +27,11 @@
  *     dnnrtSetFilterLayout, dnnrtLayerNorm,
  *     dnnrtGelu, dnnrtHostAlloc/Free, dnnrtLastError.
  *
+ * A tensor with no elements (a zero batch, a zero row count) is accepted by
+ * every operator: nothing is launched, the output buffer is left as it is and
+ * the call returns it, as the reference's zero-block launches do nothing.
+ * Negative dims and empty reduction ranges (K = 0) are refused.
+ *
  * The library is not re-entrant per handle; calls on one handle must come
  * from one host thread at a time (the reference keeps its handles in
  * file-scope globals, src/Conversion/DNNToLLVM/Ops/cudnn/ConvForward.cpp:15).

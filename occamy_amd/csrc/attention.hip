@@ -166,7 +166,9 @@ extern "C" void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void 
   if (!handle) DNNRT_FAIL("dnnrtAttention: null handle");
   if (!Q || !K || !V || !Y) DNNRT_FAIL("dnnrtAttention: null argument");
   if (dtype != DNNRT_F32) DNNRT_FAIL("dnnrtAttention: dtype %d (fp32 only)", dtype);
-  if (batch <= 0 || seqQ <= 0 || seqK <= 0 || heads <= 0) DNNRT_FAIL("dnnrtAttention: bad dims");
+  if (batch < 0 || seqQ < 0) DNNRT_FAIL("dnnrtAttention: bad dims");
+  if (batch == 0 || seqQ == 0) return Y;  // no queries: no work
+  if (seqK <= 0 || heads <= 0) DNNRT_FAIL("dnnrtAttention: bad dims");
   if (batch > 65535 || heads > 65535 || seqQ > (1 << 24) || seqK > (1 << 24)) DNNRT_FAIL("dnnrtAttention: dims too large");
   if (headDim != 32 && headDim != 64 && headDim != 128) DNNRT_FAIL("dnnrtAttention: head dim %ld (32, 64, 128)", (long)headDim);
   if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(Y)) DNNRT_FAIL("dnnrtAttention: operands must be 16-byte aligned");

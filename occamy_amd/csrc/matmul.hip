@@ -127,6 +127,7 @@ void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A, const int
   if (!A || !B || !Out || !dimA || !dimB || !dimOut) DNNRT_FAIL("dnnrtMatmul2d: null argument");
   const int64_t M = transA ? dimA[1] : dimA[0], K = transA ? dimA[0] : dimA[1];
   const int64_t Kb = transB ? dimB[1] : dimB[0], N = transB ? dimB[0] : dimB[1];
+  if (K == Kb && dimOut[0] == M && dimOut[1] == N && M >= 0 && N >= 0 && K > 0 && (M == 0 || N == 0)) return Out;  // empty product: no work
   if (K != Kb || dimOut[0] != M || dimOut[1] != N || M <= 0 || N <= 0 || K <= 0)
     DNNRT_FAIL("dnnrtMatmul2d: shapes [%ld,%ld] x [%ld,%ld] -> [%ld,%ld] do not agree", (long)M,
                (long)K, (long)Kb, (long)N, (long)dimOut[0], (long)dimOut[1]);
@@ -161,6 +162,13 @@ static void *matmul_nd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
   if (rankA < 2 || rankB < 2 || rankA > 4 || rankB > 4 || rankY != (rankA > rankB ? rankA : rankB))
     DNNRT_FAIL("dnnrtMatmulNd: ranks %d x %d -> %d (2..4 supported)", rankA, rankB, rankY);
   const int64_t M = dimA[rankA - 2], K = dimA[rankA - 1], N = dimB[rankB - 1];
+  {
+    bool neg = false;
+    for (int i = 0; i < rankA; i++) neg = neg || dimA[i] < 0;
+    for (int i = 0; i < rankB; i++) neg = neg || dimB[i] < 0;
+    for (int i = 0; i < rankY; i++) neg = neg || dimY[i] < 0;
+    if (!neg && K > 0 && dimB[rankB - 2] == K && numel(dimY, rankY) == 0) return Y;  // empty product (a zero batch or row count): no work
+  }
   if (dimB[rankB - 2] != K || dimY[rankY - 2] != M || dimY[rankY - 1] != N || M <= 0 || N <= 0 || K <= 0)
     DNNRT_FAIL("dnnrtMatmulNd: inner/outer dims do not agree");
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) DNNRT_FAIL("dnnrtMatmulNd: dims exceed 32 bits");

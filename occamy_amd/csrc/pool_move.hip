@@ -102,9 +102,11 @@ static void *pool_entry(const char *who, dnnrtHandle_t h, const void *X, const i
                         bool is_max, int32_t dtype) {
   if (!h) DNNRT_FAIL("%s: null handle", who);
   if (!X || !Y || !dX || !dY || !kr || !pads || !st) DNNRT_FAIL("%s: null argument", who);
+  if (dY[0] != dX[0] || dY[1] != dX[1]) DNNRT_FAIL("%s: N and C of X and Y differ", who);
+  // an empty batch is no work: nothing is launched and Y is left as it is (the reference's zero-block launches do nothing either)
+  if (dX[0] == 0 || dX[1] == 0) return Y;
   for (int i = 0; i < 4; i++)
     if (dX[i] <= 0 || dY[i] <= 0 || dX[i] > INT32_MAX) DNNRT_FAIL("%s: bad dims", who);
-  if (dY[0] != dX[0] || dY[1] != dX[1]) DNNRT_FAIL("%s: N and C of X and Y differ", who);
   if (kr[0] < 1 || kr[1] < 1 || st[0] < 1 || st[1] < 1 || pads[0] < 0 || pads[1] < 0)
     DNNRT_FAIL("%s: bad kernel/strides/pads", who);
   PoolGeom g;
@@ -491,12 +493,13 @@ void *dnnrtTranspose(dnnrtHandle_t handle, const void *X, const int64_t *dimX, v
   for (int i = 0; i < rank; i++) {
     if (perm[i] < 0 || perm[i] >= rank || seen[perm[i]]) DNNRT_FAIL("dnnrtTranspose: perm is not a permutation");
     seen[perm[i]] = true;
-    if (dimY[i] != dimX[perm[i]] || dimY[i] <= 0) DNNRT_FAIL("dnnrtTranspose: dimY[%d] != dimX[perm[%d]]", i, i);
+    if (dimY[i] != dimX[perm[i]] || dimY[i] < 0) DNNRT_FAIL("dnnrtTranspose: dimY[%d] != dimX[perm[%d]]", i, i);
     g.dy[i] = dimY[i];
     g.sx[i] = sx[perm[i]];
   }
   const int64_t es = esize(dtype);
   if (!es) DNNRT_FAIL("dnnrtTranspose: dtype %d", dtype);
+  if (s == 0) return Y;  // an empty tensor: nothing to move
   if (s > 0 && s < (1ll << 31)) {
     // size-1 dims dropped, runs of dims that stay together merged
     int64_t my[6], ms[6];

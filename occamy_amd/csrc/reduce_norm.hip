@@ -223,6 +223,10 @@ void *dnnrtReduce(dnnrtHandle_t handle, int32_t rank, const void *X, const int64
   if (rank < 1 || rank > 8) DNNRT_FAIL("dnnrtReduce: rank %d", rank);
   int64_t dx[8], dy[8];
   for (int i = 0; i < rank; i++) { dx[i] = dimX[i]; dy[i] = dimY[i]; }
+  for (int i = 0; i < rank; i++)
+    if (dimX[i] < 0 || dimY[i] < 0) DNNRT_FAIL("dnnrtReduce: negative dim");
+  // an empty batch is no work: nothing is launched and Y is left as it is (the reference's zero-block launches do nothing either)
+  if (numel(dimX, rank) == 0 || numel(dimY, rank) == 0) return Y;
   if (handle->format != DNNRT_NCHW && rank == 4) {  // channels-last: dense [N,H,W,C]
     dx[1] = dimX[2]; dx[2] = dimX[3]; dx[3] = dimX[1];
     dy[1] = dimY[2]; dy[2] = dimY[3]; dy[3] = dimY[1];
@@ -263,7 +267,10 @@ void *dnnrtSoftmax(dnnrtHandle_t handle, const void *X, const int64_t *dimX, voi
   const int64_t L = dimX[axis];
   for (int64_t i = 0; i < axis; i++) outer *= dimX[i];
   for (int64_t i = axis + 1; i < rank; i++) inner *= dimX[i];
-  if (L <= 0 || L > INT32_MAX || outer <= 0 || inner <= 0) DNNRT_FAIL("dnnrtSoftmax: bad dims");
+  if (L < 0 || outer < 0 || inner < 0) DNNRT_FAIL("dnnrtSoftmax: negative dim");
+  // an empty batch is no work: nothing is launched and Y is left as it is (the reference's zero-block launches do nothing either)
+  if (L == 0 || outer == 0 || inner == 0) return Y;
+  if (L > INT32_MAX) DNNRT_FAIL("dnnrtSoftmax: bad dims");
 #define SOFTMAX_LAUNCH(T)                                                                           \
   do {                                                                                              \
     if (inner == 1) {                                                                               \
@@ -292,7 +299,10 @@ void *dnnrtLayerNorm(dnnrtHandle_t handle, const void *X, const int64_t *dimX, i
   if (!X || !Y || !dimX || !gamma || !beta) DNNRT_FAIL("dnnrtLayerNorm: null argument");
   if (rank < 1 || rank > 8) DNNRT_FAIL("dnnrtLayerNorm: rank %ld", (long)rank);
   const int64_t L = dimX[rank - 1], rows = numel(dimX, rank - 1);
-  if (L <= 0 || L > INT32_MAX || rows <= 0) DNNRT_FAIL("dnnrtLayerNorm: bad dims");
+  if (L < 0 || rows < 0) DNNRT_FAIL("dnnrtLayerNorm: negative dim");
+  // an empty batch is no work: nothing is launched and Y is left as it is (the reference's zero-block launches do nothing either)
+  if (L == 0 || rows == 0) return Y;
+  if (L > INT32_MAX) DNNRT_FAIL("dnnrtLayerNorm: bad dims");
   const int64_t blocks = ceil_div(rows, 4);
   if (blocks > INT32_MAX) DNNRT_FAIL("dnnrtLayerNorm: too many rows");
   if (dtype == DNNRT_F32 && layernorm_in_registers<float>(handle, X, gamma, beta, Y, rows, L, eps)) {

@@ -524,6 +524,7 @@ void *dnnrtReduce(dnnrtHandle_t h, int32_t rank, const void *X, const int64_t *d
   for (int i = 0; i < rank; i++)
     if (dY[i] != dX[i] && dY[i] != 1) FAIL("reduce: dimY[%d]", i);
   const int64_t nx = numel(dX, rank), ny = numel(dY, rank);
+  if (nx == 0 || ny == 0) return Y;  /* nothing to average, nothing to write */
   float *tx, *ty;
   const float *x = widen(X, nx, dtype, &tx);
   float *y = outbuf(Y, ny, dtype, &ty);
@@ -772,7 +773,9 @@ void *dnnrtAttention(dnnrtHandle_t h, const void *Q, const void *K, const void *
                      int32_t dtype) {
   (void)h;
   if (dtype != DNNRT_F32) FAIL("attention: fp32 only");
-  if (B <= 0 || Sq <= 0 || Sk <= 0 || H <= 0 || D <= 0) FAIL("attention: bad dims");
+  if (B < 0 || Sq < 0) FAIL("attention: bad dims");
+  if (B == 0 || Sq == 0) return Y;  /* no queries */
+  if (Sk <= 0 || H <= 0 || D <= 0) FAIL("attention: bad dims");
   const float *q = (const float *)Q, *k = (const float *)K, *v = (const float *)V;
   float *y = (float *)Y;
   const int64_t ldy = H * D, ld = ldIn ? ldIn : ldy;

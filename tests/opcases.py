@@ -275,3 +275,65 @@ def attention_packed(be, qkv, heads, scale):
                      DT[qkv.dtype], ld_in=three)
     be.sync()
     return be.get(Y)
+
+
+def empty_tensor_behaviour(be):
+    """Every entry point with a tensor that has a zero dim.  Buffers are real
+    (64 sentinel floats) so that only the dims say "empty".  Returns
+    {entry point: "refused" | "untouched" | "wrote"}: a clean error, or a
+    successful call that left the output alone."""
+    f32 = np.float32
+    o = be.ops
+    out = {}
+
+    def probe(name, call, outputs):
+        try:
+            call()
+            be.sync()
+        except RuntimeError:
+            out[name] = "refused"
+            return
+        out[name] = "untouched" if all(np.array_equal(be.get(y), np.full(64, 7.0, f32)) for y in outputs) else "wrote"
+
+    def buf():
+        return be.put(np.full(64, 7.0, f32))
+
+    def idx():
+        return be.put(np.zeros(8, np.int64))
+
+    X, W, B, Z, Y = buf(), buf(), buf(), buf(), buf()
+    p = be.ptr
+    probe("conv", lambda: o.conv(p(X), (0, 4, 3, 3), p(W), (2, 4, 1, 1), (0, 0), (1, 1), p(Y)), [Y])
+    probe("conv_bias_activ", lambda: o.conv_bias_activ(p(X), (0, 4, 3, 3), p(W), (2, 4, 1, 1), p(B), (0, 0), (1, 1), _abi.ACT_RELU, p(Y)), [Y])
+    probe("conv_bias_add_activ", lambda: o.conv_bias_add_activ(p(X), (0, 4, 3, 3), p(W), (2, 4, 1, 1), p(B), p(Z), (0, 0), (1, 1), _abi.ACT_RELU, p(Y)), [Y])
+    probe("active", lambda: o.active(p(X), (0, 4), _abi.ACT_RELU, p(Y)), [Y])
+    probe("tensor_op", lambda: o.tensor_op(_abi.OP_ADD, p(X), (0, 4), p(B), (1, 4), p(Y)), [Y])
+    probe("clip", lambda: o.clip(p(X), p(Y), (0, 4), 0.0, 1.0), [Y])
+    probe("leaky_relu", lambda: o.leaky_relu(p(X), p(Y), (0, 4), 0.1), [Y])
+    probe("prelu", lambda: o.prelu(p(X), p(Y), (0, 4), p(B), (1, 4)), [Y])
+    probe("erf", lambda: o.erf(p(X), p(Y), (0, 4)), [Y])
+    probe("gelu", lambda: o.gelu(p(X), p(Y), (0, 4)), [Y])
+    probe("pow", lambda: o.pow(p(X), p(B), p(Y), (0, 4)), [Y])
+    probe("cast", lambda: o.cast_i64_to_float(p(idx()), p(Y), (0, 4)), [Y])
+    probe("reduce_mean", lambda: o.reduce_mean(p(X), (0, 4), p(Y), (0, 1)), [Y])
+    probe("softmax", lambda: o.softmax(p(X), (0, 4), p(Y), 1), [Y])
+    probe("layernorm", lambda: o.layernorm(p(X), (0, 4), p(W), p(B), 1e-5, p(Y)), [Y])
+    probe("maxpool", lambda: o.maxpool(p(X), (0, 2, 4, 4), p(Y), (0, 2, 2, 2), (2, 2), (0, 0, 0, 0), (2, 2)), [Y])
+    probe("avgpool", lambda: o.avgpool(p(X), (0, 2, 4, 4), p(Y), (0, 2, 2, 2), (2, 2), (0, 0, 0, 0), (2, 2)), [Y])
+    probe("matmul2d", lambda: o.matmul2d(p(X), (0, 4), p(W), (4, 3), p(Y), (0, 3)), [Y])
+    probe("matmul_nd", lambda: o.matmul_nd(p(X), (0, 2, 4), p(W), (4, 3), p(Y), (0, 2, 3)), [Y])
+    probe("matmul_nd_bias", lambda: o.matmul_nd_bias(p(X), (0, 2, 4), p(W), (4, 3), p(B), p(Y), (0, 2, 3)), [Y])
+    probe("attention", lambda: o.attention(p(X), p(W), p(Z), p(Y), 0, 4, 4, 1, 32, 1.0), [Y])
+    probe("flatten", lambda: o.flatten(p(X), (0, 2, 2), p(Y), (0, 4), 1), [Y])
+    probe("reshape", lambda: o.reshape(p(X), (0, 4), p(Y)), [Y])
+    probe("squeeze", lambda: o.squeeze(p(X), (0, 1, 4), p(Y), (0, 4)), [Y])
+    probe("unsqueeze", lambda: o.unsqueeze(p(X), (0, 4), p(Y), (0, 1, 4)), [Y])
+    probe("expand", lambda: o.expand(p(X), (0, 1), p(Y), (0, 4), _abi.F32), [Y])
+    probe("nonzero", lambda: o.nonzero(p(X), (0, 4), p(Y), (0,), _abi.F32), [Y])
+    probe("concat", lambda: o.concat([p(X), p(W)], [(0, 2), (0, 3)], p(Y), (0, 5), 1), [Y])
+    probe("transpose", lambda: o.transpose(p(X), (0, 4), p(Y), (1, 0)), [Y])
+    probe("gather", lambda: o.gather(p(X), (4, 0), p(Y), (2, 0), p(idx()), (2,), 0), [Y])
+    # the handle is still good: a real call after all of the above
+    a = np.arange(6, dtype=f32).reshape(2, 3)
+    assert np.array_equal(tensor_op(be, _abi.OP_ADD, a, a), a + a)
+    return out

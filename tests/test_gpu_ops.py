@@ -478,6 +478,14 @@ def test_expand_and_nonzero(gpu, cpu):
     np.testing.assert_array_equal(oc.nonzero(gpu, z, (5,), -1.0), np.array([2, 3, -1, -1, -1], np.float32))
 
 
+def test_empty_tensors_are_no_ops(gpu, cpu):
+    # an empty batch (or an empty tensor of any kind) launches nothing, writes nothing, raises nothing,
+    # and leaves no error behind; the oracle agrees entry point by entry point
+    got = oc.empty_tensor_behaviour(gpu)
+    assert got == oc.empty_tensor_behaviour(cpu)
+    assert set(got.values()) == {"untouched"}, got
+
+
 # ---- fp16, channels-last -----------------------------------------------------------------
 
 def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt, z=None):

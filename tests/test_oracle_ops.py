@@ -509,6 +509,12 @@ def test_nonzero_lists_flat_indices_in_order(be):
     np.testing.assert_array_equal(oc.nonzero(be, np.zeros((4, 4), np.float32), (16,), 5.0), np.full(16, 5.0, np.float32))
 
 
+def test_empty_tensors_are_no_ops(be):
+    # The reference's wrappers launch zero blocks for an empty tensor and return: no work, no error.
+    got = oc.empty_tensor_behaviour(be)
+    assert len(got) >= 30 and set(got.values()) == {"untouched"}, got
+
+
 def test_layouts_the_oracle_lacks_are_refused(be):
     # The oracle restates the reference, which knows N,C,H,W tensors and
     # K,C,R,S filters only; asking it for anything else must fail, not drift.
