@@ -56,6 +56,8 @@ bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a);
 // The variant for problems too small to fill the chip with LDS-staged tiles
 // (igemm_f32_direct.hip); rsmode / layout as computed by launch_igemm_f32.
 bool launch_igemm_f32_direct(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout);
+// 3x3 convolutions large enough for LDS-staged tiles (igemm_f32_3x3.hip); `launched` says whether it applied.
+bool launch_conv3x3_f32_tiled(const dnnrtContext *ctx, const IgemmArgs &a, int layout, bool &launched);
 // Row-major products with a few hundred rows (gemm_f32_rows.hip); `launched` says whether it applied.
 bool launch_gemm_f32_rows(const dnnrtContext *ctx, const IgemmArgs &a, bool &launched);
 // 3x3 / 1x1 specialisations of the above (igemm_f32_small.hip); `launched` says whether one applied.

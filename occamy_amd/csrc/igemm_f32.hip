@@ -296,6 +296,11 @@ bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a) {
   const int layout = (a.b_kcontig ? 1 : 0) | (a.a_mcontig ? 2 : 0);
   if ((layout & 1) && rsmode != 1) { set_error("igemm_f32: a k-contiguous right operand needs a 1x1 geometry"); return false; }
 
+  if (rsmode == 3) {  // the 3x3 specialisation takes the problems the tiles below would get
+    bool launched = false;
+    if (!launch_conv3x3_f32_tiled(ctx, a, layout, launched)) return false;
+    if (launched) return true;
+  }
   // Largest tile that still gives every CU a workgroup; small problems fall
   // through to the one-wave 32x32 tile.
   const int64_t want = ctx->num_cu;

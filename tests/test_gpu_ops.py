@@ -54,6 +54,11 @@ CONV_CASES = [
     (1, 64, 96, 80, 3, 3, 3, 1, 1, 1),      # image-producing last layer: three output channels
     (2, 16, 21, 17, 4, 3, 3, 2, 1, 1),      # four output channels, stride 2
     (2, 24, 9, 9, 2, 1, 1, 1, 0, 1),        # two output channels, 1x1
+    # 3x3 layers that fill the chip (the LDS-tiled 3x3 kernel): 128x128 tiles with an odd channel count and
+    # ragged rows; 64x64 tiles, stride 2, no padding; groups
+    (1, 5, 190, 180, 130, 3, 3, 1, 1, 1),
+    (2, 8, 260, 130, 64, 3, 3, 2, 0, 1),
+    (1, 8, 182, 182, 256, 3, 3, 1, 1, 2),
 ]
 
 
