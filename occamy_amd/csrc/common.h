@@ -60,6 +60,20 @@ constexpr int ACT_GELU = 7;
 
 // The activations a convolution epilogue can apply (sigmoid and tanh are
 // separate calls, as in the reference).
+// x / d for 0 <= x < 2^31 with magic = magic_of(d) from the host: one
+// multiply-high and a correction instead of ~40 instructions of integer division.
+__device__ __forceinline__ int div_magic(int x, int d, unsigned magic) {
+  int q = (int)__umulhi((unsigned)x, magic);
+  int r = x - q * d;
+  if (r < 0) { q--; r += d; }
+  if (r >= d) q++;
+  return q;
+}
+inline unsigned magic_of(int d) {  // ceil(2^32 / d), saturated (d == 1)
+  const uint64_t m = (((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d;
+  return (unsigned)(m > 0xffffffffull ? 0xffffffffull : m);
+}
+
 __device__ __forceinline__ float apply_act(float v, int act, float coef) {
   if (act == DNNRT_ACT_RELU) return v < 0.f ? 0.f : v;
   if (act == DNNRT_ACT_CLIPPED_RELU) { v = v < 0.f ? 0.f : v; return v > coef ? coef : v; }

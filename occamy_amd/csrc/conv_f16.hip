@@ -63,16 +63,6 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // own: the kernel renumbers them so that one XCD works on a contiguous run of
 // tiles (k_out tiles of one pixel tile first), which then share their
 // operands in that L2.
-// x / d for 0 <= x < 2^31 with magic = ceil(2^32 / d) from the host: one
-// multiply-high and a correction instead of ~40 instructions of integer division.
-__device__ __forceinline__ int div_magic(int x, int d, unsigned magic) {
-  int q = (int)__umulhi((unsigned)x, magic);
-  int r = x - q * d;
-  if (r < 0) { q--; r += d; }
-  if (r >= d) q++;
-  return q;
-}
-
 //
 // KG = 2 doubles the workgroup to eight wavefronts: wavefronts 4-7 own the
 // same output blocks as 0-3 and take the second half of every 64-k step (the
@@ -498,8 +488,6 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
                     (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0;
   if (fast) {
     ConvF16Args am = a;
-    auto magic_of = [](int d) { return (unsigned)((((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d > 0xffffffffull
-                                                   ? 0xffffffffull : (((uint64_t)1 << 32) + (uint64_t)d - 1) / (uint64_t)d); };
     am.magic_pq = magic_of(a.P * a.Q);
     am.magic_q = magic_of(a.Q);
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };

@@ -33,6 +33,7 @@ struct IgemmArgs {
   // blockIdx.z: group of a grouped convolution or batch of a batched matmul
   int Z;
   int64_t a_z_stride, x_z_stride, y_z_stride, bias_z_stride;
+  unsigned magic_rs, magic_s;  // filled in by launch_igemm_f32: magic_of(R * S), magic_of(S), for the generic filter sizes
   bool b_kcontig;     // B stored [Ncols][Kdim] (k contiguous): GEMM with transB
   bool a_mcontig;     // A stored [Kdim][M]: GEMM with transA
   bool a_vec4;        // A rows may be read as aligned float4

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(64 * WM * WN) void igemm_f32_kernel(const IgemmArgs
           int c, r, s;
           if (RSMODE == 3) { c = k / 9; const int rs = k - c * 9; r = rs / 3; s = rs - r * 3; }
           else if (RSMODE == 7) { c = k / 49; const int rs = k - c * 49; r = rs / 7; s = rs - r * 7; }
-          else { const int RS = a.R * a.S; c = k / RS; const int rs = k - c * RS; r = rs / a.S; s = rs - r * a.S; }
+          else { const int RS = a.R * a.S; c = div_magic(k, RS, a.magic_rs); const int rs = k - c * RS; r = div_magic(rs, a.S, a.magic_s); s = rs - r * a.S; }
           const int ih = ih0 + r, iw = iw0 + s;
           if (b_col_ok && k < a.Kdim && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W)
             v = Xg[b_pix_off + ((int64_t)c * a.H + ih) * a.W + iw];
@@ -286,7 +286,10 @@ static bool launch_tile(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode,
   return true;
 }
 
-bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &a) {
+bool launch_igemm_f32(const dnnrtContext *ctx, const IgemmArgs &args) {
+  IgemmArgs a = args;
+  a.magic_rs = magic_of(a.R * a.S > 0 ? a.R * a.S : 1);
+  a.magic_s = magic_of(a.S > 0 ? a.S : 1);
   if (a.M <= 0 || a.Ncols <= 0 || a.Kdim <= 0 || a.Z <= 0) { set_error("igemm_f32: empty problem"); return false; }
   if (a.Z > 65535) { set_error("igemm_f32: more than 65535 groups/batches"); return false; }
   int rsmode = 0;

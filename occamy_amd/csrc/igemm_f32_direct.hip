@@ -116,7 +116,7 @@ __global__ __launch_bounds__(64 * KS) void igemm_f32_direct_kernel(const IgemmAr
           int c, r, s;
           if (RSMODE == 3) { c = kc / 9; const int rs = kc - c * 9; r = rs / 3; s = rs - r * 3; }
           else if (RSMODE == 7) { c = kc / 49; const int rs = kc - c * 49; r = rs / 7; s = rs - r * 7; }
-          else { const int RS = a.R * a.S; c = kc / RS; const int rs = kc - c * RS; r = rs / a.S; s = rs - r * a.S; }
+          else { const int RS = a.R * a.S; c = div_magic(kc, RS, a.magic_rs); const int rs = kc - c * RS; r = div_magic(rs, a.S, a.magic_s); s = rs - r * a.S; }
           const int ih = ih0 + r, iw = iw0 + s;
           ok = ok && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
           const int64_t off = ok ? ((int64_t)c * a.H + ih) * a.W + iw : 0;
