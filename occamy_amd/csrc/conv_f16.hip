@@ -247,31 +247,35 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[i], qb[j], acc[i][j], 0, 0, 0);
   };
 
-  // prologue: steps 0 .. DEPTH-1 in flight, step 0 into LDS stage 0
-#pragma unroll
-  for (int d = 0; d < DEPTH; d++) load_step(ra[d], rb[d], rm[d]);
+  // prologue: steps 0 and 1 in flight, step 0 into LDS stage 0
+  static_assert(DEPTH == 2, "the step sequence below is written for two register slots");
+  load_step(ra[0], rb[0], rm[0]);
+  if (nk > 1) load_step(ra[1], rb[1], rm[1]);
   store_step(0, ra[0], rb[0], rm[0]);
   __syncthreads();
 
-  // Step kt (register slot U = kt % DEPTH, LDS stage U & 1): refill slot U with
-  // step kt + DEPTH; four k16 sub-steps, the operands of each read from LDS
-  // while the MFMAs of the one before run; half way, step kt + 1 goes from its
-  // slot into the other LDS stage (nobody reads that stage during this step);
-  // one barrier.  The body has no branch, so the scheduler is free to spread
-  // the loads, LDS traffic and address arithmetic between the MFMAs.  Loads
-  // and LDS stores for steps past the end are harmless (the cursor stops, the
-  // LDS rows written are never read).  (A ring of 4 register stages was
-  // measured and bought nothing over 2 on any ResNet-50 layer; only 2 is built.)
-  auto step = [&](auto slot_c) {
+  // Step kt (register slot U = kt % 2, LDS stage U): refill slot U with step
+  // kt + 2 if there is one; four k16 sub-steps, the operands of each read from
+  // LDS while the MFMAs of the one before run; half way, step kt + 1 (if there
+  // is one) goes from its slot into the other LDS stage (nobody reads that
+  // stage during this step); one barrier.  The body has no branch, so the
+  // scheduler is free to spread the loads, LDS traffic and address arithmetic
+  // between the MFMAs.  Whether a step refills and whether it has a successor
+  // are compile-time properties of its place in the sequence: nothing is
+  // loaded or staged for steps past the end (a 1x1 layer over 64 channels is a
+  // single step: it used to issue three steps' worth of loads).  (A ring of 4
+  // register stages was measured and bought nothing over 2 on any ResNet-50 layer.)
+  auto step = [&](auto slot_c, auto refill_c, auto next_c) {
     constexpr int U = decltype(slot_c)::value, S = U & 1, N = (U + 1) % DEPTH;
-    load_step(ra[U], rb[U], rm[U]);
+    constexpr bool REFILL = decltype(refill_c)::value, HAS_NEXT = decltype(next_c)::value;
+    if constexpr (REFILL) load_step(ra[U], rb[U], rm[U]);
     if constexpr (KG == 1) {
       read_frags(S, fa[0], fb[0], 0);
       read_frags(S, fa[1], fb[1], 1);
       mfma_frags(fa[0], fb[0]);
       read_frags(S, fa[0], fb[0], 2);
       mfma_frags(fa[1], fb[1]);
-      store_step(S ^ 1, ra[N], rb[N], rm[N]);
+      if constexpr (HAS_NEXT) store_step(S ^ 1, ra[N], rb[N], rm[N]);
       read_frags(S, fa[1], fb[1], 3);
       mfma_frags(fa[0], fb[0]);
       mfma_frags(fa[1], fb[1]);
@@ -279,26 +283,31 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
       read_frags(S, fa[0], fb[0], 2 * kg);
       read_frags(S, fa[1], fb[1], 2 * kg + 1);
       mfma_frags(fa[0], fb[0]);
-      store_step(S ^ 1, ra[N], rb[N], rm[N]);
+      if constexpr (HAS_NEXT) store_step(S ^ 1, ra[N], rb[N], rm[N]);
       mfma_frags(fa[1], fb[1]);
     }
     __syncthreads();
   };
   using std::integral_constant;
+  using std::true_type;
+  using std::false_type;
+  const integral_constant<int, 0> slot0{};
+  const integral_constant<int, 1> slot1{};
   int kt = 0;
-  for (; kt + DEPTH <= nk; kt += DEPTH) {
-    step(integral_constant<int, 0>{});
-    step(integral_constant<int, 1>{});
-    if constexpr (DEPTH == 4) {
-      step(integral_constant<int, 2>{});
-      step(integral_constant<int, 3>{});
-    }
+  for (; kt + 4 <= nk; kt += 2) {  // both steps have a step two ahead to request
+    step(slot0, true_type{}, true_type{});
+    step(slot1, true_type{}, true_type{});
   }
-  const int rem = nk - kt;  // < DEPTH
-  if (rem > 0) step(integral_constant<int, 0>{});
-  if constexpr (DEPTH == 4) {
-    if (rem > 1) step(integral_constant<int, 1>{});
-    if (rem > 2) step(integral_constant<int, 2>{});
+  const int rem = nk - kt;  // 1, 2 or 3
+  if (rem == 3) {
+    step(slot0, true_type{}, true_type{});
+    step(slot1, false_type{}, true_type{});
+    step(slot0, false_type{}, false_type{});
+  } else if (rem == 2) {
+    step(slot0, false_type{}, true_type{});
+    step(slot1, false_type{}, false_type{});
+  } else if (rem == 1) {
+    step(slot0, false_type{}, false_type{});
   }
 
   // ---- epilogue: bias, activation, fp16, transpose through LDS ------------
