@@ -71,7 +71,10 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // arithmetic with its MFMAs, so where a CU holds a single workgroup (few
 // tiles: the 14x14 and 7x7 layers) the MFMA pipe otherwise idles during all
 // address, mask and LDS work.
-template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG>
+// ONE_STEP: the whole reduction is one 64-k step (a 1x1 layer over 64
+// channels): one LDS stage instead of two, so more workgroups fit a CU, and
+// what these layers need is memory requests in flight, not MFMA time.
+template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG, bool ONE_STEP = false>
 __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefronts per SIMD the register budget must allow
  void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
@@ -82,7 +85,8 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   static_assert(A_CH >= 1 && B_CH >= 1, "tile too small");
   constexpr int STAGE = (BM + BN) * LDS_ROW;               // halfs per pipeline stage
   constexpr int CROW = BM + 8;                             // halfs per row of the output staging tile
-  constexpr int SMEM = (2 * STAGE > BN * CROW) ? 2 * STAGE : BN * CROW;
+  constexpr int STAGES = ONE_STEP ? 1 : 2;
+  constexpr int SMEM = (STAGES * STAGE > BN * CROW) ? STAGES * STAGE : BN * CROW;
   static_assert(DEPTH == 2 || DEPTH == 4, "ring slots and LDS stages are indexed at compile time");
   __shared__ __attribute__((aligned(16))) _Float16 smem[SMEM];
 
@@ -250,7 +254,7 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   // prologue: steps 0 and 1 in flight, step 0 into LDS stage 0
   static_assert(DEPTH == 2, "the step sequence below is written for two register slots");
   load_step(ra[0], rb[0], rm[0]);
-  if (nk > 1) load_step(ra[1], rb[1], rm[1]);
+  if (!ONE_STEP && nk > 1) load_step(ra[1], rb[1], rm[1]);
   store_step(0, ra[0], rb[0], rm[0]);
   __syncthreads();
 
@@ -294,12 +298,16 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   const integral_constant<int, 0> slot0{};
   const integral_constant<int, 1> slot1{};
   int kt = 0;
-  for (; kt + 4 <= nk; kt += 2) {  // both steps have a step two ahead to request
-    step(slot0, true_type{}, true_type{});
-    step(slot1, true_type{}, true_type{});
+  if constexpr (!ONE_STEP) {
+    for (; kt + 4 <= nk; kt += 2) {  // both steps have a step two ahead to request
+      step(slot0, true_type{}, true_type{});
+      step(slot1, true_type{}, true_type{});
+    }
   }
-  const int rem = nk - kt;  // 1, 2 or 3
-  if (rem == 3) {
+  const int rem = ONE_STEP ? 1 : nk - kt;  // 1, 2 or 3
+  if (ONE_STEP) {
+    step(slot0, false_type{}, false_type{});
+  } else if (rem == 3) {
     step(slot0, true_type{}, true_type{});
     step(slot1, false_type{}, true_type{});
     step(slot0, false_type{}, false_type{});
@@ -501,16 +509,16 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     am.magic_q = magic_of(a.Q);
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
     const bool pad = a.ph != 0 || a.pw != 0;
-#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, KG_)                                                    \
+#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, KG_, ONE_)                                                  \
   do {                                                                                                     \
     const int64_t tiles = tiles_of(BM_, BN_);                                                              \
     if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                  \
     const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                              \
     if (pad || NPQ % BN_ != 0 || a.K % BM_ != 0)                                                           \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, true, KG_>), dim3(grid), \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, true, KG_, ONE_>), dim3(grid), \
                          dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
     else                                                                                                   \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, false, KG_>), dim3(grid), \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, false, KG_, ONE_>), dim3(grid), \
                          dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
   } while (0)
     // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
@@ -518,7 +526,9 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     // 128x128 when there are enough tiles for more than one workgroup per CU;
     // with about one per CU or fewer, the eight-wavefront variants (128x128,
     // then 128x64), which keep two wavefronts on every SIMD; 128x64 for very
-    // short reductions; 64x64 when K_out <= 64 (64x128 for its 3x3 layers;
+    // short reductions; 64x64 when K_out <= 64 (64x128, case 15, was ahead on
+    // its 3x3 layers until the step sequence stopped loading past the end and
+    // fell behind after: 37 vs 33 us;
     // walking an XCD's run of tiles pixel tiles first instead of k_out tiles
     // first, so that an XCD touches a slice of a large filter only, changed
     // nothing on the 7x7 layers).
@@ -527,19 +537,26 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     if (sel == 0) {
       const int nk = a.R * a.S * (a.C / BKF);
       const int64_t t128 = tiles_of(128, 128), cus = ctx->num_cu;
-      if (a.K <= 64) sel = nk >= 9 ? 15 : 4;
+      if (nk == 1) sel = 18;  // one step: the single-stage 64x64 variant (27 vs 34 us on 64 -> 256 at 56x56)
+      else if (a.K <= 64) sel = 4;
       else if (nk <= 2) sel = 7;
       else if (4 * t128 >= 5 * cus) sel = 3;
       else if (5 * t128 >= 3 * cus) sel = 12;
       else sel = 11;
     }
     switch (sel) {
-      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1); break;
-      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1); break;
-      case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2); break;
-      case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2); break;
-      case 15: LAUNCH_FAST(64, 128, 2, 2, 2, 2, 1); break;
-      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1); break;
+      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, false); break;
+      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, false); break;
+      case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2, false); break;
+      case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2, false); break;
+      case 15: LAUNCH_FAST(64, 128, 2, 2, 2, 2, 1, false); break;
+      case 17: if (a.R * a.S * (a.C / BKF) != 1) { set_error("conv(fp16): tile 17 is for one-step reductions"); return false; }
+               LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, true); break;
+      case 18: if (a.R * a.S * (a.C / BKF) != 1) { set_error("conv(fp16): tile 18 is for one-step reductions"); return false; }
+               LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, true); break;
+      case 19: if (a.R * a.S * (a.C / BKF) != 1) { set_error("conv(fp16): tile 19 is for one-step reductions"); return false; }
+               LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, true); break;
+      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, false); break;
     }
 #undef LAUNCH_FAST
   } else {
