@@ -71,10 +71,11 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // arithmetic with its MFMAs, so where a CU holds a single workgroup (few
 // tiles: the 14x14 and 7x7 layers) the MFMA pipe otherwise idles during all
 // address, mask and LDS work.
-// ONE_STEP: the whole reduction is one 64-k step (a 1x1 layer over 64
-// channels): one LDS stage instead of two, so more workgroups fit a CU, and
+// FEW_STEPS = n > 0: the whole reduction is exactly n 64-k steps (a 1x1 layer
+// over 64 n channels) and they take turns in ONE LDS stage instead of
+// alternating between two: half the LDS, so more workgroups fit a CU, and
 // what these layers need is memory requests in flight, not MFMA time.
-template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG, bool ONE_STEP = false>
+template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG, int FEW_STEPS = 0>
 __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefronts per SIMD the register budget must allow
  void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
   static_assert(WM * WN == 4, "four wavefronts");
@@ -85,7 +86,9 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   static_assert(A_CH >= 1 && B_CH >= 1, "tile too small");
   constexpr int STAGE = (BM + BN) * LDS_ROW;               // halfs per pipeline stage
   constexpr int CROW = BM + 8;                             // halfs per row of the output staging tile
-  constexpr int STAGES = ONE_STEP ? 1 : 2;
+  constexpr bool ONE_STAGE = FEW_STEPS > 0;
+  static_assert(!ONE_STAGE || KG == 1, "the single-stage sequence is written for one k group");
+  constexpr int STAGES = ONE_STAGE ? 1 : 2;
   constexpr int SMEM = (STAGES * STAGE > BN * CROW) ? STAGES * STAGE : BN * CROW;
   static_assert(DEPTH == 2 || DEPTH == 4, "ring slots and LDS stages are indexed at compile time");
   __shared__ __attribute__((aligned(16))) _Float16 smem[SMEM];
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   // prologue: steps 0 and 1 in flight, step 0 into LDS stage 0
   static_assert(DEPTH == 2, "the step sequence below is written for two register slots");
   load_step(ra[0], rb[0], rm[0]);
-  if (!ONE_STEP && nk > 1) load_step(ra[1], rb[1], rm[1]);
+  if (ONE_STAGE ? FEW_STEPS > 1 : nk > 1) load_step(ra[1], rb[1], rm[1]);
   store_step(0, ra[0], rb[0], rm[0]);
   __syncthreads();
 
@@ -298,15 +301,30 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   const integral_constant<int, 0> slot0{};
   const integral_constant<int, 1> slot1{};
   int kt = 0;
-  if constexpr (!ONE_STEP) {
+  if constexpr (!ONE_STAGE) {
     for (; kt + 4 <= nk; kt += 2) {  // both steps have a step two ahead to request
       step(slot0, true_type{}, true_type{});
       step(slot1, true_type{}, true_type{});
     }
   }
-  const int rem = ONE_STEP ? 1 : nk - kt;  // 1, 2 or 3
-  if (ONE_STEP) {
-    step(slot0, false_type{}, false_type{});
+  const int rem = ONE_STAGE ? 0 : nk - kt;  // 1, 2 or 3
+  if constexpr (ONE_STAGE) {
+    // step T: its data goes from register slot T % 2 into the one stage (step 0's is there already), the
+    // slot is refilled with step T + 2 if there is one, then the MFMAs read the stage
+    auto turn = [&](auto t_c) {
+      constexpr int T = decltype(t_c)::value, U = T & 1;
+      if constexpr (T > 0) {
+        store_step(0, ra[U], rb[U], rm[U]);
+        __syncthreads();
+      }
+      if constexpr (T + 2 < FEW_STEPS) load_step(ra[U], rb[U], rm[U]);
+      step(slot0, false_type{}, false_type{});  // reads stage 0, loads and stages nothing, ends on a barrier
+    };
+    turn(integral_constant<int, 0>{});
+    if constexpr (FEW_STEPS > 1) turn(integral_constant<int, 1>{});
+    if constexpr (FEW_STEPS > 2) turn(integral_constant<int, 2>{});
+    if constexpr (FEW_STEPS > 3) turn(integral_constant<int, 3>{});
+    static_assert(FEW_STEPS <= 4, "up to four turns are written out");
   } else if (rem == 3) {
     step(slot0, true_type{}, true_type{});
     step(slot1, false_type{}, true_type{});
@@ -509,16 +527,16 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     am.magic_q = magic_of(a.Q);
     auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
     const bool pad = a.ph != 0 || a.pw != 0;
-#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, KG_, ONE_)                                                  \
+#define LAUNCH_FAST(BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, KG_, FEW_)                                                  \
   do {                                                                                                     \
     const int64_t tiles = tiles_of(BM_, BN_);                                                              \
     if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                  \
     const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                              \
     if (pad || NPQ % BN_ != 0 || a.K % BM_ != 0)                                                           \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, true, KG_, ONE_>), dim3(grid), \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, true, KG_, FEW_>), dim3(grid), \
                          dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
     else                                                                                                   \
-      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, false, KG_, ONE_>), dim3(grid), \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, WM_, WN_, DEPTH_, MIN_WAVES_, false, KG_, FEW_>), dim3(grid), \
                          dim3(256 * KG_), 0, ctx->stream, am, (int)tiles);                                 \
   } while (0)
     // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
@@ -537,7 +555,8 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     if (sel == 0) {
       const int nk = a.R * a.S * (a.C / BKF);
       const int64_t t128 = tiles_of(128, 128), cus = ctx->num_cu;
-      if (nk == 1) sel = 18;  // one step: the single-stage 64x64 variant (27 vs 34 us on 64 -> 256 at 56x56)
+      if (nk <= 4) sel = 18;  // up to four steps (1x1 over up to 256 channels): the single-stage 64x64 variant
+                              // (27 vs 34 us on 64 -> 256 at 56x56, 22.6 vs 26.6 on 128 -> 512 at 28x28, 18.3 vs 21.7 on 256 -> 1024 at 14x14)
       else if (a.K <= 64) sel = 4;
       else if (nk <= 2) sel = 7;
       else if (4 * t128 >= 5 * cus) sel = 3;
@@ -545,18 +564,29 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       else sel = 11;
     }
     switch (sel) {
-      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, false); break;
-      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, false); break;
-      case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2, false); break;
-      case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2, false); break;
-      case 15: LAUNCH_FAST(64, 128, 2, 2, 2, 2, 1, false); break;
-      case 17: if (a.R * a.S * (a.C / BKF) != 1) { set_error("conv(fp16): tile 17 is for one-step reductions"); return false; }
-               LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, true); break;
-      case 18: if (a.R * a.S * (a.C / BKF) != 1) { set_error("conv(fp16): tile 18 is for one-step reductions"); return false; }
-               LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, true); break;
-      case 19: if (a.R * a.S * (a.C / BKF) != 1) { set_error("conv(fp16): tile 19 is for one-step reductions"); return false; }
-               LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, true); break;
-      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, false); break;
+      case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, 0); break;
+      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, 0); break;
+      case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2, 0); break;
+      case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2, 0); break;
+      case 15: LAUNCH_FAST(64, 128, 2, 2, 2, 2, 1, 0); break;
+      case 18: {  // 64 x 64, one LDS stage, for reductions of one to four steps
+        const int steps = a.R * a.S * (a.C / BKF);
+        if (steps == 1) LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 1);
+        else if (steps == 2) LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 2);
+        else if (steps == 3) LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 3);
+        else if (steps == 4) LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 4);
+        else { set_error("conv(fp16): tile 18 is for reductions of one to four steps"); return false; }
+        break;
+      }
+      case 17: {  // the same with 128 x 64 tiles
+        const int steps = a.R * a.S * (a.C / BKF);
+        if (steps == 1) LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, 1);
+        else if (steps == 2) LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, 2);
+        else if (steps == 4) LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, 4);
+        else { set_error("conv(fp16): tile 17 is for reductions of one, two or four steps"); return false; }
+        break;
+      }
+      default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 0); break;
     }
 #undef LAUNCH_FAST
   } else {

@@ -530,6 +530,9 @@ F16_CASES = [
     (2, 64, 9, 11, 40, 3, 1, 1),       # 64 x 128 tile, ragged in both directions
     (2, 64, 9, 11, 40, 1, 1, 0),       # one-step reduction (single LDS stage), ragged in both directions
     (1, 64, 12, 12, 72, 1, 2, 0),      # the same with stride 2 and two k_out tiles
+    (2, 128, 9, 11, 40, 1, 1, 0),      # two, three and four steps taking turns in the one LDS stage
+    (1, 192, 10, 7, 72, 1, 1, 0),
+    (2, 256, 7, 7, 136, 1, 1, 0),
     (2, 3, 32, 32, 64, 7, 2, 3),       # 3 channels: first-layer kernel (NCHW in, NHWC out), generic otherwise
     (2, 3, 45, 37, 64, 7, 2, 3),       # first-layer kernel, ragged tiles (23 x 19 output pixels)
     (1, 3, 224, 224, 64, 7, 2, 3),     # the ResNet first layer at full size
