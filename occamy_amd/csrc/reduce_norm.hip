@@ -51,6 +51,43 @@ __global__ __launch_bounds__(256) void mean_cols_kernel(const T *__restrict__ x,
   st_f(y + i, s / (float)red);
 }
 
+// The same with V consecutive inner elements (8 bytes) per thread and the
+// loads of seven reduction steps in flight at a time; the sums run in the
+// same order as above.  A channels-last global average pool is this shape
+// (49 steps over 2048 channels): with one 2-byte load in flight per lane it
+// ran at a tenth of the memory rate.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void mean_cols_vec_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                            int64_t outer, int red, int64_t inner_v) {
+  struct alignas(sizeof(T) * V) Vec { T v[V]; };
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= outer * inner_v) return;
+  const int64_t o = i / inner_v, in = i - o * inner_v;
+  const Vec *xp = reinterpret_cast<const Vec *>(x) + o * red * inner_v + in;
+  float s[V];
+#pragma unroll
+  for (int e = 0; e < V; e++) s[e] = 0.f;
+  int r = 0;
+  for (; r + 7 <= red; r += 7) {
+    Vec t[7];
+#pragma unroll
+    for (int u = 0; u < 7; u++) t[u] = xp[(int64_t)(r + u) * inner_v];
+#pragma unroll
+    for (int u = 0; u < 7; u++)
+#pragma unroll
+      for (int e = 0; e < V; e++) s[e] += ld_f(&t[u].v[e]);
+  }
+  for (; r < red; r++) {
+    const Vec t = xp[(int64_t)r * inner_v];
+#pragma unroll
+    for (int e = 0; e < V; e++) s[e] += ld_f(&t.v[e]);
+  }
+  Vec out;
+#pragma unroll
+  for (int e = 0; e < V; e++) st_f(&out.v[e], s[e] / (float)red);
+  reinterpret_cast<Vec *>(y)[i] = out;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(const T *__restrict__ x, T *__restrict__ y,
                                                            int64_t rows, int L) {
@@ -199,10 +236,16 @@ static bool run_reduce(const dnnrtContext *ctx, const void *X, void *Y, int64_t 
     hipLaunchKernelGGL((mean_rows_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
                        (const T *)X, (T *)Y, outer, (int)red);
   } else {
-    const int64_t blocks = ceil_div(outer * inner, 256);
+    constexpr int V = 8 / (int)sizeof(T);
+    const bool vec = inner % V == 0 && (reinterpret_cast<uintptr_t>(X) & 7u) == 0 && (reinterpret_cast<uintptr_t>(Y) & 7u) == 0;
+    const int64_t blocks = ceil_div(vec ? outer * (inner / V) : outer * inner, 256);
     if (blocks > INT32_MAX) { set_error("reduce: tensor too large"); return false; }
-    hipLaunchKernelGGL((mean_cols_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
-                       (const T *)X, (T *)Y, outer, (int)red, inner);
+    if (vec)
+      hipLaunchKernelGGL((mean_cols_vec_kernel<T, V>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                         (const T *)X, (T *)Y, outer, (int)red, inner / V);
+    else
+      hipLaunchKernelGGL((mean_cols_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                         (const T *)X, (T *)Y, outer, (int)red, inner);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("reduce: launch failed: %s", hipGetErrorString(e)); return false; }

@@ -190,6 +190,14 @@ def test_reduce_mean(gpu, cpu):
                        ((1, 128, 768), (1, 128, 1)), ((3, 1000), (3, 1)), ((1, 1280, 7, 7), (1, 1280, 1, 1))]:
         x = r.standard_normal(shape).astype(np.float32)
         close(oc.reduce_mean(gpu, x, out), oc.reduce_mean(cpu, x, out))
+    # a middle dim reduced over an inner run of whole 8-byte units (what a channels-last global average
+    # pool is): 7 + 3, 49 and 5 reduction steps, both element types, against numpy's float64 mean
+    for shape, out in [((3, 10, 16), (3, 1, 16)), ((4, 49, 256), (4, 1, 256)), ((2, 5, 3, 8), (2, 1, 3, 8)), ((1, 7, 6), (1, 1, 6))]:
+        for dtype, tol in ((np.float32, 1e-5), (np.float16, 2e-3)):
+            x = r.standard_normal(shape).astype(dtype)
+            got = oc.reduce_mean(gpu, x, out)
+            close(got, oc.reduce_mean(cpu, x, out), tol, tol)
+            np.testing.assert_allclose(got.astype(np.float64), x.astype(np.float64).mean(1, keepdims=True), rtol=tol, atol=tol)
     with pytest.raises(RuntimeError):
         oc.reduce_mean(gpu, np.zeros((2, 3, 4, 5), np.float32), (1, 3, 1, 5))
 
