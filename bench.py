@@ -30,7 +30,7 @@ def build_workload(name):
     if name == "resnet50_fp32_bs1":
         return models.resnet50(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
-        return models.resnet50(64, np.float16, seed=5), dict(fusion=True, fuse_residual=True, channels_last=True), 64, "img/s", "f16"
+        return models.resnet50(64, np.float16, seed=5), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True), 64, "img/s", "f16"
     if name == "mobilenet_v2_fp32_bs1":
         return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":

@@ -289,7 +289,8 @@ void *dnnrtAveragePool(dnnrtHandle_t handle, const void *X,
  * (src/Tools/dnn-wrapper/cublas/CUBLASMatmul2dFunc.cu:9-153):
  * Out = alpha op(A) op(B) + beta C, row-major; C may be NULL when beta == 0.
  * C is [M,N] as in the reference (which sizes it by dimOut, :32) or, with
- * dimC = [1,N], one row added to every row of the product (fp32 only). */
+ * dimC = [1,N], one row added to every row of the product (fp16: only with
+ * beta = 1, where it is the convolution kernel's per-filter bias). */
 void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A,
                     const int64_t *dimA, const void *B, const int64_t *dimB,
                     const void *C, const int64_t *dimC, void *Out,

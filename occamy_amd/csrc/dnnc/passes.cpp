@@ -240,7 +240,10 @@ void fuse_matmul_bias(Program &p) {
   for (Op *mm : gemms) {
     // the add works on the product's BUFFER (first operand and output), not on the product's result value
     Value *buf = mm->operands[2];
-    if (mm->result->dtype != F32 || !mm->result->uses.empty()) continue;
+    if (!mm->result->uses.empty()) continue;
+    // fp16: only the shape the fp16 product is built for, with the bias as one row
+    if (mm->result->dtype == F16 && !(mm->alpha == 1.f && !mm->trans_a && mm->trans_b)) continue;
+    if (mm->result->dtype != F32 && mm->result->dtype != F16) continue;
     Op *add = nullptr;
     for (const auto &u : buf->uses) {
       Op *o = u.first;
@@ -251,6 +254,7 @@ void fuse_matmul_bias(Program &p) {
         add->operands[1] == buf)
       continue;
     if (add->dimB.size() != 2 || add->dimB[1] != mm->dimOut[1] || (add->dimB[0] != 1 && add->dimB[0] != mm->dimOut[0])) continue;
+    if (mm->result->dtype == F16 && add->dimB[0] != 1) continue;
     Value *out = buf;
     Op *fused = p.new_op(OP_MATMUL2D);
     fused->dimA = mm->dimA;

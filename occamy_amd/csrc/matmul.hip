@@ -144,10 +144,9 @@ void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A, const int
       return nullptr;
     return Out;
   }
-  if (dtype == DNNRT_F16 && c_is_row) DNNRT_FAIL("dnnrtMatmul2d: a one-row C is not built for fp16");
   if (dtype == DNNRT_F16) {
     if (!gemm_f16(handle, (const __half *)A, (const __half *)B, (const __half *)Cin, (__half *)Out,
-                  (int)M, (int)N, (int)K, alpha, beta, transA != 0, transB != 0, 1, 0, 0, 0))
+                  (int)M, (int)N, (int)K, alpha, beta, transA != 0, transB != 0, 1, 0, 0, 0, c_is_row || (Cin && M == 1)))
       return nullptr;
     return Out;
   }

@@ -700,7 +700,9 @@ void *dnnrtMatmul2d(dnnrtHandle_t h, int64_t rank, const void *A, const int64_t 
     for (int64_t m = 0; m < M; m++)
       for (int64_t n = 0; n < N; n++) {
         const float t = beta * cc[n];
-        o[m * N + n] = o[m * N + n] + t;
+        /* fp16: the product is stored (rounded) before the add reads it */
+        const float prod = dtype == DNNRT_F16 ? h2f(f2h(o[m * N + n])) : o[m * N + n];
+        o[m * N + n] = prod + t;
       }
   free(cc);
   narrow(Out, to, M * N, dtype); free(ta); free(tb); free(tc);

@@ -129,6 +129,10 @@ def test_resnet50_fp16_channels_last(batch, image):
     got, want = out16[0].astype(np.float32), ref[0]
     assert np.isfinite(got).all()
     np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    # the classifier's bias folded into the product: one launch fewer, same tolerance
+    fused, _ = run(build16, fusion=True, channels_last=True, fuse_residual=True, fuse_matmul_bias=True)
+    np.testing.assert_allclose(fused[0].astype(np.float32), want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    assert "dimC=[1," in build16()[0].compile(fusion=True, channels_last=True, fuse_matmul_bias=True).text
     # resident + graph replay gives the same bits as the per-inference mode
     g, inputs = build16()
     p = g.compile(fusion=True, channels_last=True)

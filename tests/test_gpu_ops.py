@@ -627,5 +627,11 @@ def test_matmul2d_f16(gpu, cpu):
         b = (r.standard_normal((N, K)) / np.sqrt(K)).astype(np.float16)
         np.testing.assert_allclose(oc.matmul2d(gpu, a, b, transB=1).astype(np.float32),
                                    oc.matmul2d(cpu, a, b, transB=1).astype(np.float32), rtol=2e-3, atol=2e-3)
+        # C as one row with beta 1 (a Gemm's bias): the convolution kernel's bias; the oracle runs product, then add
+        row = r.standard_normal(N).astype(np.float16)
+        np.testing.assert_allclose(oc.matmul2d_row(gpu, a, b, row, transB=1).astype(np.float32),
+                                   oc.matmul2d_row(cpu, a, b, row, transB=1).astype(np.float32), rtol=2e-3, atol=4e-3)
     with pytest.raises(RuntimeError):
         oc.matmul2d(gpu, np.zeros((4, 8), np.float16), np.zeros((8, 4), np.float16))  # layout not built: loud
+    with pytest.raises(RuntimeError):
+        oc.matmul2d_row(gpu, a, b, row, beta=0.5, transB=1)                           # only beta = 1 is built
