@@ -97,6 +97,58 @@ __global__ __launch_bounds__(256) void pool_nhwc_f16x8_kernel(const _Float16 *__
   *reinterpret_cast<pl_half8 *>(y + i * 8) = o;
 }
 
+// The same for a window size known at compile time: every tap is loaded
+// unconditionally from an address clamped into the image (all R * S loads in
+// flight at once) and a tap outside the image is replaced by -inf / 0 with a
+// select.  With the loads under the bounds checks of the loops above each tap
+// was a memory round trip of its own.
+template <bool IS_MAX, int R, int S>
+__global__ __launch_bounds__(256) void pool_nhwc_f16x8_fixed_kernel(const _Float16 *__restrict__ x, _Float16 *__restrict__ y,
+                                                                    PoolGeom g, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c8 = g.C >> 3;
+  int64_t t = i;
+  const int cg = (int)(t % c8); t /= c8;
+  const int q = (int)(t % g.Q); t /= g.Q;
+  const int p = (int)(t % g.P);
+  const int n = (int)(t / g.P);
+  const _Float16 *xb = x + (int64_t)n * g.H * g.W * g.C + cg * 8;
+  const int ih0 = p * g.sh - g.ph, iw0 = q * g.sw - g.pw;
+  pl_half8 v8[R][S];
+  bool ok[R][S];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int ss = 0; ss < S; ss++) {
+      const int ih = ih0 + r, iw = iw0 + ss;
+      ok[r][ss] = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+      const int ihc = min(max(ih, 0), g.H - 1), iwc = min(max(iw, 0), g.W - 1);
+      v8[r][ss] = *reinterpret_cast<const pl_half8 *>(xb + ((int64_t)ihc * g.W + iwc) * g.C);
+    }
+  float m[8], sum[8];
+  bool nan[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) { m[e] = -INFINITY; sum[e] = 0.f; nan[e] = false; }
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int ss = 0; ss < S; ss++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const float raw = (float)v8[r][ss][e];
+        const float v = ok[r][ss] ? raw : (IS_MAX ? -INFINITY : 0.f);
+        nan[e] = nan[e] || (v != v);
+        m[e] = v > m[e] ? v : m[e];
+        sum[e] += v;
+      }
+  pl_half8 o;
+#pragma unroll
+  for (int e = 0; e < 8; e++)
+    o[e] = (_Float16)(IS_MAX ? (nan[e] ? __builtin_nanf("") : m[e]) : sum[e] / (float)(R * S));
+  *reinterpret_cast<pl_half8 *>(y + i * 8) = o;
+}
+
 static void *pool_entry(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX, void *Y,
                         const int64_t *dY, const int64_t *kr, const int64_t *pads, const int64_t *st,
                         bool is_max, int32_t dtype) {
@@ -122,6 +174,18 @@ static void *pool_entry(const char *who, dnnrtHandle_t h, const void *X, const i
   if (blocks > INT32_MAX) DNNRT_FAIL("%s: tensor too large", who);
   if (dtype == DNNRT_F16 && g.nhwc && g.C % 8 == 0 && aligned16(X) && aligned16(Y)) {
     const int64_t tot8 = total / 8, blocks8 = ceil_div(tot8, 256);
+#define POOL_FIXED(R_, S_)                                                                                                  \
+  do {                                                                                                                      \
+    if (is_max) hipLaunchKernelGGL((pool_nhwc_f16x8_fixed_kernel<true, R_, S_>), dim3((unsigned)blocks8), dim3(256), 0, h->stream,  \
+                                   (const _Float16 *)X, (_Float16 *)Y, g, tot8);                                            \
+    else hipLaunchKernelGGL((pool_nhwc_f16x8_fixed_kernel<false, R_, S_>), dim3((unsigned)blocks8), dim3(256), 0, h->stream,        \
+                            (const _Float16 *)X, (_Float16 *)Y, g, tot8);                                                   \
+    DNNRT_CHECK_LAUNCH(who);                                                                                                \
+    return Y;                                                                                                               \
+  } while (0)
+    if (g.R == 3 && g.S == 3) POOL_FIXED(3, 3);
+    if (g.R == 2 && g.S == 2) POOL_FIXED(2, 2);
+#undef POOL_FIXED
     if (is_max)
       hipLaunchKernelGGL((pool_nhwc_f16x8_kernel<true>), dim3((unsigned)blocks8), dim3(256), 0, h->stream,
                          (const _Float16 *)X, (_Float16 *)Y, g, tot8);
