@@ -22,7 +22,7 @@ struct dnnrtContext {
   // the handle; kernels of one handle run in stream order, so they share it.
   float *splitk_partials;
   unsigned *splitk_counters;
-  int f16_tile;        // 0 = pick the fp16 convolution tile by problem size; 3, 4, 7, 11, 12, 15 (and 17-19 for one-step reductions) force one
+  int f16_tile;        // 0 = pick the fp16 convolution tile by problem size; 3, 4, 7, 11, 12, 15 (17 and 18 for reductions of up to four steps) force one; any forced tile switches the few-pixel 1x1 kernel off, 19 leaves it on
                        // (environment variable DNNRT_F16_TILE at dnnrtCreate; for tuning)
 };
 

@@ -16,6 +16,9 @@ struct ConvF16Args {
 };
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a);
+// Channels-last 1x1 stride-1 layers over at most this many output pixels (a fully connected layer at small batch).
+constexpr int FEWPIX_MAX_PIXELS = 64;
+bool launch_conv_f16_fewpix(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 // The 3-channel 7x7 stride-2 first layer (NCHW in, NHWC out); `launched` says whether it took the problem.
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 

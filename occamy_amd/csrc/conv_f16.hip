@@ -516,6 +516,9 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
   bool stem_launched = false;
   if (!launch_conv_f16_stem(ctx, a, stem_launched)) return false;
   if (stem_launched) return true;
+  bool few_launched = false;
+  if (!launch_conv_f16_fewpix(ctx, a, few_launched)) return false;
+  if (few_launched) return true;
   const int64_t NPQ = (int64_t)a.N * a.P * a.Q;
   const bool fast = a.format == DNNRT_NHWC && a.group == 1 && a.C % 64 == 0 && a.K % 8 == 0 && a.R * a.S <= 32 &&
                     (int64_t)a.N * a.H * a.W * a.C < (1ll << 31) && (int64_t)a.K * a.C * a.R * a.S < (1ll << 31) &&

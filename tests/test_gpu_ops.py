@@ -541,6 +541,10 @@ F16_CASES = [
     (2, 128, 9, 11, 40, 1, 1, 0),      # two, three and four steps taking turns in the one LDS stage
     (1, 192, 10, 7, 72, 1, 1, 0),
     (2, 256, 7, 7, 136, 1, 1, 0),
+    (64, 2048, 1, 1, 1000, 1, 1, 0),   # few pixels (a fully connected layer): 16 filters x 32 pixels per workgroup
+    (1, 512, 1, 1, 1000, 1, 1, 0),     # the same with one pixel
+    (3, 320, 3, 5, 72, 1, 1, 0),       # 45 pixels, five chunks over four wavefronts, half a block of filters
+    (1, 1088, 7, 7, 24, 1, 1, 0),      # 49 pixels, 17 chunks
     (2, 3, 32, 32, 64, 7, 2, 3),       # 3 channels: first-layer kernel (NCHW in, NHWC out), generic otherwise
     (2, 3, 45, 37, 64, 7, 2, 3),       # first-layer kernel, ragged tiles (23 x 19 output pixels)
     (1, 3, 224, 224, 64, 7, 2, 3),     # the ResNet first layer at full size
