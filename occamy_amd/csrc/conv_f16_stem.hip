@@ -44,8 +44,11 @@ constexpr int OROW = 72;                     // halfs per pixel in the output st
 __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args a, const int tiles_p, const int tiles_q,
                                                                const int total) {
   using namespace stem;
-  __shared__ __attribute__((aligned(16))) _Float16 patch[2][PATCH];
-  __shared__ __attribute__((aligned(16))) _Float16 ostage[4][32 * OROW];
+  // one LDS block: the two patch buffers, then the four wavefronts' output staging; at start-up the whole filter passes through it
+  __shared__ __attribute__((aligned(16))) _Float16 smem[2 * PATCH + 4 * 32 * OROW];
+  static_assert(2 * PATCH + 4 * 32 * OROW >= 64 * 147, "the filter is staged in the same block");
+  _Float16(*patch)[PATCH] = reinterpret_cast<_Float16(*)[PATCH]>(smem);
+  _Float16 *ostage = smem + 2 * PATCH;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, half = lane >> 5;
@@ -54,6 +57,16 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
   _Float16 *__restrict__ Yg = reinterpret_cast<_Float16 *>(a.Y);
 
   // ---- filter into A-operand registers ---------------------------------
+  // Through LDS: read from global memory a lane's 176 two-byte elements lie in
+  // 64 different cache lines per load instruction (one filter per lane, 294
+  // bytes apart), which kept the vector memory pipe busy for longer than all
+  // the tiles of the workgroup together; the copy below reads each line once.
+  {
+    const unsigned *__restrict__ w32 = reinterpret_cast<const unsigned *>(Wg);  // the launcher checked the alignment
+    unsigned *s32 = reinterpret_cast<unsigned *>(smem);
+    for (int e = tid; e < 64 * 147 / 2; e += 256) s32[e] = w32[e];
+  }
+  __syncthreads();
   half8 afr[2][STEPS];
 #pragma unroll
   for (int i = 0; i < 2; i++)
@@ -64,7 +77,7 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
 #pragma unroll
       for (int s = 0; s < 8; s++) {
         _Float16 v = (_Float16)0.f;
-        if (s < 7 && cr < 21) v = Wg[((k_out * 7 + r) * 7 + s) * 3 + c];
+        if (s < 7 && cr < 21) v = smem[((k_out * 7 + r) * 7 + s) * 3 + c];
         afr[i][j][s] = v;
       }
     }
@@ -80,6 +93,7 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
           bias4[i][g][e] = biasg ? biasg[32 * i + 8 * g + 4 * half + e] : (_Float16)0.f;
   }
 
+  __syncthreads();  // every lane has its part of the filter: the block is free
   // zero both patch buffers once: the columns past PX stay zero for good
   for (int e = tid; e < 2 * PATCH / 8; e += 256)
     reinterpret_cast<u32x4 *>(&patch[0][0])[e] = (u32x4){0u, 0u, 0u, 0u};
@@ -150,7 +164,7 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
 
     // ---- epilogue: bias, activation, 128-byte lines per pixel -------------
     const int tq = tile % tiles_q, t2 = tile / tiles_q, tp = t2 % tiles_p, n = t2 / tiles_p;
-    _Float16 *os = &ostage[wave][0];
+    _Float16 *os = ostage + wave * (32 * OROW);
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -183,7 +197,7 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched) {
   launched = false;
   if (a.format != DNNRT_NCHW_TO_NHWC || a.group != 1 || a.C != 3 || a.R != 7 || a.S != 7 || a.sh != 2 || a.sw != 2 ||
-      a.ph != 3 || a.pw != 3 || a.K != 64 || a.Z != nullptr || !aligned16(a.Y) ||
+      a.ph != 3 || a.pw != 3 || a.K != 64 || a.Z != nullptr || !aligned16(a.Y) || (reinterpret_cast<uintptr_t>(a.Wt) & 3u) != 0 ||
       (a.act != DNNRT_ACT_RELU && a.act != DNNRT_ACT_IDENTITY))
     return true;
   if ((int64_t)3 * a.H * a.W >= (1ll << 31)) return true;
