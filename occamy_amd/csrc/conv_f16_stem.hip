@@ -62,9 +62,17 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
   // bytes apart), which kept the vector memory pipe busy for longer than all
   // the tiles of the workgroup together; the copy below reads each line once.
   {
-    const unsigned *__restrict__ w32 = reinterpret_cast<const unsigned *>(Wg);  // the launcher checked the alignment
-    unsigned *s32 = reinterpret_cast<unsigned *>(smem);
-    for (int e = tid; e < 64 * 147 / 2; e += 256) s32[e] = w32[e];
+    // 64 * 147 halfs = 1176 units of 16 bytes (the launcher checked the alignment): five loads per thread, all
+    // issued before the first store (a loop of load-then-store would pay the memory latency once per unit)
+    constexpr int UNITS = 64 * 147 / 8, PER = (UNITS + 255) / 256;
+    const u32x4 *__restrict__ w128 = reinterpret_cast<const u32x4 *>(Wg);
+    u32x4 *s128 = reinterpret_cast<u32x4 *>(smem);
+    u32x4 wv[PER];
+#pragma unroll
+    for (int k = 0; k < PER; k++) wv[k] = w128[min(tid + k * 256, UNITS - 1)];
+#pragma unroll
+    for (int k = 0; k < PER; k++)
+      if (tid + k * 256 < UNITS) s128[tid + k * 256] = wv[k];
   }
   __syncthreads();
   half8 afr[2][STEPS];
@@ -83,14 +91,18 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
     }
   half4 bias4[2][4];
   {
-    const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
+    // eight unconditional 8-byte loads (from the filter when there is no bias, then zeroed): a load under a
+    // branch is waited for before the next one is issued, and 32 of them in a row took longer than ten tiles
+    const bool has_bias = a.bias != nullptr;
+    const _Float16 *__restrict__ biasg = has_bias ? reinterpret_cast<const _Float16 *>(a.bias) : Wg;
+    const half4 zero4 = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-      for (int g = 0; g < 4; g++)
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-          bias4[i][g][e] = biasg ? biasg[32 * i + 8 * g + 4 * half + e] : (_Float16)0.f;
+      for (int g = 0; g < 4; g++) {
+        const half4 b = *reinterpret_cast<const half4 *>(biasg + 32 * i + 8 * g + 4 * half);
+        bias4[i][g] = has_bias ? b : zero4;
+      }
   }
 
   __syncthreads();  // every lane has its part of the filter: the block is free
@@ -197,7 +209,7 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched) {
   launched = false;
   if (a.format != DNNRT_NCHW_TO_NHWC || a.group != 1 || a.C != 3 || a.R != 7 || a.S != 7 || a.sh != 2 || a.sw != 2 ||
-      a.ph != 3 || a.pw != 3 || a.K != 64 || a.Z != nullptr || !aligned16(a.Y) || (reinterpret_cast<uintptr_t>(a.Wt) & 3u) != 0 ||
+      a.ph != 3 || a.pw != 3 || a.K != 64 || a.Z != nullptr || !aligned16(a.Y) || !aligned16(a.Wt) || (reinterpret_cast<uintptr_t>(a.bias) & 7u) != 0 ||
       (a.act != DNNRT_ACT_RELU && a.act != DNNRT_ACT_IDENTITY))
     return true;
   if ((int64_t)3 * a.H * a.W >= (1ll << 31)) return true;
