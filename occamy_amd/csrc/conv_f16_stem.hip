@@ -41,6 +41,7 @@ constexpr int STEPS = 11;
 constexpr int OROW = 72;                     // halfs per pixel in the output staging buffer (64 + 8 pad)
 }  // namespace stem
 
+template <bool RELU>
 __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args a, const int tiles_p, const int tiles_q,
                                                                const int total) {
   using namespace stem;
@@ -111,25 +112,27 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
     reinterpret_cast<u32x4 *>(&patch[0][0])[e] = (u32x4){0u, 0u, 0u, 0u};
 
   // patch element e of this thread: (c, y, x), fixed for the whole kernel
-  int pe_lds[PER_THREAD], pe_c[PER_THREAD], pe_y[PER_THREAD], pe_x[PER_THREAD];
+  int pe_lds[PER_THREAD], pe_off[PER_THREAD], pe_y[PER_THREAD], pe_x[PER_THREAD];
+  const int HW = a.H * a.W;
 #pragma unroll
   for (int k = 0; k < PER_THREAD; k++) {
     const int e = tid + k * 256;
     const int ee = e < NEL ? e : 0;
     const int c = ee / (PY * PX), rem = ee - c * (PY * PX), y = rem / PX, x = rem - y * PX;
-    pe_c[k] = c; pe_y[k] = y; pe_x[k] = e < NEL ? x : -100000;  // far outside: reads as zero
+    pe_y[k] = y; pe_x[k] = e < NEL ? x : -100000;  // far outside: reads as zero
+    pe_off[k] = c * HW + y * a.W + x;                // offset from the patch's corner (which may lie outside the image)
     pe_lds[k] = (c * PY + y) * PROW + x;
   }
-  const int HW = a.H * a.W;
   auto load_patch = [&](int tile, _Float16 (&v)[PER_THREAD]) {
     const int tq = tile % tiles_q, t2 = tile / tiles_q, tp = t2 % tiles_p, n = t2 / tiles_p;
     const int iy0 = 2 * tp * TP - 3, ix0 = 2 * tq * TQ - 3;
     const _Float16 *xb = Xg + (int64_t)n * 3 * HW;
+    const int corner = iy0 * a.W + ix0;              // uniform; negative at the top and left borders
 #pragma unroll
     for (int k = 0; k < PER_THREAD; k++) {
       const int iy = iy0 + pe_y[k], ix = ix0 + pe_x[k];
       const bool ok = (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
-      const _Float16 t = xb[ok ? pe_c[k] * HW + iy * a.W + ix : 0];
+      const _Float16 t = xb[ok ? corner + pe_off[k] : 0];
       v[k] = ok ? t : (_Float16)0.f;
     }
   };
@@ -158,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+      for (int r = 0; r < 16; r++) acc[i][r] = (float)bias4[i][r >> 2][r & 3];  // the sum starts from the bias
     const _Float16 *pb = &patch[cur][0];
 #pragma unroll
     for (int j = 0; j < STEPS; j++) {
@@ -184,20 +187,23 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_kernel(const ConvF16Args
         half4 o;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          float v = acc[i][4 * g + e] + (float)bias4[i][g][e];
-          if (a.act == DNNRT_ACT_RELU) v = v < 0.f ? 0.f : v;
+          float v = acc[i][4 * g + e];
+          if (RELU) v = v < 0.f ? 0.f : v;
           o[e] = (_Float16)v;
         }
         *reinterpret_cast<half4 *>(os + l32 * OROW + 32 * i + 8 * g + 4 * half) = o;
       }
     // same wavefront reads what it wrote: LDS keeps a wavefront's accesses in order
+    // pixel (row it / 2 of the wavefront's two, column 8 * (it % 2) + lane / 8), channels 8 * (lane % 8) ... + 7:
+    // a uniform base per tile and wavefront, one per-lane offset, and constants per `it`
+    const int p_w = tp * TP + 2 * wave, q_l = tq * TQ + (lane >> 3);
+    _Float16 *yt = Yg + (((int64_t)n * a.P + p_w) * a.Q + tq * TQ) * 64 + (lane >> 3) * 64 + (lane & 7) * 8;
 #pragma unroll
     for (int it = 0; it < 4; it++) {
-      const int pl = it * 8 + (lane >> 3), ch = lane & 7;
-      const int p = tp * TP + 2 * wave + (pl >> 4), q = tq * TQ + (pl & 15);
-      const u32x4 v = *reinterpret_cast<const u32x4 *>(os + pl * OROW + ch * 8);
-      if (p < a.P && q < a.Q)
-        *reinterpret_cast<u32x4 *>(Yg + (((int64_t)n * a.P + p) * a.Q + q) * 64 + ch * 8) = v;
+      const int pl = it * 8 + (lane >> 3);
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(os + pl * OROW + (lane & 7) * 8);
+      if (p_w + (it >> 1) < a.P && q_l + 8 * (it & 1) < a.Q)
+        *reinterpret_cast<u32x4 *>(yt + (int64_t)(it >> 1) * a.Q * 64 + (it & 1) * 512) = v;
     }
 
     store_patch(cur ^ 1, pv);
@@ -217,7 +223,10 @@ bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &l
   const int64_t total = (int64_t)a.N * tiles_p * tiles_q;
   if (total > INT32_MAX) return true;
   const int64_t grid = total < 2 * (int64_t)ctx->num_cu ? total : 2 * (int64_t)ctx->num_cu;
-  hipLaunchKernelGGL(conv_f16_stem_kernel, dim3((unsigned)grid), dim3(256), 0, ctx->stream, a, tiles_p, tiles_q, (int)total);
+  if (a.act == DNNRT_ACT_RELU)
+    hipLaunchKernelGGL(conv_f16_stem_kernel<true>, dim3((unsigned)grid), dim3(256), 0, ctx->stream, a, tiles_p, tiles_q, (int)total);
+  else
+    hipLaunchKernelGGL(conv_f16_stem_kernel<false>, dim3((unsigned)grid), dim3(256), 0, ctx->stream, a, tiles_p, tiles_q, (int)total);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("conv(fp16 stem): launch failed: %s", hipGetErrorString(e)); return false; }
   launched = true;
