@@ -14,8 +14,9 @@
 // non-finite input value cannot leak through 0 * x).
 //
 // The filter (64 x 147) lives in registers as MFMA A operands for the whole
-// kernel: workgroups are persistent and walk over tiles, loading the next
-// tile's patch into registers while the current one is computed.
+// kernel (it gets there through LDS, see below): workgroups are persistent and
+// walk over tiles, loading the next tile's patch into registers while the
+// current one is computed.  The bias is the accumulators' starting value.
 //
 // Wavefront w owns output rows 2w, 2w+1 of the tile (32 pixels) and all 64
 // output channels (two 32x32 MFMA blocks).  Results go through a
