@@ -545,9 +545,8 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     // Tile choice, from per-layer timings of the ResNet-50 shapes at batch 64
     // (14.8 GFLOP 3x3 layers run in 25-35 us, 1x1 layers near their HBM time):
     // 128x128 when there are enough tiles for more than one workgroup per CU;
-    // with about one per CU or fewer, the eight-wavefront variants (128x128,
-    // then 128x64), which keep two wavefronts on every SIMD; 128x64 for very
-    // short reductions; 64x64 when K_out <= 64 (64x128, case 15, was ahead on
+    // with about one per CU, the eight-wavefront 128x128 variant, which keeps
+    // two wavefronts on every SIMD; with fewer still, 64x64 (see below); 64x64 when K_out <= 64 (64x128, case 15, was ahead on
     // its 3x3 layers until the step sequence stopped loading past the end and
     // fell behind after: 37 vs 33 us;
     // walking an XCD's run of tiles pixel tiles first instead of k_out tiles
@@ -564,7 +563,10 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       else if (nk <= 2) sel = 7;
       else if (4 * t128 >= 5 * cus) sel = 3;
       else if (5 * t128 >= 3 * cus) sel = 12;
-      else sel = 11;
+      else sel = 4;  // fewer 128x128 tiles than that (7x7 layers at batch 64): 64x64, as many workgroups in flight as possible.
+                     // The eight-wavefront 128x64 tile (11) is ahead when the launch is repeated on warm caches
+                     // (3x3 512 -> 512: 32.5 vs 35.3 us) and behind inside the network, where the filter comes from
+                     // HBM (43.3 vs 38.2 us; 1x1 2048 -> 512: 21.7 vs 19.3 us)
     }
     switch (sel) {
       case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, 0); break;
