@@ -24,7 +24,7 @@
  *     fully overwrites its output.
  *   - one dnnrtTranspose replaces the per-rank Transpose{2,3,4,6}D symbols.
  *   - new: dnnrtSync, dnnrtSetStream, dnnrtSetTensorFormat,
- *     dnnrtSetFilterLayout, dnnrtLayerNorm,
+ *     dnnrtSetFilterLayout, dnnrtSetConvTile, dnnrtListConvTiles, dnnrtLayerNorm,
  *     dnnrtGelu, dnnrtHostAlloc/Free, dnnrtLastError.
  *
  * A tensor with no elements (a zero batch, a zero row count) is accepted by
@@ -103,6 +103,19 @@ int32_t dnnrtSetTensorFormat(dnnrtHandle_t handle, int32_t format);
 /* New.  Physical layout of fp32 convolution filters for subsequent calls
  * (DNNRT_FILTER_KCRS is the default and the reference's). */
 int32_t dnnrtSetFilterLayout(dnnrtHandle_t handle, int32_t layout);
+/* New, for tuning and tests; no counterpart in the reference (cuDNN picks its
+ * algorithm from the `algo` argument, which the reference always passes as 0).
+ * The fp16 channels-last convolution is compiled in several variants (tile
+ * shape, wavefronts per workgroup, pipeline depth); by default each call picks
+ * one from the problem size.  dnnrtListConvTiles writes the ids of the
+ * variants of this build into ids[0..capacity) and returns how many there
+ * are; dnnrtSetConvTile(handle, id) makes every following fp16 channels-last
+ * convolution of the handle use that variant (and switches the few-pixel 1x1
+ * kernel off), 0 restores the automatic choice.  A variant that cannot run a
+ * given problem makes that convolution call fail with an error, never
+ * fall back. */
+int32_t dnnrtListConvTiles(int32_t *ids, int32_t capacity);
+int32_t dnnrtSetConvTile(dnnrtHandle_t handle, int32_t tile);
 /* The coefficient of the activation modes that take one: the ceiling of
  * DNNRT_ACT_CLIPPED_RELU, the slope of DNNRT_ACT_LEAKY_RELU.  It stands where
  * the `coef` of cudnnSetActivationDescriptor stands (the reference sets up one

@@ -23,6 +23,8 @@ SIGNATURES = {
     "dnnrtSetStream": (i32, [P, P]),
     "dnnrtSetTensorFormat": (i32, [P, i32]),
     "dnnrtSetFilterLayout": (i32, [P, i32]),
+    "dnnrtListConvTiles": (i32, [C.POINTER(i32), i32]),
+    "dnnrtSetConvTile": (i32, [P, i32]),
     "dnnrtSetActivationCoef": (i32, [P, f32]),
     "dnnrtSync": (i32, [P]),
     "dnnrtGraphBegin": (i32, [P]),

@@ -60,8 +60,7 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
     delete c;
     return 1;
   }
-  const char *tile = getenv("DNNRT_F16_TILE");
-  c->f16_tile = tile ? atoi(tile) : 0;
+  c->f16_tile = 0;
   *handle = c;
   return 0;
 }
@@ -107,6 +106,22 @@ int32_t dnnrtSetActivationCoef(dnnrtHandle_t handle, float coef) {
   if (!handle) { dnnrt::set_error("dnnrtSetActivationCoef: null handle"); return 1; }
   if (coef != coef) { dnnrt::set_error("dnnrtSetActivationCoef: NaN"); return 1; }
   handle->act_coef = coef;
+  return 0;
+}
+
+int32_t dnnrtListConvTiles(int32_t *ids, int32_t capacity) {
+  int n = 0;
+  for (const int *t = dnnrt::F16_TILE_IDS; *t; t++, n++)
+    if (ids && n < capacity) ids[n] = *t;
+  return n;
+}
+
+int32_t dnnrtSetConvTile(dnnrtHandle_t handle, int32_t tile) {
+  if (!handle) { set_error("dnnrtSetConvTile: null handle"); return 1; }
+  bool known = tile == 0;
+  for (const int *t = dnnrt::F16_TILE_IDS; *t; t++) known = known || *t == tile;
+  if (!known) { set_error("dnnrtSetConvTile: no fp16 convolution variant %d in this build", tile); return 1; }
+  handle->f16_tile = tile;
   return 0;
 }
 

@@ -22,14 +22,17 @@ struct dnnrtContext {
   // the handle; kernels of one handle run in stream order, so they share it.
   float *splitk_partials;
   unsigned *splitk_counters;
-  int f16_tile;        // 0 = pick the fp16 convolution tile by problem size; 3, 4, 7, 11, 12, 15 (17 and 18 for reductions of up to four steps) force one; any forced tile switches the few-pixel 1x1 kernel off, 19 leaves it on
-                       // (environment variable DNNRT_F16_TILE at dnnrtCreate; for tuning)
+  int f16_tile;        // dnnrtSetConvTile: 0 = pick the fp16 convolution variant by problem size, otherwise one of F16_TILE_IDS
 };
 
 namespace dnnrt {
 
 constexpr int64_t SPLITK_PARTIAL_BYTES = 8ll << 20;  // 2048 partial 32x32 fp32 tiles
 constexpr int SPLITK_MAX_TILES = 16384;               // arrival counters
+
+// The fp16 channels-last convolution variants dnnrtSetConvTile can force
+// (zero-terminated; what each one is: launch_conv_f16 in conv_f16.hip).
+constexpr int F16_TILE_IDS[] = {3, 4, 11, 12, 15, 17, 18, 0};
 
 void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 

@@ -560,7 +560,6 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       if (nk <= 4) sel = 18;  // up to four steps (1x1 over up to 256 channels): the single-stage 64x64 variant
                               // (27 vs 34 us on 64 -> 256 at 56x56, 22.6 vs 26.6 on 128 -> 512 at 28x28, 18.3 vs 21.7 on 256 -> 1024 at 14x14)
       else if (a.K <= 64) sel = 4;
-      else if (nk <= 2) sel = 7;
       else if (4 * t128 >= 5 * cus) sel = 3;
       else if (5 * t128 >= 3 * cus) sel = 12;
       else sel = 4;  // fewer 128x128 tiles than that (7x7 layers at batch 64): 64x64, as many workgroups in flight as possible.
@@ -570,7 +569,6 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     }
     switch (sel) {
       case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, 0); break;
-      case 7: LAUNCH_FAST(128, 64, 2, 2, 2, 2, 1, 0); break;
       case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2, 0); break;
       case 12: LAUNCH_FAST(128, 128, 2, 2, 2, 1, 2, 0); break;
       case 15: LAUNCH_FAST(64, 128, 2, 2, 2, 2, 1, 0); break;

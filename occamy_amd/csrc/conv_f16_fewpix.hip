@@ -113,7 +113,7 @@ bool launch_conv_f16_fewpix(const dnnrtContext *ctx, const ConvF16Args &a, bool 
                     aligned16(a.X) && aligned16(a.Wt) && (reinterpret_cast<uintptr_t>(a.Y) & 7u) == 0 &&
                     (reinterpret_cast<uintptr_t>(a.Z) & 7u) == 0 && (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0;
   const int forced = ctx->f16_tile;
-  if (!fits || (forced != 0 && forced != 19)) return true;  // another kernel's problem (or another tile is forced)
+  if (!fits || forced != 0) return true;  // another kernel's problem (or another tile is forced)
   const dim3 grid((unsigned)ceil_div(a.K, 16), (unsigned)ceil_div(npix, 32));
   hipLaunchKernelGGL(conv_f16_fewpix_kernel, grid, dim3(256), 0, ctx->stream, a, (int)npix);
   hipError_t e = hipGetLastError();

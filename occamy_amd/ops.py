@@ -55,6 +55,17 @@ class Ops:
     def set_filter_layout(self, layout):
         self._check(self.lib.dnnrtSetFilterLayout(self.handle, layout), "dnnrtSetFilterLayout")
 
+    def conv_tiles(self):
+        """Ids of the fp16 channels-last convolution variants in the library."""
+        n = self.lib.dnnrtListConvTiles(None, 0)
+        ids = (C.c_int32 * max(n, 1))()
+        self.lib.dnnrtListConvTiles(ids, n)
+        return list(ids[:n])
+
+    def set_conv_tile(self, tile):
+        """Force one fp16 convolution variant for the calls that follow (0: automatic)."""
+        self._check(self.lib.dnnrtSetConvTile(self.handle, tile), "dnnrtSetConvTile")
+
     def sync(self):
         self._check(self.lib.dnnrtSync(self.handle), "dnnrtSync")
 

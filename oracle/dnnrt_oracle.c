@@ -155,6 +155,13 @@ int32_t dnnrtSetFilterLayout(dnnrtHandle_t h, int32_t layout) {
   }
   return 0;
 }
+/* The oracle has one convolution (the 7-loop definition): no variants to list, only "automatic" to select. */
+int32_t dnnrtListConvTiles(int32_t *ids, int32_t capacity) { (void)ids; (void)capacity; return 0; }
+int32_t dnnrtSetConvTile(dnnrtHandle_t h, int32_t tile) {
+  (void)h;
+  if (tile != 0) { snprintf(g_err, sizeof g_err, "oracle: no convolution variants"); return 1; }
+  return 0;
+}
 int32_t dnnrtSetActivationCoef(dnnrtHandle_t h, float coef) {
   if (!h || coef != coef) { snprintf(g_err, sizeof g_err, "setActivationCoef: bad argument"); return 1; }
   h->act_coef = coef;

@@ -104,6 +104,61 @@ def test_new_input_same_session():
     so.close()
 
 
+def as_fp32_graph(g16, inputs):
+    """The same graph with every constant and input widened to fp32 (the values stay fp16-representable)."""
+    g = compiler.Graph()
+    for name, (shape, _) in g16.input_shapes.items():
+        g.input(name, shape, np.float32)
+    for name, arr in g16.constants.items():
+        g.constant(arr.astype(np.float32), name)
+    for op, ins, out, at in g16.nodes:
+        g.node(op, ins, out, **at)
+    for o in g16.outputs:
+        g.output(o)
+    return g, [a.astype(np.float32) for a in inputs]
+
+
+def test_resnet50_fp16_batch_64_as_benchmarked():
+    """The throughput configuration at its own size and with the benchmark's own flags (64 x 3 x 224 x 224,
+    fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
+    oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True)
+    build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
+    out16, info = run(build16, **flags)
+    assert info["requested"] == info["pool"]
+    ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
+    got, want = out16[0].astype(np.float32), ref[0]
+    assert got.shape == (64, 1000) and np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    assert (got.argmax(1) == want.argmax(1)).mean() > 0.9
+    # resident mode, replayed from a captured graph (what bench.py times): the same bits
+    import torch
+    g, inputs = build16()
+    p = g.compile(**flags)
+    s = p.session(compiler.MODE_RESIDENT)
+    dev_in = [torch.from_numpy(a).cuda() for a in inputs]
+    dev_out = torch.empty((64, 1000), dtype=torch.float16, device="cuda")
+    for _ in range(3):
+        dev_out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        s.run_device([t.data_ptr() for t in dev_in], [dev_out.data_ptr()], use_graph=True)
+        s.sync()
+        np.testing.assert_array_equal(dev_out.cpu().numpy(), out16[0])
+    s.close()
+
+
+def test_bert_base_12_layers_as_benchmarked():
+    """BERT-base at its full depth with the benchmark's four flags, against the oracle running the unfused
+    program (tolerance: rtol 1e-4, atol 1e-4 on outputs of order one after the final LayerNorm)."""
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)
+    ref, _ = run(models.bert_encoder, ORACLE_PATH)
+    out, info = run(models.bert_encoder, **flags)
+    assert info["requested"] == info["pool"]
+    close(out[0], ref[0], 1e-4, 1e-4)
+    out, _ = run(models.bert_encoder, mode=compiler.MODE_RESIDENT, **flags)
+    close(out[0], ref[0], 1e-4, 1e-4)
+
+
 @pytest.mark.parametrize("batch,image", [(2, 64), (4, 224)])
 def test_resnet50_fp16_channels_last(batch, image):
     """fp16 weights/activations, fp32 accumulation, NHWC on the device, against
@@ -112,20 +167,7 @@ def test_resnet50_fp16_channels_last(batch, image):
     out16, info = run(build16, fusion=True, channels_last=True)
     assert info["requested"] == info["pool"]
 
-    def build32():
-        g16, inputs = build16()
-        g = compiler.Graph()
-        for name, (shape, _) in g16.input_shapes.items():
-            g.input(name, shape, np.float32)
-        for name, arr in g16.constants.items():
-            g.constant(arr.astype(np.float32), name)
-        for op, ins, out, at in g16.nodes:
-            g.node(op, ins, out, **at)
-        for o in g16.outputs:
-            g.output(o)
-        return g, [a.astype(np.float32) for a in inputs]
-
-    ref, _ = run(build32, ORACLE_PATH, fusion=True)
+    ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
     got, want = out16[0].astype(np.float32), ref[0]
     assert np.isfinite(got).all()
     np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))

@@ -574,6 +574,78 @@ def test_conv_f16(gpu, cpu, case, fmt):
     np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
 
 
+# Problems of the size ResNet-50 has at batch 64: the dispatcher picks its large tiles (128 x 128 and up,
+# four or eight wavefronts) only when a launch has hundreds of tiles, so these are the only cases that reach
+# them.  N, C, H, W, K, R, stride, pad
+F16_BATCH64_CASES = [
+    (64, 128, 28, 28, 128, 3, 1, 1),   # 392 tiles of 128 x 128, padded taps
+    (32, 128, 28, 28, 128, 3, 1, 1),   # 196 tiles: about one per CU
+    (64, 512, 28, 28, 128, 1, 1, 0),   # 1x1, no taps to mask, eight steps
+    (64, 256, 14, 14, 256, 3, 1, 1),   # 14 x 14: 196 tiles
+    (64, 128, 56, 56, 128, 3, 2, 1),   # strided 3x3
+    (64, 256, 56, 56, 512, 1, 2, 0),   # strided 1x1 (downsample branch)
+    (64, 64, 56, 56, 64, 3, 1, 1),     # K_out = 64: 64-filter tiles
+    (61, 128, 28, 28, 136, 3, 1, 1),   # ragged in pixels (47824 = 373.6 x 128) and in filters
+    (64, 512, 7, 7, 512, 3, 1, 1),     # 7 x 7: few, deep tiles
+    (64, 1024, 14, 14, 256, 1, 1, 0),  # sixteen steps
+]
+
+
+def f16_problem(case, seed):
+    N, C, H, W, K, R, st, pd = case
+    r = rng(seed)
+    x = r.standard_normal((N, C, H, W), dtype=np.float32).astype(np.float16)
+    w = (r.standard_normal((K, C, R, R), dtype=np.float32) * np.sqrt(2.0 / (C * R * R))).astype(np.float16)
+    b = r.uniform(-0.1, 0.1, K).astype(np.float16)
+    return x, w, b, (pd, pd), (st, st)
+
+
+@pytest.mark.parametrize("case", F16_BATCH64_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_conv_f16_at_batch_64_sizes(gpu, cpu, case):
+    x, w, b, pads, strides = f16_problem(case, sum(case))
+    ref = oc.conv(cpu, x, w, b, pads, strides, 1, _abi.ACT_RELU)
+    got = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC)
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3)
+    z = rng(1 + sum(case)).standard_normal(ref.shape, dtype=np.float32).astype(np.float16)
+    refz = oc.conv(cpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, z=z)
+    gotz = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC, z=z)
+    np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
+
+
+def test_every_compiled_f16_conv_variant(gpu, cpu):
+    """Each variant dnnrtListConvTiles names, forced with dnnrtSetConvTile, on a padded 3x3 problem, a 1x1
+    problem over 128 channels and one over 512, all ragged in both directions: it either matches the
+    oracle or refuses the problem loudly (the single-stage variants take reductions of up to four steps)."""
+    tiles = gpu.ops.conv_tiles()
+    assert tiles and 0 not in tiles
+    cases = [(3, 128, 19, 23, 200, 3, 1, 1), (5, 128, 19, 23, 200, 1, 1, 0), (5, 512, 9, 13, 136, 1, 2, 0)]
+    ran = {t: 0 for t in tiles}
+    for case in cases:
+        x, w, b, pads, strides = f16_problem(case, 5 + sum(case))
+        z = rng(6).standard_normal((case[0], case[4]) + oc.conv_out_hw(case[2], case[3], case[5], case[5], pads, strides),
+                                   dtype=np.float32).astype(np.float16)
+        ref = oc.conv(cpu, x, w, b, pads, strides, 1, _abi.ACT_RELU)
+        refz = oc.conv(cpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, z=z)
+        for t in tiles:
+            gpu.ops.set_conv_tile(t)
+            try:
+                got = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC)
+                gotz = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC, z=z)
+            except RuntimeError as e:
+                assert "tile" in str(e) or "variant" in str(e), str(e)
+                continue
+            finally:
+                gpu.ops.set_conv_tile(0)
+            ran[t] += 1
+            np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3,
+                                       err_msg=f"variant {t} on {case}")
+            np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3,
+                                       err_msg=f"variant {t} on {case} with a residual")
+    assert all(ran.values()), f"variants that ran no case: {[t for t, n in ran.items() if not n]}"
+    with pytest.raises(RuntimeError):
+        gpu.ops.set_conv_tile(9999)
+
+
 def test_f16_channels_last_ops(gpu, cpu):
     r = rng(77)
     x = r.standard_normal((2, 64, 28, 28)).astype(np.float16)
