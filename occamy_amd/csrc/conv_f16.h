@@ -22,4 +22,9 @@ bool launch_conv_f16_fewpix(const dnnrtContext *ctx, const ConvF16Args &a, bool 
 // The 3-channel 7x7 stride-2 first layer (NCHW in, NHWC out); `launched` says whether it took the problem.
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 
+// Channels-last convolutions whose operands are loaded straight into LDS (conv_f16_dma.hip): `variant` is one of
+// that file's tile ids, `a` must satisfy dma_conv_applies and carry the division constants.
+bool dma_conv_applies(const ConvF16Args &a);
+bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int variant);
+
 }  // namespace dnnrt

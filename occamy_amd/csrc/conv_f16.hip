@@ -567,6 +567,13 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
                      // (3x3 512 -> 512: 32.5 vs 35.3 us) and behind inside the network, where the filter comes from
                      // HBM (43.3 vs 38.2 us; 1x1 2048 -> 512: 21.7 vs 19.3 us)
     }
+    if (sel >= 31 && sel <= 39) {
+      if (!dma_conv_applies(am)) { set_error("conv(fp16): tile %d needs tensors below 2 GiB", sel); return false; }
+      if (!launch_conv_f16_dma(ctx, am, sel)) return false;
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
+      return true;
+    }
     switch (sel) {
       case 3: LAUNCH_FAST(128, 128, 2, 2, 2, 2, 1, 0); break;
       case 11: LAUNCH_FAST(128, 64, 2, 2, 2, 1, 2, 0); break;
