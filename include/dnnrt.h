@@ -204,6 +204,30 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X,
                             int64_t algo, int64_t group, const int64_t *pads,
                             const int64_t *strides, int64_t activMode, void *Y,
                             int32_t dtype);
+/* No counterpart in the reference.  dnnrtConvBiasActiv for callers that cannot
+ * allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It takes the stream where the other calls
+ * take a handle (dnnrtCreate allocates the handle's reduction scratch) and
+ * calls no hipMalloc, hipFree or allocating library routine; the scratch its
+ * split-reduction kernels need (partial tiles and arrival counters) is a static
+ * device array of 1 MiB + 4 KiB that every GPU the library runs on holds until
+ * the process ends.  Tensors are NCHW, filters K,C,R,S, the activation
+ * coefficient is 0 (the defaults of a fresh handle); DNNRT_ACT_RELU and
+ * DNNRT_ACT_IDENTITY are the useful modes.  A convolution whose split reduction
+ * would need more than the static array holds (more than one partial 32x32
+ * tile per compute unit of a 256-unit device, or more than 1024 output tiles
+ * under a split) is refused with an error, never run with another split:
+ * results are bit-identical to dnnrtConvBiasActiv's on a fresh handle.
+ * All calls on one GPU share that GPU's array: two calls that overlap in time
+ * on one GPU (different streams, or several threads) race; calls on one stream
+ * do not.  The arrival counters are cleared by a fill kernel ahead of every
+ * launch that uses them, so a launch that died half-way leaves nothing behind. */
+void *dnnrtConvBiasActivNoAlloc(dnnrtStream_t stream, const void *X,
+                                const int64_t *dimX, const void *W,
+                                const int64_t *dimW, const void *B,
+                                const int64_t *dimB, int64_t group,
+                                const int64_t *pads, const int64_t *strides,
+                                int64_t activMode, void *Y, int32_t dtype);
 
 /* ---- elementwise / broadcast ----------------------------------------- */
 

@@ -60,6 +60,9 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
     delete c;
     return 1;
   }
+  c->splitk_partial_bytes = dnnrt::SPLITK_PARTIAL_BYTES;
+  c->splitk_max_tiles = dnnrt::SPLITK_MAX_TILES;
+  c->splitk_shared = false;
   c->f16_tile = 0;
   *handle = c;
   return 0;

@@ -22,13 +22,23 @@ struct dnnrtContext {
   // the handle; kernels of one handle run in stream order, so they share it.
   float *splitk_partials;
   unsigned *splitk_counters;
+  int64_t splitk_partial_bytes;  // what the two buffers hold
+  int splitk_max_tiles;
+  // The buffers are shared with callers this handle knows nothing of (the process-wide static scratch of
+  // dnnrtConvBiasActivNoAlloc): clear the counters a launch uses before it, and refuse a problem whose
+  // split would have to shrink to fit instead of shrinking it.
+  bool splitk_shared;
   int f16_tile;        // dnnrtSetConvTile: 0 = pick the fp16 convolution variant by problem size, otherwise one of F16_TILE_IDS
 };
 
 namespace dnnrt {
 
-constexpr int64_t SPLITK_PARTIAL_BYTES = 8ll << 20;  // 2048 partial 32x32 fp32 tiles
-constexpr int SPLITK_MAX_TILES = 16384;               // arrival counters
+constexpr int64_t SPLITK_PARTIAL_BYTES = 8ll << 20;  // a handle's scratch: 2048 partial 32x32 fp32 tiles
+constexpr int SPLITK_MAX_TILES = 16384;               // ... and arrival counters
+// The static scratch of dnnrtConvBiasActivNoAlloc (conv.hip): the split-reduction convolution kernels ask for
+// at most one partial tile per compute unit, 1 MiB on 256 of them.
+constexpr int64_t NOALLOC_PARTIAL_BYTES = 1ll << 20;
+constexpr int NOALLOC_MAX_TILES = 1024;
 
 // The fp16 channels-last convolution variants dnnrtSetConvTile can force
 // (zero-terminated; what each one is: launch_conv_f16 in conv_f16.hip).

@@ -9,6 +9,10 @@
 #include "igemm_f32.h"
 #include "conv_f16.h"
 
+#include <string.h>
+
+#include <mutex>
+
 namespace dnnrt {
 
 // ---- depthwise, fp32, NCHW ------------------------------------------------
@@ -272,9 +276,82 @@ static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, cons
   DNNRT_FAIL("%s: dtype %d", who, dtype);
 }
 
+// ---- the process-wide scratch of dnnrtConvBiasActivNoAlloc -----------------
+// Partial tiles, then arrival counters, in one file-scope device array: every
+// GPU the library runs on holds its own copy from the moment the code object
+// is loaded until the process ends.  Host code never uses the array's name as
+// an address (on the host it is a stand-in, not device memory): the per-device
+// address comes from hipGetSymbolAddress, once, with that device current.
+constexpr int64_t NOALLOC_SCRATCH_BYTES = NOALLOC_PARTIAL_BYTES + (int64_t)NOALLOC_MAX_TILES * sizeof(unsigned);
+static __device__ __align__(256) unsigned char noalloc_scratch[NOALLOC_SCRATCH_BYTES];
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+struct NoAllocDevice {
+  bool ready;
+  unsigned char *scratch;  // this device's copy of noalloc_scratch
+  int num_cu;
+};
+static NoAllocDevice noalloc_devices[NOALLOC_MAX_DEVICES];
+static std::mutex noalloc_mutex;
+
+// The current device's entry, set up on first use (no allocation: the array is part of the loaded code object).
+static const NoAllocDevice *noalloc_device(int &dev) {
+  if (hipGetDevice(&dev) != hipSuccess) { set_error("dnnrtConvBiasActivNoAlloc: hipGetDevice failed"); return nullptr; }
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { set_error("dnnrtConvBiasActivNoAlloc: device ordinal %d", dev); return nullptr; }
+  std::lock_guard<std::mutex> lock(noalloc_mutex);
+  NoAllocDevice &d = noalloc_devices[dev];
+  if (d.ready) return &d;
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) { set_error("dnnrtConvBiasActivNoAlloc: hipGetDeviceProperties: %s", hipGetErrorString(e)); return nullptr; }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error("dnnrtConvBiasActivNoAlloc: this library holds gfx950 code only, device is %s", prop.gcnArchName);
+    return nullptr;
+  }
+  void *ptr = nullptr;
+  e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(noalloc_scratch));
+  if (e != hipSuccess || !ptr) {
+    set_error("dnnrtConvBiasActivNoAlloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    return nullptr;
+  }
+  d.scratch = static_cast<unsigned char *>(ptr);
+  d.num_cu = prop.multiProcessorCount;
+  d.ready = true;
+  return &d;
+}
+
 }  // namespace dnnrt
 
 extern "C" {
+
+void *dnnrtConvBiasActivNoAlloc(dnnrtStream_t stream, const void *X, const int64_t *dimX, const void *W,
+                                const int64_t *dimW, const void *B, const int64_t *dimB, int64_t group,
+                                const int64_t *pads, const int64_t *strides, int64_t activMode, void *Y,
+                                int32_t dtype) {
+  if (!dnnrt::fusable_act(activMode))
+    DNNRT_FAIL("dnnrtConvBiasActivNoAlloc: activMode %ld (1 ReLU, 3 clipped ReLU, 5 identity, 6 leaky ReLU)", (long)activMode);
+  if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
+    DNNRT_FAIL("dnnrtConvBiasActivNoAlloc: bias must hold K values");
+  int dev = 0;
+  const dnnrt::NoAllocDevice *d = dnnrt::noalloc_device(dev);
+  if (!d) return nullptr;
+  // A handle on the stack: the defaults of dnnrtCreate, and the static scratch where a handle has its own.
+  dnnrtContext ctx{};
+  ctx.stream = (hipStream_t)stream;
+  ctx.format = DNNRT_NCHW;
+  ctx.filter_layout = DNNRT_FILTER_KCRS;
+  ctx.act_coef = 0.f;
+  ctx.device = dev;
+  ctx.num_cu = d->num_cu;
+  ctx.splitk_partials = reinterpret_cast<float *>(d->scratch);
+  ctx.splitk_counters = reinterpret_cast<unsigned *>(d->scratch + dnnrt::NOALLOC_PARTIAL_BYTES);
+  ctx.splitk_partial_bytes = dnnrt::NOALLOC_PARTIAL_BYTES;
+  ctx.splitk_max_tiles = dnnrt::NOALLOC_MAX_TILES;
+  ctx.splitk_shared = true;
+  ctx.f16_tile = 0;
+  return dnnrt::conv_dispatch("dnnrtConvBiasActivNoAlloc", &ctx, X, dimX, W, dimW, B, nullptr, group, pads, strides,
+                              (int)activMode, Y, dtype);
+}
 
 void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
                 const int64_t *dimW, void *workspace, int64_t workspaceBytes, int64_t algo,

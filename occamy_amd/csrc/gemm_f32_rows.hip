@@ -226,9 +226,10 @@ bool launch_gemm_f32_rows(const dnnrtContext *ctx, const IgemmArgs &a, bool &lau
   int64_t splits = tiles >= want ? 1 : (want + tiles / 2) / tiles;
   splits = splits > 16 ? 16 : splits;
   splits = splits > nchunks ? nchunks : splits;
-  while (splits > 1 && (tiles * 4 * splits * 4096 > SPLITK_PARTIAL_BYTES || tiles * 4 > SPLITK_MAX_TILES)) splits--;
+  while (splits > 1 && (tiles * 4 * splits * 4096 > ctx->splitk_partial_bytes || tiles * 4 > ctx->splitk_max_tiles)) splits--;
   const int cps = (int)ceil_div(nchunks, splits);
   splits = ceil_div(nchunks, cps);  // no empty split: every arrival carries a partial tile
+  if (ctx->splitk_shared && splits > 1) clear_split_counters(ctx, (int)tiles * 4);
   hipLaunchKernelGGL(gemm_f32_rows_kernel, dim3((unsigned)tiles, (unsigned)splits, 1), dim3(512), 0, ctx->stream, a, cps,
                      ctx->splitk_partials, ctx->splitk_counters);
   hipError_t e = hipGetLastError();

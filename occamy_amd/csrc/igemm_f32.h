@@ -61,6 +61,9 @@ bool launch_igemm_f32_direct(const dnnrtContext *ctx, const IgemmArgs &a, int rs
 bool launch_conv3x3_f32_tiled(const dnnrtContext *ctx, const IgemmArgs &a, int layout, bool &launched);
 // Row-major products with a few hundred rows (gemm_f32_rows.hip); `launched` says whether it applied.
 bool launch_gemm_f32_rows(const dnnrtContext *ctx, const IgemmArgs &a, bool &launched);
+// Zeroes the first n arrival counters of the context's split-reduction scratch on its stream.  For scratch that
+// is shared beyond one handle (splitk_shared): whoever used the counters last may have died half-way.
+void clear_split_counters(const dnnrtContext *ctx, int n);
 // 3x3 / 1x1 specialisations of the above (igemm_f32_small.hip); `launched` says whether one applied.
 bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout, bool &launched);
 

@@ -365,6 +365,16 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   reduce_and_store<KS, false>(a, acc, bias_r, bias_c, red, wave, lane, m0, img, pq, col_ok, z, (unsigned)(z * tiles + tile_id), partials, counters);
 }
 
+// A fill kernel rather than hipMemsetAsync: a caller may be recording the stream into a graph.
+__global__ void zero_counters_kernel(unsigned *counters, int n) {
+  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+  if (i < n) counters[i] = 0u;
+}
+
+void clear_split_counters(const dnnrtContext *ctx, int n) {
+  hipLaunchKernelGGL(zero_counters_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, ctx->stream, ctx->splitk_counters, n);
+}
+
 // Returns true if one of the specialised kernels took the problem.
 bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsmode, int layout, bool &launched) {
   launched = false;
@@ -390,10 +400,19 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
   // over a reduction of thousands): split the reduction over workgroups too.
   int splits = 1;
   while (splits < 16 && (int64_t)tiles * a.Z * splits * 2 <= ctx->num_cu &&
-         ceil_div(red_len, ks * splits * 2) >= min_slice &&
-         (int64_t)tiles * a.Z * splits * 2 * 4096 <= SPLITK_PARTIAL_BYTES && (int64_t)tiles * a.Z <= SPLITK_MAX_TILES)
+         ceil_div(red_len, ks * splits * 2) >= min_slice) {
+    if ((int64_t)tiles * a.Z * splits * 2 * 4096 > ctx->splitk_partial_bytes || (int64_t)tiles * a.Z > ctx->splitk_max_tiles) {
+      if (!ctx->splitk_shared) break;  // a handle's own scratch: a shallower split is as good
+      set_error("igemm_f32(small): the split reduction of this problem needs %lld bytes of scratch and %lld counters, "
+                "the static scratch holds %lld and %d",
+                (long long)tiles * a.Z * splits * 2 * 4096, (long long)tiles * a.Z, (long long)ctx->splitk_partial_bytes,
+                ctx->splitk_max_tiles);
+      return false;
+    }
     splits *= 2;
+  }
   dim3 grid((unsigned)(ceil_div(tiles, 8) * 8), splits, a.Z);
+  if (ctx->splitk_shared && splits > 1) clear_split_counters(ctx, tiles * a.Z);
 #define LAUNCH_KS2(KERNEL, AMC_, ARG)                                                                  \
   switch (ks) {                                                                                          \
     case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break;  \

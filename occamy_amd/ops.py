@@ -103,6 +103,13 @@ class Ops:
                                                      dims(strides), activ, Y, dtype),
                          "dnnrtConvBiasActiv")
 
+    def conv_bias_activ_no_alloc(self, stream, X, dimX, W, dimW, B, pads, strides, activ, Y, group=1, dtype=_abi.F32):
+        """dnnrtConvBiasActivNoAlloc: takes a stream (may be None: the default stream), not this object's handle."""
+        dimB = [1, dimW[0], 1, 1]
+        return self._ret(self.lib.dnnrtConvBiasActivNoAlloc(stream, X, dims(dimX), W, dims(dimW), B, dims(dimB), group,
+                                                            dims(pads), dims(strides), activ, Y, dtype),
+                         "dnnrtConvBiasActivNoAlloc")
+
     def conv_bias_add_activ(self, X, dimX, W, dimW, B, Z, pads, strides, activ, Y, group=1, dtype=_abi.F32):
         dimB = [1, dimW[0], 1, 1]
         return self._ret(self.lib.dnnrtConvBiasAddActiv(self.handle, X, dims(dimX), W, dims(dimW), B,

@@ -320,6 +320,16 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
     FAIL("convBiasActiv: activMode %ld", (long)act);
   return conv_entry(X, dX, W, dW, B, group, pads, strides, act, Y, dtype);
 }
+/* No reference counterpart: dnnrtConvBiasActiv on the defaults of a fresh
+ * handle (the GPU library's variant differs only in where its scratch lives). */
+void *dnnrtConvBiasActivNoAlloc(dnnrtStream_t stream, const void *X, const int64_t *dX,
+                                const void *W, const int64_t *dW, const void *B,
+                                const int64_t *dB, int64_t group, const int64_t *pads,
+                                const int64_t *strides, int64_t act, void *Y, int32_t dtype) {
+  (void)stream;
+  struct dnnrtContext fresh = {DNNRT_NCHW, 0.f};
+  return dnnrtConvBiasActiv(&fresh, X, dX, W, dW, B, dB, NULL, 0, 0, group, pads, strides, act, Y, dtype);
+}
 /* No reference wrapper of its own: the reference runs this as three calls,
  * conv+bias (CUDNNConvBiasReluFunc.cpp, identity), cudnnAddTensor
  * (CUDNNAddFunc.cpp) and cudnnActivationForward (CUDNNActiveFunc.cpp), each
