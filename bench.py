@@ -6,14 +6,20 @@ already resident in HBM: input copy into its pool slot (device to device),
 every kernel of the compiled DNN program (replayed from a captured graph),
 output copy to the caller's device buffer.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--layers FILE]
 
-workloads: resnet50_fp32_bs1 (default), resnet50_fp16_bs64, mobilenet_v2_fp32_bs1,
-bert_base_fp32_seq128, single_conv_fp32
+The default workload, "resnet50", is the metric's two halves in one line: the
+headline record (value, roofline, cpu_baseline ...) is ResNet-50 fp16 batch 64
+and the key "fp32_bs1" holds the same record for ResNet-50 fp32 batch 1.
+Other workloads: resnet50_fp32_bs1, resnet50_fp16_bs64, mobilenet_v2_fp32_bs1,
+bert_base_fp32_seq128, single_conv_fp32, alexnet_fp32_bs1, yolo_v1_fp32_bs2,
+srgan_fp32_96x96.  --layers writes a per-operation table (algorithmic FLOP and
+bytes, the roofline bound, measured time) of the headline workload to FILE.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -23,14 +29,20 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
+RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention")
 
 
-def build_workload(name):
+def build_workload(name, batch=None):
+    """((graph, inputs), compile flags, batch, unit, dtype); `batch` overrides the workload's own batch size."""
     from occamy_amd import models
     if name == "resnet50_fp32_bs1":
-        return models.resnet50(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True), 1, "img/s", "f32"
+        b = batch or 1
+        return models.resnet50(b, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True), b, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
-        return models.resnet50(64, np.float16, seed=5), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True), 64, "img/s", "f16"
+        b = batch or 64
+        return models.resnet50(b, np.float16, seed=5), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True), b, "img/s", "f16"
+    if batch is not None:
+        raise SystemExit(f"{name}: no batch override")
     if name == "mobilenet_v2_fp32_bs1":
         return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
@@ -60,14 +72,209 @@ def recorded_traffic(workload, cls):
     return None
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def measure(name, steps, warmup):
+    """One workload on the GPU: K graph-replayed steps timed as a whole (value), individually timed steps (median,
+    P90), per-class and per-operation device times, and the reference's per-inference semantics."""
+    import torch
+    from occamy_amd import compiler
+    (graph, inputs), flags, batch, unit, dtype = build_workload(name)
+    prog = graph.compile(**flags)
+    sess = prog.session(compiler.MODE_RESIDENT)
+    dev_in = [torch.from_numpy(a).cuda() for a in inputs]
+    dev_out = [torch.empty(s, dtype=torch.from_numpy(np.empty(0, d)).dtype, device="cuda") for s, d in prog.output_info()]
+    ip, op = [t.data_ptr() for t in dev_in], [t.data_ptr() for t in dev_out]
+    torch.cuda.synchronize()
+    for _ in range(max(warmup, 1)):
+        sess.run_device(ip, op, use_graph=True)
+    sess.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sess.run_device(ip, op, use_graph=True)
+    sess.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    # the distribution: the same step, each one waited for (what a caller that needs every answer sees)
+    lat = []
+    for _ in range(max(20, min(steps, 100))):
+        t1 = time.perf_counter()
+        sess.run_device(ip, op, use_graph=True)
+        sess.sync()
+        lat.append(1e3 * (time.perf_counter() - t1))
+    res = dict(name=name, batch=batch, unit=unit, dtype=dtype, ms_per_step=1e3 * dt / steps,
+               value=batch * steps / dt, pool_bytes=prog.pool_bytes, weights_bytes=sess.weights_bytes,
+               kernels_per_step=prog.num_ops(compute_only=True), flags=flags,
+               latency_ms={"median": float(np.median(lat)), "p90": float(np.percentile(lat, 90)), "samples": len(lat),
+                           "what": "one step at a time, each waited for on the host"})
+    # device timestamps on the session's own stream, eager launches: one pair per operation
+    # class around that class's launches issued back to back (a timestamp between two kernels
+    # of a few microseconds costs about as much as the kernels themselves)
+    ops = prog.compute_ops()
+    acc = np.zeros(len(ops))
+    reps = 20
+    sess.profile(ip, on_device=True, by_class=True)
+    for _ in range(reps):
+        acc += np.array(sess.profile(ip, on_device=True, by_class=True))
+    acc /= reps
+    by_class = {}
+    for (mn, cls, fl, by), ms in zip(ops, acc):
+        c = by_class.setdefault(cls, dict(launches=0, flops=0.0, bytes=0.0, ms=0.0))
+        c["launches"] += 1
+        c["flops"] += fl
+        c["bytes"] += by
+        c["ms"] += float(ms)
+    res["by_class"] = by_class
+    # ... and one pair per operation, in program order (each kernel finds the caches as the network leaves them)
+    per_op = np.zeros(len(ops))
+    sess.profile(ip, on_device=True)
+    for _ in range(reps):
+        per_op += np.array(sess.profile(ip, on_device=True))
+    res["per_op_ms"] = list(per_op / reps)
+    res["ops"] = ops
+    res["text"] = prog.text
+    # the reference's per-inference semantics: pool alloc, all weights H2D, kernels, D2H, sync, pool free
+    # (compiled with the reference's own flags: no residual fusion)
+    (ref_graph, _), _, _, _, _ = build_workload(name)  # a graph compiles once; the builders are seeded
+    ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k not in RESIDENT_ONLY_FLAGS})
+    res["pool_bytes_reference_flags"] = ref_prog.pool_bytes
+    so = ref_prog.session(compiler.MODE_OCCAMY)
+    so.run(*inputs)
+    n = max(3, min(20, steps // 10))
+    t0 = time.perf_counter()
+    for _ in range(n):
+        so.run(*inputs)
+    res["occamy_semantics_value"] = batch * n / (time.perf_counter() - t0)
+    so.close()
+    sess.close()
+    return res
+
+
+def roofline_of(res):
+    """The roofline record of the workload's dominant kernel class (by measured time)."""
+    cls, c = max(res["by_class"].items(), key=lambda kv: kv[1]["ms"])
+    if cls in ("conv_dense", "gemm", "matmul"):
+        peak = PEAK["mfma_f16" if res["dtype"] == "f16" else "mfma_f32"]
+        achieved = c["flops"] / (c["ms"] * 1e-3)
+        roof = dict(bound="mfma", achieved=achieved / 1e12, peak=peak / 1e12, unit="TFLOP/s", frac=achieved / peak)
+    else:
+        achieved = c["bytes"] / (c["ms"] * 1e-3)
+        roof = dict(bound="hbm", achieved=achieved / 1e9, peak=PEAK["hbm"] / 1e9, unit="GB/s", frac=achieved / PEAK["hbm"])
+    roof.update(kernel=cls, launches_per_step=c["launches"], avg_launch_us=1e3 * c["ms"] / c["launches"],
+                traffic=recorded_traffic(res["name"], cls))
+    return roof
+
+
+def cpu_leg(name, threads, seconds, batch=None):
+    """The same DNN program through the oracle build of the same ABI on `threads` host threads; images (sequences)
+    per second over a bounded number of inferences."""
+    import ctypes
+    from occamy_amd import compiler
+    oracle_path = os.path.join(ROOT, "oracle", "libdnnrt_oracle.so")
+    ctypes.CDLL(oracle_path).dnnrtOracleSetThreads(threads)
+    (graph, inputs), flags, b, unit, _ = build_workload(name, batch)
+    # the oracle keeps the reference's N,C,H,W layout: same graph, same flags otherwise
+    prog = graph.compile(**{k: v for k, v in flags.items() if k != "channels_last"})
+    so = prog.session(compiler.MODE_RESIDENT, runtime_library=oracle_path)
+    t0 = time.perf_counter()
+    so.run(*inputs)
+    first = time.perf_counter() - t0
+    n = int(max(1, min(50, (seconds - first) / max(first, 1e-3))))
+    times = [first] if first > seconds / 3 else []  # a long first inference is itself a sample
+    for _ in range(n):
+        t0 = time.perf_counter()
+        so.run(*inputs)
+        times.append(time.perf_counter() - t0)
+    so.close()
+    return b / float(np.median(times)), len(times), b
+
+
+def cpu_baseline(res, seconds):
+    name, batch = res["name"], res["batch"]
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    threads = max(1, min(threads, os.cpu_count() or 1))
+    value, n, _ = cpu_leg(name, threads, seconds)
+    small = None if batch <= 2 else 2  # one thread gets a batch it finishes in seconds (same per-image work)
+    v1, n1, b1 = cpu_leg(name, 1, seconds / 2, small)
+    return dict(value=value, unit=res["unit"], cores=threads, kind="port", cpu=cpu_model(), host_cpus=os.cpu_count(),
+                sample=f"median of {n} inference(s) of {name} (batch {batch}) through the in-repo CPU oracle (plain C, "
+                       f"double accumulation) on {threads} OpenMP threads = this job's share of the host "
+                       f"(OMP_NUM_THREADS); the reference's onnx-mlir CPU lowering is not available",
+                one_thread=dict(value=v1, unit=res["unit"], cores=1,
+                                sample=f"median of {n1} inference(s) of the same network at batch {b1} on one thread"))
+
+
+def record(res, steps, warmup, cpu_seconds):
+    """The JSON record of one measured workload (the keys of the headline line)."""
+    return {
+        "value": res["value"], "unit": res["unit"], "steps": steps, "warmup": warmup, "ms_per_step": res["ms_per_step"],
+        "latency_ms": res["latency_ms"], "dtype": res["dtype"], "data": "synthetic",
+        "config": {"workload": res["name"], "batch": res["batch"],
+                   "fusion": ", ".join(k for k, v in res["flags"].items() if v and (k.startswith("fus") or k == "recompose")),
+                   "mode": "weights and input resident in HBM, kernels replayed from a captured graph",
+                   "kernels_per_step": res["kernels_per_step"]},
+        "roofline": roofline_of(res),
+        "cpu_baseline": cpu_baseline(res, cpu_seconds) if cpu_seconds > 0 else None,
+        "pool_bytes": res["pool_bytes"], "pool_bytes_reference_flags": res["pool_bytes_reference_flags"],
+        "weights_bytes": res["weights_bytes"],
+        "occamy_semantics": {"value": res["occamy_semantics_value"], "unit": res["unit"],
+                             "what": "reference flags (no residual fusion); per inference: pool hipMalloc, every weight H2D into its pool slot, kernels, D2H, sync, pool free"},
+        "by_class": {k: {"launches": v["launches"], "ms": round(v["ms"], 4),
+                         "TFLOP/s": round(v["flops"] / max(v["ms"], 1e-9) / 1e9, 3),
+                         "GB/s": round(v["bytes"] / max(v["ms"], 1e-9) / 1e6, 1)} for k, v in res["by_class"].items()},
+    }
+
+
+def layer_table(res):
+    """Per operation, in program order: algorithmic FLOP and bytes, the time the roofline allows
+    (max of FLOP / MFMA peak and bytes / HBM peak), the measured time, and their ratio."""
+    peak = PEAK["mfma_f16" if res["dtype"] == "f16" else "mfma_f32"]
+    names = {o[0] for o in res["ops"]}
+    lines = [l for l in res["text"].splitlines() if any(f"= {n} " in l for n in names)]
+    out = [f"{res['name']}: per operation, program order.  t_mfma = FLOP / {peak / 1e12:.1f} TFLOP/s, t_hbm = bytes / 8 TB/s,",
+           "bound = the larger; measured = device timestamps around each launch inside the network (a pair of",
+           f"timestamps adds to a kernel of a few microseconds; the graph-replayed step takes {res['ms_per_step'] * 1e3:.0f} us,",
+           f"the measured column sums to {sum(res['per_op_ms']) * 1e3:.0f} us); frac = bound / measured.", "",
+           f"{'#':>3s} {'operation':28s} {'result':22s} {'red.':>5s} {'attrs':28s} {'MFLOP':>9s} {'KB':>9s} {'t_mfma':>7s} {'t_hbm':>7s} "
+           f"{'by':>4s} {'meas_us':>8s} {'frac':>5s} {'TF/s':>7s} {'GB/s':>7s}"]
+    for i, ((mn, cls, fl, by), ms) in enumerate(zip(res["ops"], res["per_op_ms"])):
+        line = lines[i] if len(lines) == len(res["ops"]) else ""
+        shape = re.search(r": \w+(\[[^\]]*\])\s*$", line)
+        attrs = re.search(r"\{([^}]*)\}", line)
+        a = attrs.group(1) if attrs else ""
+        a = re.sub(r"group=1, |activMode=\d+|, $", "", a).strip(", ")
+        n_out = np.prod([int(v) for v in shape.group(1)[1:-1].split(",")]) if shape else 0
+        red = f"{int(round(fl / (2 * n_out)))}" if cls == "conv_dense" and n_out else ""
+        t_m, t_h = fl / peak * 1e6, by / PEAK["hbm"] * 1e6
+        bound = max(t_m, t_h)
+        us = ms * 1e3
+        out.append(f"{i:3d} {mn[4:]:28s} {shape.group(1) if shape else '':22s} {red:>5s} {a[:28]:28s} {fl / 1e6:9.1f} {by / 1e3:9.1f} "
+                   f"{t_m:7.2f} {t_h:7.2f} {'mfma' if t_m >= t_h else 'hbm':>4s} {us:8.2f} {bound / max(us, 1e-9):5.2f} "
+                   f"{fl / max(us, 1e-9) / 1e6:7.1f} {by / max(us, 1e-9) / 1e3:7.1f}")
+    tot_b = sum(max(fl / peak, by / PEAK["hbm"]) for _, _, fl, by in res["ops"]) * 1e6
+    out.append("")
+    out.append(f"sum of bounds {tot_b:.0f} us; sum of measured {sum(res['per_op_ms']) * 1e3:.0f} us")
+    return "\n".join(out) + "\n"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="resnet50_fp32_bs1")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU-baseline leg")
+    ap.add_argument("--workload", default="resnet50")
+    ap.add_argument("--cpu-seconds", type=float, default=24.0, help="budget of the CPU-baseline leg of the headline workload")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--layers", metavar="FILE", help="write the per-operation table of the headline workload to FILE")
     ap.add_argument("--extra", action="store_true", help="also time the other workloads (reported under 'extra')")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only launch the library's plain copy kernel on 256 MiB a few times: the run that the "
@@ -78,7 +285,6 @@ def main():
                          "N GPUs are N independent copies of this run (run with --gpus 1)")
 
     import torch
-    from occamy_amd import compiler
 
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
@@ -97,132 +303,31 @@ def main():
                           "bytes_written_per_launch": 4 * n}))
         return
 
-    def measure(name, steps, warmup, want_profile):
-        (graph, inputs), flags, batch, unit, dtype = build_workload(name)
-        prog = graph.compile(**flags)
-        sess = prog.session(compiler.MODE_RESIDENT)
-        dev_in = [torch.from_numpy(a).cuda() for a in inputs]
-        dev_out = [torch.empty(s, dtype=torch.from_numpy(np.empty(0, d)).dtype, device="cuda") for s, d in prog.output_info()]
-        ip, op = [t.data_ptr() for t in dev_in], [t.data_ptr() for t in dev_out]
-        torch.cuda.synchronize()
-        for _ in range(max(warmup, 1)):
-            sess.run_device(ip, op, use_graph=True)
-        sess.sync()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            sess.run_device(ip, op, use_graph=True)
-        sess.sync()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        res = dict(name=name, batch=batch, unit=unit, dtype=dtype, ms_per_step=1e3 * dt / steps,
-                   value=batch * steps / dt, pool_bytes=prog.pool_bytes, weights_bytes=sess.weights_bytes,
-                   kernels_per_step=prog.num_ops(compute_only=True), flags=flags)
-        if want_profile:
-            # device timestamps on the session's own stream, eager launches: one pair per operation
-            # class around that class's launches issued back to back (a timestamp between two kernels
-            # of a few microseconds costs about as much as the kernels themselves)
-            ops = prog.compute_ops()
-            acc = np.zeros(len(ops))
-            reps = 20
-            sess.profile(ip, on_device=True, by_class=True)
-            for _ in range(reps):
-                acc += np.array(sess.profile(ip, on_device=True, by_class=True))
-            acc /= reps
-            by_class = {}
-            for (mn, cls, fl, by), ms in zip(ops, acc):
-                c = by_class.setdefault(cls, dict(launches=0, flops=0.0, bytes=0.0, ms=0.0))
-                c["launches"] += 1
-                c["flops"] += fl
-                c["bytes"] += by
-                c["ms"] += float(ms)
-            res["by_class"] = by_class
-        # the reference's per-inference semantics: pool alloc, all weights H2D, kernels, D2H, sync, pool free
-        # (compiled with the reference's own flags: no residual fusion)
-        (ref_graph, _), _, _, _, _ = build_workload(name)  # a graph compiles once; the builders are seeded
-        ref_prog = ref_graph.compile(**{k: v for k, v in flags.items() if k not in ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention")})
-        res["pool_bytes_reference_flags"] = ref_prog.pool_bytes
-        so = ref_prog.session(compiler.MODE_OCCAMY)
-        so.run(*inputs)
-        n = max(3, min(20, steps // 10))
-        t0 = time.perf_counter()
-        for _ in range(n):
-            so.run(*inputs)
-        res["occamy_semantics_value"] = batch * n / (time.perf_counter() - t0)
-        so.close()
-        sess.close()
-        return res, (graph, inputs, prog)
-
-    main_res, (graph, inputs, prog) = measure(args.workload, args.steps, args.warmup, True)
-
-    # dominant kernel class by measured time
-    cls, c = max(main_res["by_class"].items(), key=lambda kv: kv[1]["ms"])
-    mfma_bound = cls in ("conv_dense", "gemm", "matmul")
-    if mfma_bound:
-        peak = PEAK["mfma_f16" if main_res["dtype"] == "f16" else "mfma_f32"]
-        achieved = c["flops"] / (c["ms"] * 1e-3)
-        roof = dict(bound="mfma", achieved=achieved / 1e12, peak=peak / 1e12, unit="TFLOP/s", frac=achieved / peak)
-    else:
-        achieved = c["bytes"] / (c["ms"] * 1e-3)
-        roof = dict(bound="hbm", achieved=achieved / 1e9, peak=PEAK["hbm"] / 1e9, unit="GB/s", frac=achieved / PEAK["hbm"])
-    roof.update(kernel=cls, launches_per_step=c["launches"], avg_launch_us=1e3 * c["ms"] / c["launches"],
-                traffic=recorded_traffic(args.workload, cls))
-
-    cpu = None
-    if not args.no_cpu:
-        # CPU baseline: the oracle build of the same ABI runs the same program on the host cores.
-        import ctypes
-        oracle_path = os.path.join(ROOT, "oracle", "libdnnrt_oracle.so")
-        olib = ctypes.CDLL(oracle_path)
-        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-        olib.dnnrtOracleSetThreads(cores)
-        cpu_prog = prog
-        _, wl_flags, _, _, _ = build_workload(args.workload)
-        if wl_flags.get("channels_last"):
-            # the oracle keeps the reference's N,C,H,W layout: same graph, same flags otherwise
-            (cpu_graph, _), _, _, _, _ = build_workload(args.workload)
-            cpu_prog = cpu_graph.compile(**{k: v for k, v in wl_flags.items() if k != "channels_last"})
-        so = cpu_prog.session(compiler.MODE_RESIDENT, runtime_library=oracle_path)
-        t0 = time.perf_counter()
-        so.run(*inputs)
-        first = time.perf_counter() - t0
-        n = int(max(1, min(50, args.cpu_seconds / max(first, 1e-3))))
-        t0 = time.perf_counter()
-        for _ in range(n):
-            so.run(*inputs)
-        dt = (time.perf_counter() - t0) / n
-        so.close()
-        cpu = dict(value=main_res["batch"] / dt, unit=main_res["unit"], cores=cores, kind="port",
-                   sample=f"{n} inference(s) of {args.workload} (batch {main_res['batch']}) through the in-repo CPU oracle, "
-                          f"OpenMP {cores} threads; the reference's onnx-mlir CPU lowering is not available")
-
-    line = {
-        "metric": "ResNet-50 img/s at bs1/bs64 on 1 GPU" if args.workload.startswith("resnet50") else f"{args.workload} throughput",
-        "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": main_res["dtype"], "data": "synthetic",
-        "config": {"workload": args.workload, "batch": main_res["batch"],
-                   "fusion": ", ".join(k for k, v in main_res["flags"].items() if v and (k.startswith("fus") or k == "recompose")),
-                   "mode": "weights and input resident in HBM, kernels replayed from a captured graph",
-                   "kernels_per_step": main_res["kernels_per_step"]},
-        "roofline": roof,
-        "cpu_baseline": cpu,
-        "pool_bytes": main_res["pool_bytes"], "pool_bytes_reference_flags": main_res["pool_bytes_reference_flags"],
-        "weights_bytes": main_res["weights_bytes"],
-        "occamy_semantics": {"value": main_res["occamy_semantics_value"], "unit": main_res["unit"],
-                             "what": "reference flags (no residual fusion); per inference: pool hipMalloc, every weight H2D into its pool slot, kernels, D2H, sync, pool free"},
-        "by_class": {k: {"launches": v["launches"], "ms": round(v["ms"], 4),
-                         "TFLOP/s": round(v["flops"] / max(v["ms"], 1e-9) / 1e9, 3),
-                         "GB/s": round(v["bytes"] / max(v["ms"], 1e-9) / 1e6, 1)} for k, v in main_res["by_class"].items()},
-    }
+    both = args.workload == "resnet50"
+    head_name = "resnet50_fp16_bs64" if both else args.workload
+    cpu_seconds = 0.0 if args.no_cpu else args.cpu_seconds
+    head = measure(head_name, args.steps, args.warmup)
+    rec = record(head, args.steps, args.warmup, cpu_seconds)
+    if args.layers:
+        with open(args.layers, "w") as f:
+            f.write(layer_table(head))
+    line = {"metric": "ResNet-50 img/s at bs1/bs64 on 1 GPU" if head_name.startswith("resnet50") else f"{head_name} throughput",
+            "value": rec.pop("value"), "unit": rec.pop("unit"), "n_gpus": 1, "steps": rec.pop("steps"), "warmup": rec.pop("warmup"),
+            "ms_per_step": rec.pop("ms_per_step"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None}
+    line.update(rec)
+    if both:
+        line["headline"] = "resnet50_fp16_bs64 (the half of the metric with a stated target); the fp32 batch-1 half is under fp32_bs1 with the same keys"
+        # batch 1: more steps for the same wall time (a step is under half a millisecond)
+        small = measure("resnet50_fp32_bs1", args.steps, args.warmup)
+        line["fp32_bs1"] = record(small, args.steps, args.warmup, cpu_seconds / 2)
     if args.extra:
         extra = {}
-        for name in ["resnet50_fp16_bs64", "mobilenet_v2_fp32_bs1", "bert_base_fp32_seq128", "single_conv_fp32",
+        for name in ["resnet50_fp32_bs1", "resnet50_fp16_bs64", "mobilenet_v2_fp32_bs1", "bert_base_fp32_seq128", "single_conv_fp32",
                      "alexnet_fp32_bs1", "yolo_v1_fp32_bs2", "srgan_fp32_96x96"]:
-            if name == args.workload:
+            if name == head_name or (both and name == "resnet50_fp32_bs1"):
                 continue
             try:
-                r, _ = measure(name, max(20, args.steps // 4), max(5, args.warmup // 2), True)
+                r = measure(name, max(20, args.steps // 4), max(5, args.warmup // 2))
                 extra[name] = {k: r[k] for k in ("value", "unit", "ms_per_step", "pool_bytes", "weights_bytes", "occamy_semantics_value")}
                 extra[name]["by_class"] = {k: {"launches": v["launches"], "ms": round(v["ms"], 4)} for k, v in r["by_class"].items()}
             except Exception as e:  # a workload that cannot run yet is reported, not hidden
