@@ -108,6 +108,9 @@ int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *o
  * wait (dnncSessionSync does); use_graph: replay the kernels from a captured graph */
 int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
 int32_t dnncSessionSync(dnncSession *s);
+/* Tuning and tests: dnnrtSetConvTile on the session's handle (0 = automatic choice); a captured
+ * graph is dropped and recorded again by the next replayed run. */
+int32_t dnncSessionSetConvTile(dnncSession *s, int32_t tile);
 /* resident mode: one eager pass with device timestamps around every compute
  * operation; ms[i] belongs to dnncProgramComputeOp(i).  Returns the count.
  * on_device bit 0: the inputs are device buffers; bit 1: one pair of

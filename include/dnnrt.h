@@ -113,7 +113,9 @@ int32_t dnnrtSetFilterLayout(dnnrtHandle_t handle, int32_t layout);
  * convolution of the handle use that variant (and switches the few-pixel 1x1
  * kernel off), 0 restores the automatic choice.  A variant that cannot run a
  * given problem makes that convolution call fail with an error, never
- * fall back. */
+ * fall back.  -id states a preference instead: the variant runs the problems
+ * it can run, every other convolution gets the automatic choice (for timing
+ * a variant inside a whole network). */
 int32_t dnnrtListConvTiles(int32_t *ids, int32_t capacity);
 int32_t dnnrtSetConvTile(dnnrtHandle_t handle, int32_t tile);
 /* The coefficient of the activation modes that take one: the ceiling of

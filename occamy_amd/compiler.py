@@ -76,6 +76,7 @@ def lib():
         "dnncSessionRun": (C.c_int32, [P, C.POINTER(P), C.POINTER(P)]),
         "dnncSessionRunResident": (C.c_int32, [P, C.POINTER(P), C.POINTER(P), C.c_int32, C.c_int32]),
         "dnncSessionSync": (C.c_int32, [P]),
+        "dnncSessionSetConvTile": (C.c_int32, [P, C.c_int32]),
         "dnncSessionWeightsBytes": (C.c_int64, [P]),
         "dnncSessionLastPoolBytes": (C.c_int64, [P]),
     }
@@ -310,6 +311,11 @@ class Session:
         if lib().dnncSessionProfile(self._s, ip, int(on_device) | (2 if by_class else 0), ms, n) < 0:
             raise RuntimeError("profile: " + _err())
         return list(ms[:n])
+
+    def set_conv_tile(self, tile):
+        """Force one fp16 convolution variant (dnnrtListConvTiles) for every following run; 0 = automatic."""
+        if lib().dnncSessionSetConvTile(self._s, tile):
+            raise RuntimeError("set_conv_tile: " + _err())
 
     def sync(self):
         if lib().dnncSessionSync(self._s):

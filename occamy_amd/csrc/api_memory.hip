@@ -122,7 +122,7 @@ int32_t dnnrtListConvTiles(int32_t *ids, int32_t capacity) {
 int32_t dnnrtSetConvTile(dnnrtHandle_t handle, int32_t tile) {
   if (!handle) { set_error("dnnrtSetConvTile: null handle"); return 1; }
   bool known = tile == 0;
-  for (const int *t = dnnrt::F16_TILE_IDS; *t; t++) known = known || *t == tile;
+  for (const int *t = dnnrt::F16_TILE_IDS; *t; t++) known = known || *t == tile || *t == -tile;
   if (!known) { set_error("dnnrtSetConvTile: no fp16 convolution variant %d in this build", tile); return 1; }
   handle->f16_tile = tile;
   return 0;

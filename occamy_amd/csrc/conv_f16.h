@@ -13,6 +13,7 @@ struct ConvF16Args {
   float act_coef;  // ceiling / slope of the last two
   int format;  // physical layout of X and Y (DNNRT_NCHW / NHWC / NCHW_TO_NHWC)
   unsigned magic_pq, magic_q;  // filled in by the launcher: ceil(2^32 / (P*Q)), ceil(2^32 / Q)
+  unsigned magic_pw, magic_hp;  // (conv_f16_patch.hip) ceil(2^32 / (W + 2)), ceil(2^32 / (H + 2))
 };
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a);
@@ -26,5 +27,14 @@ bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &l
 // that file's tile ids, `a` must satisfy dma_conv_applies and carry the division constants.
 bool dma_conv_applies(const ConvF16Args &a);
 bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int variant);
+
+// 3x3 stride-1 pad-1 channels-last convolutions over at least 128 channels with the input patch kept in LDS
+// (conv_f16_patch.hip): `variant` is one of that file's tile ids, `a` must satisfy patch_conv_applies and carry the
+// division constants of P * Q and Q.  patch_conv_capacity: the smallest compiled patch capacity that holds this
+// problem's patches at tile width bn, or 0.
+bool patch_conv_applies(const ConvF16Args &a);
+int patch_conv_capacity(const ConvF16Args &a, int bn);
+bool patch_variant_fits(const ConvF16Args &a, int variant);  // the variant's patch capacity holds this problem's patches
+bool launch_conv_f16_patch(const dnnrtContext *ctx, const ConvF16Args &a, int variant);
 
 }  // namespace dnnrt

@@ -552,24 +552,53 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     // walking an XCD's run of tiles pixel tiles first instead of k_out tiles
     // first, so that an XCD touches a slice of a large filter only, changed
     // nothing on the 7x7 layers).
-    const int tile_sel = ctx->f16_tile;  // 0 = automatic; otherwise forced (tuning and tests)
+    // 0 = automatic; > 0 forced (tuning and tests); < 0: that variant where it can run the problem, else automatic
+    const int tile_sel = ctx->f16_tile;
     int sel = tile_sel;
+    if (sel < 0) {
+      const int want = -sel, steps = a.R * a.S * (a.C / BKF);
+      bool can = true;
+      if ((want >= 31 && want <= 40) || (want >= 60 && want <= 69)) can = dma_conv_applies(am);
+      else if (want >= 41 && want <= 59) can = patch_conv_applies(am) && patch_variant_fits(am, want);
+      else if (want == 18) can = steps <= 4;
+      else if (want == 17) can = steps == 1 || steps == 2 || steps == 4;
+      sel = can ? want : 0;
+    }
     if (sel == 0) {
       const int nk = a.R * a.S * (a.C / BKF);
       const int64_t t128 = tiles_of(128, 128), cus = ctx->num_cu;
-      if (nk <= 4) sel = 18;  // up to four steps (1x1 over up to 256 channels): the single-stage 64x64 variant
+      const bool dma_ok = dma_conv_applies(am);
+      const int patch_cap = patch_conv_applies(am) ? patch_conv_capacity(am, 128) : 0;
+      const bool one_per_cu = 5 * t128 >= 3 * cus && 4 * t128 < 5 * cus, fewer = 5 * t128 < 3 * cus;
+      // 3x3 stride-1 layers with at most about one 128x128 tile per CU (14x14 and 7x7 images at batch 64): the
+      // input patch stays in LDS (inside the network 33 -> 24 us on 256 -> 256 at 14x14, 41 -> 27 us on 512 -> 512
+      // at 7x7, where 64-row tiles give twice the workgroups); with more tiles per CU the im2col tiles are as fast
+      // Inside a network the filters come from HBM (activations pass through the caches in between), so the
+      // variants that keep three (128-row tiles) or six (64-row tiles) filter steps in flight are the ones
+      // chosen: 27 -> 25 us and 36 -> 26 us against two steps in flight.
+      if (patch_cap && one_per_cu) sel = patch_cap == 256 ? 48 : 52;
+      else if (patch_cap && fewer) sel = patch_cap == 256 ? 47 : 49;
+      else if (nk <= 4) sel = 18;  // up to four steps (1x1 over up to 256 channels): the single-stage 64x64 variant
                               // (27 vs 34 us on 64 -> 256 at 56x56, 22.6 vs 26.6 on 128 -> 512 at 28x28, 18.3 vs 21.7 on 256 -> 1024 at 14x14)
       else if (a.K <= 64) sel = 4;
       else if (4 * t128 >= 5 * cus) sel = 3;
-      else if (5 * t128 >= 3 * cus) sel = 12;
-      else sel = 4;  // fewer 128x128 tiles than that (7x7 layers at batch 64): 64x64, as many workgroups in flight as possible.
-                     // The eight-wavefront 128x64 tile (11) is ahead when the launch is repeated on warm caches
-                     // (3x3 512 -> 512: 32.5 vs 35.3 us) and behind inside the network, where the filter comes from
-                     // HBM (43.3 vs 38.2 us; 1x1 2048 -> 512: 21.7 vs 19.3 us)
+      else if (one_per_cu) sel = dma_ok ? 33 : 12;  // operands straight into a four-stage LDS ring, two steps in flight
+                                                    // (inside the network 37 -> 30 us on the strided 3x3 256 -> 256,
+                                                    // 20 -> 18 us on 1x1 1024 -> 256 at 14x14)
+      else sel = dma_ok && nk >= 8 ? 62 : 4;  // fewer 128x128 tiles than that (7x7 layers at batch 64): 64-row tiles with a six-stage
+                     // ring, four steps of the filter in flight (strided 3x3 512 -> 512: 37.5 -> 32 us inside the
+                     // network, 1x1 2048 -> 512: 21 -> 18.7 us); short reductions keep the 64x64 tiles
     }
-    if (sel >= 31 && sel <= 39) {
+    if ((sel >= 31 && sel <= 40) || (sel >= 60 && sel <= 69)) {
       if (!dma_conv_applies(am)) { set_error("conv(fp16): tile %d needs tensors below 2 GiB", sel); return false; }
       if (!launch_conv_f16_dma(ctx, am, sel)) return false;
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
+      return true;
+    }
+    if (sel >= 41 && sel <= 59) {
+      if (!patch_conv_applies(am)) { set_error("conv(fp16): tile %d is for 3x3 stride-1 pad-1 layers over 128 channels or more", sel); return false; }
+      if (!launch_conv_f16_patch(ctx, am, sel)) return false;
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
       return true;

@@ -20,9 +20,10 @@
 // padded chunk (none without padding: the tap offset rides in the scalar
 // offset of the instruction).
 //
-// Pipeline: a ring of NS LDS stages, the loads of step i + NS - 1 issued right
-// after the barrier of step i, one barrier per step, waits by exact count
-// (vmcnt) so that only the step about to be read has to have landed.
+// Pipeline: a ring of NS LDS stages, NS - 2 steps in flight beyond the one
+// being computed, one barrier per step, waits by exact count (vmcnt) so that
+// only the step about to be read has to have landed; within a step, fragment
+// reads, MFMA groups and the next loads alternate in a pinned order.
 #include "conv_f16.h"
 
 #include <type_traits>
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
   constexpr int A_L = BM / 8 / NW, B_L = BN / 8 / NW;  // loads (8 rows each) per wavefront and step
   constexpr int L = A_L + B_L;
   static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && TM >= 1 && TN >= 1, "tile does not divide over the wavefronts");
-  static_assert(NS >= 2 && (NS - 2) * L < 64, "ring depth");
+  static_assert(NS >= 3, "ring depth");
   constexpr int STAGE = (BM + BN) * 128;  // bytes
   constexpr int CROW = BM + 8;            // halfs per row of the output staging tile
   static_assert(BN * CROW * 2 <= NS * STAGE, "the output tile is staged in the operand ring");
@@ -134,24 +135,32 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
   // cursor of the next step to load (all scalar)
   int l_r = 0, l_s = 0, l_c0 = 0, l_stage = 0, l_k = 0;
 
-  auto issue_step = [&]() {
+  // The loads of one step, in three parts so that they can be issued between the MFMA groups of another step
+  // (a wavefront that issues them all at once sits in the memory pipeline's queue while its MFMA queue drains).
+  auto issue_loads = [&](auto lo_c, auto hi_c) {
+    constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
     char *As = smem + l_stage * STAGE, *Bs = As + BM * 128;
     const int tap = l_r * a.S + l_s;
     const int x_tap = 2 * ((l_r * a.W + l_s) * a.C);  // bytes from tap (0, 0) to this tap
 #pragma unroll
-    for (int i = 0; i < A_L; i++)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_ptr)(As + 1024 * (wave + i * NW)), 16, a_off[i], 2 * l_k, 0, 0);
-#pragma unroll
-    for (int i = 0; i < B_L; i++) {
-      if (MASKED) {
-        // bit 31 set when the tap is outside (or the address is negative): out of range, zeros
-        const unsigned voff = (unsigned)(b_base[i] + x_tap) | ((b_out[i] >> tap) << 31);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr)(Bs + 1024 * (wave + i * NW)), 16, voff, 2 * l_c0, 0, 0);
+    for (int n = LO; n < HI; n++) {
+      if (n < A_L) {
+        const int i = n;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_ptr)(As + 1024 * (wave + i * NW)), 16, a_off[i], 2 * l_k, 0, 0);
       } else {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr)(Bs + 1024 * (wave + i * NW)), 16, (unsigned)b_base[i],
-                                                 x_tap + 2 * l_c0, 0, 0);
+        const int i = n - A_L;
+        if (MASKED) {
+          // bit 31 set when the tap is outside (or the address is negative): out of range, zeros
+          const unsigned voff = (unsigned)(b_base[i] + x_tap) | ((b_out[i] >> tap) << 31);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr)(Bs + 1024 * (wave + i * NW)), 16, voff, 2 * l_c0, 0, 0);
+        } else {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr)(Bs + 1024 * (wave + i * NW)), 16, (unsigned)b_base[i],
+                                                   x_tap + 2 * l_c0, 0, 0);
+        }
       }
     }
+  };
+  auto advance_loader = [&]() {
     l_k += 64;
     l_stage = l_stage + 1 == NS ? 0 : l_stage + 1;
     const int c0n = l_c0 + 64, sn = l_s + 1;
@@ -159,6 +168,17 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
     l_c0 = wrap_c ? 0 : c0n;
     l_s = wrap_c ? (wrap_s ? 0 : sn) : l_s;
     l_r = wrap_s ? l_r + 1 : l_r;
+  };
+  constexpr int L1 = (L + 2) / 3, L2 = L1 + (L - L1 + 1) / 2;  // part boundaries
+  auto issue_part = [&](auto part_c) {
+    constexpr int PART = decltype(part_c)::value;
+    if constexpr (PART == 0) issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, L1>{});
+    if constexpr (PART == 1) issue_loads(std::integral_constant<int, L1>{}, std::integral_constant<int, L2>{});
+    if constexpr (PART == 2) { issue_loads(std::integral_constant<int, L2>{}, std::integral_constant<int, L>{}); advance_loader(); }
+  };
+  auto issue_step = [&]() {
+    issue_loads(std::integral_constant<int, 0>{}, std::integral_constant<int, L>{});
+    advance_loader();
   };
 
   floatx16 acc[TM][TN];
@@ -206,44 +226,68 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
       for (int j = 0; j < TN; j++)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[i], qb[j], acc[i][j], 0, 0, 0);
   };
-  int c_stage = 0;
-  auto compute_step = [&]() {
-    const char *stage = smem + c_stage * STAGE;
-    read_frags(stage, fa[0], fb[0], 0);
-    read_frags(stage, fa[1], fb[1], 1);
-    mfma_frags(fa[0], fb[0]);
-    read_frags(stage, fa[0], fb[0], 2);
-    mfma_frags(fa[1], fb[1]);
-    read_frags(stage, fa[1], fb[1], 3);
-    mfma_frags(fa[0], fb[0]);
-    mfma_frags(fa[1], fb[1]);
-    c_stage = c_stage + 1 == NS ? 0 : c_stage + 1;
-  };
-
   // ---- the ring -------------------------------------------------------------
-#pragma unroll
-  for (int s = 0; s < NS - 1; s++)
-    if (s < nk) issue_step();
-  int it = 0;
-  for (; it < nk - (NS - 1); it++) {
-    wait_vmcnt<(NS - 2) * L>();  // step `it` has landed (this wavefront's part; the barrier covers the others')
-    ring_barrier();              // ... and everybody is done reading the stage that is refilled next
-    issue_step();
-    compute_step();
-  }
-  auto tail = [&](auto t_c) {
-    constexpr int T = decltype(t_c)::value;
-    if (nk - (NS - 1) + T >= 0) {
-      wait_vmcnt<(NS - 2 - T) * L>();
+  // P = NS - 2 steps are in flight beyond the one being computed.  Inside step `it` a wavefront alternates
+  // fragment reads, MFMA groups and the loads of step it + P, each a sub-step ahead of its use:
+  //   read(sub 1)  mfma(sub 0)  loads 1/3  |  read(sub 2)  mfma(sub 1)  loads 2/3  |  read(sub 3)  mfma(sub 2)  loads 3/3
+  //   wait until step it + 1 has landed, barrier, read(sub 0 of step it + 1), mfma(sub 3)
+  // so an MFMA group never waits for the LDS read issued right before it, and the MFMA pipe has a group queued
+  // while the wavefront sits at the barrier or in the memory pipeline's queue.  The compiler's scheduler would
+  // sink the reads below the MFMAs that do not depend on them: scheduling barriers pin the order.
+  // The stage step it + P lands in was last read in step it - 2; the barrier inside step it - 1 came after
+  // everybody's reads of it (their MFMAs of sub-step 3 had those operands).
+  constexpr int P = NS - 2;
+  static_assert(P >= 1 && P <= 6 && (P - 1) * L < 64, "ring depth");
+  int c_stage = 0;
+  auto stage_ptr = [&]() { return smem + c_stage * STAGE; };
+  auto next_stage = [&]() { c_stage = c_stage + 1 == NS ? 0 : c_stage + 1; };
+#define PIN() __builtin_amdgcn_sched_barrier(0)
+  // G: steps still in flight behind step `it` when it ends (P while loads are being issued); LOADS: issue step it + P
+  auto step_body = [&](auto g_c, auto loads_c) {
+    constexpr int G = decltype(g_c)::value;
+    constexpr bool LOADS = decltype(loads_c)::value;
+    const char *stage = stage_ptr();
+    read_frags(stage, fa[1], fb[1], 1); PIN();
+    mfma_frags(fa[0], fb[0]); PIN();
+    if constexpr (LOADS) { issue_part(std::integral_constant<int, 0>{}); PIN(); }
+    read_frags(stage, fa[0], fb[0], 2); PIN();
+    mfma_frags(fa[1], fb[1]); PIN();
+    if constexpr (LOADS) { issue_part(std::integral_constant<int, 1>{}); PIN(); }
+    read_frags(stage, fa[1], fb[1], 3); PIN();
+    mfma_frags(fa[0], fb[0]); PIN();
+    if constexpr (LOADS) { issue_part(std::integral_constant<int, 2>{}); PIN(); }
+    next_stage();
+    if constexpr (G > 0) {
+      wait_vmcnt<(G - 1) * L>();  // this wavefront's part of the next step has landed; the barrier covers the others'
       ring_barrier();
-      compute_step();
+      read_frags(stage_ptr(), fa[0], fb[0], 0); PIN();
     }
+    mfma_frags(fa[1], fb[1]); PIN();
   };
-  tail(std::integral_constant<int, 0>{});
-  if constexpr (NS > 2) tail(std::integral_constant<int, 1>{});
-  if constexpr (NS > 3) tail(std::integral_constant<int, 2>{});
-  if constexpr (NS > 4) tail(std::integral_constant<int, 3>{});
-  static_assert(NS <= 5, "tail steps are written out up to a ring of five");
+  {
+    // prologue: steps 0 .. P - 1 (those that exist), then wait for step 0
+    const int pre = nk < P ? nk : P;
+#pragma unroll
+    for (int q = 0; q < P; q++)
+      if (q < pre) issue_step();
+    if (pre == 1) wait_vmcnt<0>();
+    else if (pre == 2) wait_vmcnt<(P > 1 ? 1 : 0) * L>();
+    else if (pre == 3) wait_vmcnt<(P > 2 ? 2 : 0) * L>();
+    else if (pre == 4) wait_vmcnt<(P > 3 ? 3 : 0) * L>();
+    else if (pre == 5) wait_vmcnt<(P > 4 ? 4 : 0) * L>();
+    else wait_vmcnt<(P > 5 ? 5 : 0) * L>();
+    ring_barrier();
+    read_frags(stage_ptr(), fa[0], fb[0], 0); PIN();
+  }
+  for (int it = 0; it < nk - P; it++) step_body(std::integral_constant<int, P>{}, std::true_type{});
+  // the last P steps (fewer if the reduction is shorter): nothing left to load, one step fewer in flight each time
+  if constexpr (P > 5) { if (nk > 5) step_body(std::integral_constant<int, 5>{}, std::false_type{}); }
+  if constexpr (P > 4) { if (nk > 4) step_body(std::integral_constant<int, 4>{}, std::false_type{}); }
+  if constexpr (P > 3) { if (nk > 3) step_body(std::integral_constant<int, 3>{}, std::false_type{}); }
+  if constexpr (P > 2) { if (nk > 2) step_body(std::integral_constant<int, 2>{}, std::false_type{}); }
+  if constexpr (P > 1) { if (nk > 1) step_body(std::integral_constant<int, 1>{}, std::false_type{}); }
+  step_body(std::integral_constant<int, 0>{}, std::false_type{});
+#undef PIN
   ring_barrier();  // nobody reads the operand stages any more
 
   // ---- epilogue: bias, activation, fp16, transpose through LDS ------------
@@ -343,7 +387,7 @@ static bool launch_dma(const dnnrtContext *ctx, const ConvF16Args &a) {
 // satisfy dma_conv_applies and carry the division constants.
 bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int variant) {
   switch (variant) {
-    case 31: return launch_dma<128, 128, 2, 2, 2>(ctx, a);
+    case 31: return launch_dma<128, 64, 2, 2, 4>(ctx, a);
     case 32: return launch_dma<128, 128, 2, 2, 3>(ctx, a);
     case 33: return launch_dma<128, 128, 2, 2, 4>(ctx, a);
     case 34: return launch_dma<128, 256, 2, 2, 3>(ctx, a);
@@ -352,6 +396,10 @@ bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int vari
     case 37: return launch_dma<64, 128, 1, 4, 4>(ctx, a);
     case 38: return launch_dma<64, 64, 2, 2, 4>(ctx, a);
     case 39: return launch_dma<256, 128, 2, 2, 3>(ctx, a);
+    case 40: return launch_dma<64, 64, 2, 2, 8>(ctx, a);    // six steps in flight: filters that come from HBM
+    case 60: return launch_dma<128, 64, 2, 2, 6>(ctx, a);
+    case 61: return launch_dma<128, 128, 2, 2, 5>(ctx, a);
+    case 62: return launch_dma<64, 128, 1, 4, 6>(ctx, a);
     default: set_error("conv(fp16): no direct-to-LDS variant %d", variant); return false;
   }
 }

@@ -280,6 +280,12 @@ int32_t dnncSessionSync(dnncSession *s) {
   return s->s.sync(err) ? 0 : fail(err);
 }
 
+int32_t dnncSessionSetConvTile(dnncSession *s, int32_t tile) {
+  if (!s) return fail("dnncSessionSetConvTile: null session");
+  std::string err;
+  return s->s.set_conv_tile(tile, err) ? 0 : fail(err);
+}
+
 int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on_device, float *ms, int64_t cap) {
   if (!s || !inputs) { fail("dnncSessionProfile: bad arguments"); return -1; }
   std::vector<float> t;

@@ -32,7 +32,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
   if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
   LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
-  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtSetConvTile); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
@@ -588,6 +588,12 @@ bool Session::profile_classes(const void *const *inputs, int on_device, const st
   rt.dnnrtEventDestroy(e0);
   rt.dnnrtEventDestroy(e1);
   return ok;
+}
+
+bool Session::set_conv_tile(int tile, std::string &err) {
+  if (rt.dnnrtSetConvTile(handle, tile)) { err = rt_error("dnnrtSetConvTile"); return false; }
+  if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
+  return true;
 }
 
 bool Session::sync(std::string &err) {

@@ -60,6 +60,7 @@ struct RuntimeApi {
   decltype(&::dnnrtTranspose) dnnrtTranspose = nullptr;
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
   decltype(&::dnnrtSetActivationCoef) dnnrtSetActivationCoef = nullptr;
+  decltype(&::dnnrtSetConvTile) dnnrtSetConvTile = nullptr;
   decltype(&::dnnrtMatmulNdBias) dnnrtMatmulNdBias = nullptr;
   decltype(&::dnnrtAttention) dnnrtAttention = nullptr;
   decltype(&::dnnrtLeakyRelu) dnnrtLeakyRelu = nullptr;
@@ -81,6 +82,8 @@ class Session {
   bool run_occamy(const void *const *inputs, void *const *outputs, std::string &err);
   bool run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err);
   bool sync(std::string &err);
+  // Tuning: dnnrtSetConvTile on the session's handle; a captured graph is dropped (it holds the old variants).
+  bool set_conv_tile(int tile, std::string &err);
   // Resident mode: one eager pass with a device timestamp around every compute
   // operation; ms[i] is the time of the i-th compute op in program order.
   // by_class: timestamps only around each operation class's launches issued

@@ -614,11 +614,13 @@ def test_conv_f16_at_batch_64_sizes(gpu, cpu, case):
 
 def test_every_compiled_f16_conv_variant(gpu, cpu):
     """Each variant dnnrtListConvTiles names, forced with dnnrtSetConvTile, on a padded 3x3 problem, a 1x1
-    problem over 128 channels and one over 512, all ragged in both directions: it either matches the
+    problem over 128 channels and one over 512, and two 3x3 problems on small images whose runs of pixels cross
+    image boundaries (one to three per tile), all ragged in both directions: it either matches the
     oracle or refuses the problem loudly (the single-stage variants take reductions of up to four steps)."""
     tiles = gpu.ops.conv_tiles()
     assert tiles and 0 not in tiles
-    cases = [(3, 128, 19, 23, 200, 3, 1, 1), (5, 128, 19, 23, 200, 1, 1, 0), (5, 512, 9, 13, 136, 1, 2, 0)]
+    cases = [(3, 128, 19, 23, 200, 3, 1, 1), (5, 128, 19, 23, 200, 1, 1, 0), (5, 512, 9, 13, 136, 1, 2, 0),
+             (11, 192, 14, 14, 136, 3, 1, 1), (23, 128, 7, 7, 72, 3, 1, 1)]
     ran = {t: 0 for t in tiles}
     for case in cases:
         x, w, b, pads, strides = f16_problem(case, 5 + sum(case))
