@@ -424,7 +424,12 @@ void *dnnrtTranspose(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
                      void *Y, const int64_t *dimY, const int64_t *perm,
                      int64_t rank, int32_t dtype);
 /* DNNAPISpecs.inc:25 "CUDAGatherFloatFunc" (cuda/CUDAGatherFloatFunc.cu:7-82):
- * numpy.take(X, indices, axis); negative indices count from the back. */
+ * numpy.take(X, indices, axis); negative indices count from the back.
+ * Indices live in device memory, so the call cannot inspect them: an index
+ * outside [-dimX[axis], dimX[axis]) reads nothing and its slice of Y is
+ * written as zeros (the reference kernel reads out of bounds there,
+ * CUDAGatherFloatFunc.cu:27-34).  A host-side build of this interface may
+ * reject such an index with an error instead. */
 void *dnnrtGather(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
                   int64_t rankX, void *Y, const int64_t *dimY, int64_t rankY,
                   const int64_t *indices, const int64_t *dimIndices,

@@ -150,6 +150,40 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
       }
       if (op->kind == OP_HOST_ALLOC) { g_err = "channels_last: a returned rank-4 tensor would come back in NHWC order"; delete pp; return nullptr; }
     }
+    // Operands: a rank-4 tensor with spatial extent may be read only by a call that has a channels-last form
+    // (a Flatten or Reshape of it would copy NHWC bytes under an NCHW shape), and a constant of that kind is
+    // uploaded as the graph holds it, N,C,H,W: only convolution filters are re-laid (K,R,S,C) at upload.
+    auto spatial4 = [](const Value *v) { return v->shape.size() == 4 && v->shape[2] * v->shape[3] > 1; };
+    auto holds_constant = [](const Value *v) {
+      for (const auto &u : v->uses)
+        if (u.first->kind == OP_MEMCPY && u.first->mode == 1 && u.second == 0 && u.first->operands[1]->def &&
+            u.first->operands[1]->def->kind == OP_HOST_CONST)
+          return true;
+      return false;
+    };
+    for (const Op *op : p.ops) {
+      bool layout_aware = false, conv = false;
+      switch (op->kind) {
+        case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: conv = true; layout_aware = true; break;
+        case OP_ACTIVATION: case OP_ADD: case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE:
+        case OP_LEAKYRELU: case OP_PRELU: case OP_CONCAT: layout_aware = true; break;
+        case OP_MALLOC: case OP_DEALLOC: case OP_MEMCPY: case OP_HOST_CONST: case OP_HOST_ALLOC: case OP_RETURN: continue;
+        default: break;
+      }
+      for (size_t i = 0; i + 1 < op->operands.size(); i++) {  // the last operand is the output buffer (checked above)
+        const Value *v = op->operands[i];
+        if (!spatial4(v)) continue;
+        if (!layout_aware) {
+          g_err = std::string("channels_last: ") + op_name(op->kind) + " reads a rank-4 tensor with spatial extent and has no channels-last form";
+          delete pp; return nullptr;
+        }
+        if (holds_constant(v) && !(conv && i == 1)) {
+          g_err = std::string("channels_last: a rank-4 constant with spatial extent feeds ") + op_name(op->kind) +
+                  ", which would read its N,C,H,W bytes as N,H,W,C";
+          delete pp; return nullptr;
+        }
+      }
+    }
     // the NCHW function arguments may feed convolutions only
     for (const Op *op : p.ops)
       if (op->kind == OP_MEMCPY && op->mode == 1 && op->operands[1]->arg_index >= 0 && op->operands[0]->shape.size() == 4)

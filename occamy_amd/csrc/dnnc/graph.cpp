@@ -542,6 +542,14 @@ static bool infer_pass(Graph &g, std::string &err) {
     } else if (t == "Relu" || t == "Sigmoid" || t == "Tanh" || t == "Sqrt" || t == "Erf" || t == "Clip" ||
                t == "Gelu" || t == "Pow" || t == "Softmax" || t == "LayerNormalization" || t == "LeakyRelu" ||
                t == "Identity" || t == "BatchNormalization") {
+      if (t == "Softmax" && g.opset > 0 && g.opset < 13) {
+        // before opset 13: axis defaults to 1 and the input is flattened to [prod(d[:axis]), prod(d[axis:])];
+        // that is the per-axis operator only when the axis is the last one
+        int64_t ax = get_int(n, "axis", 1);
+        if (ax < 0) ax += (int64_t)x.size();
+        if (ax != (int64_t)x.size() - 1) return fail("Softmax of opset " + std::to_string(g.opset) + " over flattened trailing dims is not supported (axis must be the last)");
+        n.ints["axis"] = {ax};
+      }
       out.shape = x;
     } else if (t == "FusedAttention") {  // produced by the recomposition only
       if (in.size() != 3 || !in[1] || !in[2] || x.size() != 3) return fail("needs Q, K and V of rank 3");
@@ -621,6 +629,10 @@ static bool infer_pass(Graph &g, std::string &err) {
       get_ints(n, "strides", strides);
       if (pads.size() != 4 || strides.size() != 2) return fail("pads must have 4 and strides 2 entries");
       if (get_int(n, "ceil_mode", 0) != 0) return fail("ceil_mode is not supported");
+      // the kernels divide by the full window, the reference's cuDNN mode (count include padding); the operator's
+      // default leaves the padding out of the count
+      if (t == "AveragePool" && (pads[0] || pads[1] || pads[2] || pads[3]) && get_int(n, "count_include_pad", 0) == 0)
+        return fail("padded AveragePool needs count_include_pad = 1 (windows are divided by their full size)");
       const int64_t P = (x[2] + pads[0] + pads[2] - k[0]) / strides[0] + 1;
       const int64_t Q = (x[3] + pads[1] + pads[3] - k[1]) / strides[1] + 1;
       if (P < 1 || Q < 1) return fail("empty output");

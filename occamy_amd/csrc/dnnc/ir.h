@@ -48,6 +48,7 @@ struct Graph {
   std::map<std::string, GTensor> tensors;
   std::vector<std::string> inputs, outputs;
   std::vector<GNode> nodes;  // block order; constants are "Constant" nodes
+  int64_t opset = 0;         // version of the default operator set an ONNX file declares; 0: built in memory (current semantics)
 };
 
 // ---------------------------------------------------------------- DNN program

@@ -308,6 +308,19 @@ bool graph_from_onnx(const uint8_t *data, size_t nbytes, Graph &g, std::string &
   uint32_t f, w;
   while (model.tag(f, w)) {
     if (f == 7 && w == 2) { Reader r = model.bytes(); graph_p = r.p; graph_end = r.end; }
+    else if (f == 8 && w == 2) {  // opset_import: OperatorSetIdProto { 1: domain, 2: version }
+      Reader r = model.bytes();
+      std::string domain;
+      int64_t version = 0;
+      uint32_t f2, w2;
+      while (r.tag(f2, w2)) {
+        if (f2 == 1 && w2 == 2) domain = r.str();
+        else if (f2 == 2 && w2 == 0) version = (int64_t)r.varint();
+        else r.skip(w2);
+      }
+      if (!r.ok) { err = "malformed opset_import"; return false; }
+      if (domain.empty() || domain == "ai.onnx") g.opset = version;
+    }
     else model.skip(w);
   }
   if (!model.ok) { err = "not an ONNX ModelProto (malformed protobuf)"; return false; }

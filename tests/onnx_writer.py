@@ -109,7 +109,7 @@ def node_proto(op_type, inputs, output, attrs, packed=True, extra_attrs=()):
 
 
 def model_bytes(g, typed_fields=False, packed=True, initializers_as_inputs=False, constants_as_nodes=False,
-                dynamic_batch=None, auto_pad=None):
+                dynamic_batch=None, auto_pad=None, opset=13):
     """g: a compiler.Graph built through its Python methods (the mirror is read, not the C++ object)."""
     graph = b""
     nodes = b""
@@ -130,5 +130,5 @@ def model_bytes(g, typed_fields=False, packed=True, initializers_as_inputs=False
             graph += f_bytes(11, value_info(name, a.shape, a.dtype))
     for name in g.outputs:
         graph += f_bytes(12, value_info(name, (), np.float32))  # the reader takes output names only
-    opset = f_string(1, "") + f_varint(2, 13)
-    return f_varint(1, 8) + f_string(2, "tests/onnx_writer.py") + f_bytes(8, opset) + f_bytes(7, graph)
+    opset_id = f_string(1, "") + f_varint(2, opset)
+    return f_varint(1, 8) + f_string(2, "tests/onnx_writer.py") + f_bytes(8, opset_id) + f_bytes(7, graph)

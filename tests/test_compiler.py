@@ -271,6 +271,32 @@ def test_fp16_channels_last_flag():
         g.compile(channels_last=True)  # fp32 graphs stay NCHW
 
 
+def test_channels_last_refuses_what_it_cannot_lay_out():
+    """A rank-4 constant with spatial extent reaches the device N,C,H,W (only convolution filters are re-laid at
+    upload), and Flatten / Reshape copy bytes: channels_last must refuse both at compile time, not at run time."""
+    def conv_graph():
+        g = compiler.Graph()
+        g.input("x", (1, 8, 8, 8), np.float16)
+        w = g.constant(np.ones((64, 8, 3, 3), np.float16))
+        return g, g.node("Conv", ["x", w], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1], group=1)
+    g, c = conv_graph()
+    k = g.constant(np.ones((1, 64, 8, 8), np.float16))
+    a = g.node("Add", [c, k])
+    g.output(g.node("ReduceMean", [a], axes=[2, 3], keepdims=1))
+    with pytest.raises(RuntimeError, match="constant"):
+        g.compile(channels_last=True)
+    g, c = conv_graph()
+    g.output(g.node("Flatten", [c], axis=1))
+    with pytest.raises(RuntimeError, match="no channels-last form"):
+        g.compile(channels_last=True)
+    # a per-channel constant and a flatten of a 1x1 map are fine
+    g, c = conv_graph()
+    k = g.constant(np.ones((1, 64, 1, 1), np.float16))
+    m = g.node("ReduceMean", [g.node("Add", [c, k])], axes=[2, 3], keepdims=1)
+    g.output(g.node("Flatten", [m], axis=1))
+    assert g.compile(channels_last=True).pool_bytes > 0
+
+
 def test_compile_errors():
     g = compiler.Graph()
     g.input("x", (1, 3, 8, 8))

@@ -156,6 +156,25 @@ def test_what_the_reader_refuses():
     # an operator the DNN dialect has no lowering for is reported by name at compile time
     with pytest.raises(RuntimeError, match="Selu"):
         compiler.load_onnx(ow.model_bytes(_single("Selu"))).compile()
+    # Softmax before opset 13 flattens the trailing dims: only the last axis means the same thing
+    def soft(axis_attr):
+        g = compiler.Graph()
+        g.input("x", (2, 3, 4))
+        g.output(g.node("Softmax", ["x"], **axis_attr))
+        return g
+    with pytest.raises(RuntimeError, match="opset 11"):
+        compiler.load_onnx(ow.model_bytes(soft({}), opset=11)).compile()          # default axis 1 of a rank-3 input
+    assert "axis=2" in compiler.load_onnx(ow.model_bytes(soft({"axis": -1}), opset=11)).compile().text
+    assert "axis=-1" in compiler.load_onnx(ow.model_bytes(soft({}), opset=13)).compile().text  # opset 13: last axis
+    # a padded AveragePool that leaves the padding out of the count
+    def avg(**extra):
+        g = compiler.Graph()
+        g.input("x", (1, 2, 6, 6))
+        g.output(g.node("AveragePool", ["x"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1], **extra))
+        return g
+    with pytest.raises(RuntimeError, match="count_include_pad"):
+        avg().compile()
+    assert avg(count_include_pad=1).compile().pool_bytes > 0
     # two outputs on one node
     n = ow.f_string(1, "x") + ow.f_string(2, "y") + ow.f_string(2, "mask") + ow.f_string(4, "MaxPool")
     vi = ow.value_info("x", (1, 1, 4, 4), np.float32)
