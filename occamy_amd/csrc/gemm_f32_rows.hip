@@ -144,10 +144,16 @@ __global__ __launch_bounds__(512) void gemm_f32_rows_kernel(const IgemmArgs a, c
     for (int r = 0; r < 16; r++) __hip_atomic_store(&mine[r * 64 + lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // device-scope accesses reach the point where all XCDs agree; waiting for
     // the stores' acknowledgements orders them before the arrival (a release
-    // fence would write back this XCD's whole L2)
+    // fence would write back this XCD's whole L2).  The signal fences keep the
+    // compiler from moving the relaxed accesses across the wait and the arrival
+    // (they emit no instruction); the hand-over protocol is described in
+    // igemm_f32_small.hip.
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_s_waitcnt(0);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     unsigned arrived = 0;
     if (lane == 0) arrived = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != (unsigned)splits - 1) return;
     // the partial tiles are requested four at a time (a memory round trip each time) and added in split order

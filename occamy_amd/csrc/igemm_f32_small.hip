@@ -106,14 +106,25 @@ __device__ __forceinline__ void reduce_and_store(const IgemmArgs &a, floatx16 ac
     float *mine = partials + ((size_t)tile * splits + blockIdx.y) * 1024;
 #pragma unroll
     for (int r = 0; r < 16; r++) __hip_atomic_store(&mine[r * 64 + lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // Partials are written and read with device-scope atomic accesses, which
-    // go past the per-XCD L2 to where all XCDs agree.  A release fence here
-    // would also write back every dirty line of this XCD's L2 (the previous
-    // layer's output), which costs more than the split saves; waiting for the
-    // stores' acknowledgements orders them before the arrival just as well.
+    // The hand-over.  Every workgroup of a tile (1) writes its partial tile with device-scope atomic
+    // stores, which go past the per-XCD L2 to the point where all XCDs agree, (2) waits until every one of
+    // them is acknowledged (s_waitcnt 0: the counters of a wavefront reach zero only when its stores have been
+    // written there), (3) adds one to the tile's arrival counter with a device-scope atomic, performed at
+    // that same point.  Whoever reads splits - 1 knows that every other workgroup's step (2) is over, so its
+    // device-scope atomic loads, issued after the counter's value has come back (the branch depends on it and
+    // a wavefront issues in order), read the finished partial tiles.  Nobody waits for anybody: a workgroup
+    // that is not last leaves.  What this rests on is the hardware's behaviour, stated above, not the
+    // language's memory model, which would ask for a release on (3) and an acquire in the reader; on this
+    // target a release at device scope also writes back every dirty line of the XCD's L2 (the previous
+    // layer's output), which costs more than the split saves.  The signal fences keep the compiler, which
+    // may reorder relaxed accesses to different addresses, from moving them across (2) and (3); they emit no
+    // instruction.
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0)
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     unsigned arrived = 0;
     if (lane == 0) arrived = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     if (arrived != (unsigned)splits - 1) return;
     // splits is a power of two >= 2: the partial tiles are requested four

@@ -293,6 +293,45 @@ def test_matmul_nd(gpu, cpu):
         close(oc.matmul_nd(gpu, a, b), ref)   # again: the split-reduction counters must be back at zero
 
 
+def test_split_reduction_hand_over_is_deterministic(gpu, cpu):
+    """Reductions split over workgroups meet through partial tiles and arrival counters in the handle's scratch;
+    partial tiles are added in split order, so the result does not depend on who arrives last.  The deepest
+    split of ResNet-50 at batch 1 (3x3 over 512 channels at 7x7), a 1x1 layer over 2048 channels and the
+    768 -> 3072 product, 200 times each on one handle: every repetition bit-identical to the first, which
+    matches the oracle."""
+    r = rng(91)
+    def repeat(call, ref):
+        first = call()
+        close(gpu.get(first), ref)
+        first = first.clone()
+        for i in range(200):
+            again = call()
+            assert gpu.torch.equal(again, first), f"repetition {i} differs"
+    for case in [(1, 512, 7, 7, 512, 3, 1, 1), (1, 2048, 7, 7, 512, 1, 1, 0), (1, 1024, 14, 14, 256, 1, 1, 0)]:
+        N, C, H, W, K, R, st, pd = case
+        x = r.standard_normal((N, C, H, W)).astype(np.float32)
+        w = (r.standard_normal((K, C, R, R)) * np.sqrt(2.0 / (C * R * R))).astype(np.float32)
+        b = r.uniform(-0.1, 0.1, K).astype(np.float32)
+        ref = oc.conv(cpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU)
+        P, Q = oc.conv_out_hw(H, W, R, R, (pd, pd), (st, st))
+        X, Wt, B, Y = gpu.put(x), gpu.put(w), gpu.put(b), gpu.empty((N, K, P, Q))
+        def conv_call():
+            gpu.ops.conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (pd, pd), (st, st), _abi.ACT_RELU,
+                                    gpu.ptr(Y), 1, _abi.F32)
+            gpu.sync()
+            return Y
+        repeat(conv_call, ref)
+    a = r.standard_normal((1, 128, 768)).astype(np.float32)
+    b = (r.standard_normal((768, 3072)) / np.sqrt(768)).astype(np.float32)
+    ref = oc.matmul_nd(cpu, a, b)
+    A, Bm, Y = gpu.put(a), gpu.put(b), gpu.empty((1, 128, 3072))
+    def mm_call():
+        gpu.ops.matmul_nd(gpu.ptr(A), a.shape, gpu.ptr(Bm), b.shape, gpu.ptr(Y), (1, 128, 3072), _abi.F32)
+        gpu.sync()
+        return Y
+    repeat(mm_call, ref)
+
+
 def test_matmul_nd_bias(gpu, cpu):
     r = rng(44)
     # transformer Linear layers (one tall product, the dot-product kernel for few rows) and batched products
