@@ -34,6 +34,7 @@ struct IgemmArgs {
   int Z;
   int64_t a_z_stride, x_z_stride, y_z_stride, bias_z_stride;
   unsigned magic_rs, magic_s;  // filled in by launch_igemm_f32: magic_of(R * S), magic_of(S), for the generic filter sizes
+  int xcd_m;          // (small kernels, set by their launcher) the XCDs form an xcd_m x (8 / xcd_m) grid over the tile plane
   bool b_kcontig;     // B stored [Ncols][Kdim] (k contiguous): GEMM with transB
   bool a_mcontig;     // A stored [Kdim][M]: GEMM with transA
   bool a_vec4;        // A rows may be read as aligned float4

@@ -193,15 +193,19 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
                                                                     unsigned *counters) {
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
-  // Workgroup ids go round-robin over the 8 XCDs (gridDim.x is a multiple of 8,
-  // so that holds for every y and z as well).  Renumbered so that one XCD owns
-  // a contiguous run of tiles, column tiles of one filter-row tile first: a
-  // slice of the filter is then fetched into one L2 instead of all eight.
-  const int tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * ((a.M + 31) / 32);
-  const int per_xcd = (int)(gridDim.x >> 3);
-  const int tile_id = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-  if (tile_id >= tiles) return;
-  const int tile_m = tile_id / tiles_n, tile_n = tile_id - tile_m * tiles_n;
+  // Workgroups go round-robin over the 8 XCDs (gridDim.x is a multiple of 8, so that holds for every y and
+  // z as well), each with its own L2.  The XCDs are laid out as a grid of xcd_m x (8 / xcd_m) over the
+  // (filter-row tile, column tile) plane and each owns one rectangle of tiles: it fetches 1 / xcd_m of the
+  // filter and xcd_m / 8 of the activations, where a run of consecutive tiles per XCD fetches all of one operand
+  // into all eight L2s.  The launcher picks xcd_m from the two operands' sizes.
+  const int tiles_m = (a.M + 31) / 32, tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * tiles_m;
+  const int xcd_n = 8 / a.xcd_m;
+  const int tm_per = (tiles_m + a.xcd_m - 1) / a.xcd_m, tn_per = (tiles_n + xcd_n - 1) / xcd_n;
+  const int xcd = (int)(blockIdx.x & 7), in_xcd = (int)(blockIdx.x >> 3);
+  const int tm_local = in_xcd / tn_per;
+  const int tile_m = (xcd / xcd_n) * tm_per + tm_local, tile_n = (xcd % xcd_n) * tn_per + (in_xcd - tm_local * tn_per);
+  if (tm_local >= tm_per || tile_m >= tiles_m || tile_n >= tiles_n) return;
+  const int tile_id = tile_m * tiles_n + tile_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
   const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
   const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
@@ -295,15 +299,19 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
                                                                     unsigned *counters) {
   __shared__ float red[KS > 1 ? KS - 1 : 1][16][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, half = lane >> 5;
-  // Workgroup ids go round-robin over the 8 XCDs (gridDim.x is a multiple of 8,
-  // so that holds for every y and z as well).  Renumbered so that one XCD owns
-  // a contiguous run of tiles, column tiles of one filter-row tile first: a
-  // slice of the filter is then fetched into one L2 instead of all eight.
-  const int tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * ((a.M + 31) / 32);
-  const int per_xcd = (int)(gridDim.x >> 3);
-  const int tile_id = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
-  if (tile_id >= tiles) return;
-  const int tile_m = tile_id / tiles_n, tile_n = tile_id - tile_m * tiles_n;
+  // Workgroups go round-robin over the 8 XCDs (gridDim.x is a multiple of 8, so that holds for every y and
+  // z as well), each with its own L2.  The XCDs are laid out as a grid of xcd_m x (8 / xcd_m) over the
+  // (filter-row tile, column tile) plane and each owns one rectangle of tiles: it fetches 1 / xcd_m of the
+  // filter and xcd_m / 8 of the activations, where a run of consecutive tiles per XCD fetches all of one operand
+  // into all eight L2s.  The launcher picks xcd_m from the two operands' sizes.
+  const int tiles_m = (a.M + 31) / 32, tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * tiles_m;
+  const int xcd_n = 8 / a.xcd_m;
+  const int tm_per = (tiles_m + a.xcd_m - 1) / a.xcd_m, tn_per = (tiles_n + xcd_n - 1) / xcd_n;
+  const int xcd = (int)(blockIdx.x & 7), in_xcd = (int)(blockIdx.x >> 3);
+  const int tm_local = in_xcd / tn_per;
+  const int tile_m = (xcd / xcd_n) * tm_per + tm_local, tile_n = (xcd % xcd_n) * tn_per + (in_xcd - tm_local * tn_per);
+  if (tm_local >= tm_per || tile_m >= tiles_m || tile_n >= tiles_n) return;
+  const int tile_id = tile_m * tiles_n + tile_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
   const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
   const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
@@ -422,14 +430,33 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
     }
     splits *= 2;
   }
-  dim3 grid((unsigned)(ceil_div(tiles, 8) * 8), splits, a.Z);
+  // The XCD grid: xcd_m x (8 / xcd_m) rectangles of tiles.  Elements fetched over all eight L2s: the filter
+  // 8 / xcd_m times, the activations xcd_m times; rectangles that do not divide the tile counts leave
+  // workgroups without a tile and XCDs with less work, which the estimate charges for.
+  IgemmArgs am = a;
+  const int tiles_m = (int)ceil_div(a.M, 32), tiles_n = (int)ceil_div(a.Ncols, 32);
+  int64_t slots = 0;
+  {
+    const double act = (double)(a.Kdim / (a.R * a.S)) * a.H * a.W * (double)ceil_div(a.Ncols, (int64_t)a.P * a.Q), filt = (double)a.M * a.Kdim;
+    double best = 0;
+    for (int xm = 1; xm <= 8; xm *= 2) {
+      const int xn = 8 / xm;
+      if ((xm > tiles_m && xm > 1) || (xn > tiles_n && xn > 1)) continue;
+      const int64_t per = ceil_div(tiles_m, xm) * ceil_div(tiles_n, xn);
+      const double cost = (act * xm + filt * xn) * ((double)(8 * per) / tiles);
+      if (slots == 0 || cost < best) { best = cost; am.xcd_m = xm; slots = 8 * per; }
+    }
+    if (slots == 0) { am.xcd_m = 1; slots = 8 * ceil_div(tiles_m, 1) * ceil_div(tiles_n, 8); }  // a single tile either way
+  }
+  if (slots > INT32_MAX) return true;
+  dim3 grid((unsigned)slots, splits, a.Z);
   if (ctx->splitk_shared && splits > 1) clear_split_counters(ctx, tiles * a.Z);
 #define LAUNCH_KS2(KERNEL, AMC_, ARG)                                                                  \
   switch (ks) {                                                                                          \
-    case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break;  \
-    case 2: hipLaunchKernelGGL((KERNEL<2, AMC_>), grid, dim3(128), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
-    case 4: hipLaunchKernelGGL((KERNEL<4, AMC_>), grid, dim3(256), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
-    default: hipLaunchKernelGGL((KERNEL<8, AMC_>), grid, dim3(512), 0, ctx->stream, a, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
+    case 1: hipLaunchKernelGGL((KERNEL<1, AMC_>), grid, dim3(64), 0, ctx->stream, am, ARG, ctx->splitk_partials, ctx->splitk_counters); break;  \
+    case 2: hipLaunchKernelGGL((KERNEL<2, AMC_>), grid, dim3(128), 0, ctx->stream, am, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
+    case 4: hipLaunchKernelGGL((KERNEL<4, AMC_>), grid, dim3(256), 0, ctx->stream, am, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
+    default: hipLaunchKernelGGL((KERNEL<8, AMC_>), grid, dim3(512), 0, ctx->stream, am, ARG, ctx->splitk_partials, ctx->splitk_counters); break; \
   }
 #define LAUNCH_KS(KERNEL, ARG)                                                                         \
   do {                                                                                                 \
