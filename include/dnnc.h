@@ -111,6 +111,10 @@ int32_t dnncSessionSync(dnncSession *s);
 /* Tuning and tests: dnnrtSetConvTile on the session's handle (0 = automatic choice); a captured
  * graph is dropped and recorded again by the next replayed run. */
 int32_t dnncSessionSetConvTile(dnncSession *s, int32_t tile);
+/* Debugging, per-inference (occamy) mode: fill the pool when it is allocated, and every tensor's slot when it
+ * is carved out of the pool, with `byte` (0..255; -1 switches it off).  With 0xFF a byte that a kernel leaves
+ * unwritten, or that is read before its producer ran, shows up as NaN in the results. */
+int32_t dnncSessionSetDebugFill(dnncSession *s, int32_t byte);
 /* resident mode: one eager pass with device timestamps around every compute
  * operation; ms[i] belongs to dnncProgramComputeOp(i).  Returns the count.
  * on_device bit 0: the inputs are device buffers; bit 1: one pair of

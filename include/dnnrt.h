@@ -156,6 +156,14 @@ int32_t dnnrtMemPoolInit(void **pool, int64_t bytes);
 /* DNNAPISpecs.inc:47 "wrapDNNMemOffset" (wrapDNNMemOffset.cpp:19-34). */
 int32_t dnnrtMemOffset(void **ptr, void *base, int64_t offset, int64_t bytes);
 /* DNNAPISpecs.inc:45 "wrapDNNMemcpy" (wrapDNNMemcpy.cpp:17-61). */
+/* New, for debugging.  Fills bytes [ptr, ptr + bytes) with `byte` on `stream` (a
+ * kernel, so it can be captured into a graph).  The reference clears every
+ * tensor's slot as it carves it out of the pool
+ * (src/Tools/dnn-wrapper/cuda/wrapDNNMemOffset.cpp:27); dnnrtMemOffset does not,
+ * and nothing needs it: every kernel writes all of its output.  A caller that
+ * wants to see that claim tested fills each slot with 0xFF (a NaN in fp16 and
+ * fp32) before its producer runs and looks for NaNs in the results. */
+int32_t dnnrtMemFill(void *ptr, int32_t byte, int64_t bytes, dnnrtStream_t stream);
 int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind,
                     dnnrtStream_t stream);
 /* DNNAPISpecs.inc:40 "wrapDNNMalloc" (wrapDNNMalloc.cpp). */

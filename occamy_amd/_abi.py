@@ -39,6 +39,7 @@ SIGNATURES = {
     "dnnrtIsHostBackend": (i32, []),
     "dnnrtMemPoolInit": (i32, [C.POINTER(P), i64]),
     "dnnrtMemOffset": (i32, [C.POINTER(P), P, i64, i64]),
+    "dnnrtMemFill": (i32, [P, i32, i64, P]),
     "dnnrtMemcpy": (i32, [P, P, i64, i32, P]),
     "dnnrtMalloc": (i32, [C.POINTER(P), i64]),
     "dnnrtDealloc": (i32, [P]),

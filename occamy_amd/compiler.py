@@ -77,6 +77,7 @@ def lib():
         "dnncSessionRunResident": (C.c_int32, [P, C.POINTER(P), C.POINTER(P), C.c_int32, C.c_int32]),
         "dnncSessionSync": (C.c_int32, [P]),
         "dnncSessionSetConvTile": (C.c_int32, [P, C.c_int32]),
+        "dnncSessionSetDebugFill": (C.c_int32, [P, C.c_int32]),
         "dnncSessionWeightsBytes": (C.c_int64, [P]),
         "dnncSessionLastPoolBytes": (C.c_int64, [P]),
     }
@@ -311,6 +312,11 @@ class Session:
         if lib().dnncSessionProfile(self._s, ip, int(on_device) | (2 if by_class else 0), ms, n) < 0:
             raise RuntimeError("profile: " + _err())
         return list(ms[:n])
+
+    def set_debug_fill(self, byte):
+        """Per-inference mode: fill the pool and every tensor's slot with `byte` before use (-1: off)."""
+        if lib().dnncSessionSetDebugFill(self._s, byte):
+            raise RuntimeError("set_debug_fill: " + _err())
 
     def set_conv_tile(self, tile):
         """Force one fp16 convolution variant (dnnrtListConvTiles) for every following run; 0 = automatic."""

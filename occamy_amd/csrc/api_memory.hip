@@ -18,6 +18,20 @@ void set_error(const char *fmt, ...) {
 
 using dnnrt::set_error;
 
+namespace dnnrt {
+// 16 bytes per thread, byte stores at the ragged ends (a slot's address is 32-byte aligned, its size is not)
+__global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *p, unsigned char byte, int64_t n) {
+  const int64_t at = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 16;
+  if (at >= n) return;
+  if (at + 16 <= n && (reinterpret_cast<uintptr_t>(p + at) & 15u) == 0) {
+    const unsigned w = byte * 0x01010101u;
+    *reinterpret_cast<uint4 *>(p + at) = make_uint4(w, w, w, w);
+  } else {
+    for (int64_t i = at; i < n && i < at + 16; i++) p[i] = byte;
+  }
+}
+}  // namespace dnnrt
+
 #define HIP_RET(call, what)                                                    \
   do {                                                                         \
     hipError_t e_ = (call);                                                    \
@@ -208,6 +222,17 @@ int32_t dnnrtMemOffset(void **ptr, void *base, int64_t offset, int64_t bytes) {
   (void)bytes;
   if (!ptr || !base || offset < 0) { set_error("dnnrtMemOffset: bad arguments"); return 1; }
   *ptr = static_cast<char *>(base) + offset;
+  return 0;
+}
+
+int32_t dnnrtMemFill(void *ptr, int32_t byte, int64_t bytes, dnnrtStream_t stream) {
+  if (bytes <= 0) return 0;
+  if (!ptr || byte < 0 || byte > 255) { set_error("dnnrtMemFill: bad arguments"); return 1; }
+  const int64_t blocks = (bytes + 256 * 16 - 1) / (256 * 16);
+  if (blocks > INT32_MAX) { set_error("dnnrtMemFill: too large"); return 1; }
+  hipLaunchKernelGGL(dnnrt::fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     static_cast<unsigned char *>(ptr), (unsigned char)byte, bytes);
+  HIP_RET(hipGetLastError(), "dnnrtMemFill");
   return 0;
 }
 

@@ -314,6 +314,12 @@ int32_t dnncSessionSync(dnncSession *s) {
   return s->s.sync(err) ? 0 : fail(err);
 }
 
+int32_t dnncSessionSetDebugFill(dnncSession *s, int32_t byte) {
+  if (!s || byte < -1 || byte > 255) return fail("dnncSessionSetDebugFill: bad arguments");
+  s->s.debug_fill = byte;
+  return 0;
+}
+
 int32_t dnncSessionSetConvTile(dnncSession *s, int32_t tile) {
   if (!s) return fail("dnncSessionSetConvTile: null session");
   std::string err;

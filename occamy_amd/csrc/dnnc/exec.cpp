@@ -32,7 +32,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
   if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
   LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
-  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtSetConvTile); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtSetConvTile); LOAD(dnnrtMemFill); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
@@ -392,11 +392,13 @@ bool Session::run_occamy(const void *const *inputs, void *const *outputs, std::s
         if (rt.dnnrtMemPoolInit(&run_pool, op->bytes)) { err = rt_error("dnnrtMemPoolInit"); ok = false; }
         ptr[(size_t)op->result->id] = run_pool;
         last_pool_bytes = op->bytes;
+        if (ok && debug_fill >= 0 && rt.dnnrtMemFill(run_pool, debug_fill, op->bytes, stream)) { err = rt_error("dnnrtMemFill"); ok = false; }
         break;
       case OP_MEM_OFFSET: {
         void *q = nullptr;
         if (rt.dnnrtMemOffset(&q, ptr[(size_t)op->operands[0]->id], op->offset, op->bytes)) { err = rt_error("dnnrtMemOffset"); ok = false; }
         ptr[(size_t)op->result->id] = q;
+        if (ok && debug_fill >= 0 && rt.dnnrtMemFill(q, debug_fill, op->bytes, stream)) { err = rt_error("dnnrtMemFill"); ok = false; }
         break;
       }
       case OP_MEMCPY:

@@ -61,6 +61,7 @@ struct RuntimeApi {
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
   decltype(&::dnnrtSetActivationCoef) dnnrtSetActivationCoef = nullptr;
   decltype(&::dnnrtSetConvTile) dnnrtSetConvTile = nullptr;
+  decltype(&::dnnrtMemFill) dnnrtMemFill = nullptr;
   decltype(&::dnnrtMatmulNdBias) dnnrtMatmulNdBias = nullptr;
   decltype(&::dnnrtAttention) dnnrtAttention = nullptr;
   decltype(&::dnnrtLeakyRelu) dnnrtLeakyRelu = nullptr;
@@ -95,6 +96,10 @@ class Session {
   const Program *prog = nullptr;
   int mode = MODE_OCCAMY;
   int64_t weights_bytes = 0;     // bytes of the constants arena (resident mode)
+  // Debugging (the reference's per-inference mode): fill the pool when it is allocated and every tensor's slot when
+  // it is carved out with this byte (-1: off); 0xFF makes any byte a kernel leaves unwritten, or reads before its
+  // producer ran, a NaN in the results.
+  int debug_fill = -1;
   int64_t last_pool_bytes = -1;  // bytes the last occamy-mode run asked the runtime for
 
  private:

@@ -203,6 +203,11 @@ int32_t dnnrtMemOffset(void **p, void *base, int64_t off, int64_t bytes) {
   return 0;
 }
 /* wrapDNNMemcpy.cpp:17-61. */
+int32_t dnnrtMemFill(void *ptr, int32_t byte, int64_t bytes, dnnrtStream_t stream) {
+  (void)stream;
+  if (bytes > 0) memset(ptr, byte, (size_t)bytes);
+  return 0;
+}
 int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind, dnnrtStream_t s) {
   (void)kind; (void)s;
   if (bytes > 0) memmove(dst, src, (size_t)bytes);

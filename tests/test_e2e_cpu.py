@@ -55,6 +55,26 @@ def test_modes_and_flags_agree():
     np.testing.assert_allclose(out[0], base[0], rtol=1e-4, atol=1e-3)
 
 
+def test_poisoned_pool_changes_nothing():
+    """The executor's debug fill: the pool, and then every tensor's slot as it is carved out, is filled with 0xFF
+    bytes (NaN in fp32 and fp16) before use.  A kernel that left part of its output unwritten, or an operator placed
+    before its producer, would carry NaNs into the result; the result must be the unpoisoned run's, bit for bit."""
+    for builder, flags in [(lambda: models.resnet50(image=32, classes=10), dict(fusion=True)),
+                           (lambda: models.mobilenet_v2(image=32, classes=10), dict()),
+                           (lambda: models.bert_encoder(layers=1, hidden=64, heads=2, ffn=128, seq=16, vocab=50), dict())]:
+        g, inputs = builder()
+        p = g.compile(**flags)
+        s = p.session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+        plain = s.run(*inputs)
+        s.set_debug_fill(0xFF)
+        poisoned = s.run(*inputs)
+        s.set_debug_fill(-1)
+        s.close()
+        for a, b in zip(plain, poisoned):
+            assert np.isfinite(b).all()
+            np.testing.assert_array_equal(a, b)
+
+
 def test_resnet50_small_image():
     check(lambda: models.resnet50(image=64, classes=100))
     check(lambda: models.resnet50(batch=2, image=32, classes=10), fusion=True)

@@ -87,6 +87,28 @@ def test_resident_mode_and_graph_replay(name, oracle_outputs):
     s.close()
 
 
+def test_poisoned_pool_changes_nothing_on_the_gpu():
+    """Every kernel writes all of its output and no operator reads a slot before its producer ran: with the pool and
+    every freshly carved slot filled with 0xFF bytes (NaN) the results are those of the plain run, bit for bit.
+    fp32 networks with and without the fused calls, BERT with its fused paths, fp16 channels-last."""
+    cases = [(lambda: models.resnet50(image=64, classes=100), dict()),
+             (lambda: models.resnet50(image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True)),
+             (lambda: models.mobilenet_v2(image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_activations=True)),
+             (lambda: models.bert_encoder(layers=2), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)),
+             (lambda: models.resnet50(4, np.float16, seed=5, image=64), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True)),
+             (lambda: models.srgan_generator(1, np.float32, height=24, width=16), dict(fusion=True, fuse_activations=True))]
+    for builder, flags in cases:
+        g, inputs = builder()
+        s = g.compile(**flags).session(compiler.MODE_OCCAMY)
+        plain = s.run(*inputs)
+        s.set_debug_fill(0xFF)
+        poisoned = s.run(*inputs)
+        s.close()
+        for a, b in zip(plain, poisoned):
+            assert np.isfinite(b.astype(np.float32)).all()
+            np.testing.assert_array_equal(a, b)
+
+
 def test_bert_fused_layernorm_gelu(oracle_outputs):
     out, _ = run(lambda: models.bert_encoder(layers=2, fused=True))
     close(out[0], oracle_outputs["bert_2_layers"][0], 1e-4, 1e-4)
