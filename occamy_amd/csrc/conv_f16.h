@@ -37,4 +37,9 @@ int patch_conv_capacity(const ConvF16Args &a, int bn);
 bool patch_variant_fits(const ConvF16Args &a, int variant);  // the variant's patch capacity holds this problem's patches
 bool launch_conv_f16_patch(const dnnrtContext *ctx, const ConvF16Args &a, int variant);
 
+// 3x3 stride-1 pad-1 channels-last convolutions over exactly 64 channels, images up to 62 wide, no residual
+// (conv_f16_c64.hip): persistent workgroups, filter in registers, input patch in LDS.
+bool c64_conv_applies(const ConvF16Args &a);
+bool launch_conv_f16_c64(const dnnrtContext *ctx, const ConvF16Args &a);
+
 }  // namespace dnnrt

@@ -560,6 +560,7 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       bool can = true;
       if ((want >= 31 && want <= 40) || (want >= 60 && want <= 69)) can = dma_conv_applies(am);
       else if (want >= 41 && want <= 59) can = patch_conv_applies(am) && patch_variant_fits(am, want);
+      else if (want == 70) can = c64_conv_applies(am);
       else if (want == 18) can = steps <= 4;
       else if (want == 17) can = steps == 1 || steps == 2 || steps == 4;
       sel = can ? want : 0;
@@ -576,7 +577,11 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       // Inside a network the filters come from HBM (activations pass through the caches in between), so the
       // variants that keep three (128-row tiles) or six (64-row tiles) filter steps in flight are the ones
       // chosen: 27 -> 25 us and 36 -> 26 us against two steps in flight.
-      if (patch_cap && one_per_cu) sel = patch_cap == 256 ? 48 : 52;
+      // 64 -> 64 channels, 3x3, on images wide enough to fill the persistent kernel's two-row tiles and with several
+      // tiles per workgroup: its filter stays in registers (inside the network 36 -> 27.5 us at 56x56, batch 64)
+      const int64_t c64_tiles = (int64_t)a.N * ((a.H + 1) / 2) * ceil_div(a.K, 64);
+      if (c64_conv_applies(am) && 2 * a.W >= 96 && c64_tiles >= 4 * cus) sel = 70;
+      else if (patch_cap && one_per_cu) sel = patch_cap == 256 ? 48 : 52;
       else if (patch_cap && fewer) sel = patch_cap == 256 ? 47 : 49;
       else if (nk <= 4) sel = 18;  // up to four steps (1x1 over up to 256 channels): the single-stage 64x64 variant
                               // (27 vs 34 us on 64 -> 256 at 56x56, 22.6 vs 26.6 on 128 -> 512 at 28x28, 18.3 vs 21.7 on 256 -> 1024 at 14x14)
@@ -592,6 +597,13 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     if ((sel >= 31 && sel <= 40) || (sel >= 60 && sel <= 69)) {
       if (!dma_conv_applies(am)) { set_error("conv(fp16): tile %d needs tensors below 2 GiB", sel); return false; }
       if (!launch_conv_f16_dma(ctx, am, sel)) return false;
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
+      return true;
+    }
+    if (sel == 70) {
+      if (!c64_conv_applies(am)) { set_error("conv(fp16): tile 70 is for 3x3 stride-1 pad-1 layers over 64 channels, at most 62 pixels wide, without a residual"); return false; }
+      if (!launch_conv_f16_c64(ctx, am)) return false;
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
       return true;
