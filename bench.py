@@ -29,7 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
-RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention")
+RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool")
 
 
 def build_workload(name, batch=None):
@@ -40,7 +40,8 @@ def build_workload(name, batch=None):
         return models.resnet50(b, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True), b, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
         b = batch or 64
-        return models.resnet50(b, np.float16, seed=5), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True), b, "img/s", "f16"
+        return (models.resnet50(b, np.float16, seed=5),
+                dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True), b, "img/s", "f16")
     if batch is not None:
         raise SystemExit(f"{name}: no batch override")
     if name == "mobilenet_v2_fp32_bs1":

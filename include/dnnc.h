@@ -64,6 +64,10 @@ typedef struct {
                              becomes one call (default 0) */
   int32_t fuse_attention; /* no reference flag: the head split, QK^T, scaling, Softmax, PV and
                              head merge of an exported attention block become one call (default 0) */
+  int32_t fuse_first_layer_maxpool; /* no reference flag: with `fusion` and `channels_last`, a ResNet's first
+                             convolution (3 -> 64 channels, 7x7, stride 2, pad 3, even image width, ReLU or
+                             identity) and the 3x3 / stride 2 / pad 1 max-pool behind it become one call
+                             that never stores the convolution's result (default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);

@@ -214,6 +214,27 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X,
                             int64_t algo, int64_t group, const int64_t *pads,
                             const int64_t *strides, int64_t activMode, void *Y,
                             int32_t dtype);
+/* New: dnnrtConvBiasActiv followed by dnnrtMaxPool in one kernel, for the
+ * first layer of an ImageNet ResNet: Y = maxpool(act(conv(X, W) + B)) with
+ * the convolution's result (four times the pooled tensor) never stored.  It
+ * replaces the reference's two calls (CUDNNConvBiasReluFunc.cpp:8-140, then
+ * CUDNNMaxPoolFunc.cpp:8-78); every element is what that chain stores: the
+ * activation's output rounded to fp16, then the maximum over the window,
+ * padding ignored, NaN propagated.  One shape only, anything else fails with
+ * an error (nothing falls back to the two calls, which would need a buffer
+ * for the intermediate tensor): fp16, tensor format DNNRT_NCHW_TO_NHWC (X is
+ * the N,C,H,W function argument, Y is N,H,W,C), filter K,R,S,C with 3 -> 64
+ * channels, 7x7, stride 2, pad 3, group 1, activMode ReLU or identity; pooling
+ * 3x3, stride 2, pad 1.  dimY = [N, 64, PP, QQ], the pooled extents. */
+void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X,
+                                const int64_t *dimX, const void *W,
+                                const int64_t *dimW, const void *B,
+                                const int64_t *dimB, int64_t group,
+                                const int64_t *pads, const int64_t *strides,
+                                int64_t activMode, const int64_t *poolKernel,
+                                const int64_t *poolPads,
+                                const int64_t *poolStrides, void *Y,
+                                const int64_t *dimY, int32_t dtype);
 /* No counterpart in the reference.  dnnrtConvBiasActiv for callers that cannot
  * allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It takes the stream where the other calls

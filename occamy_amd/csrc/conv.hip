@@ -374,6 +374,35 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dim
                               strides, (int)activMode, Y, dtype);
 }
 
+void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
+                                const int64_t *dimW, const void *B, const int64_t *dimB, int64_t group,
+                                const int64_t *pads, const int64_t *strides, int64_t activMode,
+                                const int64_t *poolKernel, const int64_t *poolPads, const int64_t *poolStrides, void *Y,
+                                const int64_t *dimY, int32_t dtype) {
+  const char *who = "dnnrtConvBiasActivMaxPool";
+  if (!handle) DNNRT_FAIL("%s: null handle", who);
+  if (!X || !W || !Y || !dimX || !dimW || !dimY || !pads || !strides || !poolKernel || !poolPads || !poolStrides)
+    DNNRT_FAIL("%s: null argument", who);
+  if (!B || !dimB || dnnrt::numel(dimB, 4) != dimW[0]) DNNRT_FAIL("%s: bias must hold K values", who);
+  if (dtype != DNNRT_F16) DNNRT_FAIL("%s: fp16 tensors only", who);
+  if (poolKernel[0] != 3 || poolKernel[1] != 3 || poolStrides[0] != 2 || poolStrides[1] != 2 || poolPads[0] != 1 || poolPads[1] != 1)
+    DNNRT_FAIL("%s: the pooling must be 3x3, stride 2, pad 1", who);
+  dnnrt::ConvShape s;
+  if (!dnnrt::parse_conv(who, dimX, dimW, group, pads, strides, s)) return nullptr;
+  const int64_t PP = (s.P + 2 - 3) / 2 + 1, QQ = (s.Q + 2 - 3) / 2 + 1;
+  if (dimY[0] != s.N || dimY[1] != s.K || dimY[2] != PP || dimY[3] != QQ)
+    DNNRT_FAIL("%s: dimY is [%ld,%ld,%ld,%ld], the pooled convolution is [%d,%d,%ld,%ld]", who, (long)dimY[0], (long)dimY[1],
+               (long)dimY[2], (long)dimY[3], s.N, s.K, (long)PP, (long)QQ);
+  if (s.N == 0) return Y;
+  dnnrt::ConvF16Args a{};
+  a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Z = nullptr; a.Y = nullptr;
+  a.N = s.N; a.C = s.C; a.H = s.H; a.W = s.W; a.K = s.K; a.Cg = s.Cg; a.R = s.R; a.S = s.S;
+  a.P = s.P; a.Q = s.Q; a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw; a.group = s.group;
+  a.act = (int)activMode; a.act_coef = handle->act_coef; a.format = handle->format;
+  if (!dnnrt::launch_conv_f16_stem_pool(handle, a, (__half *)Y, (int)PP, (int)QQ)) return nullptr;
+  return Y;
+}
+
 void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
                             const int64_t *dimW, const void *B, const int64_t *dimB, const void *Z,
                             void *workspace, int64_t workspaceBytes, int64_t algo, int64_t group,

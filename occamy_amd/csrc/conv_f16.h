@@ -22,6 +22,9 @@ constexpr int FEWPIX_MAX_PIXELS = 64;
 bool launch_conv_f16_fewpix(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 // The 3-channel 7x7 stride-2 first layer (NCHW in, NHWC out); `launched` says whether it took the problem.
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
+// The same layer with the 3x3 stride-2 pad-1 max-pool behind it in one kernel: `a` is the convolution (a.Y unused),
+// Yp the pooled tensor N x PP x QQ x 64.  Fails with an error on any other shape.
+bool launch_conv_f16_stem_pool(const dnnrtContext *ctx, const ConvF16Args &a, __half *Yp, int PP, int QQ);
 
 // Channels-last convolutions whose operands are loaded straight into LDS (conv_f16_dma.hip): `variant` is one of
 // that file's tile ids, `a` must satisfy dma_conv_applies and carry the division constants.

@@ -133,6 +133,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (opt->fusion && opt->fuse_activations) fuse_conv_activations(p);
   if (opt->fusion && opt->fuse_matmul_bias) fuse_matmul_bias(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
+  if (opt->fusion && opt->fuse_first_layer_maxpool && opt->channels_last) fuse_first_layer_maxpool(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {
     // Only fp16 programs whose rank-4 tensors flow through layout-aware calls
@@ -143,7 +144,8 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
       if (!r4) continue;
       if (op->result->dtype != F16) { g_err = "channels_last needs an fp16 graph"; delete pp; return nullptr; }
       switch (op->kind) {
-        case OP_MALLOC: case OP_HOST_ALLOC: case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_ACTIVATION: case OP_ADD:
+        case OP_MALLOC: case OP_HOST_ALLOC: case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_CONV_BIAS_ACTIV_MAXPOOL:
+        case OP_ACTIVATION: case OP_ADD:
         case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE: case OP_LEAKYRELU: case OP_PRELU:
         case OP_CONCAT: break;
         default: g_err = std::string("channels_last: ") + op_name(op->kind) + " has no channels-last form"; delete pp; return nullptr;
@@ -164,7 +166,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
     for (const Op *op : p.ops) {
       bool layout_aware = false, conv = false;
       switch (op->kind) {
-        case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: conv = true; layout_aware = true; break;
+        case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_CONV_BIAS_ACTIV_MAXPOOL: conv = true; layout_aware = true; break;
         case OP_ACTIVATION: case OP_ADD: case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE:
         case OP_LEAKYRELU: case OP_PRELU: case OP_CONCAT: layout_aware = true; break;
         case OP_MALLOC: case OP_DEALLOC: case OP_MEMCPY: case OP_HOST_CONST: case OP_HOST_ALLOC: case OP_RETURN: continue;
@@ -189,6 +191,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
       if (op->kind == OP_MEMCPY && op->mode == 1 && op->operands[1]->arg_index >= 0 && op->operands[0]->shape.size() == 4)
         for (const auto &u : op->operands[0]->uses)
           if (u.first->kind != OP_MEMCPY && u.first->kind != OP_DEALLOC && u.first->kind != OP_CONVFWD && u.first->kind != OP_CONV_BIAS_ACTIV &&
+              !(u.first->kind == OP_CONV_BIAS_ACTIV_MAXPOOL && u.second == 0) &&
               !(u.first->kind == OP_CONV_BIAS_ADD_ACTIV && u.second == 0)) {
             g_err = "channels_last: a rank-4 function argument may only feed convolutions"; delete pp; return nullptr;
           }

@@ -37,7 +37,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
   LOAD(dnnrtMalloc); LOAD(dnnrtDealloc); LOAD(dnnrtHostAlloc); LOAD(dnnrtHostFree);
-  LOAD(dnnrtConv); LOAD(dnnrtConvBiasActiv); LOAD(dnnrtConvBiasAddActiv); LOAD(dnnrtActive); LOAD(dnnrtTensorOp); LOAD(dnnrtClip);
+  LOAD(dnnrtConv); LOAD(dnnrtConvBiasActiv); LOAD(dnnrtConvBiasAddActiv); LOAD(dnnrtConvBiasActivMaxPool); LOAD(dnnrtActive); LOAD(dnnrtTensorOp); LOAD(dnnrtClip);
   LOAD(dnnrtErf); LOAD(dnnrtNegative); LOAD(dnnrtReciprocal); LOAD(dnnrtPow); LOAD(dnnrtCastI64toFloat);
   LOAD(dnnrtGelu); LOAD(dnnrtReduce); LOAD(dnnrtSoftmax); LOAD(dnnrtLayerNorm); LOAD(dnnrtMaxPool);
   LOAD(dnnrtAveragePool); LOAD(dnnrtMatmul2d); LOAD(dnnrtMatmulNd); LOAD(dnnrtFlatten);
@@ -112,7 +112,7 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
     for (const auto &u : op->operands[0]->uses) {
       if (u.first == op) continue;
       const bool conv = u.first->kind == OP_CONVFWD || u.first->kind == OP_CONV_BIAS_ACTIV ||
-                        u.first->kind == OP_CONV_BIAS_ADD_ACTIV;
+                        u.first->kind == OP_CONV_BIAS_ADD_ACTIV || u.first->kind == OP_CONV_BIAS_ACTIV_MAXPOOL;
       if (conv && u.second == 1) any = true;
       else if (is_compute(u.first->kind)) only_filter = false;
     }
@@ -201,7 +201,7 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
 
 int Session::format_for(const Op *op) const {
   if (!prog->channels_last) return 0;  // NCHW
-  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV) {
+  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL) {
     const Value *x = op->operands[0];
     // the function argument's slot holds what the host sent: NCHW
     const bool from_arg = x->def && x->def->kind == OP_MEM_OFFSET;
@@ -223,7 +223,7 @@ bool Session::issue(const Op *op, std::string &err) {
       cur_format = f;
     }
   }
-  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV) {
+  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL) {
     const int lay = filter_crsk[(size_t)op->operands[1]->id] ? DNNRT_FILTER_CRSK : DNNRT_FILTER_KCRS;
     if (lay != cur_filter_layout) {
       if (rt.dnnrtSetFilterLayout(handle, lay)) { err = rt_error("dnnrtSetFilterLayout"); return false; }
@@ -251,6 +251,13 @@ bool Session::issue(const Op *op, std::string &err) {
       const int64_t dimB[4] = {1, op->dimB[0], 1, 1};
       r = rt.dnnrtConvBiasAddActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, P(4), P(3), 0, 1,
                                    op->group, op->pads.data(), op->strides.data(), op->mode, out, dt);
+      break;
+    }
+    case OP_CONV_BIAS_ACTIV_MAXPOOL: {  // operands: x, w, bias, workspace, out
+      const int64_t dimB[4] = {1, op->dimB[0], 1, 1};
+      r = rt.dnnrtConvBiasActivMaxPool(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, op->group, op->pads.data(),
+                                       op->strides.data(), op->mode, op->kernel.data(), op->pool_pads.data(), op->pool_strides.data(),
+                                       out, op->dimOut.data(), dt);
       break;
     }
     case OP_ACTIVATION: {

@@ -39,6 +39,7 @@ struct RuntimeApi {
   decltype(&::dnnrtConv) dnnrtConv = nullptr;
   decltype(&::dnnrtConvBiasActiv) dnnrtConvBiasActiv = nullptr;
   decltype(&::dnnrtConvBiasAddActiv) dnnrtConvBiasAddActiv = nullptr;
+  decltype(&::dnnrtConvBiasActivMaxPool) dnnrtConvBiasActivMaxPool = nullptr;
   decltype(&::dnnrtActive) dnnrtActive = nullptr;
   decltype(&::dnnrtTensorOp) dnnrtTensorOp = nullptr;
   decltype(&::dnnrtClip) dnnrtClip = nullptr;

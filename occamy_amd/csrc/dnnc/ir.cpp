@@ -48,6 +48,7 @@ const char *op_name(OpKind k) {
     case OP_CONV_BIAS_ADD_ACTIV: return "dnn.conv-bias-add-relufwd";
     case OP_MATMUL_BIAS: return "dnn.matmulnd-bias";
     case OP_ATTENTION: return "dnn.attention";
+    case OP_CONV_BIAS_ACTIV_MAXPOOL: return "dnn.conv-bias-relu-maxpoolfwd";
     case OP_RETURN: return "return";
   }
   return "?";
@@ -181,6 +182,19 @@ std::string Program::to_text() const {
         os << ", group=" << op->group;
         if (op->kind != OP_CONVFWD) os << ", activMode=" << op->mode;
         if (op->kind != OP_CONVFWD && (op->mode == 3 || op->mode == 6)) os << ", activCoef=" << op->coef;
+        os << "}";
+        break;
+      case OP_CONV_BIAS_ACTIV_MAXPOOL:
+        os << " {pads=";
+        print_shape(os, op->pads);
+        os << ", strides=";
+        print_shape(os, op->strides);
+        os << ", group=" << op->group << ", activMode=" << op->mode << ", poolKernel=";
+        print_shape(os, op->kernel);
+        os << ", poolPads=";
+        print_shape(os, op->pool_pads);
+        os << ", poolStrides=";
+        print_shape(os, op->pool_strides);
         os << "}";
         break;
       case OP_ACTIVATION: os << " {mode=" << op->mode << "}"; break;

@@ -129,6 +129,59 @@ void fuse_residual_add(Program &p) {
   }
 }
 
+// The first two layers of an ImageNet ResNet, conv 7x7 / stride 2 / pad 3 over the 3-channel function argument
+// (+ bias, ReLU or identity) -> max-pool 3x3 / stride 2 / pad 1, the convolution's result read by nothing else,
+// become one call that never stores that result (four times the pooled tensor).  Channels-last fp16 programs
+// only, and only this shape with an even image width: it is the one the runtime's kernel is written for, and the
+// runtime refuses everything else rather than fall back.  The reference has no such pattern
+// (src/Dialect/DNN/Transforms/fuseConvBiasRelu.cpp stops at the activation).
+void fuse_first_layer_maxpool(Program &p) {
+  std::vector<Op *> convs;
+  for (Op *op : p.ops)
+    if (op->kind == OP_CONV_BIAS_ACTIV && (op->mode == 1 || op->mode == 5)) convs.push_back(op);
+  for (Op *conv : convs) {
+    const Shape &dx = conv->dimA, &dw = conv->dimB;
+    if (dx.size() != 4 || dw.size() != 4 || conv->result->dtype != F16) continue;
+    if (dw[0] != 64 || dw[1] != 3 || dw[2] != 7 || dw[3] != 7 || conv->group != 1 || (dx[3] & 1)) continue;
+    if (conv->pads != Shape{3, 3} || conv->strides != Shape{2, 2}) continue;
+    // the input must be the device copy of a function argument (N,C,H,W as the host sent it)
+    bool from_arg = false;
+    for (const auto &u : conv->operands[0]->uses)
+      if (u.first->kind == OP_MEMCPY && u.first->mode == 1 && u.second == 0 && u.first->operands[1]->arg_index >= 0) from_arg = true;
+    if (!from_arg || conv->result->uses.size() != 1) continue;
+    Op *pool = conv->result->uses.front().first;
+    if (pool->kind != OP_MAXPOOL || pool->operands[0] != conv->result) continue;
+    if (pool->kernel != Shape{3, 3} || pool->strides != Shape{2, 2} || pool->pads.size() < 2 || pool->pads[0] != 1 || pool->pads[1] != 1)
+      continue;
+    if (pool->pads.size() == 4 && (pool->pads[2] != 1 || pool->pads[3] != 1)) continue;
+    Value *out = pool->operands[1];
+    Op *fused = p.new_op(OP_CONV_BIAS_ACTIV_MAXPOOL);
+    fused->pads = conv->pads;
+    fused->strides = conv->strides;
+    fused->group = conv->group;
+    fused->dimA = conv->dimA;
+    fused->dimB = conv->dimB;
+    fused->mode = conv->mode;
+    fused->kernel = pool->kernel;
+    fused->pool_pads = pool->pads;
+    fused->pool_strides = pool->strides;
+    fused->dimOut = pool->dimOut;
+    fused->result = p.new_value(out->dtype, out->shape);
+    fused->result->def = fused;
+    p.insert_after(fused, pool);  // where the pooling stood: its output buffer exists by then
+    p.set_operands(fused, {conv->operands[0], conv->operands[1], conv->operands[2], conv->operands[3], out});
+    p.replace_all_uses(pool->result, fused->result);
+    Value *conv_buf = conv->operands[4];
+    p.erase(pool);
+    p.erase(conv);
+    std::vector<Op *> deallocs;
+    for (const auto &u : conv_buf->uses)
+      if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+    for (Op *d : deallocs) p.erase(d);
+    if (conv_buf->uses.empty() && conv_buf->def) p.erase(conv_buf->def);
+  }
+}
+
 // conv+bias (identity) -> Clip(0, c) | LeakyRelu(alpha) | PRelu(one constant
 // slope), the convolution's result read by nothing else, becomes one fused
 // call with activation mode 3 (clipped ReLU, ceiling c) or 6 (leaky ReLU,

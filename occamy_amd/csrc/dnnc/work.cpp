@@ -11,6 +11,7 @@ const char *op_class(const Op *op) {
     case OP_CONVFWD:
     case OP_CONV_BIAS_ACTIV:
     case OP_CONV_BIAS_ADD_ACTIV: return (op->dimB[1] == 1 && op->group > 1) ? "conv_depthwise" : "conv_dense";
+    case OP_CONV_BIAS_ACTIV_MAXPOOL: return "conv_dense";
     case OP_MATMUL2D: return "gemm";
     case OP_MATMULND:
     case OP_MATMUL_BIAS: return "matmul";
@@ -48,6 +49,13 @@ void op_work(const Op *op, double &flops, double &bytes) {
       bytes = ((double)shape_numel(op->dimA) + (double)shape_numel(op->dimB) + n_out +
                (op->kind != OP_CONVFWD ? (double)op->dimB[0] : 0.0) +
                (op->kind == OP_CONV_BIAS_ADD_ACTIV ? n_out : 0.0)) * es;
+      break;
+    }
+    case OP_CONV_BIAS_ACTIV_MAXPOOL: {  // the convolution's products (its output extents, not the pooled ones); the pooling's compares are not counted
+      const Shape &dx = op->dimA, &dw = op->dimB;
+      const double P = (double)((dx[2] + 2 * op->pads[0] - dw[2]) / op->strides[0] + 1), Q = (double)((dx[3] + 2 * op->pads[1] - dw[3]) / op->strides[1] + 1);
+      flops = 2.0 * (double)dx[0] * (double)dw[0] * P * Q * (double)(dw[1] * dw[2] * dw[3]);
+      bytes = ((double)shape_numel(dx) + (double)shape_numel(dw) + (double)dw[0] + n_out) * es;
       break;
     }
     case OP_MATMUL2D: {

@@ -117,6 +117,14 @@ class Ops:
                                                         dims(strides), activ, Y, dtype),
                          "dnnrtConvBiasAddActiv")
 
+    def conv_bias_activ_max_pool(self, X, dimX, W, dimW, B, pads, strides, activ, kernel, pool_pads, pool_strides, Y, dimY,
+                                 group=1, dtype=_abi.F16):
+        dimB = [1, dimW[0], 1, 1]
+        return self._ret(self.lib.dnnrtConvBiasActivMaxPool(self.handle, X, dims(dimX), W, dims(dimW), B, dims(dimB), group,
+                                                            dims(pads), dims(strides), activ, dims(kernel), dims(pool_pads),
+                                                            dims(pool_strides), Y, dims(dimY), dtype),
+                         "dnnrtConvBiasActivMaxPool")
+
     def active(self, X, dimX, mode, Y, dtype=_abi.F32):
         d = list(dimX) + [1] * (4 - len(dimX))
         return self._ret(self.lib.dnnrtActive(self.handle, X, dims(d), mode, Y, dtype), "dnnrtActive")

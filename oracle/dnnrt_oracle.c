@@ -673,6 +673,31 @@ void *dnnrtAveragePool(dnnrtHandle_t h, const void *X, const int64_t *dX, void *
   (void)h; return pool_entry(X, dX, Y, dY, k, p, s, 0, dtype);
 }
 
+/* No reference wrapper of its own: the reference runs this as two calls,
+ * CUDNNConvBiasReluFunc.cpp:8-140 and CUDNNMaxPoolFunc.cpp:8-78, the first
+ * storing its result in the tensor's type.  Restated as exactly that chain,
+ * for any shape the two calls take (the GPU library's kernel takes one). */
+void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t h, const void *X, const int64_t *dX,
+                                const void *W, const int64_t *dW, const void *B,
+                                const int64_t *dB, int64_t group, const int64_t *pads,
+                                const int64_t *strides, int64_t act, const int64_t *pk,
+                                const int64_t *pp, const int64_t *ps, void *Y,
+                                const int64_t *dY, int32_t dtype) {
+  if (bad_dtype(dtype)) FAIL("convBiasActivMaxPool: bad dtype");
+  const int64_t P = (dX[2] + 2 * pads[0] - dW[2]) / strides[0] + 1,
+                Q = (dX[3] + 2 * pads[1] - dW[3]) / strides[1] + 1;
+  if (P < 1 || Q < 1) FAIL("convBiasActivMaxPool: empty convolution output");
+  const int64_t dC[4] = {dX[0], dW[0], P, Q};
+  const int64_t PP = (P + 2 * pp[0] - pk[0]) / ps[0] + 1, QQ = (Q + 2 * pp[1] - pk[1]) / ps[1] + 1;
+  if (dY[0] != dC[0] || dY[1] != dC[1] || dY[2] != PP || dY[3] != QQ) FAIL("convBiasActivMaxPool: dimY");
+  void *mid = malloc((size_t)(numel(dC, 4) * (dtype == DNNRT_F16 ? 2 : 4)));
+  if (!mid) FAIL("convBiasActivMaxPool: out of memory");
+  void *r = dnnrtConvBiasActiv(h, X, dX, W, dW, B, dB, NULL, 0, 0, group, pads, strides, act, mid, dtype);
+  if (r) r = dnnrtMaxPool(h, mid, dC, Y, dY, pk, pp, ps, dtype);
+  free(mid);
+  return r ? Y : NULL;
+}
+
 /* ---- matrix products ----------------------------------------------------- */
 
 /* C[M,N] = alpha * sum_k A(m,k) B(k,n) (+ beta * Cin), element strides given */

@@ -271,6 +271,39 @@ def test_fp16_channels_last_flag():
         g.compile(channels_last=True)  # fp32 graphs stay NCHW
 
 
+def test_first_layer_maxpool_fusion():
+    """conv 7x7/2 over the 3-channel argument + ReLU + max-pool 3x3/2 -> one call, in channels-last fp16 programs with
+    an even image width only; the convolution's buffer (the largest activation of the network) is never allocated."""
+    flags = dict(fusion=True, fuse_residual=True, channels_last=True)
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    plain = g.compile(**flags)
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    fused = g.compile(fuse_first_layer_maxpool=True, **flags)
+    assert plain.text.count("dnn.maxpool") == 1 and "maxpoolfwd" not in plain.text
+    assert fused.text.count("dnn.conv-bias-relu-maxpoolfwd") == 1 and "dnn.maxpool " not in fused.text
+    line = next(l for l in fused.text.splitlines() if "maxpoolfwd" in l)
+    assert "pads=[3,3], strides=[2,2], group=1, activMode=1, poolKernel=[3,3], poolPads=[1,1,1,1], poolStrides=[2,2]" in line
+    assert fused.num_ops(compute_only=True) == plain.num_ops(compute_only=True) - 1
+    assert fused.pool_bytes <= plain.pool_bytes
+    conv_bytes = 1 * 64 * 32 * 32 * 2  # the convolution's result at a 64 x 64 image, batch 1
+    sizes = lambda prog: sorted(b for k, _, b, _ in prog.events() if k == 0)
+    gone = list(sizes(plain))
+    gone.remove(conv_bytes)
+    assert sizes(fused) == gone
+    check_lifetimes(lambda: models.resnet50(dtype=np.float16, **SMALL), fuse_first_layer_maxpool=True, **flags)
+    # not without channels-last (the kernel writes N,H,W,C), not for fp32, not for an odd width
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    assert "maxpoolfwd" not in g.compile(fusion=True, fuse_first_layer_maxpool=True).text
+    g, _ = models.resnet50(dtype=np.float32, **SMALL)
+    assert "maxpoolfwd" not in g.compile(fusion=True, fuse_first_layer_maxpool=True).text
+    odd = dict(SMALL, image=SMALL.get("image", 32) + 1)
+    g, _ = models.resnet50(dtype=np.float16, **odd)
+    assert "maxpoolfwd" not in g.compile(fuse_first_layer_maxpool=True, **flags).text
+    # nor when something else reads the convolution's result
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    assert "maxpoolfwd" not in g.compile(fuse_first_layer_maxpool=True, channels_last=True).text  # no fusion flag: conv, add, relu apart
+
+
 def test_channels_last_refuses_what_it_cannot_lay_out():
     """A rank-4 constant with spatial extent reaches the device N,C,H,W (only convolution filters are re-laid at
     upload), and Flatten / Reshape copy bytes: channels_last must refuse both at compile time, not at run time."""

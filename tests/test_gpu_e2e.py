@@ -96,6 +96,8 @@ def test_poisoned_pool_changes_nothing_on_the_gpu():
              (lambda: models.mobilenet_v2(image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_activations=True)),
              (lambda: models.bert_encoder(layers=2), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)),
              (lambda: models.resnet50(4, np.float16, seed=5, image=64), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True)),
+             (lambda: models.resnet50(4, np.float16, seed=5, image=64),
+              dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True)),
              (lambda: models.srgan_generator(1, np.float32, height=24, width=16), dict(fusion=True, fuse_activations=True))]
     for builder, flags in cases:
         g, inputs = builder()
@@ -144,7 +146,7 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     """The throughput configuration at its own size and with the benchmark's own flags (64 x 3 x 224 x 224,
     fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
     oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
-    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True)
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True)
     build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
     out16, info = run(build16, **flags)
     assert info["requested"] == info["pool"]
@@ -203,6 +205,24 @@ def test_resnet50_fp16_channels_last(batch, image):
     s = p.session(compiler.MODE_RESIDENT)
     np.testing.assert_array_equal(s.run(*inputs)[0], out16[0])
     s.close()
+
+
+@pytest.mark.parametrize("batch,image", [(3, 64), (2, 224), (1, 90)])
+def test_first_layer_maxpool_fusion_fp16_channels_last(batch, image):
+    """The first convolution and its max-pool as one call: the same bits as this library's own two calls (same
+    products in the same order, an exact maximum), per inference and replayed from a captured graph, and the
+    fp32 oracle's result to the fp16 tolerance.  90 x 90: strips and steps that hang over the edge."""
+    build16 = lambda: models.resnet50(batch, np.float16, seed=5, image=image)  # noqa: E731
+    flags = dict(fusion=True, channels_last=True, fuse_residual=True, fuse_matmul_bias=True)
+    assert "maxpoolfwd" in build16()[0].compile(fuse_first_layer_maxpool=True, **flags).text
+    two, _ = run(build16, **flags)
+    one, info = run(build16, fuse_first_layer_maxpool=True, **flags)
+    assert info["requested"] == info["pool"]
+    np.testing.assert_array_equal(one[0], two[0])
+    res, _ = run(build16, mode=compiler.MODE_RESIDENT, fuse_first_layer_maxpool=True, **flags)
+    np.testing.assert_array_equal(res[0], one[0])
+    ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
+    np.testing.assert_allclose(one[0].astype(np.float32), ref[0], rtol=2e-2, atol=2e-2 * float(np.abs(ref[0]).max()))
 
 
 @pytest.mark.parametrize("name", ["resnet50", "mobilenet_v2"])

@@ -613,6 +613,89 @@ def test_conv_f16(gpu, cpu, case, fmt):
     np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
 
 
+def stem_pool_f16(gpu, x, w, b, activ, fmt=_abi.NCHW_TO_NHWC, kernel=(3, 3), ppads=(1, 1, 1, 1), pstrides=(2, 2)):
+    """The fused first layer through the C-ABI; x in N,C,H,W, w logical K,C,R,S; returns logical N,K,PP,QQ."""
+    N, C, H, W = x.shape
+    K = w.shape[0]
+    P, Q = oc.conv_out_hw(H, W, 7, 7, (3, 3), (2, 2))
+    PP, QQ = oc.conv_out_hw(P, Q, 3, 3, (1, 1), (2, 2))
+    X, Wt, B = gpu.put(x), gpu.put(np.ascontiguousarray(w.transpose(0, 2, 3, 1))), gpu.put(b)
+    Y = gpu.empty((N * K * PP * QQ,), np.float16)
+    gpu.ops.set_format(fmt)
+    try:
+        gpu.ops.conv_bias_activ_max_pool(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (3, 3), (2, 2), activ, kernel,
+                                         ppads, pstrides, gpu.ptr(Y), (N, K, PP, QQ))
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    return gpu.get(Y).reshape(N, PP, QQ, K).transpose(0, 3, 1, 2)
+
+
+@pytest.mark.parametrize("case", [(2, 32, 32), (2, 45, 38), (3, 64, 80), (1, 224, 224), (5, 23, 62), (70, 16, 16), (1, 7, 2)],
+                         ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("activ", [_abi.ACT_RELU, _abi.ACT_IDENTITY])
+def test_first_layer_with_its_max_pool_in_one_call(gpu, cpu, case, activ):
+    """dnnrtConvBiasActivMaxPool against the two calls it replaces: the oracle's chain to the convolution's
+    tolerance (one rounding to fp16 of an fp32 sum; the maximum adds none), and this library's own two calls
+    bit for bit (same products in the same order, then an exact maximum).  Identity activation leaves negative
+    values, so a padding of zeros instead of -inf would show; odd heights and widths that are not multiples of 28
+    leave ragged strips and a last pooled row and column whose windows hang over the edge."""
+    N, H, W = case
+    r = rng(N + H + W + activ)
+    x = r.standard_normal((N, 3, H, W)).astype(np.float16)
+    w = (r.standard_normal((64, 3, 7, 7)) * np.sqrt(2.0 / 147)).astype(np.float16)
+    b = r.uniform(-0.5, 0.1, 64).astype(np.float16)
+    if case == (5, 23, 62):
+        x[1, 2, 11, 30] = np.nan  # reaches a 4 x 4 block of convolution outputs of image 1, every channel
+        x[3, 0, 5, 40] = np.inf   # infinities of both signs in one window's reach: inf - inf is a NaN as well,
+        x[3, 1, 6, 41] = -np.inf  # and around it results of +inf and -inf
+    got = stem_pool_f16(gpu, x, w, b, activ)
+    conv_ref = oc.conv(cpu, x, w, b, (3, 3), (2, 2), 1, activ)
+    ref = oc.pool(cpu, "max", conv_ref, (3, 3), (1, 1), (2, 2))
+    assert got.shape == ref.shape
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3)
+    if case == (5, 23, 62):
+        assert np.isnan(got[1]).any() and np.isnan(got[3]).any() and not np.isnan(got[[0, 2, 4]]).any()
+        assert (np.isnan(got) == np.isnan(ref)).all()
+    # the two calls on the GPU, channels-last in between
+    conv_gpu = conv_f16(gpu, x, w, b, (3, 3), (2, 2), 1, activ, _abi.NCHW_TO_NHWC)       # logical NCHW
+    mid = gpu.put(np.ascontiguousarray(conv_gpu.transpose(0, 2, 3, 1)))
+    P, Q = conv_gpu.shape[2:]
+    PP, QQ = ref.shape[2:]
+    Y2 = gpu.empty((N * 64 * PP * QQ,), np.float16)
+    gpu.ops.set_format(_abi.NHWC)
+    try:
+        gpu.ops.maxpool(gpu.ptr(mid), (N, 64, P, Q), gpu.ptr(Y2), (N, 64, PP, QQ), (3, 3), (1, 1, 1, 1), (2, 2), _abi.F16)
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    two = gpu.get(Y2).reshape(N, PP, QQ, 64).transpose(0, 3, 1, 2)
+    np.testing.assert_array_equal(got, two)
+
+
+def test_first_layer_with_its_max_pool_refuses_other_shapes(gpu):
+    r = rng(3)
+    x = r.standard_normal((1, 3, 32, 32)).astype(np.float16)
+    w = r.standard_normal((64, 3, 7, 7)).astype(np.float16)
+    b = np.zeros(64, np.float16)
+    for kw, word in ((dict(fmt=_abi.NHWC), "NCHW_TO_NHWC"), (dict(kernel=(2, 2)), "3x3"), (dict(pstrides=(1, 1)), "stride 2"),
+                     (dict(ppads=(0, 0, 0, 0)), "pad 1")):
+        with pytest.raises(RuntimeError, match=word):
+            stem_pool_f16(gpu, x, w, b, _abi.ACT_RELU, **kw)
+    with pytest.raises(RuntimeError, match="even width"):
+        stem_pool_f16(gpu, r.standard_normal((1, 3, 32, 33)).astype(np.float16), w, b, _abi.ACT_RELU)
+    with pytest.raises(RuntimeError, match="7x7"):
+        w5 = r.standard_normal((64, 3, 5, 5)).astype(np.float16)
+        X, Wt, B = gpu.put(x), gpu.put(np.ascontiguousarray(w5.transpose(0, 2, 3, 1))), gpu.put(b)
+        Y = gpu.empty((64 * 8 * 8,), np.float16)
+        gpu.ops.set_format(_abi.NCHW_TO_NHWC)
+        try:
+            gpu.ops.conv_bias_activ_max_pool(gpu.ptr(X), x.shape, gpu.ptr(Wt), w5.shape, gpu.ptr(B), (2, 2), (2, 2), _abi.ACT_RELU,
+                                             (3, 3), (1, 1, 1, 1), (2, 2), gpu.ptr(Y), (1, 64, 8, 8))
+        finally:
+            gpu.ops.set_format(_abi.NCHW)
+
+
 # Problems of the size ResNet-50 has at batch 64: the dispatcher picks its large tiles (128 x 128 and up,
 # four or eight wavefronts) only when a launch has hundreds of tiles, so these are the only cases that reach
 # them.  N, C, H, W, K, R, stride, pad

@@ -274,6 +274,36 @@ def test_layernorm(be):
 
 # ---- pooling -----------------------------------------------------------------------------
 
+def test_conv_bias_activ_max_pool_is_the_chain_of_its_two_calls(be):
+    """The oracle's dnnrtConvBiasActivMaxPool against torch (fp64 convolution rounded to the tensor's type, then
+    max_pool2d: an independent statement of the chain) and against the oracle's own two calls, fp32 and fp16,
+    ReLU and identity, on a first-layer shape and on one that is not (the oracle takes any)."""
+    r = rng(21)
+    for dt, (N, C, H, W, K, R, st, pd), (pk, pp, ps) in [(np.float32, (2, 3, 33, 36, 64, 7, 2, 3), (3, 1, 2)),
+                                                        (np.float16, (2, 3, 33, 36, 64, 7, 2, 3), (3, 1, 2)),
+                                                        (np.float16, (1, 5, 12, 11, 7, 3, 1, 1), (2, 0, 2))]:
+        x = r.standard_normal((N, C, H, W)).astype(dt)
+        w = (r.standard_normal((K, C, R, R)) * 0.2).astype(dt)
+        b = r.uniform(-0.5, 0.5, K).astype(dt)
+        for act in (_abi.ACT_RELU, _abi.ACT_IDENTITY):
+            conv = oc.conv(be, x, w, b, (pd, pd), (st, st), 1, act)
+            chain = oc.pool(be, "max", conv, (pk, pk), (pp, pp), (ps, ps))
+            X, Wt, B = be.put(x), be.put(w), be.put(b)
+            Y = be.empty(chain.shape, dt)
+            be.ops.conv_bias_activ_max_pool(be.ptr(X), x.shape, be.ptr(Wt), w.shape, be.ptr(B), (pd, pd), (st, st), act, (pk, pk),
+                                            (pp, pp, pp, pp), (ps, ps), be.ptr(Y), chain.shape, dtype=oc.DT[np.dtype(dt)])
+            got = be.get(Y)
+            np.testing.assert_array_equal(got, chain)
+            c64 = F.conv2d(t64(x), t64(w), t64(b), st, pd)
+            if act == _abi.ACT_RELU:
+                c64 = c64.relu()
+            ref = F.max_pool2d(torch.from_numpy(c64.numpy().astype(dt).astype(np.float32)), pk, ps, pp).numpy()
+            np.testing.assert_allclose(got.astype(np.float32), ref, rtol=2e-3 if dt == np.float16 else 1e-5, atol=2e-3 if dt == np.float16 else 1e-5)
+    with pytest.raises(RuntimeError, match="dimY"):
+        be.ops.conv_bias_activ_max_pool(be.ptr(X), x.shape, be.ptr(Wt), w.shape, be.ptr(B), (pd, pd), (st, st), act, (pk, pk),
+                                        (pp, pp, pp, pp), (ps, ps), be.ptr(Y), (1, 7, 5, 5), dtype=_abi.F16)
+
+
 def test_pooling(be):
     r = rng(13)
     x = r.standard_normal((2, 3, 13, 12)).astype(np.float32)
