@@ -29,7 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
-RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool")
+RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool", "alias_copies")
 
 
 def build_workload(name, batch=None):
@@ -37,17 +37,18 @@ def build_workload(name, batch=None):
     from occamy_amd import models
     if name == "resnet50_fp32_bs1":
         b = batch or 1
-        return models.resnet50(b, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True), b, "img/s", "f32"
+        return models.resnet50(b, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, alias_copies=True), b, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
         b = batch or 64
         return (models.resnet50(b, np.float16, seed=5),
-                dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True), b, "img/s", "f16")
+                dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True, alias_copies=True),
+                b, "img/s", "f16")
     if batch is not None:
         raise SystemExit(f"{name}: no batch override")
     if name == "mobilenet_v2_fp32_bs1":
-        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True), 1, "img/s", "f32"
+        return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True, alias_copies=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
-        return models.bert_encoder(), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True), 1, "seq/s", "f32"
+        return models.bert_encoder(), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True, alias_copies=True), 1, "seq/s", "f32"
     if name == "single_conv_fp32":
         return models.single_conv(), dict(fusion=True), 1, "img/s", "f32"
     if name == "alexnet_fp32_bs1":
@@ -220,7 +221,7 @@ def record(res, steps, warmup, cpu_seconds):
         "value": res["value"], "unit": res["unit"], "steps": steps, "warmup": warmup, "ms_per_step": res["ms_per_step"],
         "latency_ms": res["latency_ms"], "dtype": res["dtype"], "data": "synthetic",
         "config": {"workload": res["name"], "batch": res["batch"],
-                   "fusion": ", ".join(k for k, v in res["flags"].items() if v and (k.startswith("fus") or k == "recompose")),
+                   "fusion": ", ".join(k for k, v in res["flags"].items() if v and (k.startswith("fus") or k in ("recompose", "alias_copies", "channels_last"))),
                    "mode": "weights and input resident in HBM, kernels replayed from a captured graph",
                    "kernels_per_step": res["kernels_per_step"]},
         "roofline": roofline_of(res),

@@ -68,6 +68,8 @@ typedef struct {
                              convolution (3 -> 64 channels, 7x7, stride 2, pad 3, even image width, ReLU or
                              identity) and the 3x3 / stride 2 / pad 1 max-pool behind it become one call
                              that never stores the convolution's result (default 0) */
+  int32_t alias_copies;   /* no reference flag: Flatten / Reshape / Squeeze / Unsqueeze name their input's buffer
+                             as their output, so nothing is copied and nothing launched (default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);

@@ -134,6 +134,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (opt->fusion && opt->fuse_matmul_bias) fuse_matmul_bias(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
   if (opt->fusion && opt->fuse_first_layer_maxpool && opt->channels_last) fuse_first_layer_maxpool(p);
+  if (opt->alias_copies) alias_copies(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {
     // Only fp16 programs whose rank-4 tensors flow through layout-aware calls
@@ -244,7 +245,7 @@ int64_t dnncProgramNumOps(const dnncProgram *p, int32_t compute_only) {
   if (!p) return -1;
   int64_t n = 0;
   for (const Op *op : p->p.ops)
-    if (!compute_only || (op->kind >= OP_CONVFWD && op->kind < OP_RETURN)) n++;
+    if (!compute_only || launches(op)) n++;
   return n;
 }
 
@@ -252,7 +253,7 @@ int32_t dnncProgramComputeOp(const dnncProgram *p, int64_t i, const char **name,
   if (!p || !name || !work_class || !flops || !bytes) return fail("dnncProgramComputeOp: bad arguments");
   int64_t n = 0;
   for (const Op *op : p->p.ops) {
-    if (op->kind < OP_CONVFWD || op->kind >= OP_RETURN) continue;
+    if (!launches(op)) continue;
     if (n++ != i) continue;
     *name = op_name(op->kind);
     *work_class = op_class(op);

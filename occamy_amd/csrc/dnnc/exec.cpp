@@ -234,6 +234,12 @@ bool Session::issue(const Op *op, std::string &err) {
       cur_act_coef = op->coef;
     }
   }
+  // a copy whose output buffer is its input's (the alias_copies pass): nothing to do
+  if ((op->kind == OP_FLATTEN || op->kind == OP_RESHAPE || op->kind == OP_SQUEEZE || op->kind == OP_UNSQUEEZE) &&
+      op->operands.size() == 2 && P(0) == out) {
+    ptr[(size_t)op->result->id] = out;
+    return true;
+  }
   void *r = nullptr;
   auto pad4 =[](const Shape &s) { Shape o = s; while (o.size() < 4) o.push_back(1); return o; };
   switch (op->kind) {
@@ -516,9 +522,17 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
 
 bool Session::profile_resident(const void *const *inputs, int on_device, bool by_class, std::vector<float> &ms, std::string &err) {
   if (mode != MODE_RESIDENT) { err = "profiling needs a resident session"; return false; }
+  // the operations that launch something, in program order (an aliased copy only hands its input's address on;
+  // a first eager pass has set those)
   std::vector<const Op *> compute;
   for (const Op *op : prog->ops)
-    if (is_compute(op->kind)) compute.push_back(op);
+    if (launches(op)) compute.push_back(op);
+  for (const Op *op : prog->ops)
+    if (is_compute(op->kind) && !launches(op) && !ptr[(size_t)op->result->id]) {
+      std::string e2;
+      if (!issue_all_compute(e2)) { err = e2; return false; }
+      break;
+    }
   if (by_class) return profile_classes(inputs, on_device, compute, ms, err);
   std::vector<void *> ev(compute.size() + 1, nullptr);
   bool ok = true;

@@ -72,6 +72,7 @@ enum OpKind {
   OP_RETURN
 };
 const char *op_name(OpKind k);
+inline bool is_compute_kind(OpKind k) { return k >= OP_CONVFWD && k < OP_RETURN; }
 
 struct Op;
 struct Value {
@@ -99,6 +100,17 @@ struct Op {
   int out_index = -1;              // OP_HOST_ALLOC: which function result
   std::list<Op *>::iterator pos;   // position in Program::ops
 };
+
+// A Flatten / Reshape / Squeeze / Unsqueeze whose output buffer is the buffer its input lives in (the alias_copies
+// pass): it launches nothing.
+inline bool is_aliased_copy(const Op *op) {
+  if ((op->kind != OP_FLATTEN && op->kind != OP_RESHAPE && op->kind != OP_SQUEEZE && op->kind != OP_UNSQUEEZE) || op->operands.size() != 2)
+    return false;
+  const Value *x = op->operands[0], *out = op->operands[1];
+  return x == out || (x->def && is_compute_kind(x->def->kind) && !x->def->operands.empty() && x->def->operands.back() == out);
+}
+// One runtime call per such operation
+inline bool launches(const Op *op) { return is_compute_kind(op->kind) && !is_aliased_copy(op); }
 
 // One allocation event of the final program, in execution order.
 struct PoolEvent {
@@ -170,6 +182,7 @@ void fuse_residual_add(Program &p);
 void fuse_conv_activations(Program &p);
 void fuse_matmul_bias(Program &p);
 void fuse_first_layer_maxpool(Program &p);
+void alias_copies(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);
 bool malloc_pool_opt(Program &p, std::string &err);

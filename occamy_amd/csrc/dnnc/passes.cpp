@@ -182,6 +182,41 @@ void fuse_first_layer_maxpool(Program &p) {
   }
 }
 
+// Flatten, Reshape, Squeeze and Unsqueeze move no element: the reference copies the tensor into a buffer of its
+// own (src/Tools/dnn-wrapper/cuda/CUDAFlattenFunc.cu and its three siblings are device-to-device copies), here the
+// operation can instead name its input's buffer as its output buffer.  The executor launches nothing for an
+// operation whose input and output are the same address; the buffer lives on under the result's readers (the
+// dealloc pass follows a result back to the buffer its producer names last), and the copy's own buffer and
+// launch are gone.  Not done when anything else writes the input's buffer.
+void alias_copies(Program &p) {
+  std::vector<Op *> copies;
+  for (Op *op : p.ops)
+    if ((op->kind == OP_FLATTEN || op->kind == OP_RESHAPE || op->kind == OP_SQUEEZE || op->kind == OP_UNSQUEEZE) &&
+        op->operands.size() == 2)
+      copies.push_back(op);
+  for (Op *op : copies) {
+    Value *x = op->operands[0], *old_out = op->operands[1];
+    Value *buf = nullptr;
+    if (x->def && x->def->kind == OP_MALLOC) buf = x;
+    else if (x->def && x->def->kind >= OP_CONVFWD && x->def->kind < OP_RETURN && !x->def->operands.empty()) buf = x->def->operands.back();
+    if (!buf || !buf->def || buf->def->kind != OP_MALLOC || buf == old_out) continue;
+    if (shape_numel(buf->shape) * dtype_bytes(buf->dtype) != shape_numel(old_out->shape) * dtype_bytes(old_out->dtype)) continue;
+    bool other_writer = false;
+    for (const auto &u : buf->uses)
+      if (u.first != x->def && u.first->kind != OP_MEMCPY && u.first->kind != OP_DEALLOC && !u.first->operands.empty() &&
+          u.first->operands.back() == buf)
+        other_writer = true;
+    if (other_writer) continue;
+    p.set_operands(op, {x, buf});
+    std::vector<Op *> deallocs;
+    for (const auto &u : old_out->uses)
+      if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
+    if (old_out->uses.size() != deallocs.size()) continue;  // something else uses the old buffer: leave it allocated
+    for (Op *d : deallocs) p.erase(d);
+    if (old_out->def && old_out->def->kind == OP_MALLOC) p.erase(old_out->def);
+  }
+}
+
 // conv+bias (identity) -> Clip(0, c) | LeakyRelu(alpha) | PRelu(one constant
 // slope), the convolution's result read by nothing else, becomes one fused
 // call with activation mode 3 (clipped ReLU, ceiling c) or 6 (leaky ReLU,

@@ -244,6 +244,39 @@ def test_activation_fusion_matches_unfused_chain(builder):
         np.testing.assert_array_equal(x, y)
 
 
+@pytest.mark.parametrize("builder,copies", [(lambda: models.resnet50(image=32, classes=10), 1), (ALEX, 1),
+                                            (lambda: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128), None),
+                                            (YOLO, None)],
+                         ids=["resnet50", "alexnet", "bert", "yolo_v1"])
+def test_aliased_copies_change_nothing(builder, copies):
+    """Flatten / Reshape / Squeeze / Unsqueeze on their input's buffer: every copy leaves the launch count and its
+    buffer leaves the pool's event trace, the results keep every bit (per inference, with the dealloc pass on and
+    off, and resident), and no tensor is read after its buffer was released (the debug fill would turn that
+    into NaN)."""
+    _, _, a = run_oracle(builder, fusion=True)
+    plain = builder()[0].compile(fusion=True)
+    aliased = builder()[0].compile(fusion=True, alias_copies=True)
+    n = sum(plain.text.count(k) for k in ("dnn.flatten", "dnn.reshape", "dnn.squeeze", "dnn.unsqueeze"))
+    assert n >= 1 and (copies is None or n == copies)
+    gone = plain.num_ops(compute_only=True) - aliased.num_ops(compute_only=True)
+    assert 1 <= gone <= n and (copies is None or gone == copies)
+    assert len(aliased.events()) == len(plain.events()) - 2 * gone
+    assert aliased.pool_bytes <= plain.pool_bytes
+    for flags in (dict(), dict(dealloc_opt=False)):
+        _, _, b = run_oracle(builder, fusion=True, alias_copies=True, **flags)
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+    _, _, c = run_oracle(builder, mode=compiler.MODE_RESIDENT, fusion=True, alias_copies=True)
+    for x, y in zip(a, c):
+        np.testing.assert_array_equal(x, y)
+    g, inputs = builder()
+    s = g.compile(fusion=True, alias_copies=True).session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+    s.set_debug_fill(0xFF)
+    for x, y in zip(a, s.run(*inputs)):
+        np.testing.assert_array_equal(x, y)
+    s.close()
+
+
 @pytest.mark.parametrize("builder", [lambda: models.resnet50(image=32, classes=10), ALEX,
                                      lambda: models.mobilenet_v2(image=32, classes=10)],
                          ids=["resnet50", "alexnet", "mobilenet_v2"])

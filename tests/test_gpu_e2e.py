@@ -146,7 +146,7 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     """The throughput configuration at its own size and with the benchmark's own flags (64 x 3 x 224 x 224,
     fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
     oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
-    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True)
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True, alias_copies=True)
     build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
     out16, info = run(build16, **flags)
     assert info["requested"] == info["pool"]
@@ -172,9 +172,9 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
 
 
 def test_bert_base_12_layers_as_benchmarked():
-    """BERT-base at its full depth with the benchmark's four flags, against the oracle running the unfused
+    """BERT-base at its full depth with the benchmark's flags, against the oracle running the unfused
     program (tolerance: rtol 1e-4, atol 1e-4 on outputs of order one after the final LayerNorm)."""
-    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True)
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True, alias_copies=True)
     ref, _ = run(models.bert_encoder, ORACLE_PATH)
     out, info = run(models.bert_encoder, **flags)
     assert info["requested"] == info["pool"]
@@ -223,6 +223,29 @@ def test_first_layer_maxpool_fusion_fp16_channels_last(batch, image):
     np.testing.assert_array_equal(res[0], one[0])
     ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
     np.testing.assert_allclose(one[0].astype(np.float32), ref[0], rtol=2e-2, atol=2e-2 * float(np.abs(ref[0]).max()))
+
+
+def test_aliased_copies_change_nothing_on_the_gpu():
+    """Flatten / Reshape on their input's buffer: one launch fewer per copy and the same bits, per inference, with
+    a poisoned pool, and replayed from a captured graph; fp32 ResNet-50, a BERT whose reshapes survive the
+    attention fusion's absence, fp16 channels-last ResNet-50."""
+    cases = [(lambda: models.resnet50(image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True)),
+             (lambda: models.bert_encoder(layers=2), dict(recompose=True, fusion=True, fuse_matmul_bias=True)),
+             (lambda: models.resnet50(4, np.float16, seed=5, image=64), dict(fusion=True, fuse_residual=True, channels_last=True))]
+    for builder, flags in cases:
+        plain, _ = run(builder, **flags)
+        g, inputs = builder()
+        p = g.compile(alias_copies=True, **flags)
+        assert p.num_ops(compute_only=True) < builder()[0].compile(**flags).num_ops(compute_only=True)
+        s = p.session(compiler.MODE_OCCAMY)
+        s.set_debug_fill(0xFF)
+        np.testing.assert_array_equal(s.run(*inputs)[0], plain[0])
+        s.close()
+        s = p.session(compiler.MODE_RESIDENT)
+        for _ in range(2):
+            np.testing.assert_array_equal(s.run(*inputs)[0], plain[0])
+        assert len(s.profile(inputs)) == p.num_ops(compute_only=True)
+        s.close()
 
 
 @pytest.mark.parametrize("name", ["resnet50", "mobilenet_v2"])
