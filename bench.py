@@ -29,7 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
-RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool", "alias_copies")
+RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool", "fuse_projection_shortcut", "alias_copies")
 
 
 def build_workload(name, batch=None):
@@ -41,7 +41,8 @@ def build_workload(name, batch=None):
     if name == "resnet50_fp16_bs64":
         b = batch or 64
         return (models.resnet50(b, np.float16, seed=5),
-                dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True, alias_copies=True),
+                dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True,
+                     alias_copies=True),
                 b, "img/s", "f16")
     if batch is not None:
         raise SystemExit(f"{name}: no batch override")

@@ -235,6 +235,23 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X,
                                 const int64_t *poolPads,
                                 const int64_t *poolStrides, void *Y,
                                 const int64_t *dimY, int32_t dtype);
+/* New: a residual block's last convolution and its projection shortcut in
+ * one kernel: Y = act((conv(X, W) + B) + (conv(X2, W2) + B2)).  It replaces
+ * dnnrtConvBiasActiv (identity) on the shortcut followed by
+ * dnnrtConvBiasAddActiv with that result as Z; the shortcut's result is then
+ * never stored or read.  Every element is what the two calls would store:
+ * each conv + bias rounded to fp16 on its own, the sum and the activation in
+ * fp32, one more rounding.  fp16, tensor format DNNRT_NHWC, filters K,R,S,C;
+ * both convolutions 1x1 without padding, the first with stride 1, the second
+ * with any stride, input channel counts multiples of 64, onto the same
+ * [N, K, P, Q] result; group 1; B and B2 may be null.  Anything else fails
+ * with an error. */
+void *dnnrtConvBiasAddConvBiasActiv(
+    dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
+    const int64_t *dimW, const void *B, const int64_t *pads,
+    const int64_t *strides, const void *X2, const int64_t *dimX2,
+    const void *W2, const int64_t *dimW2, const void *B2, const int64_t *pads2,
+    const int64_t *strides2, int64_t activMode, void *Y, int32_t dtype);
 /* No counterpart in the reference.  dnnrtConvBiasActiv for callers that cannot
  * allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It takes the stream where the other calls

@@ -49,6 +49,7 @@ SIGNATURES = {
     "dnnrtConvBiasActiv": (P, [P, P, I64P, P, I64P, P, I64P, P, i64, i64, i64, I64P, I64P, i64, P, i32]),
     "dnnrtConvBiasAddActiv": (P, [P, P, I64P, P, I64P, P, I64P, P, P, i64, i64, i64, I64P, I64P, i64, P, i32]),
     "dnnrtConvBiasActivMaxPool": (P, [P, P, I64P, P, I64P, P, I64P, i64, I64P, I64P, i64, I64P, I64P, I64P, P, I64P, i32]),
+    "dnnrtConvBiasAddConvBiasActiv": (P, [P, P, I64P, P, I64P, P, I64P, I64P, P, I64P, P, I64P, P, I64P, I64P, i64, P, i32]),
     "dnnrtConvBiasActivNoAlloc": (P, [P, P, I64P, P, I64P, P, I64P, i64, I64P, I64P, i64, P, i32]),
     "dnnrtActive": (P, [P, P, I64P, i32, P, i32]),
     "dnnrtTensorOp": (P, [P, i64, P, I64P, i32, P, I64P, i32, P, I64P, i32, f32, i32]),

@@ -403,6 +403,35 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64
   return Y;
 }
 
+void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W, const int64_t *dimW,
+                                    const void *B, const int64_t *pads, const int64_t *strides, const void *X2,
+                                    const int64_t *dimX2, const void *W2, const int64_t *dimW2, const void *B2,
+                                    const int64_t *pads2, const int64_t *strides2, int64_t activMode, void *Y, int32_t dtype) {
+  const char *who = "dnnrtConvBiasAddConvBiasActiv";
+  if (!handle) DNNRT_FAIL("%s: null handle", who);
+  if (!X || !W || !X2 || !W2 || !Y) DNNRT_FAIL("%s: null tensor", who);
+  if (dtype != DNNRT_F16) DNNRT_FAIL("%s: fp16 tensors only", who);
+  if (!dnnrt::fusable_act(activMode)) DNNRT_FAIL("%s: activMode %ld (1 ReLU, 3 clipped ReLU, 5 identity, 6 leaky ReLU)", who, (long)activMode);
+  dnnrt::ConvShape s1, s2;
+  if (!dnnrt::parse_conv(who, dimX, dimW, 1, pads, strides, s1) || !dnnrt::parse_conv(who, dimX2, dimW2, 1, pads2, strides2, s2)) return nullptr;
+  if (s1.N != s2.N || s1.K != s2.K || s1.P != s2.P || s1.Q != s2.Q)
+    DNNRT_FAIL("%s: the two convolutions give [%d,%d,%d,%d] and [%d,%d,%d,%d]", who, s1.N, s1.K, s1.P, s1.Q, s2.N, s2.K, s2.P, s2.Q);
+  if (s1.R != 1 || s1.S != 1 || s2.R != 1 || s2.S != 1 || s1.ph || s1.pw || s2.ph || s2.pw || s1.sh != 1 || s1.sw != 1)
+    DNNRT_FAIL("%s: both convolutions must be 1x1 without padding, the first with stride 1", who);
+  dnnrt::ConvF16Args a{};
+  a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Z = nullptr; a.Y = (__half *)Y;
+  a.N = s1.N; a.C = s1.C; a.H = s1.H; a.W = s1.W; a.K = s1.K; a.Cg = s1.Cg; a.R = 1; a.S = 1;
+  a.P = s1.P; a.Q = s1.Q; a.ph = 0; a.pw = 0; a.sh = 1; a.sw = 1; a.group = 1;
+  a.act = (int)activMode; a.act_coef = handle->act_coef; a.format = handle->format;
+  a.X2 = (const __half *)X2; a.Wt2 = (const __half *)W2; a.bias2 = (const __half *)B2;
+  a.C2 = s2.C; a.H2 = s2.H; a.W2 = s2.W; a.sh2 = s2.sh; a.sw2 = s2.sw;
+  if (!dnnrt::dual_conv_applies(a))
+    DNNRT_FAIL("%s: channels-last (DNNRT_NHWC) tensors with channel counts that are multiples of 64 (inputs) and 8 (result), "
+               "16-byte aligned, below 2^31 elements", who);
+  if (!dnnrt::launch_conv_f16_dual(handle, a)) return nullptr;
+  return Y;
+}
+
 void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
                             const int64_t *dimW, const void *B, const int64_t *dimB, const void *Z,
                             void *workspace, int64_t workspaceBytes, int64_t algo, int64_t group,

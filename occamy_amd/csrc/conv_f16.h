@@ -14,9 +14,17 @@ struct ConvF16Args {
   int format;  // physical layout of X and Y (DNNRT_NCHW / NHWC / NCHW_TO_NHWC)
   unsigned magic_pq, magic_q;  // filled in by the launcher: ceil(2^32 / (P*Q)), ceil(2^32 / Q)
   unsigned magic_pw, magic_hp;  // (conv_f16_patch.hip) ceil(2^32 / (W + 2)), ceil(2^32 / (H + 2))
+  // a second 1x1 convolution onto the same result (launch_conv_f16_dual): input N x H2 x W2 x C2 read with strides
+  // sh2, sw2, filter K x C2, bias or null
+  const __half *X2, *Wt2, *bias2;
+  int C2, H2, W2, sh2, sw2;
 };
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a);
+// Y = act(fp16(conv(X, W) + bias) + fp16(conv(X2, W2) + bias2)), both convolutions 1x1 without padding (a residual
+// block's last convolution and its projection shortcut); `a` must satisfy dual_conv_applies.
+bool dual_conv_applies(const ConvF16Args &a);
+bool launch_conv_f16_dual(const dnnrtContext *ctx, const ConvF16Args &a);
 // Channels-last 1x1 stride-1 layers over at most this many output pixels (a fully connected layer at small batch).
 constexpr int FEWPIX_MAX_PIXELS = 64;
 bool launch_conv_f16_fewpix(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);

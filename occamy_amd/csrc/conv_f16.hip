@@ -75,9 +75,17 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // over 64 n channels) and they take turns in ONE LDS stage instead of
 // alternating between two: half the LDS, so more workgroups fit a CU, and
 // what these layers need is memory requests in flight, not MFMA time.
-template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG, int FEW_STEPS = 0>
+// DUAL: two 1x1 convolutions (no padding) onto the same output tile, Y = act(fp16(conv(X, W) + bias) +
+// fp16(conv(X2, W2) + bias2)) — a residual block's last convolution and its projection shortcut.  The second
+// convolution's steps come first, into the same accumulators; where its reduction ends they are rounded to fp16
+// with its bias, exactly what it would have stored as a convolution of its own, and set aside; the epilogue adds
+// them as it adds a residual tensor, which is then never written or read.  With FEW_STEPS the turns are
+// DUAL_FIRST steps of the second convolution, then the first's.
+template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG, int FEW_STEPS = 0, bool DUAL = false,
+          int DUAL_FIRST = 0>
 __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefronts per SIMD the register budget must allow
  void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
+  static_assert(!DUAL || KG == 1, "the two-convolution form is written for one k group");
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(KG == 1 || KG == 2, "one or two k groups");
@@ -109,6 +117,8 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
 
   const char *__restrict__ Xg = reinterpret_cast<const char *>(a.X);
   const char *__restrict__ Wg = reinterpret_cast<const char *>(a.Wt);
+  const char *__restrict__ X2g = reinterpret_cast<const char *>(a.X2);
+  const char *__restrict__ W2g = reinterpret_cast<const char *>(a.Wt2);
 
   // ---- loader constants ------------------------------------------------
   // chunk id -> (row of the tile, 16-byte chunk of the row's 64-byte k slice).
@@ -116,18 +126,19 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   // dispatcher checks the tensors are below 4 GiB), so the loads use the
   // scalar-base + 32-bit vector-offset form: no 64-bit address arithmetic and
   // no address registers that outlive the load.
-  unsigned a_off[A_CH], a_msk[A_CH];
+  unsigned a_off[A_CH], a_msk[A_CH], a_off2[DUAL ? A_CH : 1];
 #pragma unroll
   for (int i = 0; i < A_CH; i++) {
     const int id = tid + i * NT, row = id >> 3, ch = id & 7;
     const int k_out = m0 + row;
     const bool ok = k_out < a.K;
     a_off[i] = 2u * (unsigned)((ok ? k_out : 0) * CRS + ch * 8);
+    if (DUAL) a_off2[i] = 2u * (unsigned)((ok ? k_out : 0) * a.C2 + ch * 8);
     a_msk[i] = ok ? 0xffffffffu : 0u;
   }
   // B (im2col): a chunk belongs to one output pixel; bit (r * S + s) of
   // b_taps says whether that tap reads inside the image.
-  int b_pix[B_CH];
+  int b_pix[B_CH], b_pix2[DUAL ? B_CH : 1];
   unsigned b_taps[B_CH];
 #pragma unroll
   for (int i = 0; i < B_CH; i++) {
@@ -139,6 +150,7 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
     const int p = div_magic(pq, a.Q, a.magic_q), q = pq - p * a.Q;
     const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
     b_pix[i] = 2 * (((n * a.H + ih0) * a.W + iw0) * a.C + ch * 8);  // bytes; negative inside the padding
+    if (DUAL) b_pix2[i] = 2 * (((n * a.H2 + p * a.sh2) * a.W2 + q * a.sw2) * a.C2 + ch * 8);
     unsigned taps = 0;
     if (MASKED && ok) {
       // taps (r, s) inside the image: r in [r_lo, r_hi), s in [s_lo, s_hi)
@@ -154,12 +166,33 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   u32x4 ra[DEPTH][A_CH], rb[DEPTH][B_CH];
   unsigned rm[DEPTH][B_CH];
 
-  const int steps_c = a.C / BKF, nk = a.R * a.S * steps_c;
+  const int steps_c = a.C / BKF, nk2 = DUAL ? a.C2 / BKF : 0, nk = a.R * a.S * steps_c + nk2;
   // cursor of the next step to load (wave-uniform); it stops at the last step,
   // so loads issued past the end re-read that step and are never used
   int lj = 0, l_r = 0, l_s = 0, l_c0 = 0;
 
   auto load_step = [&](u32x4 (&qa)[A_CH], u32x4 (&qb)[B_CH], unsigned (&qm)[B_CH]) {
+    if (DUAL) {  // both convolutions 1x1: step lj is 64 channels of the second one (lj < nk2), then of the first
+      const bool second = lj < nk2;
+      const unsigned k_off = 2u * (unsigned)(second ? lj : lj - nk2) * BKF;
+      const char *__restrict__ wb = second ? W2g : Wg;
+      const char *__restrict__ xb = second ? X2g : Xg;
+#pragma unroll
+      for (int i = 0; i < A_CH; i++) qa[i] = load_global_16(wb + ((second ? a_off2[i] : a_off[i]) + k_off));
+#pragma unroll
+      for (int i = 0; i < B_CH; i++) {
+        const unsigned off = (unsigned)(second ? b_pix2[i] : b_pix[i]) + k_off;
+        if (MASKED) {
+          const unsigned m = 0u - (b_taps[i] & 1u);
+          qm[i] = m;
+          qb[i] = load_global_16(xb + (off & m));
+        } else {
+          qb[i] = load_global_16(xb + off);
+        }
+      }
+      lj = lj + 1 < nk ? lj + 1 : lj;
+      return;
+    }
     const unsigned w_off = 2u * (unsigned)lj * BKF;
     const int x_off = 2 * ((l_r * a.W + l_s) * a.C + l_c0);
     const int tap = l_r * a.S + l_s;
@@ -236,6 +269,27 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
       }
   }
 
+  // the second convolution's result, as it would have been stored: set aside when its steps are done
+  floatx16 zacc[DUAL ? TM : 1][DUAL ? TN : 1];
+  auto set_aside = [&]() __attribute__((always_inline)) {
+    const _Float16 *__restrict__ bias2g = reinterpret_cast<const _Float16 *>(a.bias2);
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int k_out = m0 + wm0 + i * 32 + 8 * g + 4 * half;
+        half4 b2 = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+        if (bias2g) b2 = *reinterpret_cast<const half4 *>(bias2g + (k_out < a.K ? k_out : 0));
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            zacc[DUAL ? i : 0][DUAL ? j : 0][4 * g + e] = (float)(_Float16)(acc[i][j][4 * g + e] + (float)b2[e]);
+            acc[i][j][4 * g + e] = 0.f;
+          }
+      }
+  };
+
   half8 fa[2][TM], fb[2][TN];
   auto read_frags = [&](int stage, half8 (&qa)[TM], half8 (&qb)[TN], int sub) {  // sub: which k16 of the step
     const _Float16 *As = smem + stage * STAGE, *Bs = As + BM * LDS_ROW;
@@ -301,18 +355,27 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   const integral_constant<int, 0> slot0{};
   const integral_constant<int, 1> slot1{};
   int kt = 0;
+  // (two-convolution form: before step nk2 the accumulators change hands; nk2 is even and at least two here, so
+  // that happens before a pair of steps: three places in the code, each a copy of 2 x 16 x TM x TN register moves)
   if constexpr (!ONE_STAGE) {
     for (; kt + 4 <= nk; kt += 2) {  // both steps have a step two ahead to request
+      if constexpr (DUAL) {
+        if (kt == nk2) set_aside();
+      }
       step(slot0, true_type{}, true_type{});
       step(slot1, true_type{}, true_type{});
     }
   }
   const int rem = ONE_STAGE ? 0 : nk - kt;  // 1, 2 or 3
+  if constexpr (DUAL && !ONE_STAGE) {
+    if (kt == nk2) set_aside();
+  }
   if constexpr (ONE_STAGE) {
     // step T: its data goes from register slot T % 2 into the one stage (step 0's is there already), the
     // slot is refilled with step T + 2 if there is one, then the MFMAs read the stage
     auto turn = [&](auto t_c) {
       constexpr int T = decltype(t_c)::value, U = T & 1;
+      if constexpr (DUAL && T == DUAL_FIRST) set_aside();
       if constexpr (T > 0) {
         store_step(0, ra[U], rb[U], rm[U]);
         __syncthreads();
@@ -328,6 +391,9 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   } else if (rem == 3) {
     step(slot0, true_type{}, true_type{});
     step(slot1, false_type{}, true_type{});
+    if constexpr (DUAL) {
+      if (kt + 2 == nk2) set_aside();  // (a single step of the first convolution behind an even number of the second's)
+    }
     step(slot0, false_type{}, false_type{});
   } else if (rem == 2) {
     step(slot0, false_type{}, true_type{});
@@ -401,8 +467,13 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
             const int kl = wm0 + i * 32 + 8 * g + 4 * half;  // k_out within the tile
             half4 o;
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-              o[e] = (_Float16)apply_act(acc[i][j][4 * g + e] + (float)bias4[i][g][e], MODE, a.act_coef);
+            for (int e = 0; e < 4; e++) {
+              if (DUAL)  // conv + bias rounded as a convolution of its own would store it, then the sum in fp32
+                o[e] = (_Float16)apply_act((float)(_Float16)(acc[i][j][4 * g + e] + (float)bias4[i][g][e]) +
+                                               zacc[DUAL ? i : 0][DUAL ? j : 0][4 * g + e], MODE, a.act_coef);
+              else
+                o[e] = (_Float16)apply_act(acc[i][j][4 * g + e] + (float)bias4[i][g][e], MODE, a.act_coef);
+            }
             *reinterpret_cast<half4 *>(Cs + (wn0 + j * 32 + l32) * CROW + kl) = o;
           }
     });
@@ -510,6 +581,50 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
     v = apply_act(v, a.act, a.act_coef);
     Yg[off] = (_Float16)v;
   }
+}
+
+// Y = act(fp16(conv(X, W) + bias) + fp16(conv(X2, W2) + bias2)): `a` with its X2 / Wt2 / bias2 / C2 / H2 / W2 / sh2 / sw2
+// fields set.  Both convolutions 1x1 without padding onto the same N x K x P x Q result (dual_conv_applies).
+bool dual_conv_applies(const ConvF16Args &a) {
+  return a.format == DNNRT_NHWC && a.group == 1 && a.R == 1 && a.S == 1 && a.ph == 0 && a.pw == 0 && a.Z == nullptr && a.X2 && a.Wt2 &&
+         a.C % 64 == 0 && a.C2 % 64 == 0 && a.K % 8 == 0 && (a.H2 - 1) / a.sh2 + 1 == a.P && (a.W2 - 1) / a.sw2 + 1 == a.Q &&
+         (int64_t)a.N * a.H * a.W * a.C < (1ll << 31) && (int64_t)a.N * a.H2 * a.W2 * a.C2 < (1ll << 31) &&
+         (int64_t)a.K * a.C < (1ll << 31) && (int64_t)a.K * a.C2 < (1ll << 31) && aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) &&
+         aligned16(a.X2) && aligned16(a.Wt2) && (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.bias2) & 7u) == 0;
+}
+
+bool launch_conv_f16_dual(const dnnrtContext *ctx, const ConvF16Args &a) {
+  const int64_t NPQ = (int64_t)a.N * a.P * a.Q;
+  ConvF16Args am = a;
+  am.magic_pq = magic_of(a.P * a.Q);
+  am.magic_q = magic_of(a.Q);
+  auto tiles_of = [&](int bm, int bn) { return ceil_div(a.K, bm) * ceil_div(NPQ, bn); };
+#define LAUNCH_DUAL(BM_, BN_, MINW_, FEW_, FIRST_)                                                                                      \
+  do {                                                                                                                         \
+    const int64_t tiles = tiles_of(BM_, BN_);                                                                                  \
+    if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }                                      \
+    const unsigned grid = (unsigned)(ceil_div(tiles, 8) * 8);                                                                  \
+    if (NPQ % BN_ != 0 || a.K % BM_ != 0)                                                                                      \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, 2, 2, 2, MINW_, true, 1, FEW_, true, FIRST_>), dim3(grid), dim3(256), 0,  \
+                         ctx->stream, am, (int)tiles);                                                                         \
+    else                                                                                                                       \
+      hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, 2, 2, 2, MINW_, false, 1, FEW_, true, FIRST_>), dim3(grid), dim3(256), 0, \
+                         ctx->stream, am, (int)tiles);                                                                         \
+  } while (0)
+  // Two steps in all (64 + 64 channels, the first block of a ResNet): the single-stage 64 x 64 tiles that such short
+  // reductions run best on; 89 -> 56 us at batch 64, where the layer is bound by the 103 MB the shortcut's result
+  // would be written and read with.  Longer reductions run on plain 64 x 64 tiles, correct but slower than the two
+  // calls they replace (second accumulator set; at 128 x 128 it no longer fits 256 registers: 73 vs 54 us on
+  // 256 + 128 -> 512 channels at 28 x 28, 53 vs 45 and 43 vs 41 us on the next two stages), so the compiler's pass
+  // asks for the fused call only in the first case.
+  if (a.C == 64 && a.C2 == 64) LAUNCH_DUAL(64, 64, 2, 2, 1);
+  else if (a.C2 % 128 != 0) { set_error("conv(fp16): the second convolution must read 64 or a multiple of 128 channels"); return false; }
+  else LAUNCH_DUAL(64, 64, 2, 0, 0);
+#undef LAUNCH_DUAL
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
+  return true;
 }
 
 bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {

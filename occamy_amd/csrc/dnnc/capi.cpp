@@ -134,6 +134,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (opt->fusion && opt->fuse_matmul_bias) fuse_matmul_bias(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
   if (opt->fusion && opt->fuse_first_layer_maxpool && opt->channels_last) fuse_first_layer_maxpool(p);
+  if (opt->fusion && opt->fuse_residual && opt->fuse_projection_shortcut && opt->channels_last) fuse_projection_shortcut(p);
   if (opt->alias_copies) alias_copies(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {
@@ -146,7 +147,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
       if (op->result->dtype != F16) { g_err = "channels_last needs an fp16 graph"; delete pp; return nullptr; }
       switch (op->kind) {
         case OP_MALLOC: case OP_HOST_ALLOC: case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_CONV_BIAS_ACTIV_MAXPOOL:
-        case OP_ACTIVATION: case OP_ADD:
+        case OP_CONV_ADD_CONV_ACTIV: case OP_ACTIVATION: case OP_ADD:
         case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE: case OP_LEAKYRELU: case OP_PRELU:
         case OP_CONCAT: break;
         default: g_err = std::string("channels_last: ") + op_name(op->kind) + " has no channels-last form"; delete pp; return nullptr;
@@ -167,7 +168,8 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
     for (const Op *op : p.ops) {
       bool layout_aware = false, conv = false;
       switch (op->kind) {
-        case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_CONV_BIAS_ACTIV_MAXPOOL: conv = true; layout_aware = true; break;
+        case OP_CONVFWD: case OP_CONV_BIAS_ACTIV: case OP_CONV_BIAS_ADD_ACTIV: case OP_CONV_BIAS_ACTIV_MAXPOOL: case OP_CONV_ADD_CONV_ACTIV:
+          conv = true; layout_aware = true; break;
         case OP_ACTIVATION: case OP_ADD: case OP_MUL: case OP_MAXPOOL: case OP_AVGPOOL: case OP_CLIP: case OP_REDUCE:
         case OP_LEAKYRELU: case OP_PRELU: case OP_CONCAT: layout_aware = true; break;
         case OP_MALLOC: case OP_DEALLOC: case OP_MEMCPY: case OP_HOST_CONST: case OP_HOST_ALLOC: case OP_RETURN: continue;
@@ -180,7 +182,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
           g_err = std::string("channels_last: ") + op_name(op->kind) + " reads a rank-4 tensor with spatial extent and has no channels-last form";
           delete pp; return nullptr;
         }
-        if (holds_constant(v) && !(conv && i == 1)) {
+        if (holds_constant(v) && !(conv && (i == 1 || (op->kind == OP_CONV_ADD_CONV_ACTIV && i == 5)))) {
           g_err = std::string("channels_last: a rank-4 constant with spatial extent feeds ") + op_name(op->kind) +
                   ", which would read its N,C,H,W bytes as N,H,W,C";
           delete pp; return nullptr;

@@ -37,7 +37,7 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
   LOAD(dnnrtMalloc); LOAD(dnnrtDealloc); LOAD(dnnrtHostAlloc); LOAD(dnnrtHostFree);
-  LOAD(dnnrtConv); LOAD(dnnrtConvBiasActiv); LOAD(dnnrtConvBiasAddActiv); LOAD(dnnrtConvBiasActivMaxPool); LOAD(dnnrtActive); LOAD(dnnrtTensorOp); LOAD(dnnrtClip);
+  LOAD(dnnrtConv); LOAD(dnnrtConvBiasActiv); LOAD(dnnrtConvBiasAddActiv); LOAD(dnnrtConvBiasActivMaxPool); LOAD(dnnrtConvBiasAddConvBiasActiv); LOAD(dnnrtActive); LOAD(dnnrtTensorOp); LOAD(dnnrtClip);
   LOAD(dnnrtErf); LOAD(dnnrtNegative); LOAD(dnnrtReciprocal); LOAD(dnnrtPow); LOAD(dnnrtCastI64toFloat);
   LOAD(dnnrtGelu); LOAD(dnnrtReduce); LOAD(dnnrtSoftmax); LOAD(dnnrtLayerNorm); LOAD(dnnrtMaxPool);
   LOAD(dnnrtAveragePool); LOAD(dnnrtMatmul2d); LOAD(dnnrtMatmulNd); LOAD(dnnrtFlatten);
@@ -112,8 +112,9 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
     for (const auto &u : op->operands[0]->uses) {
       if (u.first == op) continue;
       const bool conv = u.first->kind == OP_CONVFWD || u.first->kind == OP_CONV_BIAS_ACTIV ||
-                        u.first->kind == OP_CONV_BIAS_ADD_ACTIV || u.first->kind == OP_CONV_BIAS_ACTIV_MAXPOOL;
-      if (conv && u.second == 1) any = true;
+                        u.first->kind == OP_CONV_BIAS_ADD_ACTIV || u.first->kind == OP_CONV_BIAS_ACTIV_MAXPOOL ||
+                        u.first->kind == OP_CONV_ADD_CONV_ACTIV;
+      if (conv && (u.second == 1 || (u.first->kind == OP_CONV_ADD_CONV_ACTIV && u.second == 5))) any = true;
       else if (is_compute(u.first->kind)) only_filter = false;
     }
     const bool f = any && only_filter;
@@ -201,7 +202,8 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
 
 int Session::format_for(const Op *op) const {
   if (!prog->channels_last) return 0;  // NCHW
-  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL) {
+  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL ||
+      op->kind == OP_CONV_ADD_CONV_ACTIV) {
     const Value *x = op->operands[0];
     // the function argument's slot holds what the host sent: NCHW
     const bool from_arg = x->def && x->def->kind == OP_MEM_OFFSET;
@@ -223,7 +225,8 @@ bool Session::issue(const Op *op, std::string &err) {
       cur_format = f;
     }
   }
-  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL) {
+  if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL ||
+      op->kind == OP_CONV_ADD_CONV_ACTIV) {
     const int lay = filter_crsk[(size_t)op->operands[1]->id] ? DNNRT_FILTER_CRSK : DNNRT_FILTER_KCRS;
     if (lay != cur_filter_layout) {
       if (rt.dnnrtSetFilterLayout(handle, lay)) { err = rt_error("dnnrtSetFilterLayout"); return false; }
@@ -266,6 +269,11 @@ bool Session::issue(const Op *op, std::string &err) {
                                        out, op->dimOut.data(), dt);
       break;
     }
+    case OP_CONV_ADD_CONV_ACTIV:  // operands: x, w, bias, workspace, x2, w2, bias2, workspace2, out
+      r = rt.dnnrtConvBiasAddConvBiasActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), op->pads.data(), op->strides.data(),
+                                           P(4), op->dimA2.data(), P(5), op->dimB2.data(), P(6), op->pads2.data(), op->strides2.data(),
+                                           op->mode, out, dt);
+      break;
     case OP_ACTIVATION: {
       const Shape d = pad4(op->dimA);  // the lowering pads the dims to 4 with trailing ones
       if (d.size() > 4) {

@@ -40,6 +40,7 @@ struct RuntimeApi {
   decltype(&::dnnrtConvBiasActiv) dnnrtConvBiasActiv = nullptr;
   decltype(&::dnnrtConvBiasAddActiv) dnnrtConvBiasAddActiv = nullptr;
   decltype(&::dnnrtConvBiasActivMaxPool) dnnrtConvBiasActivMaxPool = nullptr;
+  decltype(&::dnnrtConvBiasAddConvBiasActiv) dnnrtConvBiasAddConvBiasActiv = nullptr;
   decltype(&::dnnrtActive) dnnrtActive = nullptr;
   decltype(&::dnnrtTensorOp) dnnrtTensorOp = nullptr;
   decltype(&::dnnrtClip) dnnrtClip = nullptr;

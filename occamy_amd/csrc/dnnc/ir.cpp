@@ -49,6 +49,7 @@ const char *op_name(OpKind k) {
     case OP_MATMUL_BIAS: return "dnn.matmulnd-bias";
     case OP_ATTENTION: return "dnn.attention";
     case OP_CONV_BIAS_ACTIV_MAXPOOL: return "dnn.conv-bias-relu-maxpoolfwd";
+    case OP_CONV_ADD_CONV_ACTIV: return "dnn.conv-bias-add-conv-bias-relufwd";
     case OP_RETURN: return "return";
   }
   return "?";
@@ -195,6 +196,19 @@ std::string Program::to_text() const {
         print_shape(os, op->pool_pads);
         os << ", poolStrides=";
         print_shape(os, op->pool_strides);
+        os << "}";
+        break;
+      case OP_CONV_ADD_CONV_ACTIV:
+        os << " {pads=";
+        print_shape(os, op->pads);
+        os << ", strides=";
+        print_shape(os, op->strides);
+        os << ", pads2=";
+        print_shape(os, op->pads2);
+        os << ", strides2=";
+        print_shape(os, op->strides2);
+        os << ", activMode=" << op->mode;
+        if (op->mode == 3 || op->mode == 6) os << ", activCoef=" << op->coef;
         os << "}";
         break;
       case OP_ACTIVATION: os << " {mode=" << op->mode << "}"; break;

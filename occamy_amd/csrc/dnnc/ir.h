@@ -69,6 +69,7 @@ enum OpKind {
   OP_MATMUL_BIAS,          // batched matrix product + one row added to every row
   OP_ATTENTION,            // softmax(scale * Q K^T) V per head on [batch, seq, heads * dim] tensors
   OP_CONV_BIAS_ACTIV_MAXPOOL,  // conv + bias + activation, then the max-pool behind it (a ResNet's first two layers)
+  OP_CONV_ADD_CONV_ACTIV,      // act((conv + bias) + (conv2 + bias2)): a residual block's last convolution and its projection shortcut
   OP_RETURN
 };
 const char *op_name(OpKind k);
@@ -92,6 +93,7 @@ struct Op {
   Shape dimA, dimB, dimOut;        // dim attributes as the reference emits them
   Shape pads, strides, kernel, perm;
   Shape pool_pads, pool_strides;   // OP_CONV_BIAS_ACTIV_MAXPOOL: the pooling's (`kernel` is its window; pads, strides: the convolution's)
+  Shape dimA2, dimB2, pads2, strides2;  // OP_CONV_ADD_CONV_ACTIV: the second convolution's input dims, filter dims, pads, strides
   int64_t group = 1, axis = 0, mode = 0, algo = 0, trans_a = 0, trans_b = 0;
   int64_t bytes = 0;               // malloc / memcpy / mem-offset size
   int64_t offset = 0;              // mem-offset
@@ -183,6 +185,7 @@ void fuse_conv_activations(Program &p);
 void fuse_matmul_bias(Program &p);
 void fuse_first_layer_maxpool(Program &p);
 void alias_copies(Program &p);
+void fuse_projection_shortcut(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);
 bool malloc_pool_opt(Program &p, std::string &err);

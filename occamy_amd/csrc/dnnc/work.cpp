@@ -12,6 +12,7 @@ const char *op_class(const Op *op) {
     case OP_CONV_BIAS_ACTIV:
     case OP_CONV_BIAS_ADD_ACTIV: return (op->dimB[1] == 1 && op->group > 1) ? "conv_depthwise" : "conv_dense";
     case OP_CONV_BIAS_ACTIV_MAXPOOL: return "conv_dense";
+    case OP_CONV_ADD_CONV_ACTIV: return "conv_dense";
     case OP_MATMUL2D: return "gemm";
     case OP_MATMULND:
     case OP_MATMUL_BIAS: return "matmul";
@@ -49,6 +50,13 @@ void op_work(const Op *op, double &flops, double &bytes) {
       bytes = ((double)shape_numel(op->dimA) + (double)shape_numel(op->dimB) + n_out +
                (op->kind != OP_CONVFWD ? (double)op->dimB[0] : 0.0) +
                (op->kind == OP_CONV_BIAS_ADD_ACTIV ? n_out : 0.0)) * es;
+      break;
+    }
+    case OP_CONV_ADD_CONV_ACTIV: {  // both convolutions' products; every tensor the call touches once
+      const double crs = (double)(op->dimB[1] * op->dimB[2] * op->dimB[3]), crs2 = (double)(op->dimB2[1] * op->dimB2[2] * op->dimB2[3]);
+      flops = 2.0 * n_out * (crs + crs2);
+      bytes = ((double)shape_numel(op->dimA) + (double)shape_numel(op->dimB) + (double)shape_numel(op->dimA2) +
+               (double)shape_numel(op->dimB2) + 2.0 * (double)op->dimB[0] + n_out) * es;
       break;
     }
     case OP_CONV_BIAS_ACTIV_MAXPOOL: {  // the convolution's products (its output extents, not the pooled ones); the pooling's compares are not counted

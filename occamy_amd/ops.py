@@ -125,6 +125,13 @@ class Ops:
                                                             dims(pool_strides), Y, dims(dimY), dtype),
                          "dnnrtConvBiasActivMaxPool")
 
+    def conv_bias_add_conv_bias_activ(self, X, dimX, W, dimW, B, pads, strides, X2, dimX2, W2, dimW2, B2, pads2, strides2, activ, Y,
+                                      dtype=_abi.F16):
+        return self._ret(self.lib.dnnrtConvBiasAddConvBiasActiv(self.handle, X, dims(dimX), W, dims(dimW), B, dims(pads), dims(strides),
+                                                                X2, dims(dimX2), W2, dims(dimW2), B2, dims(pads2), dims(strides2),
+                                                                activ, Y, dtype),
+                         "dnnrtConvBiasAddConvBiasActiv")
+
     def active(self, X, dimX, mode, Y, dtype=_abi.F32):
         d = list(dimX) + [1] * (4 - len(dimX))
         return self._ret(self.lib.dnnrtActive(self.handle, X, dims(d), mode, Y, dtype), "dnnrtActive")

@@ -698,6 +698,33 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t h, const void *X, const int64_t *d
   return r ? Y : NULL;
 }
 
+/* No reference wrapper of its own: the reference runs this as dnnrtConvBiasActiv
+ * (identity) on the second convolution and then the chain of
+ * dnnrtConvBiasAddActiv with that result as Z, every call storing its result
+ * in the tensor's type.  Restated as exactly that, for any shapes the two
+ * calls take. */
+void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t h, const void *X, const int64_t *dX, const void *W,
+                                    const int64_t *dW, const void *B, const int64_t *pads,
+                                    const int64_t *strides, const void *X2, const int64_t *dX2,
+                                    const void *W2, const int64_t *dW2, const void *B2,
+                                    const int64_t *pads2, const int64_t *strides2, int64_t act,
+                                    void *Y, int32_t dtype) {
+  if (bad_dtype(dtype)) FAIL("convBiasAddConvBiasActiv: bad dtype");
+  const int64_t P = (dX2[2] + 2 * pads2[0] - dW2[2]) / strides2[0] + 1,
+                Q = (dX2[3] + 2 * pads2[1] - dW2[3]) / strides2[1] + 1;
+  if (P < 1 || Q < 1) FAIL("convBiasAddConvBiasActiv: empty second convolution");
+  const int64_t dZ[4] = {dX2[0], dW2[0], P, Q};
+  const int64_t dB[4] = {1, dW[0], 1, 1}, dB2[4] = {1, dW2[0], 1, 1};
+  const size_t es = dtype == DNNRT_F16 ? 2 : 4;
+  void *z = malloc((size_t)numel(dZ, 4) * es);
+  void *zero = calloc((size_t)(dW[0] > dW2[0] ? dW[0] : dW2[0]), es);
+  if (!z || !zero) { free(z); free(zero); FAIL("convBiasAddConvBiasActiv: out of memory"); }
+  void *r = dnnrtConvBiasActiv(h, X2, dX2, W2, dW2, B2 ? B2 : zero, dB2, NULL, 0, 0, 1, pads2, strides2, DNNRT_ACT_IDENTITY, z, dtype);
+  if (r) r = dnnrtConvBiasAddActiv(h, X, dX, W, dW, B ? B : zero, dB, z, NULL, 0, 0, 1, pads, strides, act, Y, dtype);
+  free(z); free(zero);
+  return r ? Y : NULL;
+}
+
 /* ---- matrix products ----------------------------------------------------- */
 
 /* C[M,N] = alpha * sum_k A(m,k) B(k,n) (+ beta * Cin), element strides given */

@@ -99,7 +99,7 @@ for rank in (2, 3, 4, 6):
 NEW = {"dnnrtLastError", "dnnrtIsHostBackend", "dnnrtSetStream", "dnnrtSetTensorFormat", "dnnrtSetFilterLayout",
        "dnnrtSetActivationCoef", "dnnrtListConvTiles", "dnnrtSetConvTile", "dnnrtSync", "dnnrtGraphBegin", "dnnrtGraphEnd",
        "dnnrtGraphLaunch", "dnnrtGraphDestroy", "dnnrtEventCreate", "dnnrtEventRecord", "dnnrtEventElapsedMs",
-       "dnnrtEventDestroy", "dnnrtHostAlloc", "dnnrtHostFree", "dnnrtMemFill", "dnnrtConvBiasAddActiv", "dnnrtConvBiasActivNoAlloc", "dnnrtConvBiasActivMaxPool",
+       "dnnrtEventDestroy", "dnnrtHostAlloc", "dnnrtHostFree", "dnnrtMemFill", "dnnrtConvBiasAddActiv", "dnnrtConvBiasActivNoAlloc", "dnnrtConvBiasActivMaxPool", "dnnrtConvBiasAddConvBiasActiv",
        "dnnrtGelu", "dnnrtLayerNorm", "dnnrtMatmulNdBias", "dnnrtAttention", "dnnrtSqrt", "dnnrtSigmoid", "dnnrtTanh"}
 
 

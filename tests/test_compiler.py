@@ -304,6 +304,33 @@ def test_first_layer_maxpool_fusion():
     assert "maxpoolfwd" not in g.compile(fuse_first_layer_maxpool=True, channels_last=True).text  # no fusion flag: conv, add, relu apart
 
 
+def test_projection_shortcut_fusion():
+    """The 1x1 projection shortcut (64 -> 256 channels) of ResNet-50's first block and the block's last 1x1 convolution
+    (+ add + ReLU) become one call; the three other projection shortcuts (longer reductions, strided) stay as they
+    are; the shortcut's buffer is never allocated."""
+    flags = dict(fusion=True, fuse_residual=True, channels_last=True)
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    plain = g.compile(**flags)
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    fused = g.compile(fuse_projection_shortcut=True, **flags)
+    assert "add-conv" not in plain.text and fused.text.count("dnn.conv-bias-add-conv-bias-relufwd") == 1
+    line = next(l for l in fused.text.splitlines() if "add-conv" in l)
+    assert "pads=[0,0], strides=[1,1], pads2=[0,0], strides2=[1,1], activMode=1" in line and line.rstrip().endswith("f16[1,256,16,16]")
+    assert fused.num_ops(compute_only=True) == plain.num_ops(compute_only=True) - 1
+    assert fused.text.count("dnn.conv-bias-add-relufwd") == plain.text.count("dnn.conv-bias-add-relufwd") - 1
+    shortcut_bytes = 1 * 256 * 16 * 16 * 2
+    sizes = lambda prog: sorted(b for k, _, b, _ in prog.events() if k == 0)
+    gone = list(sizes(plain))
+    gone.remove(shortcut_bytes)
+    assert sizes(fused) == gone
+    check_lifetimes(lambda: models.resnet50(dtype=np.float16, **SMALL), fuse_projection_shortcut=True, **flags)
+    # needs the residual fusion (it extends that call) and channels-last fp16
+    g, _ = models.resnet50(dtype=np.float16, **SMALL)
+    assert "add-conv" not in g.compile(fusion=True, channels_last=True, fuse_projection_shortcut=True).text
+    g, _ = models.resnet50(dtype=np.float32, **SMALL)
+    assert "add-conv" not in g.compile(fusion=True, fuse_residual=True, fuse_projection_shortcut=True).text
+
+
 def test_channels_last_refuses_what_it_cannot_lay_out():
     """A rank-4 constant with spatial extent reaches the device N,C,H,W (only convolution filters are re-laid at
     upload), and Flatten / Reshape copy bytes: channels_last must refuse both at compile time, not at run time."""

@@ -146,7 +146,8 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     """The throughput configuration at its own size and with the benchmark's own flags (64 x 3 x 224 x 224,
     fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
     oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
-    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True, alias_copies=True)
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
+                 fuse_projection_shortcut=True, alias_copies=True)
     build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
     out16, info = run(build16, **flags)
     assert info["requested"] == info["pool"]
@@ -246,6 +247,21 @@ def test_aliased_copies_change_nothing_on_the_gpu():
             np.testing.assert_array_equal(s.run(*inputs)[0], plain[0])
         assert len(s.profile(inputs)) == p.num_ops(compute_only=True)
         s.close()
+
+
+@pytest.mark.parametrize("batch,image", [(3, 64), (2, 224)])
+def test_projection_shortcut_fusion_fp16_channels_last(batch, image):
+    """The first block's projection shortcut and last convolution as one call: the same bits as the two calls, per
+    inference and replayed from a captured graph."""
+    build16 = lambda: models.resnet50(batch, np.float16, seed=5, image=image)  # noqa: E731
+    flags = dict(fusion=True, channels_last=True, fuse_residual=True, fuse_matmul_bias=True)
+    assert "add-conv" in build16()[0].compile(fuse_projection_shortcut=True, **flags).text
+    two, _ = run(build16, **flags)
+    one, info = run(build16, fuse_projection_shortcut=True, **flags)
+    assert info["requested"] == info["pool"]
+    np.testing.assert_array_equal(one[0], two[0])
+    res, _ = run(build16, mode=compiler.MODE_RESIDENT, fuse_projection_shortcut=True, **flags)
+    np.testing.assert_array_equal(res[0], one[0])
 
 
 @pytest.mark.parametrize("name", ["resnet50", "mobilenet_v2"])

@@ -696,6 +696,75 @@ def test_first_layer_with_its_max_pool_refuses_other_shapes(gpu):
             gpu.ops.set_format(_abi.NCHW)
 
 
+def dual_conv_f16(gpu, x, w, b, x2, w2, b2, stride2, activ):
+    """dnnrtConvBiasAddConvBiasActiv through the C-ABI; tensors in logical NCHW / KCRS order; returns logical NCHW."""
+    N, C, P, Q = x.shape
+    K = w.shape[0]
+    nhwc = lambda t: np.ascontiguousarray(t.transpose(0, 2, 3, 1))  # noqa: E731
+    X, Wt, B, X2, Wt2, B2 = gpu.put(nhwc(x)), gpu.put(nhwc(w)), gpu.put(b), gpu.put(nhwc(x2)), gpu.put(nhwc(w2)), gpu.put(b2)
+    Y = gpu.empty((N * K * P * Q,), np.float16)
+    gpu.ops.set_format(_abi.NHWC)
+    try:
+        gpu.ops.conv_bias_add_conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), gpu.ptr(X2), x2.shape,
+                                              gpu.ptr(Wt2), w2.shape, gpu.ptr(B2), (0, 0), (stride2, stride2), activ, gpu.ptr(Y))
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    return gpu.get(Y).reshape(N, P, Q, K).transpose(0, 3, 1, 2)
+
+
+@pytest.mark.parametrize("case", [(2, 9, 11, 64, 64, 72, 1), (3, 13, 13, 128, 256, 200, 2), (2, 14, 10, 192, 128, 256, 2), (8, 56, 56, 64, 64, 256, 1), (2, 10, 10, 128, 128, 72, 1), (2, 12, 12, 64, 256, 64, 2), (1, 9, 9, 192, 256, 40, 1),
+                                  (1, 7, 7, 64, 128, 64, 1)], ids=lambda c: "x".join(map(str, c)))
+def test_last_convolution_and_projection_shortcut_in_one_call(gpu, cpu, case):
+    """dnnrtConvBiasAddConvBiasActiv against the two calls it replaces: the oracle's chain to the fp16 convolutions'
+    tolerance, and this library's own two calls bit for bit (each conv + bias rounded to fp16 on its own, the sum
+    and ReLU in fp32).  N, H2, W2, C, C2, K, stride of the shortcut; ragged tiles in both directions; 64 + 64
+    channels take the single-stage kernel, the rest the general one."""
+    N, H2, W2, C, C2, K, st = case
+    P, Q = (H2 - 1) // st + 1, (W2 - 1) // st + 1
+    r = rng(sum(case))
+    x = r.standard_normal((N, C, P, Q)).astype(np.float16)
+    x2 = r.standard_normal((N, C2, H2, W2)).astype(np.float16)
+    w = (r.standard_normal((K, C, 1, 1)) * np.sqrt(2.0 / C)).astype(np.float16)
+    w2 = (r.standard_normal((K, C2, 1, 1)) * np.sqrt(2.0 / C2)).astype(np.float16)
+    b, b2 = r.uniform(-0.2, 0.2, K).astype(np.float16), r.uniform(-0.2, 0.2, K).astype(np.float16)
+    got = dual_conv_f16(gpu, x, w, b, x2, w2, b2, st, _abi.ACT_RELU)
+    z_ref = oc.conv(cpu, x2, w2, b2, (0, 0), (st, st), 1, _abi.ACT_IDENTITY)
+    ref = oc.conv(cpu, x, w, b, (0, 0), (1, 1), 1, _abi.ACT_RELU, z=z_ref)
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=4e-3, atol=4e-3)
+    z_gpu = conv_f16(gpu, x2, w2, b2, (0, 0), (st, st), 1, _abi.ACT_IDENTITY, _abi.NHWC)
+    two = conv_f16(gpu, x, w, b, (0, 0), (1, 1), 1, _abi.ACT_RELU, _abi.NHWC, z=z_gpu)
+    np.testing.assert_array_equal(got, two)
+    if case[0] == 2 and C == 64:  # the oracle's own entry point is that chain
+        X, Wt, B, X2, Wt2, B2 = cpu.put(x), cpu.put(w), cpu.put(b), cpu.put(x2), cpu.put(w2), cpu.put(b2)
+        Y = cpu.empty(ref.shape, np.float16)
+        cpu.ops.conv_bias_add_conv_bias_activ(cpu.ptr(X), x.shape, cpu.ptr(Wt), w.shape, cpu.ptr(B), (0, 0), (1, 1), cpu.ptr(X2), x2.shape,
+                                              cpu.ptr(Wt2), w2.shape, cpu.ptr(B2), (0, 0), (st, st), _abi.ACT_RELU, cpu.ptr(Y))
+        np.testing.assert_array_equal(cpu.get(Y), ref)
+
+
+def test_last_convolution_and_projection_shortcut_refuses_other_shapes(gpu):
+    r = rng(4)
+    x = r.standard_normal((1, 64, 8, 8)).astype(np.float16)
+    w = r.standard_normal((64, 64, 1, 1)).astype(np.float16)
+    b = np.zeros(64, np.float16)
+    w3 = r.standard_normal((64, 64, 3, 3)).astype(np.float16)
+    X, Wt, B, W3 = gpu.put(x), gpu.put(w), gpu.put(b), gpu.put(w3)
+    Y = gpu.empty((64 * 64,), np.float16)
+    call = lambda fmt, wt2, dw2, pads2, dx2=(1, 64, 8, 8): (gpu.ops.set_format(fmt), gpu.ops.conv_bias_add_conv_bias_activ(  # noqa: E731
+        gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), gpu.ptr(X), dx2, gpu.ptr(wt2), dw2, gpu.ptr(B), pads2, (1, 1),
+        _abi.ACT_RELU, gpu.ptr(Y)))
+    try:
+        with pytest.raises(RuntimeError, match="1x1"):
+            call(_abi.NHWC, W3, w3.shape, (1, 1))
+        with pytest.raises(RuntimeError, match="DNNRT_NHWC"):
+            call(_abi.NCHW, Wt, w.shape, (0, 0))
+        with pytest.raises(RuntimeError, match="give"):
+            call(_abi.NHWC, Wt, w.shape, (0, 0), (1, 64, 4, 16))
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+
+
 # Problems of the size ResNet-50 has at batch 64: the dispatcher picks its large tiles (128 x 128 and up,
 # four or eight wavefronts) only when a launch has hundreds of tiles, so these are the only cases that reach
 # them.  N, C, H, W, K, R, stride, pad
