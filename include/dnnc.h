@@ -70,8 +70,8 @@ typedef struct {
                              that never stores the convolution's result (default 0) */
   int32_t fuse_projection_shortcut; /* no reference flag: with `fusion`, `fuse_residual` and `channels_last`, the
                              1x1 projection shortcut of a residual block and the block's last 1x1 convolution
-                             (+ add + activation), both over 64 input channels, become one call that never
-                             stores the shortcut's result (default 0) */
+                             (+ add + activation), over 64 + 64 or 256 + 128 input channels, become one call
+                             that never stores the shortcut's result (default 0) */
   int32_t alias_copies;   /* no reference flag: Flatten / Reshape / Squeeze / Unsqueeze name their input's buffer
                              as their output, so nothing is copied and nothing launched (default 0) */
 } dnncOptions;

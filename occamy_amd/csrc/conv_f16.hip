@@ -387,7 +387,9 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
     if constexpr (FEW_STEPS > 1) turn(integral_constant<int, 1>{});
     if constexpr (FEW_STEPS > 2) turn(integral_constant<int, 2>{});
     if constexpr (FEW_STEPS > 3) turn(integral_constant<int, 3>{});
-    static_assert(FEW_STEPS <= 4, "up to four turns are written out");
+    if constexpr (FEW_STEPS > 4) turn(integral_constant<int, 4>{});
+    if constexpr (FEW_STEPS > 5) turn(integral_constant<int, 5>{});
+    static_assert(FEW_STEPS <= 6, "up to six turns are written out");
   } else if (rem == 3) {
     step(slot0, true_type{}, true_type{});
     step(slot1, false_type{}, true_type{});
@@ -612,13 +614,14 @@ bool launch_conv_f16_dual(const dnnrtContext *ctx, const ConvF16Args &a) {
       hipLaunchKernelGGL((conv_f16_nhwc_kernel<BM_, BN_, 2, 2, 2, MINW_, false, 1, FEW_, true, FIRST_>), dim3(grid), dim3(256), 0, \
                          ctx->stream, am, (int)tiles);                                                                         \
   } while (0)
-  // Two steps in all (64 + 64 channels, the first block of a ResNet): the single-stage 64 x 64 tiles that such short
-  // reductions run best on; 89 -> 56 us at batch 64, where the layer is bound by the 103 MB the shortcut's result
-  // would be written and read with.  Longer reductions run on plain 64 x 64 tiles, correct but slower than the two
-  // calls they replace (second accumulator set; at 128 x 128 it no longer fits 256 registers: 73 vs 54 us on
-  // 256 + 128 -> 512 channels at 28 x 28, 53 vs 45 and 43 vs 41 us on the next two stages), so the compiler's pass
-  // asks for the fused call only in the first case.
+  // Two steps in all (64 + 64 channels, the first block of a ResNet), or six (256 strided + 128, the first block of its
+  // second stage): the single-stage 64 x 64 tiles that such short reductions run best on; 89 -> 56 us and 55 -> 50 us
+  // at batch 64, where the pair is bound by the bytes the shortcut's result would be written and read with.  Other
+  // reductions run on plain 64 x 64 tiles, correct but slower than the two calls they replace (second accumulator
+  // set; at 128 x 128 it no longer fits 256 registers: 53 vs 45 us on 512 + 256 -> 1024 channels at 14 x 14, 43 vs
+  // 41 us on the last stage), so the compiler's pass asks for the fused call only in the first two cases.
   if (a.C == 64 && a.C2 == 64) LAUNCH_DUAL(64, 64, 2, 2, 1);
+  else if (a.C == 128 && a.C2 == 256) LAUNCH_DUAL(64, 64, 2, 6, 4);
   else if (a.C2 % 128 != 0) { set_error("conv(fp16): the second convolution must read 64 or a multiple of 128 channels"); return false; }
   else LAUNCH_DUAL(64, 64, 2, 0, 0);
 #undef LAUNCH_DUAL

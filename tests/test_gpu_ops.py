@@ -713,7 +713,7 @@ def dual_conv_f16(gpu, x, w, b, x2, w2, b2, stride2, activ):
     return gpu.get(Y).reshape(N, P, Q, K).transpose(0, 3, 1, 2)
 
 
-@pytest.mark.parametrize("case", [(2, 9, 11, 64, 64, 72, 1), (3, 13, 13, 128, 256, 200, 2), (2, 14, 10, 192, 128, 256, 2), (8, 56, 56, 64, 64, 256, 1), (2, 10, 10, 128, 128, 72, 1), (2, 12, 12, 64, 256, 64, 2), (1, 9, 9, 192, 256, 40, 1),
+@pytest.mark.parametrize("case", [(2, 9, 11, 64, 64, 72, 1), (3, 13, 13, 128, 256, 200, 2), (2, 14, 10, 192, 128, 256, 2), (8, 56, 56, 64, 64, 256, 1), (4, 56, 56, 128, 256, 512, 2), (3, 9, 13, 128, 256, 136, 2), (2, 10, 10, 128, 128, 72, 1), (2, 12, 12, 64, 256, 64, 2), (1, 9, 9, 192, 256, 40, 1),
                                   (1, 7, 7, 64, 128, 64, 1)], ids=lambda c: "x".join(map(str, c)))
 def test_last_convolution_and_projection_shortcut_in_one_call(gpu, cpu, case):
     """dnnrtConvBiasAddConvBiasActiv against the two calls it replaces: the oracle's chain to the fp16 convolutions'
