@@ -68,10 +68,10 @@ typedef struct {
                              convolution (3 -> 64 channels, 7x7, stride 2, pad 3, even image width, ReLU or
                              identity) and the 3x3 / stride 2 / pad 1 max-pool behind it become one call
                              that never stores the convolution's result (default 0) */
-  int32_t fuse_projection_shortcut; /* no reference flag: with `fusion`, `fuse_residual` and `channels_last`, the
-                             1x1 projection shortcut of a residual block and the block's last 1x1 convolution
-                             (+ add + activation), over 64 + 64 or 256 + 128 input channels, become one call
-                             that never stores the shortcut's result (default 0) */
+  int32_t fuse_projection_shortcut; /* no reference flag: with `fusion` and `fuse_residual`, the projection shortcut of a
+                             residual block (conv + bias) and the block's last convolution (+ add + activation)
+                             become one call, and the shortcut's result has no tensor of its own (fp16 programs:
+                             with `channels_last` only; default 0) */
   int32_t alias_copies;   /* no reference flag: Flatten / Reshape / Squeeze / Unsqueeze name their input's buffer
                              as their output, so nothing is copied and nothing launched (default 0) */
 } dnncOptions;

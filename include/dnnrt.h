@@ -236,16 +236,21 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X,
                                 const int64_t *poolStrides, void *Y,
                                 const int64_t *dimY, int32_t dtype);
 /* New: a residual block's last convolution and its projection shortcut in
- * one kernel: Y = act((conv(X, W) + B) + (conv(X2, W2) + B2)).  It replaces
+ * one call: Y = act((conv(X, W) + B) + (conv(X2, W2) + B2)).  It replaces
  * dnnrtConvBiasActiv (identity) on the shortcut followed by
- * dnnrtConvBiasAddActiv with that result as Z; the shortcut's result is then
- * never stored or read.  Every element is what the two calls would store:
- * each conv + bias rounded to fp16 on its own, the sum and the activation in
- * fp32, one more rounding.  fp16, tensor format DNNRT_NHWC, filters K,R,S,C;
- * both convolutions 1x1 without padding, the first with stride 1, the second
- * with any stride, input channel counts multiples of 64, onto the same
- * [N, K, P, Q] result; group 1; B and B2 may be null.  Anything else fails
- * with an error. */
+ * dnnrtConvBiasAddActiv with that result as Z; no tensor for the shortcut's
+ * result is needed.  Any two convolutions (group 1) onto the same
+ * [N, K, P, Q] result, fp32 or fp16, in the handle's tensor format and filter
+ * layout; B and B2 may be null.
+ * One kernel where that is the faster way: fp16 DNNRT_NHWC, both 1x1 without
+ * padding, the first with stride 1, over 64 + 64 or 128 + 256 input channels
+ * (every element is then what the two calls would store: each conv + bias
+ * rounded to fp16 on its own, the sum and the activation in fp32); fp32
+ * DNNRT_NCHW, both 1x1 without padding, on problems small enough for the
+ * batch-1 kernels (the two reductions are then one sum, rounded once: within
+ * an fp32 ulp or two of the chain).  Everywhere else the call runs the two
+ * convolutions one after the other with the shortcut's result passing through
+ * Y, which gives the chain's bits. */
 void *dnnrtConvBiasAddConvBiasActiv(
     dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
     const int64_t *dimW, const void *B, const int64_t *pads,

@@ -79,13 +79,13 @@ constexpr int LDS_ROW_G = 40; // generic kernel: 32 + 8 pad (80 bytes)
 // fp16(conv(X2, W2) + bias2)) — a residual block's last convolution and its projection shortcut.  The second
 // convolution's steps come first, into the same accumulators; where its reduction ends they are rounded to fp16
 // with its bias, exactly what it would have stored as a convolution of its own, and set aside; the epilogue adds
-// them as it adds a residual tensor, which is then never written or read.  With FEW_STEPS the turns are
-// DUAL_FIRST steps of the second convolution, then the first's.
+// them as it adds a residual tensor, which is then never written or read.  The turns of the single-stage sequence
+// are DUAL_FIRST steps of the second convolution, then the first's.
 template <int BM, int BN, int WM, int WN, int DEPTH, int MIN_WAVES, bool MASKED, int KG, int FEW_STEPS = 0, bool DUAL = false,
           int DUAL_FIRST = 0>
 __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefronts per SIMD the register budget must allow
  void conv_f16_nhwc_kernel(const ConvF16Args a, const int tiles_total) {
-  static_assert(!DUAL || KG == 1, "the two-convolution form is written for one k group");
+  static_assert(!DUAL || (KG == 1 && FEW_STEPS > 0), "the two-convolution form is written for the single-stage sequence");
   static_assert(WM * WN == 4, "four wavefronts");
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert(KG == 1 || KG == 2, "one or two k groups");
@@ -355,21 +355,13 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   const integral_constant<int, 0> slot0{};
   const integral_constant<int, 1> slot1{};
   int kt = 0;
-  // (two-convolution form: before step nk2 the accumulators change hands; nk2 is even and at least two here, so
-  // that happens before a pair of steps: three places in the code, each a copy of 2 x 16 x TM x TN register moves)
   if constexpr (!ONE_STAGE) {
     for (; kt + 4 <= nk; kt += 2) {  // both steps have a step two ahead to request
-      if constexpr (DUAL) {
-        if (kt == nk2) set_aside();
-      }
       step(slot0, true_type{}, true_type{});
       step(slot1, true_type{}, true_type{});
     }
   }
   const int rem = ONE_STAGE ? 0 : nk - kt;  // 1, 2 or 3
-  if constexpr (DUAL && !ONE_STAGE) {
-    if (kt == nk2) set_aside();
-  }
   if constexpr (ONE_STAGE) {
     // step T: its data goes from register slot T % 2 into the one stage (step 0's is there already), the
     // slot is refilled with step T + 2 if there is one, then the MFMAs read the stage
@@ -393,9 +385,6 @@ __global__ __launch_bounds__(256 * KG, MIN_WAVES)  // second argument: wavefront
   } else if (rem == 3) {
     step(slot0, true_type{}, true_type{});
     step(slot1, false_type{}, true_type{});
-    if constexpr (DUAL) {
-      if (kt + 2 == nk2) set_aside();  // (a single step of the first convolution behind an even number of the second's)
-    }
     step(slot0, false_type{}, false_type{});
   } else if (rem == 2) {
     step(slot0, false_type{}, true_type{});
@@ -616,14 +605,13 @@ bool launch_conv_f16_dual(const dnnrtContext *ctx, const ConvF16Args &a) {
   } while (0)
   // Two steps in all (64 + 64 channels, the first block of a ResNet), or six (256 strided + 128, the first block of its
   // second stage): the single-stage 64 x 64 tiles that such short reductions run best on; 89 -> 56 us and 55 -> 50 us
-  // at batch 64, where the pair is bound by the bytes the shortcut's result would be written and read with.  Other
-  // reductions run on plain 64 x 64 tiles, correct but slower than the two calls they replace (second accumulator
-  // set; at 128 x 128 it no longer fits 256 registers: 53 vs 45 us on 512 + 256 -> 1024 channels at 14 x 14, 43 vs
-  // 41 us on the last stage), so the compiler's pass asks for the fused call only in the first two cases.
+  // at batch 64, where the pair is bound by the bytes the shortcut's result would be written and read with.  Longer
+  // reductions were slower this way than as two calls (on plain 64 x 64 tiles, and on 128 x 128 ones, where the
+  // second accumulator set no longer fits 256 registers: 53 vs 45 us on 512 + 256 -> 1024 channels at 14 x 14, 43 vs
+  // 41 us on the last stage); the entry point runs those as the two calls.
   if (a.C == 64 && a.C2 == 64) LAUNCH_DUAL(64, 64, 2, 2, 1);
   else if (a.C == 128 && a.C2 == 256) LAUNCH_DUAL(64, 64, 2, 6, 4);
-  else if (a.C2 % 128 != 0) { set_error("conv(fp16): the second convolution must read 64 or a multiple of 128 channels"); return false; }
-  else LAUNCH_DUAL(64, 64, 2, 0, 0);
+  else { set_error("conv(fp16): the two-convolution kernel takes 64 + 64 or 128 + 256 input channels"); return false; }
 #undef LAUNCH_DUAL
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("conv(fp16): launch failed: %s", hipGetErrorString(e)); return false; }

@@ -129,12 +129,13 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (!emit_program(g->g, p, err)) { g_err = err; delete pp; return nullptr; }
   func_args_to_device(p);
   erase_dummy_constants(p);
+  p.channels_last_requested = opt->channels_last != 0;
   if (opt->fusion) fuse_conv_bias_activ(p);
   if (opt->fusion && opt->fuse_activations) fuse_conv_activations(p);
   if (opt->fusion && opt->fuse_matmul_bias) fuse_matmul_bias(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
   if (opt->fusion && opt->fuse_first_layer_maxpool && opt->channels_last) fuse_first_layer_maxpool(p);
-  if (opt->fusion && opt->fuse_residual && opt->fuse_projection_shortcut && opt->channels_last) fuse_projection_shortcut(p);
+  if (opt->fusion && opt->fuse_residual && opt->fuse_projection_shortcut) fuse_projection_shortcut(p);
   if (opt->alias_copies) alias_copies(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {

@@ -228,6 +228,10 @@ bool Session::issue(const Op *op, std::string &err) {
   if (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_BIAS_ACTIV_MAXPOOL ||
       op->kind == OP_CONV_ADD_CONV_ACTIV) {
     const int lay = filter_crsk[(size_t)op->operands[1]->id] ? DNNRT_FILTER_CRSK : DNNRT_FILTER_KCRS;
+    if (op->kind == OP_CONV_ADD_CONV_ACTIV && filter_crsk[(size_t)op->operands[5]->id] != filter_crsk[(size_t)op->operands[1]->id]) {
+      err = "executor: the two filters of a fused shortcut pair were uploaded in different layouts";
+      return false;
+    }
     if (lay != cur_filter_layout) {
       if (rt.dnnrtSetFilterLayout(handle, lay)) { err = rt_error("dnnrtSetFilterLayout"); return false; }
       cur_filter_layout = lay;

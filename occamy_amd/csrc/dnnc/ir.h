@@ -134,6 +134,7 @@ struct Program {
   int64_t pool_bytes = -1;           // set by the pool pass: the size the reference planner reports
   int64_t pool_extent = -1;          // highest planned byte + 1 (equals pool_bytes unless the planner under-reports)
   bool channels_last = false;        // fp16 programs: rank-4 activations are NHWC on the device
+  bool channels_last_requested = false;  // set before the passes run (channels_last itself after the layout checks)
 
   Value *new_value(DType dt, const Shape &s);
   Op *new_op(OpKind k);                       // not yet in the block

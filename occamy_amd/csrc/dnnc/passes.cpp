@@ -182,29 +182,23 @@ void fuse_first_layer_maxpool(Program &p) {
   }
 }
 
-// conv 1x1 + bias (identity: the projection shortcut of a residual block) whose only reader is the residual operand of a
-// conv 1x1 + bias + add + activation (the block's last convolution), both without padding, the closer with stride 1:
-// one call computes both convolutions onto the same tile and the shortcut's result, the largest tensor of the
-// block, is never stored or read.  Channels-last fp16 programs only, and only for the two pairs of channel counts
-// the runtime has single-stage kernels for (64 + 64 and 128 + 256: the first blocks of an ImageNet ResNet's first
-// two stages): there the pair is bound by memory traffic (89 -> 56 us and 55 -> 50 us at batch 64); with longer
-// reductions the runtime's fused kernel is slower than the two calls.  The reference has no such pattern.
+// conv + bias (identity: the projection shortcut of a residual block) whose only reader is the residual operand of a
+// conv + bias + add + activation (the block's last convolution): one call computes both, and no tensor is allocated
+// for the shortcut's result, the largest of the block.  The runtime runs the pair as one kernel where that is faster
+// (fp16 channels-last over 64 + 64 and 128 + 256 channels: 89 -> 56 us and 55 -> 50 us at batch 64; fp32 at batch-1
+// sizes: one launch fewer per shortcut) and as the two convolutions through the output buffer elsewhere.  fp16
+// programs must be channels-last.  The reference has no such pattern.
 void fuse_projection_shortcut(Program &p) {
   std::vector<Op *> closers;
   for (Op *op : p.ops)
     if (op->kind == OP_CONV_BIAS_ADD_ACTIV) closers.push_back(op);
-  auto plain_1x1 = [](const Op *c) {
-    return c->dimB.size() == 4 && c->dimB[2] == 1 && c->dimB[3] == 1 && c->group == 1 && c->pads == Shape{0, 0};
-  };
   for (Op *m : closers) {  // operands: x, w, bias, workspace, z, out
-    if (m->result->dtype != F16 || !plain_1x1(m) || m->strides != Shape{1, 1}) continue;
+    if (m->group != 1 || m->dimB.size() != 4) continue;
+    if (m->result->dtype == F16 && !p.channels_last_requested) continue;
     Value *z = m->operands[4];
     Op *sc = z->def;
-    if (!sc || sc->kind != OP_CONV_BIAS_ACTIV || sc->mode != 5 || !plain_1x1(sc) || z->uses.size() != 1) continue;
+    if (!sc || sc->kind != OP_CONV_BIAS_ACTIV || sc->mode != 5 || sc->group != 1 || sc->dimB.size() != 4 || z->uses.size() != 1) continue;
     if (z->shape != m->result->shape || sc->operands[0]->shape.size() != 4) continue;
-    // the two channel counts the runtime has single-stage kernels for (ResNet-50's first and second stage)
-    const int64_t c1 = m->dimB[1], c2 = sc->dimB[1];
-    if (!((c1 == 64 && c2 == 64) || (c1 == 128 && c2 == 256))) continue;
     Value *out = m->operands[5];
     Op *fused = p.new_op(OP_CONV_ADD_CONV_ACTIV);
     fused->pads = m->pads; fused->strides = m->strides; fused->group = 1;

@@ -35,6 +35,12 @@ struct IgemmArgs {
   int64_t a_z_stride, x_z_stride, y_z_stride, bias_z_stride;
   unsigned magic_rs, magic_s;  // filled in by launch_igemm_f32: magic_of(R * S), magic_of(S), for the generic filter sizes
   int xcd_m;          // (small kernels, set by their launcher) the XCDs form an xcd_m x (8 / xcd_m) grid over the tile plane
+  // (conv1x1_f32_small_kernel) a second 1x1 convolution onto the same result, its reduction appended to the first's:
+  // filter A2 ([M][Kdim2] or, a_mcontig, [Kdim2][a_ld]), input X2 of H2 x W2 pixels per channel read with strides sh2, sw2,
+  // bias2 per row or null.  A2 == nullptr: none.
+  const float *A2, *X2, *bias2;
+  int Kdim2, H2, W2, sh2, sw2;
+  int64_t x2_img_stride;
   bool b_kcontig;     // B stored [Ncols][Kdim] (k contiguous): GEMM with transB
   bool a_mcontig;     // A stored [Kdim][M]: GEMM with transA
   bool a_vec4;        // A rows may be read as aligned float4

@@ -313,22 +313,32 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   if (tm_local >= tm_per || tile_m >= tiles_m || tile_n >= tiles_n) return;
   const int tile_id = tile_m * tiles_n + tile_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
-  const float *__restrict__ Ag = a.A + (int64_t)z * a.a_z_stride;
-  const float *__restrict__ Xg = a.X + (int64_t)z * a.x_z_stride;
+  // With a second convolution (a.A2) the reduction is the first's followed by the second's; a wavefront's slice
+  // lies in one of them (the launcher makes k_per_wave divide Kdim), so it only picks its operands here.
+  const int kbeg_all = ((int)blockIdx.y * KS + wave) * k_per_wave;
+  const bool second = a.A2 != nullptr && kbeg_all >= a.Kdim;
+  const float *__restrict__ Ag = second ? a.A2 : a.A + (int64_t)z * a.a_z_stride;
+  const float *__restrict__ Xg = second ? a.X2 : a.X + (int64_t)z * a.x_z_stride;
+  const int Kd = second ? a.Kdim2 : a.Kdim;
 
   const int m = m0 + l32, mrow = m < a.M ? m : 0;
   const int col = n0 + l32;
   const bool col_ok = col < a.Ncols;
-  const int PQ = a.P * a.Q, HW = a.H * a.W;
+  const int PQ = a.P * a.Q, HW = second ? a.H2 * a.W2 : a.H * a.W;
   float bias_r[16];
   prefetch_bias(a, z, m0, half, bias_r);
+  if (a.A2 != nullptr && a.bias2 != nullptr) {  // both biases ride in the one epilogue
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias_r[r] += a.bias2[min(acc_row(m0, half, r), a.M - 1)];
+  }
   const float bias_c = load_bias_col(a, col_ok ? col : 0);  // requested up front as well
   const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
   const int p = pq / a.Q, q = pq - p * a.Q;
-  const unsigned x_pix = (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
-  const unsigned a_row = (unsigned)mrow * (unsigned)a.Kdim, lda = (unsigned)a.a_ld;
+  const unsigned x_pix = second ? (unsigned)((int64_t)img * a.x2_img_stride + (int64_t)(p * a.sh2) * a.W2 + q * a.sw2)
+                                : (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
+  const unsigned a_row = (unsigned)mrow * (unsigned)Kd, lda = (unsigned)a.a_ld;
 
-  const int kbeg = ((int)blockIdx.y * KS + wave) * k_per_wave, kend = min(a.Kdim, kbeg + k_per_wave);
+  const int kbeg = second ? kbeg_all - a.Kdim : kbeg_all, kend = min(Kd, kbeg + k_per_wave);
   const int niter = k_per_wave >> 3;
 
   constexpr int DEPTH = 4;
@@ -337,7 +347,7 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   unsigned km[DEPTH];
   auto load_iter = [&](int i, float4 &av, float (&bv)[4], unsigned &kmask) {
     const int ka = kbeg + 8 * i + 4 * half;
-    const unsigned kc = (unsigned)min(ka, a.Kdim - 4);
+    const unsigned kc = (unsigned)min(ka, Kd - 4);
     kmask = ka < kend ? 0xffffffffu : 0u;
     if (AMC) {
       const unsigned ao = kc * lda + (unsigned)mrow;
@@ -406,12 +416,19 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
   const bool is3x3 = rsmode == 3 && a.Kdim % 9 == 0 && !a.bias_col;
   const bool is1x1 = rsmode == 1 && (amc || a.a_vec4) && a.Kdim % 4 == 0 && a.Kdim >= 4;
   if (!is3x3 && !is1x1) return true;
+  const bool dual = a.A2 != nullptr;
+  if (dual) {
+    const int64_t x2_elems = (int64_t)((a.Ncols + a.P * a.Q - 1) / (a.P * a.Q)) * a.x2_img_stride + (int64_t)a.Kdim2 * a.H2 * a.W2;
+    if (!is1x1 || a.Z != 1 || a.Kdim2 % 8 != 0 || a.Kdim % 8 != 0 || x2_elems >= (1ll << 31) || (int64_t)a.Kdim2 * a.a_ld >= (1ll << 31) ||
+        (int64_t)a.M * a.Kdim2 >= (1ll << 31))
+      return true;
+  }
 
   const int64_t tiles64 = ceil_div(a.M, 32) * ceil_div(a.Ncols, 32);
   if (tiles64 > INT32_MAX) return true;
   const int tiles = (int)tiles64;
   const int64_t want_waves = (int64_t)ctx->num_cu * 8;
-  const int red_len = is3x3 ? a.Kdim / 9 : a.Kdim;   // channels
+  const int red_len = is3x3 ? a.Kdim / 9 : a.Kdim + (dual ? a.Kdim2 : 0);   // channels
   const int min_slice = is3x3 ? 4 : 32;              // reduction slice worth a wavefront
   int ks = 1;
   while (ks < 8 && (int64_t)tiles * a.Z * ks < want_waves && ceil_div(red_len, ks * 2) >= min_slice) ks *= 2;
@@ -429,6 +446,15 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
       return false;
     }
     splits *= 2;
+  }
+  int k_per_wave_1x1 = (int)(ceil_div(ceil_div(red_len, ks * splits), 8) * 8);
+  if (dual) {
+    // a slice must not straddle the two reductions: the next power of two, which has to divide the first one's
+    // length (wavefronts whose slice starts past the end find every k masked)
+    int p2 = 8;
+    while (p2 < k_per_wave_1x1) p2 *= 2;
+    if (a.Kdim % p2 != 0) return true;  // not launched: the caller runs the two convolutions one after the other
+    k_per_wave_1x1 = p2;
   }
   // The XCD grid: xcd_m x (8 / xcd_m) rectangles of tiles.  Elements fetched over all eight L2s: the filter
   // 8 / xcd_m times, the activations xcd_m times; rectangles that do not divide the tile counts leave
@@ -466,8 +492,7 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
     const int c_per_wave = (int)(ceil_div(ceil_div(red_len, ks * splits), 2) * 2);
     LAUNCH_KS(conv3x3_f32_small_kernel, c_per_wave);
   } else {
-    const int k_per_wave = (int)(ceil_div(ceil_div(red_len, ks * splits), 8) * 8);
-    LAUNCH_KS(conv1x1_f32_small_kernel, k_per_wave);
+    LAUNCH_KS(conv1x1_f32_small_kernel, k_per_wave_1x1);
   }
 #undef LAUNCH_KS
 #undef LAUNCH_KS2

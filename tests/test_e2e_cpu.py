@@ -244,6 +244,26 @@ def test_activation_fusion_matches_unfused_chain(builder):
         np.testing.assert_array_equal(x, y)
 
 
+def test_projection_shortcut_fusion_matches_unfused_chain():
+    """The oracle runs the fused shortcut + closer call as the chain of the two calls: not a bit may change, per
+    inference (with the debug fill), without the dealloc pass, and resident; four launches fewer."""
+    small = lambda: models.resnet50(image=32, classes=10)  # noqa: E731
+    flags = dict(fusion=True, fuse_residual=True)
+    _, _, a = run_oracle(small, **flags)
+    assert small()[0].compile(fuse_projection_shortcut=True, **flags).text.count("add-conv") == 4
+    for more in (dict(), dict(dealloc_opt=False)):
+        _, _, b = run_oracle(small, fuse_projection_shortcut=True, **flags, **more)
+        np.testing.assert_array_equal(a[0], b[0])
+    _, _, c = run_oracle(small, mode=compiler.MODE_RESIDENT, fuse_projection_shortcut=True, **flags)
+    np.testing.assert_array_equal(a[0], c[0])
+    check(small, fuse_projection_shortcut=True, **flags)
+    g, inputs = small()
+    s = g.compile(fuse_projection_shortcut=True, **flags).session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+    s.set_debug_fill(0xFF)
+    np.testing.assert_array_equal(s.run(*inputs)[0], a[0])
+    s.close()
+
+
 @pytest.mark.parametrize("builder,copies", [(lambda: models.resnet50(image=32, classes=10), 1), (ALEX, 1),
                                             (lambda: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128), None),
                                             (YOLO, None)],

@@ -264,6 +264,18 @@ def test_projection_shortcut_fusion_fp16_channels_last(batch, image):
     np.testing.assert_array_equal(res[0], one[0])
 
 
+def test_projection_shortcut_fusion_fp32(oracle_outputs):
+    """fp32 ResNet-50 at batch 1 with every shortcut pair as one call (four launches fewer; the pairs' sums are rounded
+    once instead of three times): the oracle's result to the usual fp32 tolerance, per inference and resident."""
+    flags = dict(fusion=True, fuse_residual=True, fuse_projection_shortcut=True)
+    assert CONFIGS["resnet50"]()[0].compile(**flags).text.count("add-conv") == 4
+    out, info = run(CONFIGS["resnet50"], **flags)
+    assert info["requested"] == info["pool"]
+    close(out[0], oracle_outputs["resnet50"][0])
+    res, _ = run(CONFIGS["resnet50"], mode=compiler.MODE_RESIDENT, **flags)
+    np.testing.assert_array_equal(res[0], out[0])
+
+
 @pytest.mark.parametrize("name", ["resnet50", "mobilenet_v2"])
 def test_residual_fusion_fp32(name, oracle_outputs):
     """conv+bias -> add -> relu as one call: against the oracle, and bit for

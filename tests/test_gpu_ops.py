@@ -718,8 +718,8 @@ def dual_conv_f16(gpu, x, w, b, x2, w2, b2, stride2, activ):
 def test_last_convolution_and_projection_shortcut_in_one_call(gpu, cpu, case):
     """dnnrtConvBiasAddConvBiasActiv against the two calls it replaces: the oracle's chain to the fp16 convolutions'
     tolerance, and this library's own two calls bit for bit (each conv + bias rounded to fp16 on its own, the sum
-    and ReLU in fp32).  N, H2, W2, C, C2, K, stride of the shortcut; ragged tiles in both directions; 64 + 64
-    channels take the single-stage kernel, the rest the general one."""
+    and ReLU in fp32).  N, H2, W2, C, C2, K, stride of the shortcut; ragged tiles in both directions; 64 + 64 and
+    128 + 256 channels take the one-kernel form, the rest run as the two convolutions through Y."""
     N, H2, W2, C, C2, K, st = case
     P, Q = (H2 - 1) // st + 1, (W2 - 1) // st + 1
     r = rng(sum(case))
@@ -743,24 +743,82 @@ def test_last_convolution_and_projection_shortcut_in_one_call(gpu, cpu, case):
         np.testing.assert_array_equal(cpu.get(Y), ref)
 
 
+@pytest.mark.parametrize("case", [(1, 56, 56, 64, 64, 256, 1), (1, 56, 56, 128, 256, 512, 2), (1, 28, 28, 256, 512, 1024, 2),
+                                  (1, 14, 14, 512, 1024, 2048, 2), (2, 9, 11, 24, 40, 72, 1), (16, 28, 28, 128, 256, 512, 2)],
+                         ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("crsk", [False, True])
+def test_last_convolution_and_projection_shortcut_fp32(gpu, cpu, case, crsk):
+    """The same call on fp32 N,C,H,W tensors with both filter layouts: ResNet-50's four shortcut pairs at batch 1 (one
+    launch of the small 1x1 kernel, the second reduction appended to the first: one rounding of the whole sum where the
+    chain has three), an odd-sized pair and a batch-16 pair (the two convolutions one after the other through Y: the
+    chain's bits).  Against the oracle's chain: rtol 1e-4, atol 1e-5 as for every fp32 convolution."""
+    N, H2, W2, C, C2, K, st = case
+    P, Q = (H2 - 1) // st + 1, (W2 - 1) // st + 1
+    r = rng(sum(case))
+    x = r.standard_normal((N, C, P, Q)).astype(np.float32)
+    x2 = r.standard_normal((N, C2, H2, W2)).astype(np.float32)
+    w = (r.standard_normal((K, C, 1, 1)) * np.sqrt(2.0 / C)).astype(np.float32)
+    w2 = (r.standard_normal((K, C2, 1, 1)) * np.sqrt(2.0 / C2)).astype(np.float32)
+    b, b2 = r.uniform(-0.2, 0.2, K).astype(np.float32), r.uniform(-0.2, 0.2, K).astype(np.float32)
+    z_ref = oc.conv(cpu, x2, w2, b2, (0, 0), (st, st), 1, _abi.ACT_IDENTITY)
+    ref = oc.conv(cpu, x, w, b, (0, 0), (1, 1), 1, _abi.ACT_RELU, z=z_ref)
+    lay = (lambda t: np.ascontiguousarray(t.transpose(1, 2, 3, 0))) if crsk else (lambda t: t)
+    X, Wt, B, X2, Wt2, B2 = gpu.put(x), gpu.put(lay(w)), gpu.put(b), gpu.put(x2), gpu.put(lay(w2)), gpu.put(b2)
+    Y = gpu.empty(ref.shape, np.float32)
+    gpu.ops.set_filter_layout(_abi.FILTER_CRSK if crsk else _abi.FILTER_KCRS)
+    try:
+        for _ in range(2):  # twice: the split reduction's counters must be back at zero
+            gpu.ops.conv_bias_add_conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), gpu.ptr(X2), x2.shape,
+                                                  gpu.ptr(Wt2), w2.shape, gpu.ptr(B2), (0, 0), (st, st), _abi.ACT_RELU, gpu.ptr(Y), dtype=_abi.F32)
+            gpu.sync()
+            np.testing.assert_allclose(gpu.get(Y), ref, rtol=1e-4, atol=1e-5)
+    finally:
+        gpu.ops.set_filter_layout(_abi.FILTER_KCRS)
+
+
+def test_last_convolution_and_projection_shortcut_with_other_convolutions(gpu, cpu):
+    """Shapes the one-kernel forms do not take run as the two convolutions through Y and give the chain's bits: a 3x3
+    closing convolution in fp16 channels-last, 192 + 128 channels, and an fp32 pair with padding."""
+    r = rng(11)
+    x = r.standard_normal((2, 64, 9, 9)).astype(np.float16)
+    x2 = r.standard_normal((2, 128, 9, 9)).astype(np.float16)
+    w = (r.standard_normal((72, 64, 3, 3)) * 0.06).astype(np.float16)
+    w2 = (r.standard_normal((72, 128, 1, 1)) * 0.1).astype(np.float16)
+    b, b2 = r.uniform(-0.2, 0.2, 72).astype(np.float16), r.uniform(-0.2, 0.2, 72).astype(np.float16)
+    nhwc = lambda t: np.ascontiguousarray(t.transpose(0, 2, 3, 1))  # noqa: E731
+    X, Wt, B, X2, Wt2, B2 = gpu.put(nhwc(x)), gpu.put(nhwc(w)), gpu.put(b), gpu.put(nhwc(x2)), gpu.put(nhwc(w2)), gpu.put(b2)
+    Y = gpu.empty((2 * 72 * 9 * 9,), np.float16)
+    gpu.ops.set_format(_abi.NHWC)
+    try:
+        gpu.ops.conv_bias_add_conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (1, 1), (1, 1), gpu.ptr(X2), x2.shape,
+                                              gpu.ptr(Wt2), w2.shape, gpu.ptr(B2), (0, 0), (1, 1), _abi.ACT_RELU, gpu.ptr(Y))
+        gpu.sync()
+    finally:
+        gpu.ops.set_format(_abi.NCHW)
+    got = gpu.get(Y).reshape(2, 9, 9, 72).transpose(0, 3, 1, 2)
+    z_gpu = conv_f16(gpu, x2, w2, b2, (0, 0), (1, 1), 1, _abi.ACT_IDENTITY, _abi.NHWC)
+    two = conv_f16(gpu, x, w, b, (1, 1), (1, 1), 1, _abi.ACT_RELU, _abi.NHWC, z=z_gpu)
+    np.testing.assert_array_equal(got, two)
+    z_ref = oc.conv(cpu, x2, w2, b2, (0, 0), (1, 1), 1, _abi.ACT_IDENTITY)
+    ref = oc.conv(cpu, x, w, b, (1, 1), (1, 1), 1, _abi.ACT_RELU, z=z_ref)
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=4e-3, atol=4e-3)
+
+
 def test_last_convolution_and_projection_shortcut_refuses_other_shapes(gpu):
     r = rng(4)
     x = r.standard_normal((1, 64, 8, 8)).astype(np.float16)
     w = r.standard_normal((64, 64, 1, 1)).astype(np.float16)
     b = np.zeros(64, np.float16)
-    w3 = r.standard_normal((64, 64, 3, 3)).astype(np.float16)
-    X, Wt, B, W3 = gpu.put(x), gpu.put(w), gpu.put(b), gpu.put(w3)
+    X, Wt, B = gpu.put(x), gpu.put(w), gpu.put(b)
     Y = gpu.empty((64 * 64,), np.float16)
-    call = lambda fmt, wt2, dw2, pads2, dx2=(1, 64, 8, 8): (gpu.ops.set_format(fmt), gpu.ops.conv_bias_add_conv_bias_activ(  # noqa: E731
-        gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), gpu.ptr(X), dx2, gpu.ptr(wt2), dw2, gpu.ptr(B), pads2, (1, 1),
-        _abi.ACT_RELU, gpu.ptr(Y)))
+    gpu.ops.set_format(_abi.NHWC)
     try:
-        with pytest.raises(RuntimeError, match="1x1"):
-            call(_abi.NHWC, W3, w3.shape, (1, 1))
-        with pytest.raises(RuntimeError, match="DNNRT_NHWC"):
-            call(_abi.NCHW, Wt, w.shape, (0, 0))
-        with pytest.raises(RuntimeError, match="give"):
-            call(_abi.NHWC, Wt, w.shape, (0, 0), (1, 64, 4, 16))
+        with pytest.raises(RuntimeError, match="give"):  # the two convolutions must land on the same tensor
+            gpu.ops.conv_bias_add_conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), gpu.ptr(X), (1, 64, 4, 16),
+                                                  gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), _abi.ACT_RELU, gpu.ptr(Y))
+        with pytest.raises(RuntimeError, match="dtype"):
+            gpu.ops.conv_bias_add_conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), gpu.ptr(X), x.shape,
+                                                  gpu.ptr(Wt), w.shape, gpu.ptr(B), (0, 0), (1, 1), _abi.ACT_RELU, gpu.ptr(Y), dtype=_abi.I64)
     finally:
         gpu.ops.set_format(_abi.NCHW)
 
