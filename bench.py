@@ -37,7 +37,7 @@ def build_workload(name, batch=None):
     from occamy_amd import models
     if name == "resnet50_fp32_bs1":
         b = batch or 1
-        return models.resnet50(b, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, fuse_projection_shortcut=True, alias_copies=True), b, "img/s", "f32"
+        return models.resnet50(b, np.float32), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True, alias_copies=True), b, "img/s", "f32"
     if name == "resnet50_fp16_bs64":
         b = batch or 64
         return (models.resnet50(b, np.float16, seed=5),

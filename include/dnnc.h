@@ -64,10 +64,11 @@ typedef struct {
                              becomes one call (default 0) */
   int32_t fuse_attention; /* no reference flag: the head split, QK^T, scaling, Softmax, PV and
                              head merge of an exported attention block become one call (default 0) */
-  int32_t fuse_first_layer_maxpool; /* no reference flag: with `fusion` and `channels_last`, a ResNet's first
-                             convolution (3 -> 64 channels, 7x7, stride 2, pad 3, even image width, ReLU or
-                             identity) and the 3x3 / stride 2 / pad 1 max-pool behind it become one call
-                             that never stores the convolution's result (default 0) */
+  int32_t fuse_first_layer_maxpool; /* no reference flag: with `fusion`, a ResNet's first convolution (3 -> 64
+                             channels, 7x7, stride 2, pad 3, ReLU or identity) and the 3x3 / stride 2 / pad 1
+                             max-pool behind it become one call that never stores the convolution's result;
+                             fp32 programs, and fp16 programs with `channels_last` and an even image width
+                             (default 0) */
   int32_t fuse_projection_shortcut; /* no reference flag: with `fusion` and `fuse_residual`, the projection shortcut of a
                              residual block (conv + bias) and the block's last convolution (+ add + activation)
                              become one call, and the shortcut's result has no tensor of its own (fp16 programs:

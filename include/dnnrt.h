@@ -219,13 +219,15 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X,
  * the convolution's result (four times the pooled tensor) never stored.  It
  * replaces the reference's two calls (CUDNNConvBiasReluFunc.cpp:8-140, then
  * CUDNNMaxPoolFunc.cpp:8-78); every element is what that chain stores: the
- * activation's output rounded to fp16, then the maximum over the window,
+ * activation's output in the tensors' type, then the maximum over the window,
  * padding ignored, NaN propagated.  One shape only, anything else fails with
  * an error (nothing falls back to the two calls, which would need a buffer
- * for the intermediate tensor): fp16, tensor format DNNRT_NCHW_TO_NHWC (X is
- * the N,C,H,W function argument, Y is N,H,W,C), filter K,R,S,C with 3 -> 64
- * channels, 7x7, stride 2, pad 3, group 1, activMode ReLU or identity; pooling
- * 3x3, stride 2, pad 1.  dimY = [N, 64, PP, QQ], the pooled extents. */
+ * for the intermediate tensor): 3 -> 64 channels, 7x7, stride 2, pad 3,
+ * group 1, activMode ReLU or identity; pooling 3x3, stride 2, pad 1; either
+ * fp16 with tensor format DNNRT_NCHW_TO_NHWC (X is the N,C,H,W function
+ * argument with an even width, Y is N,H,W,C, filter K,R,S,C) or fp32 with
+ * format DNNRT_NCHW (filter in the handle's filter layout).
+ * dimY = [N, 64, PP, QQ], the pooled extents. */
 void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X,
                                 const int64_t *dimX, const void *W,
                                 const int64_t *dimW, const void *B,

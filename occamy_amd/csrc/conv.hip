@@ -8,6 +8,7 @@
 #include "common.h"
 #include "igemm_f32.h"
 #include "conv_f16.h"
+#include "conv_f32_stem.h"
 
 #include <string.h>
 
@@ -187,6 +188,11 @@ __global__ __launch_bounds__(256) void conv_f32_narrow_kernel(
     }
 }
 
+// 3 -> 64 channels, 7x7, stride 2, pad 3: the shape conv_f32_stem.hip is written for.
+static bool stem_f32_shape(const ConvShape &s) {
+  return s.group == 1 && s.C == 3 && s.K == 64 && s.R == 7 && s.S == 7 && s.sh == 2 && s.sw == 2 && s.ph == 3 && s.pw == 3;
+}
+
 static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const float *X,
                            const float *Wt, const float *bias, const float *Z, int act, float *Y) {
   // Filter storage: K,C,R,S (the reference's) or C,R,S,K (k_out contiguous),
@@ -222,6 +228,11 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
       hipLaunchKernelGGL((conv_f32_narrow_kernel<4, 1, 1>), grid, block, lds, ctx->stream, X, Wt, bias, Z, Y, s.C, s.H, s.W, s.K,
                          s.P, s.Q, s.ph, s.pw, s.sh, s.sw, act, ctx->act_coef, w_k, w_tap);
     DNNRT_CHECK_LAUNCH("conv(narrow)");
+    return Y;
+  }
+  if (stem_f32_shape(s) && bias && !Z && (int64_t)s.N * ceil_div(s.P, 5) * ceil_div(s.Q, 16) <= 4 * (int64_t)ctx->num_cu) {
+    // the first layer of the ImageNet networks at small batches: one workgroup per 5 x 16 pixels, patch in LDS
+    if (!launch_conv_f32_stem(ctx, s.N, s.H, s.W, s.P, s.Q, X, Wt, bias, act, Y, false, 0, 0)) return nullptr;
     return Y;
   }
   IgemmArgs a{};
@@ -384,7 +395,7 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64
   if (!X || !W || !Y || !dimX || !dimW || !dimY || !pads || !strides || !poolKernel || !poolPads || !poolStrides)
     DNNRT_FAIL("%s: null argument", who);
   if (!B || !dimB || dnnrt::numel(dimB, 4) != dimW[0]) DNNRT_FAIL("%s: bias must hold K values", who);
-  if (dtype != DNNRT_F16) DNNRT_FAIL("%s: fp16 tensors only", who);
+  if (dtype != DNNRT_F16 && dtype != DNNRT_F32) DNNRT_FAIL("%s: dtype %d", who, dtype);
   if (poolKernel[0] != 3 || poolKernel[1] != 3 || poolStrides[0] != 2 || poolStrides[1] != 2 || poolPads[0] != 1 || poolPads[1] != 1)
     DNNRT_FAIL("%s: the pooling must be 3x3, stride 2, pad 1", who);
   dnnrt::ConvShape s;
@@ -394,6 +405,14 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64
     DNNRT_FAIL("%s: dimY is [%ld,%ld,%ld,%ld], the pooled convolution is [%d,%d,%ld,%ld]", who, (long)dimY[0], (long)dimY[1],
                (long)dimY[2], (long)dimY[3], s.N, s.K, (long)PP, (long)QQ);
   if (s.N == 0) return Y;
+  if (dtype == DNNRT_F32) {
+    if (handle->format != DNNRT_NCHW) DNNRT_FAIL("%s: fp32 tensors are NCHW only", who);
+    if (!dnnrt::stem_f32_shape(s)) DNNRT_FAIL("%s: the convolution must be 3 -> 64 channels, 7x7, stride 2, pad 3", who);
+    if (!dnnrt::launch_conv_f32_stem(handle, s.N, s.H, s.W, s.P, s.Q, (const float *)X, (const float *)W, (const float *)B,
+                                     (int)activMode, (float *)Y, true, (int)PP, (int)QQ))
+      return nullptr;
+    return Y;
+  }
   dnnrt::ConvF16Args a{};
   a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Z = nullptr; a.Y = nullptr;
   a.N = s.N; a.C = s.C; a.H = s.H; a.W = s.W; a.K = s.K; a.Cg = s.Cg; a.R = s.R; a.S = s.S;

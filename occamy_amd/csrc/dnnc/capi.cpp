@@ -134,7 +134,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (opt->fusion && opt->fuse_activations) fuse_conv_activations(p);
   if (opt->fusion && opt->fuse_matmul_bias) fuse_matmul_bias(p);
   if (opt->fusion && opt->fuse_residual) fuse_residual_add(p);
-  if (opt->fusion && opt->fuse_first_layer_maxpool && opt->channels_last) fuse_first_layer_maxpool(p);
+  if (opt->fusion && opt->fuse_first_layer_maxpool) fuse_first_layer_maxpool(p);
   if (opt->fusion && opt->fuse_residual && opt->fuse_projection_shortcut) fuse_projection_shortcut(p);
   if (opt->alias_copies) alias_copies(p);
   if (opt->dealloc_opt) dealloc_opt(p);

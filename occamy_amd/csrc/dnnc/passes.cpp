@@ -131,9 +131,10 @@ void fuse_residual_add(Program &p) {
 
 // The first two layers of an ImageNet ResNet, conv 7x7 / stride 2 / pad 3 over the 3-channel function argument
 // (+ bias, ReLU or identity) -> max-pool 3x3 / stride 2 / pad 1, the convolution's result read by nothing else,
-// become one call that never stores that result (four times the pooled tensor).  Channels-last fp16 programs
-// only, and only this shape with an even image width: it is the one the runtime's kernel is written for, and the
-// runtime refuses everything else rather than fall back.  The reference has no such pattern
+// become one call that never stores that result (four times the pooled tensor).  Channels-last fp16 programs (even
+// image width, input straight from the function argument) and N,C,H,W fp32 programs, and only this shape: it is
+// the one the runtime's kernels are written for, and the runtime refuses everything else rather than fall back.
+// The reference has no such pattern
 // (src/Dialect/DNN/Transforms/fuseConvBiasRelu.cpp stops at the activation).
 void fuse_first_layer_maxpool(Program &p) {
   std::vector<Op *> convs;
@@ -141,14 +142,16 @@ void fuse_first_layer_maxpool(Program &p) {
     if (op->kind == OP_CONV_BIAS_ACTIV && (op->mode == 1 || op->mode == 5)) convs.push_back(op);
   for (Op *conv : convs) {
     const Shape &dx = conv->dimA, &dw = conv->dimB;
-    if (dx.size() != 4 || dw.size() != 4 || conv->result->dtype != F16) continue;
-    if (dw[0] != 64 || dw[1] != 3 || dw[2] != 7 || dw[3] != 7 || conv->group != 1 || (dx[3] & 1)) continue;
+    const bool f16 = conv->result->dtype == F16;
+    if (dx.size() != 4 || dw.size() != 4) continue;
+    if (f16 ? !p.channels_last_requested : (conv->result->dtype != F32 || p.channels_last_requested)) continue;
+    if (dw[0] != 64 || dw[1] != 3 || dw[2] != 7 || dw[3] != 7 || conv->group != 1 || (f16 && (dx[3] & 1))) continue;
     if (conv->pads != Shape{3, 3} || conv->strides != Shape{2, 2}) continue;
     // the input must be the device copy of a function argument (N,C,H,W as the host sent it)
     bool from_arg = false;
     for (const auto &u : conv->operands[0]->uses)
       if (u.first->kind == OP_MEMCPY && u.first->mode == 1 && u.second == 0 && u.first->operands[1]->arg_index >= 0) from_arg = true;
-    if (!from_arg || conv->result->uses.size() != 1) continue;
+    if ((f16 && !from_arg) || conv->result->uses.size() != 1) continue;
     Op *pool = conv->result->uses.front().first;
     if (pool->kind != OP_MAXPOOL || pool->operands[0] != conv->result) continue;
     if (pool->kernel != Shape{3, 3} || pool->strides != Shape{2, 2} || pool->pads.size() < 2 || pool->pads[0] != 1 || pool->pads[1] != 1)

@@ -273,7 +273,8 @@ def test_fp16_channels_last_flag():
 
 def test_first_layer_maxpool_fusion():
     """conv 7x7/2 over the 3-channel argument + ReLU + max-pool 3x3/2 -> one call, in channels-last fp16 programs with
-    an even image width only; the convolution's buffer (the largest activation of the network) is never allocated."""
+    an even image width and in fp32 programs; the convolution's buffer (the largest activation of the network) is
+    never allocated."""
     flags = dict(fusion=True, fuse_residual=True, channels_last=True)
     g, _ = models.resnet50(dtype=np.float16, **SMALL)
     plain = g.compile(**flags)
@@ -291,11 +292,18 @@ def test_first_layer_maxpool_fusion():
     gone.remove(conv_bytes)
     assert sizes(fused) == gone
     check_lifetimes(lambda: models.resnet50(dtype=np.float16, **SMALL), fuse_first_layer_maxpool=True, **flags)
-    # not without channels-last (the kernel writes N,H,W,C), not for fp32, not for an odd width
+    # fp16: not without channels-last (the kernel writes N,H,W,C), not for an odd width
     g, _ = models.resnet50(dtype=np.float16, **SMALL)
     assert "maxpoolfwd" not in g.compile(fusion=True, fuse_first_layer_maxpool=True).text
-    g, _ = models.resnet50(dtype=np.float32, **SMALL)
-    assert "maxpoolfwd" not in g.compile(fusion=True, fuse_first_layer_maxpool=True).text
+    # fp32 N,C,H,W programs: any width
+    for shape in (SMALL, dict(SMALL, image=SMALL.get("image", 32) + 1)):
+        g, _ = models.resnet50(dtype=np.float32, **shape)
+        plain32 = g.compile(fusion=True)
+        g, _ = models.resnet50(dtype=np.float32, **shape)
+        fused32 = g.compile(fusion=True, fuse_first_layer_maxpool=True)
+        assert fused32.text.count("dnn.conv-bias-relu-maxpoolfwd") == 1 and "dnn.maxpool " not in fused32.text
+        assert fused32.num_ops(compute_only=True) == plain32.num_ops(compute_only=True) - 1
+    check_lifetimes(lambda: models.resnet50(dtype=np.float32, **SMALL), fusion=True, fuse_residual=True, fuse_first_layer_maxpool=True)
     odd = dict(SMALL, image=SMALL.get("image", 32) + 1)
     g, _ = models.resnet50(dtype=np.float16, **odd)
     assert "maxpoolfwd" not in g.compile(fuse_first_layer_maxpool=True, **flags).text

@@ -98,6 +98,8 @@ def test_poisoned_pool_changes_nothing_on_the_gpu():
              (lambda: models.resnet50(4, np.float16, seed=5, image=64), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True)),
              (lambda: models.resnet50(4, np.float16, seed=5, image=64),
               dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True)),
+             (lambda: models.resnet50(image=64, classes=100),
+              dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True)),
              (lambda: models.srgan_generator(1, np.float32, height=24, width=16), dict(fusion=True, fuse_activations=True))]
     for builder, flags in cases:
         g, inputs = builder()
@@ -224,6 +226,25 @@ def test_first_layer_maxpool_fusion_fp16_channels_last(batch, image):
     np.testing.assert_array_equal(res[0], one[0])
     ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
     np.testing.assert_allclose(one[0].astype(np.float32), ref[0], rtol=2e-2, atol=2e-2 * float(np.abs(ref[0]).max()))
+
+
+@pytest.mark.parametrize("batch,image", [(1, 224), (2, 75)])
+def test_first_layer_maxpool_fusion_fp32(batch, image):
+    """fp32 N,C,H,W programs: the first convolution and its max-pool as one call, per inference and replayed from a
+    captured graph, against the oracle running the unfused program to the fp32 tolerance of every ResNet-50 test
+    here; and against this library's own two calls bit for bit (the unfused first layer runs the same kernel's
+    arithmetic, the maximum is exact)."""
+    build = lambda: models.resnet50(batch, seed=6, image=image, classes=100)  # noqa: E731
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, fuse_projection_shortcut=True, alias_copies=True)  # the benchmark's
+    assert "maxpoolfwd" in build()[0].compile(fuse_first_layer_maxpool=True, **flags).text
+    two, _ = run(build, **flags)
+    one, info = run(build, fuse_first_layer_maxpool=True, **flags)
+    assert info["requested"] == info["pool"]
+    np.testing.assert_array_equal(one[0], two[0])
+    res, _ = run(build, mode=compiler.MODE_RESIDENT, fuse_first_layer_maxpool=True, **flags)
+    np.testing.assert_array_equal(res[0], one[0])
+    ref, _ = run(build, ORACLE_PATH, fusion=True)
+    close(one[0], ref[0], 1e-4, 1e-4)
 
 
 def test_aliased_copies_change_nothing_on_the_gpu():

@@ -696,6 +696,68 @@ def test_first_layer_with_its_max_pool_refuses_other_shapes(gpu):
             gpu.ops.set_format(_abi.NCHW)
 
 
+@pytest.mark.parametrize("case", [(1, 224, 224), (2, 64, 64), (3, 37, 51), (1, 9, 9), (2, 30, 61)], ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("crsk", [False, True])
+@pytest.mark.parametrize("activ", [_abi.ACT_RELU, _abi.ACT_IDENTITY])
+def test_first_layer_fp32_alone_and_with_its_max_pool(gpu, cpu, case, crsk, activ):
+    """The fp32 N,C,H,W first layer (3 -> 64 channels, 7x7, stride 2, pad 3) through dnnrtConvBiasActiv and, with the
+    3x3 stride-2 pooling behind it, through dnnrtConvBiasActivMaxPool, against the oracle's convolution and its chain:
+    rtol 1e-4, atol 1e-5 as for every fp32 convolution (the maximum adds no rounding).  Both filter layouts; the
+    benchmark's size, odd sizes with ragged tiles in both directions, an image smaller than one tile; identity
+    activation leaves negative values, so a padding of zeros instead of -inf would show."""
+    N, H, W = case
+    r = rng(N + H + W + activ)
+    x = r.standard_normal((N, 3, H, W)).astype(np.float32)
+    w = (r.standard_normal((64, 3, 7, 7)) * np.sqrt(2.0 / 147)).astype(np.float32)
+    b = r.uniform(-0.5, 0.1, 64).astype(np.float32)
+    if case == (3, 37, 51):
+        x[1, 2, 11, 30] = np.nan
+        x[2, 0, 5, 40] = np.inf
+        x[2, 1, 6, 41] = -np.inf
+    conv_ref = oc.conv(cpu, x, w, b, (3, 3), (2, 2), 1, activ)
+    ref = oc.pool(cpu, "max", conv_ref, (3, 3), (1, 1), (2, 2))
+    lay = (lambda t: np.ascontiguousarray(t.transpose(1, 2, 3, 0))) if crsk else (lambda t: t)
+    X, Wt, B = gpu.put(x), gpu.put(lay(w)), gpu.put(b)
+    Yc, Yp = gpu.empty(conv_ref.shape, np.float32), gpu.empty(ref.shape, np.float32)
+    gpu.ops.set_filter_layout(_abi.FILTER_CRSK if crsk else _abi.FILTER_KCRS)
+    try:
+        gpu.ops.conv_bias_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (3, 3), (2, 2), activ, gpu.ptr(Yc))
+        gpu.ops.conv_bias_activ_max_pool(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), (3, 3), (2, 2), activ,
+                                         (3, 3), (1, 1, 1, 1), (2, 2), gpu.ptr(Yp), ref.shape, dtype=_abi.F32)
+        gpu.sync()
+    finally:
+        gpu.ops.set_filter_layout(_abi.FILTER_KCRS)
+    got_c, got = gpu.get(Yc), gpu.get(Yp)
+    finite = np.isfinite(conv_ref)
+    assert (np.isnan(got_c) == np.isnan(conv_ref)).all() and (np.isnan(got) == np.isnan(ref)).all()
+    np.testing.assert_allclose(got_c[finite], conv_ref[finite], rtol=1e-4, atol=1e-5)
+    np.testing.assert_array_equal(got_c[~finite & ~np.isnan(conv_ref)], conv_ref[~finite & ~np.isnan(conv_ref)])
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
+    if case == (3, 37, 51):
+        assert np.isnan(got[1]).any() and np.isnan(got[2]).any() and not np.isnan(got[0]).any()
+    # the pooled result is the exact maximum of this library's own convolution
+    Y2 = gpu.empty(ref.shape, np.float32)
+    gpu.ops.maxpool(gpu.ptr(Yc), conv_ref.shape, gpu.ptr(Y2), ref.shape, (3, 3), (1, 1, 1, 1), (2, 2), _abi.F32)
+    gpu.sync()
+    np.testing.assert_array_equal(got, gpu.get(Y2))
+
+
+def test_first_layer_fp32_with_its_max_pool_refuses_other_shapes(gpu):
+    r = rng(4)
+    x = r.standard_normal((1, 3, 32, 32)).astype(np.float32)
+    b = np.zeros(64, np.float32)
+    X, B = gpu.put(x), gpu.put(b)
+    Y = gpu.empty((64 * 8 * 8,), np.float32)
+    w5 = r.standard_normal((64, 3, 5, 5)).astype(np.float32)
+    with pytest.raises(RuntimeError, match="7x7"):
+        gpu.ops.conv_bias_activ_max_pool(gpu.ptr(X), x.shape, gpu.ptr(gpu.put(w5)), w5.shape, gpu.ptr(B), (2, 2), (2, 2), _abi.ACT_RELU,
+                                         (3, 3), (1, 1, 1, 1), (2, 2), gpu.ptr(Y), (1, 64, 8, 8), dtype=_abi.F32)
+    w7 = r.standard_normal((64, 3, 7, 7)).astype(np.float32)
+    with pytest.raises(RuntimeError, match="ReLU or identity"):
+        gpu.ops.conv_bias_activ_max_pool(gpu.ptr(X), x.shape, gpu.ptr(gpu.put(w7)), w7.shape, gpu.ptr(B), (3, 3), (2, 2), _abi.ACT_LEAKY_RELU,
+                                         (3, 3), (1, 1, 1, 1), (2, 2), gpu.ptr(Y), (1, 64, 8, 8), dtype=_abi.F32)
+
+
 def dual_conv_f16(gpu, x, w, b, x2, w2, b2, stride2, activ):
     """dnnrtConvBiasAddConvBiasActiv through the C-ABI; tensors in logical NCHW / KCRS order; returns logical NCHW."""
     N, C, P, Q = x.shape
