@@ -75,6 +75,9 @@ typedef struct {
                              with `channels_last` only; default 0) */
   int32_t alias_copies;   /* no reference flag: Flatten / Reshape / Squeeze / Unsqueeze name their input's buffer
                              as their output, so nothing is copied and nothing launched (default 0) */
+  int32_t inplace_residual; /* no reference flag: with `fusion` and `fuse_residual`, a fused conv + add + activation
+                             whose residual operand nothing reads afterwards writes its result over that operand
+                             (one tensor fewer in the pool, one fewer in the caches; default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);

@@ -202,8 +202,11 @@ void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X,
 /* New: the same call with the residual operand that
  * cudnnConvolutionBiasActivationForward has and the reference passes with a
  * zero weight (CUDNNConvBiasReluFunc.cpp:94-112: alpha2 = 0, z = y).
- * Y = act((conv(X, W) + B) + Z), Z shaped and laid out like Y, not
- * overlapping it.
+ * Y = act((conv(X, W) + B) + Z), Z shaped and laid out like Y: either Y
+ * itself (the result is written over the residual operand, which
+ * cudnnConvolutionBiasActivationForward allows as well: every kernel adds an
+ * element of Z in the thread that stores that element of Y) or not
+ * overlapping Y at all; X must not overlap Y.
  * It replaces the conv -> add -> relu chain that closes a residual block; the
  * sums are formed in that chain's order. */
 void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X,

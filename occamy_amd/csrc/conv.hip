@@ -230,9 +230,9 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
     DNNRT_CHECK_LAUNCH("conv(narrow)");
     return Y;
   }
-  if (stem_f32_shape(s) && bias && !Z && (int64_t)s.N * ceil_div(s.P, 5) * ceil_div(s.Q, 16) <= 4 * (int64_t)ctx->num_cu) {
+  if (stem_f32_shape(s) && bias && (int64_t)s.N * ceil_div(s.P, 5) * ceil_div(s.Q, 16) <= 4 * (int64_t)ctx->num_cu) {
     // the first layer of the ImageNet networks at small batches: one workgroup per 5 x 16 pixels, patch in LDS
-    if (!launch_conv_f32_stem(ctx, s.N, s.H, s.W, s.P, s.Q, X, Wt, bias, act, Y, false, 0, 0)) return nullptr;
+    if (!launch_conv_f32_stem(ctx, s.N, s.H, s.W, s.P, s.Q, X, Wt, bias, Z, act, Y, false, 0, 0)) return nullptr;
     return Y;
   }
   IgemmArgs a{};
@@ -409,7 +409,7 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64
     if (handle->format != DNNRT_NCHW) DNNRT_FAIL("%s: fp32 tensors are NCHW only", who);
     if (!dnnrt::stem_f32_shape(s)) DNNRT_FAIL("%s: the convolution must be 3 -> 64 channels, 7x7, stride 2, pad 3", who);
     if (!dnnrt::launch_conv_f32_stem(handle, s.N, s.H, s.W, s.P, s.Q, (const float *)X, (const float *)W, (const float *)B,
-                                     (int)activMode, (float *)Y, true, (int)PP, (int)QQ))
+                                     nullptr, (int)activMode, (float *)Y, true, (int)PP, (int)QQ))
       return nullptr;
     return Y;
   }

@@ -65,7 +65,10 @@ __global__ __launch_bounds__(256, 2) void conv3x3_f16_c64_kernel(const ConvF16Ar
   const int l32 = lane & 31, half = lane >> 5;
   const int m0 = (int)blockIdx.y * 64;
   const int PW = a.W + 2;
-  const int worker = (int)blockIdx.x, workers = (int)gridDim.x;
+  // Workgroup b runs on XCD b % 8.  Neighbouring tiles share two of their four input rows: the workgroups of one XCD
+  // take a run of consecutive tiles at a time, so that the second reader of a row finds it in that XCD's L2.
+  const int workers = (int)gridDim.x;
+  const int worker = (workers & 7) == 0 ? (int)(blockIdx.x & 7) * (workers >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
   if (worker >= tiles_n) return;
 
   const __amdgpu_buffer_rsrc_t rsrc_x =

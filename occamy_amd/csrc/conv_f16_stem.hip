@@ -425,7 +425,10 @@ __global__ __launch_bounds__(256, 2) void conv_f16_stem_pool_kernel(const ConvF1
   // ---- the walk: patches are loaded two steps ahead (registers), stored to LDS one step ahead --------------
   // Step i: issue the loads of step i + 2; pool step i - 1 (its tile is complete since the last barrier);
   // multiply step i; stage its tile; store the patch of step i + 1, loaded a whole step ago; barrier.
-  int u0 = blockIdx.x, t0 = 0;  // this step
+  // Workgroup b runs on XCD b % 8; neighbouring strips of an image read overlapping input columns (and every strip
+  // whole 128-byte lines of them): an XCD's workgroups take consecutive strips, so the overlap is read from its L2.
+  const int first_unit = (gridDim.x & 7) == 0 ? (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  int u0 = first_unit, t0 = 0;  // this step
   int u1 = u0, t1 = 0;          // the next one
   advance(u1, t1);
   int u2 = u1, t2 = t1;         // the one after

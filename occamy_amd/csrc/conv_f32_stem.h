@@ -5,9 +5,10 @@
 
 namespace dnnrt {
 
-// X: N x 3 x H x W, filter in the context's layout, Y: N x 64 x P x Q, or with `pool` the pooled N x 64 x PP x QQ
-// (activation ReLU or identity then).  P, Q: the convolution's output size.
+// X: N x 3 x H x W, filter in the context's layout, Y: N x 64 x P x Q (Z: a residual operand shaped like Y, or null),
+// or with `pool` the pooled N x 64 x PP x QQ (activation ReLU or identity, no residual).  P, Q: the convolution's
+// output size.
 bool launch_conv_f32_stem(const dnnrtContext *ctx, int N, int H, int W, int P, int Q, const float *X, const float *Wt,
-                          const float *bias, int act, float *Y, bool pool, int PP, int QQ);
+                          const float *bias, const float *Z, int act, float *Y, bool pool, int PP, int QQ);
 
 }  // namespace dnnrt

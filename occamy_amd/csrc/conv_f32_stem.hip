@@ -46,7 +46,7 @@ __device__ __forceinline__ float nan_max(float a, float b) {
 
 template <bool POOL, bool RELU>
 __global__ __launch_bounds__(256) void conv_f32_stem_kernel(const float *__restrict__ X, const float *__restrict__ Wt,
-                                                            const float *__restrict__ bias, float *__restrict__ Y,
+                                                            const float *__restrict__ bias, const float *Zr, float *Y,
                                                             const int H, const int W, const int P, const int Q, const int PP,
                                                             const int QQ, const int tiles_r, const int tiles_c,
                                                             const int w_filter_stride, const int w_tap_stride, const int act,
@@ -148,17 +148,22 @@ __global__ __launch_bounds__(256) void conv_f32_stem_kernel(const float *__restr
     for (int i = 0; i < 4; i++)
 #pragma unroll
       for (int j = 0; j < ROWS; j++)
-        if (col_ok && cr0 + j < P)
-          Y[(((int64_t)n * 64 + f0 + i) * P + cr0 + j) * Q + cc0 + col] = apply_act(acc[j][i] + bv[i], act, act_coef);
+        if (col_ok && cr0 + j < P) {
+          const int64_t at = (((int64_t)n * 64 + f0 + i) * P + cr0 + j) * Q + cc0 + col;
+          float v = acc[j][i] + bv[i];
+          if (Zr) v += Zr[at];  // the residual operand (which may be Y itself: same thread, same element)
+          Y[at] = apply_act(v, act, act_coef);
+        }
   }
 }
 
 bool launch_conv_f32_stem(const dnnrtContext *ctx, int N, int H, int W, int P, int Q, const float *X, const float *Wt,
-                          const float *bias, int act, float *Y, bool pool, int PP, int QQ) {
+                          const float *bias, const float *Z, int act, float *Y, bool pool, int PP, int QQ) {
   using namespace stem32;
   if ((int64_t)3 * H * W >= (1ll << 31)) { set_error("first-layer kernel: image too large"); return false; }
   if (!bias) { set_error("first-layer kernel: needs a bias"); return false; }
   if (pool && act != DNNRT_ACT_RELU && act != DNNRT_ACT_IDENTITY) { set_error("conv+maxpool: activation must be ReLU or identity"); return false; }
+  if (pool && Z) { set_error("conv+maxpool: no residual operand"); return false; }
   const bool crsk = ctx->filter_layout == DNNRT_FILTER_CRSK;
   const int fs = crsk ? 1 : TAPS, ts = crsk ? 64 : 1;
   const int tiles_r = pool ? (PP + 1) / 2 : (P + ROWS - 1) / ROWS;
@@ -167,7 +172,7 @@ bool launch_conv_f32_stem(const dnnrtContext *ctx, int N, int H, int W, int P, i
   if (grid > INT32_MAX) { set_error("first-layer kernel: batch too large"); return false; }
   if (grid == 0) return true;
 #define STEM32(POOL, RELU)                                                                                                  \
-  hipLaunchKernelGGL((conv_f32_stem_kernel<POOL, RELU>), dim3((unsigned)grid), dim3(256), 0, ctx->stream, X, Wt, bias, Y, H,     \
+  hipLaunchKernelGGL((conv_f32_stem_kernel<POOL, RELU>), dim3((unsigned)grid), dim3(256), 0, ctx->stream, X, Wt, bias, Z, Y, H,     \
                      W, P, Q, PP, QQ, tiles_r, tiles_c, fs, ts, act, ctx->act_coef)
   if (pool) {
     if (act == DNNRT_ACT_RELU) STEM32(true, true);

@@ -137,6 +137,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
   if (opt->fusion && opt->fuse_first_layer_maxpool) fuse_first_layer_maxpool(p);
   if (opt->fusion && opt->fuse_residual && opt->fuse_projection_shortcut) fuse_projection_shortcut(p);
   if (opt->alias_copies) alias_copies(p);
+  if (opt->fusion && opt->fuse_residual && opt->inplace_residual) inplace_residual(p);
   if (opt->dealloc_opt) dealloc_opt(p);
   if (opt->channels_last) {
     // Only fp16 programs whose rank-4 tensors flow through layout-aware calls

@@ -186,6 +186,7 @@ void fuse_conv_activations(Program &p);
 void fuse_matmul_bias(Program &p);
 void fuse_first_layer_maxpool(Program &p);
 void alias_copies(Program &p);
+void inplace_residual(Program &p);
 void fuse_projection_shortcut(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);

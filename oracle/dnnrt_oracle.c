@@ -350,11 +350,24 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
     FAIL("convBiasAddActiv: activMode %ld", (long)act);
   if (numel(dB, 4) != dW[0]) FAIL("convBiasAddActiv: bias must hold K values");
   if (!Z) FAIL("convBiasAddActiv: null residual tensor");
-  if (!conv_entry(X, dX, W, dW, B, group, pads, strides, DNNRT_ACT_IDENTITY, Y, dtype))
-    return NULL;
   const int64_t P = (dX[2] + 2 * pads[0] - dW[2]) / strides[0] + 1,
                 Q = (dX[3] + 2 * pads[1] - dW[3]) / strides[1] + 1;
   const int64_t ny = dX[0] * dW[0] * P * Q;
+  /* Z may be Y itself (cudnnConvolutionBiasActivationForward allows zData == yData;
+   * the GPU library's in-place residual relies on it): the chain below stores the
+   * convolution in Y first, so the residual is set aside. */
+  void *z_copy = NULL;
+  if (Z == Y && ny > 0) {
+    const size_t bytes = (size_t)ny * (dtype == DNNRT_F16 ? 2 : 4);
+    z_copy = malloc(bytes);
+    if (!z_copy) FAIL("convBiasAddActiv: out of memory");
+    memcpy(z_copy, Z, bytes);
+    Z = z_copy;
+  }
+  if (!conv_entry(X, dX, W, dW, B, group, pads, strides, DNNRT_ACT_IDENTITY, Y, dtype)) {
+    free(z_copy);
+    return NULL;
+  }
   float *ty, *tz, *to;
   const float *y = widen(Y, ny, dtype, &ty);
   const float *z = widen(Z, ny, dtype, &tz);
@@ -363,7 +376,7 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t h, const void *X, const int64_t *dX,
    * end stands for the add's and the activation's stores */
   for (int64_t i = 0; i < ny; i++) o[i] = act_apply(y[i] + z[i], act, h->act_coef);
   narrow(Y, to, ny, dtype);
-  free(ty); free(tz);
+  free(ty); free(tz); free(z_copy);
   return Y;
 }
 

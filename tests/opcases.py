@@ -12,9 +12,10 @@ def conv_out_hw(H, W, R, S, pads, strides):
     return (H + 2 * pads[0] - R) // strides[0] + 1, (W + 2 * pads[1] - S) // strides[1] + 1
 
 
-def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crsk=False, z=None, coef=None):
+def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crsk=False, z=None, coef=None, inplace=False):
     """crsk: hand the filter over stored C,R,S,K (the dims stay logical K,C,R,S).
-    z: residual tensor shaped like the result (needs b): act((conv + b) + z).
+    z: residual tensor shaped like the result (needs b): act((conv + b) + z); inplace: the result buffer holds z
+    and is passed as both Z and Y.
     coef: the handle's activation coefficient (ceiling of ACT_CLIPPED_RELU, slope of ACT_LEAKY_RELU)."""
     N, C, H, W = x.shape
     K, Cg, R, S = w.shape
@@ -33,6 +34,8 @@ def conv(be, x, w, b=None, pads=(0, 0), strides=(1, 1), group=1, activ=None, crs
             be.ops.conv(be.ptr(X), x.shape, be.ptr(Wt), w.shape, pads, strides, be.ptr(Y), group, dt)
         elif z is not None:
             B, Z = be.put(b), be.put(z)
+            if inplace:
+                Y = Z
             be.ops.conv_bias_add_activ(be.ptr(X), x.shape, be.ptr(Wt), w.shape, be.ptr(B), be.ptr(Z), pads, strides,
                                        activ if activ is not None else _abi.ACT_IDENTITY, be.ptr(Y), group, dt)
         else:

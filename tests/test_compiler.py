@@ -312,6 +312,53 @@ def test_first_layer_maxpool_fusion():
     assert "maxpoolfwd" not in g.compile(fuse_first_layer_maxpool=True, channels_last=True).text  # no fusion flag: conv, add, relu apart
 
 
+def test_inplace_residual():
+    """A fused conv + add + activation whose residual operand nothing reads afterwards names that operand's buffer
+    as its output: ResNet-50's twelve identity blocks (and, without the shortcut fusion, its four projection blocks)
+    lose their output buffers, chains of blocks walk down one buffer, and every tensor is still alive when read."""
+    for dt, flags in ((np.float32, dict(fusion=True, fuse_residual=True)), (np.float16, dict(fusion=True, fuse_residual=True, channels_last=True))):
+        g, _ = models.resnet50(dtype=dt, **SMALL)
+        plain = g.compile(**flags)
+        g, _ = models.resnet50(dtype=dt, **SMALL)
+        inpl = g.compile(inplace_residual=True, **flags)
+        mallocs = lambda prog: sum(1 for k, _, _, _ in prog.events() if k == 0)  # noqa: E731
+        assert mallocs(inpl) == mallocs(plain) - 16
+        assert inpl.num_ops(compute_only=True) == plain.num_ops(compute_only=True)
+        closers = [l for l in inpl.text.splitlines() if "conv-bias-add-relufwd" in l]
+        assert len(closers) == 16
+        for l in closers:  # operands: x, w, bias, workspace, z, out; z is a result, out the buffer it lives in
+            ops = l.split("conv-bias-add-relufwd")[1].split("{")[0].replace(" ", "").split(",")
+            assert len(ops) == 6 and ops[4] != ops[5]
+        g, _ = models.resnet50(dtype=dt, **SMALL)
+        with_pairs = g.compile(inplace_residual=True, fuse_projection_shortcut=True, **flags)
+        assert mallocs(with_pairs) == mallocs(plain) - 16  # four shortcut results, twelve identity blocks' outputs
+        check_lifetimes(lambda: models.resnet50(dtype=dt, **SMALL), inplace_residual=True, **flags)
+        check_lifetimes(lambda: models.resnet50(dtype=dt, **SMALL), inplace_residual=True, fuse_projection_shortcut=True, alias_copies=True, **flags)
+        # nothing without the residual fusion
+        g, _ = models.resnet50(dtype=dt, **SMALL)
+        assert mallocs(g.compile(fusion=True, inplace_residual=True)) == mallocs(models.resnet50(dtype=dt, **SMALL)[0].compile(fusion=True))
+    # a residual operand that is read again later keeps its buffer
+    def again():
+        g = compiler.Graph()
+        g.input("x", (1, 8, 6, 6), np.float32)
+        r = np.random.default_rng(0)
+        g.constant(r.standard_normal((8, 8, 1, 1)).astype(np.float32), "w")
+        g.constant(r.standard_normal(8).astype(np.float32), "b")
+        g.node("Conv", ["x", "w", "b"], "c", kernel_shape=[1, 1])
+        g.node("Relu", ["c"], "z")
+        g.node("Conv", ["z", "w", "b"], "d", kernel_shape=[1, 1])
+        g.node("Add", ["d", "z"], "s")
+        g.node("Relu", ["s"], "y")
+        g.node("Add", ["y", "z"], "t")  # z again
+        g.output("t")
+        return g
+    flags = dict(fusion=True, fuse_residual=True)
+    mallocs = lambda prog: sum(1 for k, _, _, _ in prog.events() if k == 0)  # noqa: E731
+    p2 = again().compile(inplace_residual=True, **flags)
+    assert "conv-bias-add-relufwd" in p2.text
+    assert mallocs(p2) == mallocs(again().compile(**flags))
+
+
 def test_projection_shortcut_fusion():
     """Every projection shortcut of ResNet-50 (conv + bias) and the last convolution (+ add + ReLU) of its block become
     one call; the shortcuts' buffers are never allocated.  fp32 programs and channels-last fp16 programs."""

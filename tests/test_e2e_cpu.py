@@ -264,6 +264,31 @@ def test_projection_shortcut_fusion_matches_unfused_chain():
     s.close()
 
 
+def test_inplace_residual_changes_nothing():
+    """A closing convolution that writes over its residual operand: the oracle (which takes Z == Y like
+    cudnnConvolutionBiasActivationForward does) gives the same bits per inference with a poisoned pool, without the
+    dealloc pass and resident, for ResNet-50 with and without the fused shortcut pairs and for MobileNetV2; the
+    pool never holds the sixteen (ten) buffers the pass removes."""
+    for small, flags in ((lambda: models.resnet50(image=32, classes=10), dict(fusion=True, fuse_residual=True)),
+                         (lambda: models.resnet50(image=32, classes=10), dict(fusion=True, fuse_residual=True, fuse_projection_shortcut=True, alias_copies=True)),
+                         (lambda: models.mobilenet_v2(image=32, classes=10), dict(fusion=True, fuse_residual=True, fuse_activations=True))):
+        _, _, a = run_oracle(small, **flags)
+        for more in (dict(), dict(dealloc_opt=False)):
+            _, _, b = run_oracle(small, inplace_residual=True, **flags, **more)
+            np.testing.assert_array_equal(a[0], b[0])
+        _, _, c = run_oracle(small, mode=compiler.MODE_RESIDENT, inplace_residual=True, **flags)
+        np.testing.assert_array_equal(a[0], c[0])
+        check(small, inplace_residual=True, **flags)
+        g, inputs = small()
+        p = g.compile(inplace_residual=True, **flags)
+        mallocs = lambda prog: sum(1 for k, _, _, _ in prog.events() if k == 0)  # noqa: E731
+        assert mallocs(p) < mallocs(small()[0].compile(**flags))
+        s = p.session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+        s.set_debug_fill(0xFF)
+        np.testing.assert_array_equal(s.run(*inputs)[0], a[0])
+        s.close()
+
+
 @pytest.mark.parametrize("builder,copies", [(lambda: models.resnet50(image=32, classes=10), 1), (ALEX, 1),
                                             (lambda: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128), None),
                                             (YOLO, None)],

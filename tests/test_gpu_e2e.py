@@ -149,7 +149,7 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
     oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
     flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
-                 fuse_projection_shortcut=True, alias_copies=True)
+                 fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True)
     build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
     out16, info = run(build16, **flags)
     assert info["requested"] == info["pool"]
@@ -245,6 +245,29 @@ def test_first_layer_maxpool_fusion_fp32(batch, image):
     np.testing.assert_array_equal(res[0], one[0])
     ref, _ = run(build, ORACLE_PATH, fusion=True)
     close(one[0], ref[0], 1e-4, 1e-4)
+
+
+@pytest.mark.parametrize("dtype,batch,image", [(np.float16, 4, 224), (np.float16, 3, 64), (np.float32, 1, 224), (np.float32, 2, 64)])
+def test_inplace_residual_on_the_gpu(dtype, batch, image):
+    """Closing convolutions that write over their residual operand: the same bits as with an output buffer of their
+    own, per inference with a poisoned pool and replayed from a captured graph; a smaller set of buffers."""
+    build = lambda: models.resnet50(batch, dtype, seed=7, image=image, classes=100)  # noqa: E731
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, fuse_projection_shortcut=True, alias_copies=True)
+    if dtype == np.float16:
+        flags.update(channels_last=True, fuse_first_layer_maxpool=True)
+    plain, _ = run(build, **flags)
+    g, inputs = build()
+    p = g.compile(inplace_residual=True, **flags)
+    mallocs = lambda prog: sum(1 for k, _, _, _ in prog.events() if k == 0)  # noqa: E731
+    assert mallocs(p) == mallocs(build()[0].compile(**flags)) - 12
+    s = p.session(compiler.MODE_OCCAMY)
+    s.set_debug_fill(0xFF)
+    np.testing.assert_array_equal(s.run(*inputs)[0], plain[0])
+    s.close()
+    s = p.session(compiler.MODE_RESIDENT)
+    for _ in range(2):
+        np.testing.assert_array_equal(s.run(*inputs)[0], plain[0])
+    s.close()
 
 
 def test_aliased_copies_change_nothing_on_the_gpu():

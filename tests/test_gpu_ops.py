@@ -89,6 +89,11 @@ def test_conv_f32(gpu, cpu, case):
     lin = oc.conv(gpu, x, w, b, *args, _abi.ACT_IDENTITY)
     np.testing.assert_array_equal(fused, oc.unary(gpu, "relu", oc.tensor_op(gpu, _abi.OP_ADD, lin, z)))
     close(oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, crsk=True, z=z), fused)
+    # the result written over the residual operand (Z == Y): the same bits, from the kernels of either filter layout
+    np.testing.assert_array_equal(oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, z=z, inplace=True), fused)
+    np.testing.assert_array_equal(oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, crsk=True, z=z, inplace=True),
+                                  oc.conv(gpu, x, w, b, *args, _abi.ACT_RELU, crsk=True, z=z))
+    np.testing.assert_array_equal(oc.conv(cpu, x, w, b, *args, _abi.ACT_RELU, z=z, inplace=True), oc.conv(cpu, x, w, b, *args, _abi.ACT_RELU, z=z))
 
 
 def test_conv_closed_forms(gpu):
@@ -540,8 +545,9 @@ def test_empty_tensors_are_no_ops(gpu, cpu):
 
 # ---- fp16, channels-last -----------------------------------------------------------------
 
-def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt, z=None):
-    """x, w (and the residual z) in logical NCHW / KCRS order; returns logical NCHW."""
+def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt, z=None, inplace=False):
+    """x, w (and the residual z) in logical NCHW / KCRS order; returns logical NCHW.  inplace: the result buffer
+    holds z and is passed as both Z and Y."""
     N, C, H, W = x.shape
     K, Cg, R, S = w.shape
     P, Q = oc.conv_out_hw(H, W, R, S, pads, strides)
@@ -556,6 +562,8 @@ def conv_f16(gpu, x, w, b, pads, strides, group, activ, fmt, z=None):
                                     gpu.ptr(Y), group, _abi.F16)
         else:  # laid out like Y
             Z = gpu.put(z if fmt == _abi.NCHW else np.ascontiguousarray(z.transpose(0, 2, 3, 1)))
+            if inplace:
+                Y = Z
             gpu.ops.conv_bias_add_activ(gpu.ptr(X), x.shape, gpu.ptr(Wt), w.shape, gpu.ptr(B), gpu.ptr(Z), pads, strides,
                                         activ, gpu.ptr(Y), group, _abi.F16)
         gpu.sync()
@@ -611,6 +619,8 @@ def test_conv_f16(gpu, cpu, case, fmt):
     refz = oc.conv(cpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, z=z)
     gotz = conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, fmt, z=z)
     np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
+    if fmt != _abi.NCHW_TO_NHWC:  # written over the residual operand: the same bits
+        np.testing.assert_array_equal(conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, fmt, z=z, inplace=True), gotz)
 
 
 def stem_pool_f16(gpu, x, w, b, activ, fmt=_abi.NCHW_TO_NHWC, kernel=(3, 3), ppads=(1, 1, 1, 1), pstrides=(2, 2)):
@@ -921,6 +931,7 @@ def test_conv_f16_at_batch_64_sizes(gpu, cpu, case):
     refz = oc.conv(cpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, z=z)
     gotz = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC, z=z)
     np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
+    np.testing.assert_array_equal(conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC, z=z, inplace=True), gotz)
 
 
 def test_every_compiled_f16_conv_variant(gpu, cpu):
@@ -945,6 +956,8 @@ def test_every_compiled_f16_conv_variant(gpu, cpu):
                 got = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC)
                 try:
                     gotz = conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC, z=z)
+                    np.testing.assert_array_equal(conv_f16(gpu, x, w, b, pads, strides, 1, _abi.ACT_RELU, _abi.NHWC, z=z, inplace=True), gotz,
+                                                  err_msg=f"variant {t} on {case} written over its residual operand")
                 except RuntimeError as e:  # a variant without the residual operand says so
                     assert "residual" in str(e), str(e)
                     gotz = None
