@@ -29,7 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK = {"mfma_f32": 157.3e12, "mfma_f16": 2.5e15, "hbm": 8.0e12}
-RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool", "fuse_projection_shortcut", "alias_copies", "inplace_residual")
+RESIDENT_ONLY_FLAGS = ("fuse_residual", "fuse_activations", "recompose", "fuse_matmul_bias", "fuse_attention", "fuse_first_layer_maxpool", "fuse_projection_shortcut", "alias_copies", "inplace_residual", "compact_pool")
 
 
 def build_workload(name, batch=None):
@@ -42,7 +42,7 @@ def build_workload(name, batch=None):
         b = batch or 64
         return (models.resnet50(b, np.float16, seed=5),
                 dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True,
-                     alias_copies=True, inplace_residual=True),
+                     alias_copies=True, inplace_residual=True, compact_pool=True),
                 b, "img/s", "f16")
     if batch is not None:
         raise SystemExit(f"{name}: no batch override")
@@ -222,7 +222,7 @@ def record(res, steps, warmup, cpu_seconds):
         "value": res["value"], "unit": res["unit"], "steps": steps, "warmup": warmup, "ms_per_step": res["ms_per_step"],
         "latency_ms": res["latency_ms"], "dtype": res["dtype"], "data": "synthetic",
         "config": {"workload": res["name"], "batch": res["batch"],
-                   "fusion": ", ".join(k for k, v in res["flags"].items() if v and (k.startswith("fus") or k in ("recompose", "alias_copies", "channels_last", "inplace_residual"))),
+                   "fusion": ", ".join(k for k, v in res["flags"].items() if v and (k.startswith("fus") or k in ("recompose", "alias_copies", "channels_last", "inplace_residual", "compact_pool"))),
                    "mode": "weights and input resident in HBM, kernels replayed from a captured graph",
                    "kernels_per_step": res["kernels_per_step"]},
         "roofline": roofline_of(res),

@@ -78,6 +78,10 @@ typedef struct {
   int32_t inplace_residual; /* no reference flag: with `fusion` and `fuse_residual`, a fused conv + add + activation
                              whose residual operand nothing reads afterwards writes its result over that operand
                              (one tensor fewer in the pool, one fewer in the caches; default 0) */
+  int32_t compact_pool;   /* no reference flag: with `pool_opt`, offsets from a planner that knows every lifetime
+                             before it places anything (largest tensor first, lowest free offset) instead of the
+                             reference's first fit in program order; the pool is then usually the bytes alive at
+                             once.  dnncProgramPoolBytes is that pool, not the reference's maxAllocByte (default 0) */
 } dnncOptions;
 /* the graph must outlive the program: constants are not copied again */
 dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt);

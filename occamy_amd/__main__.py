@@ -27,6 +27,7 @@ def main():
     ap.add_argument("--fuse-projection-shortcut", action="store_true",
                     help="with --dnn-kernel-fusion, --fuse-residual and --channels-last: a residual block's projection shortcut and last convolution in one call")
     ap.add_argument("--alias-copies", action="store_true", help="Flatten / Reshape / Squeeze / Unsqueeze reuse their input's buffer")
+    ap.add_argument("--compact-pool", action="store_true", help="plan the pool with every lifetime known (largest first) instead of the reference's first fit")
     ap.add_argument("--inplace-residual", action="store_true", help="a fused conv + add + activation writes over its residual operand when nothing reads it afterwards")
     ap.add_argument("--fuse-first-layer-maxpool", action="store_true",
                     help="with --dnn-kernel-fusion and --channels-last: a ResNet's first convolution and its max-pool in one call")
@@ -41,7 +42,7 @@ def main():
     prog = graph.compile(fusion=args.fusion, fuse_residual=args.fuse_residual, fuse_activations=args.fuse_activations, recompose=args.recompose, fuse_matmul_bias=args.fuse_matmul_bias, fuse_attention=args.fuse_attention, dealloc_opt=args.dealloc_opt,
                          const_at_use=args.const_at_use, channels_last=args.channels_last,
                          fuse_first_layer_maxpool=args.fuse_first_layer_maxpool, alias_copies=args.alias_copies, fuse_projection_shortcut=args.fuse_projection_shortcut,
-                         inplace_residual=args.inplace_residual)
+                         inplace_residual=args.inplace_residual, compact_pool=args.compact_pool)
     print(f"inputs: {graph.input_shapes}")
     print(f"pool: {prog.pool_bytes} bytes (maxAllocByte); {prog.num_ops(compute_only=True)} runtime calls per inference")
     if args.emit:

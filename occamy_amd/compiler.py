@@ -29,7 +29,7 @@ class _Options(C.Structure):
                 ("pool_opt", C.c_int32), ("channels_last", C.c_int32), ("fuse_residual", C.c_int32),
                 ("fuse_activations", C.c_int32), ("recompose", C.c_int32), ("fuse_matmul_bias", C.c_int32),
                 ("fuse_attention", C.c_int32), ("fuse_first_layer_maxpool", C.c_int32),
-                ("fuse_projection_shortcut", C.c_int32), ("alias_copies", C.c_int32), ("inplace_residual", C.c_int32)]
+                ("fuse_projection_shortcut", C.c_int32), ("alias_copies", C.c_int32), ("inplace_residual", C.c_int32), ("compact_pool", C.c_int32)]
 
 
 _lib = None
@@ -197,11 +197,11 @@ class Graph:
     def compile(self, fusion=False, dealloc_opt=True, pool_opt=True, const_at_use=True, channels_last=False,
                 fuse_residual=False, fuse_activations=False, recompose=False, fuse_matmul_bias=False,
                 fuse_attention=False, fuse_first_layer_maxpool=False, alias_copies=False, fuse_projection_shortcut=False,
-                inplace_residual=False):
+                inplace_residual=False, compact_pool=False):
         opt = _Options(int(const_at_use), int(fusion), int(dealloc_opt), int(pool_opt), int(channels_last),
                        int(fuse_residual), int(fuse_activations), int(recompose), int(fuse_matmul_bias),
                        int(fuse_attention), int(fuse_first_layer_maxpool), int(fuse_projection_shortcut), int(alias_copies),
-                       int(inplace_residual))
+                       int(inplace_residual), int(compact_pool))
         p = lib().dnncCompile(self._g, C.byref(opt))
         if not p:
             raise RuntimeError("compile: " + _err())

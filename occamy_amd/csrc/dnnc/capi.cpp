@@ -202,7 +202,7 @@ dnncProgram *dnncCompile(dnncGraph *g, const dnncOptions *opt) {
           }
     p.channels_last = true;
   }
-  if (opt->pool_opt && !malloc_pool_opt(p, err)) { g_err = err; delete pp; return nullptr; }
+  if (opt->pool_opt && !malloc_pool_opt(p, err, opt->compact_pool != 0)) { g_err = err; delete pp; return nullptr; }
   return pp;
 }
 

@@ -190,6 +190,6 @@ void inplace_residual(Program &p);
 void fuse_projection_shortcut(Program &p);
 void dealloc_opt(Program &p);
 std::vector<PoolEvent> pool_events(const Program &p);
-bool malloc_pool_opt(Program &p, std::string &err);
+bool malloc_pool_opt(Program &p, std::string &err, bool compact = false);
 
 }  // namespace dnnc

@@ -359,6 +359,47 @@ def test_inplace_residual():
     assert mallocs(p2) == mallocs(again().compile(**flags))
 
 
+def test_compact_pool():
+    """The planner that knows every lifetime before it places anything: no two tensors alive together overlap, the
+    pool is not larger than the reference's first fit on these programs (up to its rounding of every tensor to 256
+    bytes where the reference rounds to 32) and reaches the bytes alive at once on ResNet-50; the events (ids,
+    sizes, order) are those of the first-fit program."""
+    def peak_and_overlap(prog):
+        live, cur, peak = {}, 0, 0
+        for k, i, b, off in prog.events():
+            if k == 0:
+                assert off >= 0 and off % 32 == 0
+                for bb, oo in live.values():
+                    assert not (b and bb and off < oo + bb and oo < off + b), "two live tensors overlap"
+                live[i] = (b, off)
+                cur += b
+                peak = max(peak, cur)
+                assert off + b <= prog.pool_bytes
+            else:
+                cur -= live.pop(i)[0]
+        return peak
+    cases = [(lambda: models.resnet50(dtype=np.float32, **SMALL), dict(fusion=True, fuse_residual=True)),
+             (lambda: models.resnet50(dtype=np.float16, **SMALL), dict(fusion=True, fuse_residual=True, channels_last=True, inplace_residual=True, fuse_projection_shortcut=True)),
+             (lambda: models.mobilenet_v2(image=32, classes=10), dict(fusion=True, fuse_residual=True, fuse_activations=True)),
+             (lambda: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128), dict()),
+             (lambda: models.single_conv(), dict())]
+    for build, flags in cases:
+        first = build()[0].compile(**flags)
+        tight = build()[0].compile(compact_pool=True, **flags)
+        assert [(k, i, b) for k, i, b, _ in first.events()] == [(k, i, b) for k, i, b, _ in tight.events()]
+        peak = peak_and_overlap(tight)
+        peak_and_overlap(first)
+        n = sum(1 for k, _, _, _ in tight.events() if k == 0)
+        assert peak <= tight.pool_bytes <= first.pool_bytes + 256 * n
+        assert first.text.count("dnn.mem-offset") == tight.text.count("dnn.mem-offset")
+    g, _ = models.resnet50(dtype=np.float32, **SMALL)
+    tight = g.compile(compact_pool=True, fusion=True, fuse_residual=True)
+    assert tight.pool_bytes <= 1.02 * peak_and_overlap(tight)  # the bytes alive at once, up to the rounding of each tensor to 256 bytes
+    # without the pool pass the flag does nothing
+    g, _ = models.single_conv()
+    assert "dnn.malloc" in g.compile(pool_opt=False, compact_pool=True).text
+
+
 def test_projection_shortcut_fusion():
     """Every projection shortcut of ResNet-50 (conv + bias) and the last convolution (+ add + ReLU) of its block become
     one call; the shortcuts' buffers are never allocated.  fp32 programs and channels-last fp16 programs."""

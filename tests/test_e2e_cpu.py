@@ -289,6 +289,30 @@ def test_inplace_residual_changes_nothing():
         s.close()
 
 
+def test_compact_pool_changes_nothing():
+    """Offsets from the planner that knows every lifetime: the same bits from the oracle, per inference with a
+    poisoned pool and resident, for ResNet-50 with every fusion, MobileNetV2, BERT and YOLOv1."""
+    cases = [(lambda: models.resnet50(image=32, classes=10), dict(fusion=True, fuse_residual=True, fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True)),
+             (lambda: models.mobilenet_v2(image=32, classes=10), dict(fusion=True, fuse_residual=True, fuse_activations=True)),
+             (lambda: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128), dict(recompose=True, fusion=True)),
+             (YOLO, dict(fusion=True, fuse_activations=True))]
+    for small, flags in cases:
+        _, _, a = run_oracle(small, **flags)
+        _, _, b = run_oracle(small, compact_pool=True, **flags)
+        _, _, c = run_oracle(small, mode=compiler.MODE_RESIDENT, compact_pool=True, **flags)
+        for x, y, z in zip(a, b, c):
+            np.testing.assert_array_equal(x, y)
+            np.testing.assert_array_equal(x, z)
+        g, inputs = small()
+        p = g.compile(compact_pool=True, **flags)
+        s = p.session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+        s.set_debug_fill(0xFF)
+        for x, y in zip(s.run(*inputs), a):
+            np.testing.assert_array_equal(x, y)
+        assert s.last_pool_bytes == p.pool_bytes
+        s.close()
+
+
 @pytest.mark.parametrize("builder,copies", [(lambda: models.resnet50(image=32, classes=10), 1), (ALEX, 1),
                                             (lambda: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128), None),
                                             (YOLO, None)],

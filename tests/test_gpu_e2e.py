@@ -149,7 +149,7 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
     oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
     flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
-                 fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True)
+                 fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True, compact_pool=True)
     build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
     out16, info = run(build16, **flags)
     assert info["requested"] == info["pool"]
@@ -268,6 +268,34 @@ def test_inplace_residual_on_the_gpu(dtype, batch, image):
     for _ in range(2):
         np.testing.assert_array_equal(s.run(*inputs)[0], plain[0])
     s.close()
+
+
+def test_compact_pool_on_the_gpu():
+    """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
+    inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured
+    graph; fp16 channels-last and fp32 ResNet-50, MobileNetV2, a two-layer BERT with its fused paths."""
+    cases = [(lambda: models.resnet50(4, np.float16, seed=5, image=64),
+              dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
+                   fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True)),
+             (lambda: models.resnet50(image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, fuse_projection_shortcut=True)),
+             (lambda: models.mobilenet_v2(image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_activations=True)),
+             (lambda: models.bert_encoder(layers=2), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True))]
+    for builder, flags in cases:
+        plain, _ = run(builder, **flags)
+        g, inputs = builder()
+        p = g.compile(compact_pool=True, **flags)
+        assert p.pool_bytes <= builder()[0].compile(**flags).pool_bytes
+        s = p.session(compiler.MODE_OCCAMY)
+        s.set_debug_fill(0xFF)
+        for a, b in zip(s.run(*inputs), plain):
+            np.testing.assert_array_equal(a, b)
+        assert s.last_pool_bytes == p.pool_bytes
+        s.close()
+        s = p.session(compiler.MODE_RESIDENT)
+        for _ in range(2):
+            for a, b in zip(s.run(*inputs), plain):
+                np.testing.assert_array_equal(a, b)
+        s.close()
 
 
 def test_aliased_copies_change_nothing_on_the_gpu():
