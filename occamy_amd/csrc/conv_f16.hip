@@ -574,6 +574,64 @@ __global__ __launch_bounds__(256) void conv_f16_generic_kernel(const ConvF16Args
   }
 }
 
+// ---- depthwise, channels-last -------------------------------------------------
+// One input channel per filter and as many filters as channels: a memory-bound elementwise operation.  A thread owns
+// eight consecutive channels of one output pixel: per tap one 16-byte load of the input and the tap's eight weights
+// from LDS, where the workgroup keeps the whole filter transposed to [tap][channel] (its global layout, K,R,S with
+// one channel, is the same whether the program calls it K,C,R,S or K,R,S,C); fp32 accumulation, bias, residual and
+// activation as in every fp16 convolution (conv + bias rounded to fp16 before the residual is added).
+__global__ __launch_bounds__(256) void dwconv_f16_nhwc_kernel(const ConvF16Args a, const int64_t total) {
+  extern __shared__ __attribute__((aligned(16))) _Float16 wt[];  // [R * S][K]
+  const int RS = a.R * a.S, K8 = a.K >> 3;
+  const _Float16 *__restrict__ Wg = reinterpret_cast<const _Float16 *>(a.Wt);
+  for (int e = threadIdx.x; e < a.K * RS; e += 256) {
+    const int k = e / RS, tap = e - k * RS;
+    wt[tap * a.K + k] = Wg[e];
+  }
+  __syncthreads();
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int c8 = (int)(i % K8);
+  const int64_t pix = i / K8;
+  const int q = (int)(pix % a.Q);
+  const int64_t t = pix / a.Q;
+  const int p = (int)(t % a.P), n = (int)(t / a.P);
+  const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
+  const _Float16 *__restrict__ Xg = reinterpret_cast<const _Float16 *>(a.X) + (int64_t)n * a.H * a.W * a.C + 8 * c8;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) acc[e] = 0.f;
+  for (int r = 0; r < a.R; r++) {
+    const int ih = ih0 + r;
+    if ((unsigned)ih >= (unsigned)a.H) continue;
+    for (int s = 0; s < a.S; s++) {
+      const int iw = iw0 + s;
+      if ((unsigned)iw >= (unsigned)a.W) continue;
+      const half8 xv = *reinterpret_cast<const half8 *>(Xg + ((int64_t)ih * a.W + iw) * a.C);
+      const half8 wv = *reinterpret_cast<const half8 *>(wt + (r * a.S + s) * a.K + 8 * c8);
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[e] = fmaf((float)xv[e], (float)wv[e], acc[e]);
+    }
+  }
+  const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
+  const _Float16 *__restrict__ Zg = reinterpret_cast<const _Float16 *>(a.Z);
+  const int64_t off = pix * a.K + 8 * c8;
+  half8 out;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    float v = acc[e];
+    if (biasg) v += (float)biasg[8 * c8 + e];
+    if (Zg) v = (float)(_Float16)v + (float)Zg[off + e];
+    out[e] = (_Float16)apply_act(v, a.act, a.act_coef);
+  }
+  *reinterpret_cast<half8 *>(reinterpret_cast<_Float16 *>(a.Y) + off) = out;
+}
+
+static bool dwconv_f16_applies(const ConvF16Args &a) {
+  return a.format == DNNRT_NHWC && a.group > 1 && a.group == a.C && a.K == a.C && a.Cg == 1 && a.C % 8 == 0 &&
+         (int64_t)a.K * a.R * a.S * 2 <= 48 * 1024 && aligned16(a.X) && aligned16(a.Y) && aligned16(a.Z);
+}
+
 // Y = act(fp16(conv(X, W) + bias) + fp16(conv(X2, W2) + bias2)): `a` with its X2 / Wt2 / bias2 / C2 / H2 / W2 / sh2 / sw2
 // fields set.  Both convolutions 1x1 without padding onto the same N x K x P x Q result (dual_conv_applies).
 bool dual_conv_applies(const ConvF16Args &a) {
@@ -746,6 +804,10 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 0); break;
     }
 #undef LAUNCH_FAST
+  } else if (dwconv_f16_applies(a)) {
+    const int64_t total = NPQ * (a.K / 8), blocks = ceil_div(total, 256);
+    if (blocks > INT32_MAX) { set_error("conv(fp16): depthwise output too large"); return false; }
+    hipLaunchKernelGGL(dwconv_f16_nhwc_kernel, dim3((unsigned)blocks), dim3(256), (size_t)a.K * a.R * a.S * 2, ctx->stream, a, total);
   } else {
     const int Kg = a.K / a.group;
     const int64_t tiles = ceil_div(Kg, 64) * ceil_div(NPQ, 64);

@@ -270,6 +270,25 @@ def test_inplace_residual_on_the_gpu(dtype, batch, image):
     s.close()
 
 
+@pytest.mark.parametrize("batch,image", [(2, 64), (8, 224)])
+def test_mobilenet_v2_fp16_channels_last(batch, image):
+    """MobileNetV2 with fp16 weights and activations, channels-last on the device: its depthwise layers on the
+    channels-last depthwise kernel, ReLU6 fused as a clipped ReLU, inverted-residual sums written in place; against
+    the fp32 oracle on the same fp16-representable weights and input (rtol 2e-2, atol 2e-2 of the largest logit),
+    per inference and replayed from a captured graph."""
+    build16 = lambda: models.mobilenet_v2(batch, np.float16, seed=4, image=image, classes=100)  # noqa: E731
+    flags = dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True, channels_last=True, alias_copies=True,
+                 inplace_residual=True, compact_pool=True)
+    out16, info = run(build16, **flags)
+    assert info["requested"] == info["pool"]
+    ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
+    got, want = out16[0].astype(np.float32), ref[0]
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    res, _ = run(build16, mode=compiler.MODE_RESIDENT, **flags)
+    np.testing.assert_array_equal(res[0], out16[0])
+
+
 def test_compact_pool_on_the_gpu():
     """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
     inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured

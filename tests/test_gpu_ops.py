@@ -623,6 +623,31 @@ def test_conv_f16(gpu, cpu, case, fmt):
         np.testing.assert_array_equal(conv_f16(gpu, x, w, b, (pd, pd), (st, st), 1, _abi.ACT_RELU, fmt, z=z, inplace=True), gotz)
 
 
+@pytest.mark.parametrize("case", [(2, 32, 14, 14, 32, 3, 1, 1, 32), (1, 96, 28, 28, 96, 3, 2, 1, 96), (2, 6, 7, 7, 12, 3, 1, 1, 6),
+                                  (1, 16, 10, 10, 32, 3, 1, 1, 4), (2, 128, 9, 9, 128, 1, 1, 0, 2), (3, 144, 13, 9, 144, 3, 2, 1, 144),
+                                  (1, 960, 7, 7, 960, 3, 1, 1, 960), (2, 24, 9, 9, 24, 5, 1, 2, 24), (1, 12, 6, 6, 12, 3, 1, 1, 12)],
+                         ids=lambda c: "x".join(map(str, c)))
+@pytest.mark.parametrize("fmt", [_abi.NHWC, _abi.NCHW])
+def test_conv_f16_grouped_and_depthwise(gpu, cpu, case, fmt):
+    """fp16 convolutions with groups (depthwise: the channels-last kernel of its own for channel counts that are
+    multiples of eight, MobileNetV2's shapes among them, the generic kernel otherwise; depthwise with a channel
+    multiplier; a few wide groups), with bias, ReLU and a residual operand, channels-last and N,C,H,W, against the
+    oracle to the fp16 convolution tolerance."""
+    N, C, H, W, K, R, st, pd, grp = case
+    r = rng(sum(case) + fmt)
+    x = r.standard_normal((N, C, H, W)).astype(np.float16)
+    w = (r.standard_normal((K, C // grp, R, R)) * np.sqrt(2.0 / (C // grp * R * R))).astype(np.float16)
+    b = r.uniform(-0.1, 0.1, K).astype(np.float16)
+    ref = oc.conv(cpu, x, w, b, (pd, pd), (st, st), grp, _abi.ACT_RELU)
+    got = conv_f16(gpu, x, w, b, (pd, pd), (st, st), grp, _abi.ACT_RELU, fmt)
+    np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3)
+    z = r.standard_normal(ref.shape).astype(np.float16)
+    refz = oc.conv(cpu, x, w, b, (pd, pd), (st, st), grp, _abi.ACT_RELU, z=z)
+    gotz = conv_f16(gpu, x, w, b, (pd, pd), (st, st), grp, _abi.ACT_RELU, fmt, z=z)
+    np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3)
+    np.testing.assert_array_equal(conv_f16(gpu, x, w, b, (pd, pd), (st, st), grp, _abi.ACT_RELU, fmt, z=z, inplace=True), gotz)
+
+
 def stem_pool_f16(gpu, x, w, b, activ, fmt=_abi.NCHW_TO_NHWC, kernel=(3, 3), ppads=(1, 1, 1, 1), pstrides=(2, 2)):
     """The fused first layer through the C-ABI; x in N,C,H,W, w logical K,C,R,S; returns logical N,K,PP,QQ."""
     N, C, H, W = x.shape
