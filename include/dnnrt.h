@@ -384,8 +384,8 @@ void *dnnrtAveragePool(dnnrtHandle_t handle, const void *X,
  * (src/Tools/dnn-wrapper/cublas/CUBLASMatmul2dFunc.cu:9-153):
  * Out = alpha op(A) op(B) + beta C, row-major; C may be NULL when beta == 0.
  * C is [M,N] as in the reference (which sizes it by dimOut, :32) or, with
- * dimC = [1,N], one row added to every row of the product (fp16: only with
- * beta = 1, where it is the convolution kernel's per-filter bias). */
+ * dimC = [1,N], one row added to every row of the product.  fp16 tensors:
+ * fp32 accumulation and one rounding of alpha op(A) op(B) + beta C. */
 void *dnnrtMatmul2d(dnnrtHandle_t handle, int64_t rank, const void *A,
                     const int64_t *dimA, const void *B, const int64_t *dimB,
                     const void *C, const int64_t *dimC, void *Out,
@@ -403,7 +403,8 @@ void *dnnrtMatmulNd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
  * tensor shaped like Y (NULL: none), act = Gelu if `gelu` != 0 else identity.
  * No reference wrapper: the reference runs CUDAMatmulNdFunc and then the
  * broadcast add of the bias (Ops/cudnn/Add.cpp), the residual add, and Gelu
- * operator by operator (Div, Erf, Add, Mul, Mul).  fp32 only. */
+ * operator by operator (Div, Erf, Add, Mul, Mul).  fp32 and fp16 (fp32
+ * accumulation, everything up to the activation in fp32, one rounding). */
 void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
                         int32_t rankA, const void *B, const int64_t *dimB,
                         int32_t rankB, const void *bias, const void *Z,
@@ -418,7 +419,8 @@ void *dnnrtMatmulNdBias(dnnrtHandle_t handle, const void *A, const int64_t *dimA
  * and V in elements (0: heads*headDim); with the three projections computed
  * by one product into a [batch, seq, 3*heads*headDim] tensor, Q, K and V are
  * that tensor's base plus 0, 1 and 2 times heads*headDim and ldIn is its row
- * length.  Y's rows are heads*headDim long.  fp32, headDim 32 / 64 / 128,
+ * length.  Y's rows are heads*headDim long.  fp32 or fp16 (widened on the way
+ * in, fp32 in between, one rounding on the way out), headDim 32 / 64 / 128,
  * 16-byte aligned operands, Y distinct from the inputs. */
 void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void *K,
                      const void *V, void *Y, int64_t batch, int64_t seqQ,

@@ -1,7 +1,8 @@
 // Multi-head attention core for transformer encoders:
 //   Y[b, q, h*DH + d] = sum_k softmax_k(scale * <Q[b,q,h,:], K[b,k,h,:]>) * V[b,k,h,d]
 // with Q, K, V, Y stored [batch, seq, heads * DH] (the layout the Linear layers
-// write), fp32.  It stands for the chain the reference runs call by call --
+// write), fp32 or fp16 (widened on the way into LDS, everything in between in
+// fp32, one rounding on the way out).  It stands for the chain the reference runs call by call --
 // Reshape + Transpose of each operand (CUDAReshapeFunc, CUDATranspose4DFloatFunc),
 // CUDAMatmulNdFunc, the scaling Mul, CUDASoftmaxFunc, CUDAMatmulNdFunc, Transpose
 // + Reshape back -- twelve launches and eleven round trips through memory.
@@ -18,13 +19,26 @@
 namespace dnnrt {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 att_half4 __attribute__((ext_vector_type(4)));
+
+// four consecutive elements of a stored tensor as fp32, and back
+__device__ __forceinline__ float4 load4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 load4(const __half *p) {
+  const att_half4 h = *reinterpret_cast<const att_half4 *>(p);
+  return make_float4((float)h[0], (float)h[1], (float)h[2], (float)h[3]);
+}
+__device__ __forceinline__ void store4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ void store4(__half *p, float4 v) {
+  const att_half4 h = {(_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w};
+  *reinterpret_cast<att_half4 *>(p) = h;
+}
 
 constexpr int ATT_QB = 32, ATT_KB = 128;
 
-template <int DH>
-__global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restrict__ Q, const float *__restrict__ K,
-                                                            const float *__restrict__ V, float *__restrict__ Y, int Sq,
-                                                            int Sk, int ld_in, int ld, float scale) {
+template <int DH, typename T>
+__global__ __launch_bounds__(256) void attention_kernel(const T *__restrict__ Q, const T *__restrict__ K,
+                                                        const T *__restrict__ V, T *__restrict__ Y, int Sq,
+                                                        int Sk, int ld_in, int ld, float scale) {
   constexpr int ROW = DH + 4;       // LDS row stride in floats: 16-byte aligned rows, 16-byte reads spread over the banks
   constexpr int TD = DH / 32;       // 32-wide tiles of the head dimension
   extern __shared__ float smem[];
@@ -35,15 +49,14 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
   float *sm = mx + 4 * 32;          // [4][32] final sums per wavefront
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
   const int q0 = blockIdx.x * ATT_QB, head = blockIdx.y, b = blockIdx.z;
-  const float *Qg = Q + (int64_t)b * Sq * ld_in + head * DH;
-  const float *Kg = K + (int64_t)b * Sk * ld_in + head * DH;
-  const float *Vg = V + (int64_t)b * Sk * ld_in + head * DH;
+  const T *Qg = Q + (int64_t)b * Sq * ld_in + head * DH;
+  const T *Kg = K + (int64_t)b * Sk * ld_in + head * DH;
+  const T *Vg = V + (int64_t)b * Sk * ld_in + head * DH;
 
   // the query tile (rows past the end repeat the last query; they are not stored)
   for (int i = tid; i < ATT_QB * (DH / 4); i += 256) {
     const int r = i / (DH / 4), c4 = i - r * (DH / 4);
-    *reinterpret_cast<float4 *>(Qs + r * ROW + c4 * 4) =
-        *reinterpret_cast<const float4 *>(Qg + (int64_t)min(q0 + r, Sq - 1) * ld_in + c4 * 4);
+    *reinterpret_cast<float4 *>(Qs + r * ROW + c4 * 4) = load4(Qg + (int64_t)min(q0 + r, Sq - 1) * ld_in + c4 * 4);
   }
 
   floatx16 o[TD];
@@ -58,8 +71,8 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
     for (int i = tid; i < ATT_KB * (DH / 4); i += 256) {
       const int r = i / (DH / 4), c4 = i - r * (DH / 4);
       const int64_t row = (int64_t)min(kb + r, Sk - 1) * ld_in + c4 * 4;
-      *reinterpret_cast<float4 *>(Ks + r * ROW + c4 * 4) = *reinterpret_cast<const float4 *>(Kg + row);
-      *reinterpret_cast<float4 *>(Vs + r * ROW + c4 * 4) = *reinterpret_cast<const float4 *>(Vg + row);
+      *reinterpret_cast<float4 *>(Ks + r * ROW + c4 * 4) = load4(Kg + row);
+      *reinterpret_cast<float4 *>(Vs + r * ROW + c4 * 4) = load4(Vg + row);
     }
     __syncthreads();
 
@@ -126,7 +139,7 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
       *reinterpret_cast<float4 *>(red + (wave * 32 + l32) * ROW + 32 * t + 8 * g + 4 * half) =
           make_float4(o[t][4 * g], o[t][4 * g + 1], o[t][4 * g + 2], o[t][4 * g + 3]);
   __syncthreads();
-  float *Yg = Y + (int64_t)b * Sq * ld + head * DH;
+  T *Yg = Y + (int64_t)b * Sq * ld + head * DH;
   for (int i = tid; i < ATT_QB * (DH / 4); i += 256) {
     const int q = i / (DH / 4), c4 = i - q * (DH / 4);
     if (q0 + q >= Sq) continue;
@@ -137,22 +150,22 @@ __global__ __launch_bounds__(256) void attention_f32_kernel(const float *__restr
       const float4 p = *reinterpret_cast<const float4 *>(red + (w * 32 + q) * ROW + c4 * 4);
       acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
     }
-    *reinterpret_cast<float4 *>(Yg + (int64_t)(q0 + q) * ld + c4 * 4) = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+    store4(Yg + (int64_t)(q0 + q) * ld + c4 * 4, make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv));
   }
 }
 
-template <int DH>
-static void launch_attention(const dnnrtContext *ctx, const float *Q, const float *K, const float *V, float *Y, int B,
+template <int DH, typename T>
+static void launch_attention(const dnnrtContext *ctx, const T *Q, const T *K, const T *V, T *Y, int B,
                              int Sq, int Sk, int H, int ld_in, float scale) {
   constexpr int ROW = DH + 4;
   const size_t lds = (size_t)((ATT_QB + 2 * ATT_KB) * ROW + 8 * 32) * sizeof(float);
   static bool raised = false;  // per instantiation: more than 64 KiB of dynamic LDS must be asked for once
   if (!raised) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attention_f32_kernel<DH>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attention_kernel<DH, T>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     raised = true;
   }
-  hipLaunchKernelGGL((attention_f32_kernel<DH>), dim3((unsigned)ceil_div(Sq, ATT_QB), (unsigned)H, (unsigned)B), dim3(256),
+  hipLaunchKernelGGL((attention_kernel<DH, T>), dim3((unsigned)ceil_div(Sq, ATT_QB), (unsigned)H, (unsigned)B), dim3(256),
                      lds, ctx->stream, Q, K, V, Y, Sq, Sk, ld_in, H * DH, scale);
 }
 
@@ -165,7 +178,7 @@ extern "C" void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void 
                                 int64_t ldIn, float scale, int32_t dtype) {
   if (!handle) DNNRT_FAIL("dnnrtAttention: null handle");
   if (!Q || !K || !V || !Y) DNNRT_FAIL("dnnrtAttention: null argument");
-  if (dtype != DNNRT_F32) DNNRT_FAIL("dnnrtAttention: dtype %d (fp32 only)", dtype);
+  if (dtype != DNNRT_F32 && dtype != DNNRT_F16) DNNRT_FAIL("dnnrtAttention: dtype %d (fp32 and fp16)", dtype);
   if (batch < 0 || seqQ < 0) DNNRT_FAIL("dnnrtAttention: bad dims");
   if (batch == 0 || seqQ == 0) return Y;  // no queries: no work
   if (seqK <= 0 || heads <= 0) DNNRT_FAIL("dnnrtAttention: bad dims");
@@ -175,10 +188,13 @@ extern "C" void *dnnrtAttention(dnnrtHandle_t handle, const void *Q, const void 
   if (Y == Q || Y == K || Y == V) DNNRT_FAIL("dnnrtAttention: Y must not alias an input");
   if (ldIn == 0) ldIn = heads * headDim;
   if (ldIn < heads * headDim || ldIn % 4 || ldIn > INT32_MAX) DNNRT_FAIL("dnnrtAttention: ldIn %ld (>= heads * headDim, multiple of 4)", (long)ldIn);
-  const float *q = (const float *)Q, *k = (const float *)K, *v = (const float *)V;
-  if (headDim == 32) launch_attention<32>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
-  else if (headDim == 64) launch_attention<64>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
-  else launch_attention<128>(handle, q, k, v, (float *)Y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
+  auto run = [&](auto *q, auto *k, auto *v, auto *y) {
+    if (headDim == 32) launch_attention<32>(handle, q, k, v, y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
+    else if (headDim == 64) launch_attention<64>(handle, q, k, v, y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
+    else launch_attention<128>(handle, q, k, v, y, (int)batch, (int)seqQ, (int)seqK, (int)heads, (int)ldIn, scale);
+  };
+  if (dtype == DNNRT_F32) run((const float *)Q, (const float *)K, (const float *)V, (float *)Y);
+  else run((const __half *)Q, (const __half *)K, (const __half *)V, (__half *)Y);
   DNNRT_CHECK_LAUNCH("dnnrtAttention");
   return Y;
 }

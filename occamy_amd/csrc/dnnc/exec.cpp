@@ -384,7 +384,8 @@ bool Session::issue(const Op *op, std::string &err) {
       if (op->axis) {  // one tensor holds [Q | K | V] per row
         const int64_t hidden = op->dimA[2];
         char *base = (char *)P(0);
-        r = rt.dnnrtAttention(handle, base, base + hidden * 4, base + 2 * hidden * 4, out, op->dimA[0], op->dimA[1], op->dimB[1],
+        const int64_t es = dt == DNNRT_F16 ? 2 : 4;  // bytes per element
+        r = rt.dnnrtAttention(handle, base, base + hidden * es, base + 2 * hidden * es, out, op->dimA[0], op->dimA[1], op->dimB[1],
                               op->group, hidden / op->group, 3 * hidden, op->alpha, dt);
       } else {
         r = rt.dnnrtAttention(handle, P(0), P(1), P(2), out, op->dimA[0], op->dimA[1], op->dimB[1], op->group,

@@ -386,7 +386,7 @@ static bool match_attention(const Matcher &m, const GNode &root, GNode &fused, s
   }
   const GTensor &q = m.g.tensors.at(r[0]->inputs[0]), &k = m.g.tensors.at(r[1]->inputs[0]), &v = m.g.tensors.at(r[2]->inputs[0]);
   const Shape &qs = m.g.tensors.at(r[0]->output).shape, &ks = m.g.tensors.at(r[1]->output).shape, &vs = m.g.tensors.at(r[2]->output).shape;
-  if (q.dtype != F32 || q.shape.size() != 3 || k.shape.size() != 3 || v.shape != k.shape || qs.size() != 4 || ks.size() != 4 || vs != ks) return false;
+  if ((q.dtype != F32 && q.dtype != F16) || k.dtype != q.dtype || v.dtype != q.dtype || q.shape.size() != 3 || k.shape.size() != 3 || v.shape != k.shape || qs.size() != 4 || ks.size() != 4 || vs != ks) return false;
   const int64_t B = qs[0], Sq = qs[1], H = qs[2], D = qs[3], Sk = ks[1];
   if (ks[0] != B || ks[2] != H || ks[3] != D || (D != 32 && D != 64 && D != 128)) return false;
   if (q.shape != Shape{B, Sq, H * D} || k.shape != Shape{B, Sk, H * D} || m.g.tensors.at(root.output).shape != q.shape) return false;
@@ -424,7 +424,8 @@ static void pack_qkv(const Matcher &m, GNode &fused, std::vector<std::string> &d
     auto wi = g.tensors.find(mm[i]->inputs[1]), bi = g.tensors.find(bias[i]);
     if (wi == g.tensors.end() || bi == g.tensors.end() || !wi->second.is_const || !bi->second.is_const) return;
     w[i] = &wi->second; b[i] = &bi->second;
-    if (w[i]->dtype != F32 || b[i]->dtype != F32 || w[i]->shape.size() != 2 || w[i]->shape != w[0]->shape ||
+    if ((w[i]->dtype != F32 && w[i]->dtype != F16) || w[i]->dtype != w[0]->dtype || b[i]->dtype != w[0]->dtype || w[i]->shape.size() != 2 ||
+        w[i]->shape != w[0]->shape ||
         b[i]->shape != Shape{w[i]->shape[1]})
       return;
   }
@@ -432,12 +433,13 @@ static void pack_qkv(const Matcher &m, GNode &fused, std::vector<std::string> &d
   const std::string base = fused.output + "_qkv", wn = base + "_w", bn = base + "_b", mn = base + "_mm";
   if (g.tensors.count(base) || g.tensors.count(wn) || g.tensors.count(bn) || g.tensors.count(mn)) return;
   GTensor wt, bt;
-  wt.name = wn; wt.dtype = F32; wt.shape = {in, 3 * hid}; wt.is_const = true; wt.data.resize((size_t)(in * 3 * hid * 4));
-  bt.name = bn; bt.dtype = F32; bt.shape = {3 * hid}; bt.is_const = true; bt.data.resize((size_t)(3 * hid * 4));
+  const int64_t es = w[0]->dtype == F32 ? 4 : 2;  // bytes per element
+  wt.name = wn; wt.dtype = w[0]->dtype; wt.shape = {in, 3 * hid}; wt.is_const = true; wt.data.resize((size_t)(in * 3 * hid * es));
+  bt.name = bn; bt.dtype = w[0]->dtype; bt.shape = {3 * hid}; bt.is_const = true; bt.data.resize((size_t)(3 * hid * es));
   for (int i = 0; i < 3; i++) {
     for (int64_t r = 0; r < in; r++)
-      std::memcpy(wt.data.data() + ((r * 3 + i) * hid) * 4, w[i]->data.data() + r * hid * 4, (size_t)hid * 4);
-    std::memcpy(bt.data.data() + (int64_t)i * hid * 4, b[i]->data.data(), (size_t)hid * 4);
+      std::memcpy(wt.data.data() + ((r * 3 + i) * hid) * es, w[i]->data.data() + r * hid * es, (size_t)(hid * es));
+    std::memcpy(bt.data.data() + (int64_t)i * hid * es, b[i]->data.data(), (size_t)(hid * es));
   }
   g.tensors[wn] = std::move(wt);
   g.tensors[bn] = std::move(bt);

@@ -1,30 +1,121 @@
 // fp16 matrix product.  Out[M,N] = A[M,K] * B[N,K]^T is exactly a channels-last
 // 1x1 convolution (M "pixels" of K channels, N filters), so it runs on the
-// fp16 convolution kernels (a bias row is the convolution's bias); other
-// operand layouts are not built yet and fail loudly.
+// fp16 convolution kernels (a bias row is the convolution's bias).  Every
+// other form -- B stored K x N, transposed A, batches, alpha / beta, a bias
+// row with a residual matrix and an activation behind it -- goes to one
+// generic kernel: a 64 x 64 tile of Out per workgroup, operands gathered
+// element by element into LDS (strides are runtime values), 32x32x16 MFMA,
+// fp32 accumulation, one rounding to fp16 at the end.
 #include "gemm_f16.h"
 
 #include "conv_f16.h"
 
 namespace dnnrt {
 
+typedef _Float16 g_half8 __attribute__((ext_vector_type(8)));
+typedef float g_floatx16 __attribute__((ext_vector_type(16)));
+
+struct GemmF16Args {
+  const __half *A, *B, *C, *bias;
+  __half *Out;
+  int M, N, K;
+  int64_t a_sm, a_sk, b_sk, b_sn;   // element strides of A along m and k, of B along k and n
+  int64_t az, bz, yz;               // batch strides (0: shared)
+  int64_t c_sm, cz;                 // C: row stride (0: one row for every m), batch stride
+  float alpha, beta;
+  int act;
+  float act_coef;
+};
+
+constexpr int G_BK = 32, G_ROW = 40;  // k per step; halfs per LDS row (32 + 8 of padding)
+
+// Tile: 64 columns n x 64 rows m; the MFMA's row operand is the B side (n), its column operand the A side (m), so
+// that a lane ends up with four consecutive n of one m: an 8-byte store.
+__global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args a) {
+  __shared__ __attribute__((aligned(16))) _Float16 Ns[64 * G_ROW];  // [n][k]
+  __shared__ __attribute__((aligned(16))) _Float16 Ms[64 * G_ROW];  // [m][k]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int wn0 = (wave >> 1) * 32, wm0 = (wave & 1) * 32;
+  const int tiles_n = (a.N + 63) / 64;
+  const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x - tile_m * tiles_n;
+  const int n0 = tile_n * 64, m0 = tile_m * 64, z = blockIdx.z;
+  const _Float16 *__restrict__ Ag = reinterpret_cast<const _Float16 *>(a.A) + (int64_t)z * a.az;
+  const _Float16 *__restrict__ Bg = reinterpret_cast<const _Float16 *>(a.B) + (int64_t)z * a.bz;
+  // Which way the 2048 elements of an operand's step are dealt to the 256 threads: along k when k is the
+  // contiguous direction in memory (eight consecutive k of one row per thread), along the row index otherwise.
+  const bool a_k_fast = a.a_sk == 1, b_k_fast = a.b_sk == 1;
+  g_floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  for (int k0 = 0; k0 < a.K; k0 += G_BK) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      // A side -> Ms[m][k]
+      const int am = a_k_fast ? tid >> 2 : ((tid & 7) << 3) + e, ak = a_k_fast ? ((tid & 3) << 3) + e : tid >> 3;
+      const int gm = m0 + am, gk = k0 + ak;
+      Ms[am * G_ROW + ak] = (gm < a.M && gk < a.K) ? Ag[(int64_t)gm * a.a_sm + (int64_t)gk * a.a_sk] : (_Float16)0.f;
+      // B side -> Ns[n][k]
+      const int bn = b_k_fast ? tid >> 2 : ((tid & 7) << 3) + e, bk = b_k_fast ? ((tid & 3) << 3) + e : tid >> 3;
+      const int gn = n0 + bn, gk2 = k0 + bk;
+      Ns[bn * G_ROW + bk] = (gn < a.N && gk2 < a.K) ? Bg[(int64_t)gk2 * a.b_sk + (int64_t)gn * a.b_sn] : (_Float16)0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < G_BK; ks += 16) {
+      const g_half8 nv = *reinterpret_cast<const g_half8 *>(Ns + (wn0 + l32) * G_ROW + ks + half * 8);
+      const g_half8 mv = *reinterpret_cast<const g_half8 *>(Ms + (wm0 + l32) * G_ROW + ks + half * 8);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(nv, mv, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  // register r of a lane: n = n0 + wn0 + 8 (r >> 2) + 4 half + (r & 3), m = m0 + wm0 + l32
+  const int m = m0 + wm0 + l32;
+  if (m >= a.M) return;
+  const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
+  const _Float16 *__restrict__ Cg = a.C ? reinterpret_cast<const _Float16 *>(a.C) + (int64_t)z * a.cz + (int64_t)m * a.c_sm : nullptr;
+  _Float16 *__restrict__ Og = reinterpret_cast<_Float16 *>(a.Out) + (int64_t)z * a.yz + (int64_t)m * a.N;
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const int n = n0 + wn0 + 8 * (r >> 2) + 4 * half + (r & 3);
+    if (n >= a.N) continue;
+    float v = a.alpha * acc[r];
+    if (biasg) v += (float)biasg[n];
+    if (Cg) v += a.beta * (float)Cg[n];
+    Og[n] = (_Float16)apply_act(v, a.act, a.act_coef);
+  }
+}
+
 bool gemm_f16(const dnnrtContext *ctx, const __half *A, const __half *B, const __half *C, __half *Out, int M,
               int N, int K, float alpha, float beta, bool transA, bool transB, int Z, int64_t az, int64_t bz,
-              int64_t yz, bool c_is_row) {
-  (void)az; (void)bz; (void)yz;
+              int64_t yz, bool c_is_row, const __half *bias, int act) {
   // C: nothing, or one row of N values with beta 1 (a Gemm's bias), which is the convolution's per-filter bias
   const bool bias_row = C && c_is_row && beta == 1.f;
-  if (transA || !transB || Z != 1 || alpha != 1.f || (!bias_row && (beta != 0.f || C))) {
-    set_error("matmul(fp16): only Out = A * B^T [+ one row] (transA=0, transB=1, alpha=1, one batch) is built");
-    return false;
+  const bool as_conv = !transA && transB && Z == 1 && alpha == 1.f && (bias_row || (!C || beta == 0.f)) && !bias && act == DNNRT_ACT_IDENTITY;
+  if (as_conv) {
+    ConvF16Args a{};
+    a.X = A; a.Wt = B; a.bias = bias_row ? C : nullptr; a.Y = Out;
+    a.N = M; a.C = K; a.H = 1; a.W = 1; a.K = N; a.Cg = K; a.R = 1; a.S = 1; a.P = 1; a.Q = 1;
+    a.ph = 0; a.pw = 0; a.sh = 1; a.sw = 1; a.group = 1;
+    a.act = DNNRT_ACT_IDENTITY;
+    a.format = DNNRT_NHWC;
+    return launch_conv_f16(ctx, a);
   }
-  ConvF16Args a{};
-  a.X = A; a.Wt = B; a.bias = bias_row ? C : nullptr; a.Y = Out;
-  a.N = M; a.C = K; a.H = 1; a.W = 1; a.K = N; a.Cg = K; a.R = 1; a.S = 1; a.P = 1; a.Q = 1;
-  a.ph = 0; a.pw = 0; a.sh = 1; a.sw = 1; a.group = 1;
-  a.act = DNNRT_ACT_IDENTITY;
-  a.format = DNNRT_NHWC;
-  return launch_conv_f16(ctx, a);
+  if (Z < 1 || Z > 65535) { set_error("matmul(fp16): %d batches (1..65535)", Z); return false; }
+  const int64_t tiles = ceil_div(M, 64) * ceil_div(N, 64);
+  if (tiles > INT32_MAX) { set_error("matmul(fp16): too many tiles"); return false; }
+  GemmF16Args g{};
+  g.A = A; g.B = B; g.C = (C && beta != 0.f) ? C : nullptr; g.bias = bias; g.Out = Out;
+  g.M = M; g.N = N; g.K = K;
+  g.a_sm = transA ? 1 : K; g.a_sk = transA ? M : 1;   // A stored M x K, or K x M when transposed
+  g.b_sk = transB ? 1 : N; g.b_sn = transB ? K : 1;   // B stored K x N, or N x K when transposed
+  g.az = az; g.bz = bz; g.yz = yz;
+  g.c_sm = c_is_row ? 0 : N; g.cz = c_is_row ? 0 : yz;
+  g.alpha = alpha; g.beta = beta; g.act = act; g.act_coef = ctx->act_coef;
+  hipLaunchKernelGGL(gemm_f16_generic_kernel, dim3((unsigned)tiles, 1, (unsigned)Z), dim3(256), 0, ctx->stream, g);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { set_error("matmul(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
+  return true;
 }
 
 }  // namespace dnnrt

@@ -200,10 +200,10 @@ static void *matmul_nd(dnnrtHandle_t handle, const void *A, const int64_t *dimA,
       return nullptr;
     return Y;
   }
-  if (dtype == DNNRT_F16 && (bias || Zr || act != DNNRT_ACT_IDENTITY)) DNNRT_FAIL("dnnrtMatmulNdBias: fp16 is not built");
   if (dtype == DNNRT_F16) {
-    if (!gemm_f16(handle, (const __half *)A, (const __half *)B, nullptr, (__half *)Y, (int)Mz, (int)N,
-                  (int)K, 1.f, 0.f, false, false, Z, azz, bz, yz))
+    // the residual is laid out like Y (one tall product or one product per batch, as above)
+    if (!gemm_f16(handle, (const __half *)A, (const __half *)B, (const __half *)Zr, (__half *)Y, (int)Mz, (int)N,
+                  (int)K, 1.f, Zr ? 1.f : 0.f, false, false, Z, azz, bz, yz, false, (const __half *)bias, act))
       return nullptr;
     return Y;
   }

@@ -861,14 +861,18 @@ void *dnnrtAttention(dnnrtHandle_t h, const void *Q, const void *K, const void *
                      int64_t B, int64_t Sq, int64_t Sk, int64_t H, int64_t D, int64_t ldIn, float scale,
                      int32_t dtype) {
   (void)h;
-  if (dtype != DNNRT_F32) FAIL("attention: fp32 only");
+  if (dtype != DNNRT_F32 && dtype != DNNRT_F16) FAIL("attention: fp32 and fp16 only");
   if (B < 0 || Sq < 0) FAIL("attention: bad dims");
   if (B == 0 || Sq == 0) return Y;  /* no queries */
   if (Sk <= 0 || H <= 0 || D <= 0) FAIL("attention: bad dims");
-  const float *q = (const float *)Q, *k = (const float *)K, *v = (const float *)V;
-  float *y = (float *)Y;
   const int64_t ldy = H * D, ld = ldIn ? ldIn : ldy;
   if (ld < ldy) FAIL("attention: ldIn");
+  /* fp16 tensors: widened here, one rounding of the result at the end (packed
+   * operands are three views of one buffer: each is widened over its own rows) */
+  float *tq, *tk, *tv, *to;
+  const int64_t nq = (B * Sq - 1) * ld + ldy, nk = (B * Sk - 1) * ld + ldy;
+  const float *q = widen(Q, nq, dtype, &tq), *k = widen(K, nk, dtype, &tk), *v = widen(V, nk, dtype, &tv);
+  float *y = outbuf(Y, B * Sq * ldy, dtype, &to);
 #pragma omp parallel for collapse(2) schedule(static)
   for (int64_t b = 0; b < B; b++)
     for (int64_t hd = 0; hd < H; hd++) {
@@ -894,6 +898,8 @@ void *dnnrtAttention(dnnrtHandle_t h, const void *Q, const void *K, const void *
       }
       free(p);
     }
+  narrow(Y, to, B * Sq * ldy, dtype);
+  free(tq); free(tk); free(tv);
   return Y;
 }
 

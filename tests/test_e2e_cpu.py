@@ -289,6 +289,31 @@ def test_inplace_residual_changes_nothing():
         s.close()
 
 
+def test_bert_fp16_fused_paths_on_the_oracle():
+    """A small fp16 BERT through the oracle: the program with the recomposed LayerNorm / GELU, the fused
+    matmul-bias and the fused attention call (packed Q | K | V, whose three views are offsets in elements of the
+    tensors' type) stays within the fp16 chain's rounding of the unfused program, and both of the fp32 network on
+    the same weights."""
+    small = lambda dt: models.bert_encoder(layers=2, hidden=64, heads=2, seq=16, vocab=50, ffn=128, dtype=dt)  # noqa: E731
+    g16, inputs = small(np.float16)
+    g32 = compiler.Graph()
+    for name, (shape, dt) in g16.input_shapes.items():
+        g32.input(name, shape, dt if np.dtype(dt).kind == "i" else np.float32)
+    for name, arr in g16.constants.items():
+        g32.constant(arr if arr.dtype.kind == "i" else arr.astype(np.float32), name)
+    for op, ins, out, at in g16.nodes:
+        g32.node(op, ins, out, **at)
+    for o in g16.outputs:
+        g32.output(o)
+    want = g32.compile().session(runtime_library=ORACLE_PATH).run(*inputs)[0]
+    _, _, plain = run_oracle(lambda: small(np.float16))
+    np.testing.assert_allclose(plain[0].astype(np.float32), want, rtol=2e-2, atol=3e-2)
+    flags = dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True, alias_copies=True)
+    assert "attention" in small(np.float16)[0].compile(**flags).text
+    _, _, fused = run_oracle(lambda: small(np.float16), **flags)
+    np.testing.assert_allclose(fused[0].astype(np.float32), want, rtol=2e-2, atol=3e-2)
+
+
 def test_compact_pool_changes_nothing():
     """Offsets from the planner that knows every lifetime: the same bits from the oracle, per inference with a
     poisoned pool and resident, for ResNet-50 with every fusion, MobileNetV2, BERT and YOLOv1."""

@@ -289,6 +289,39 @@ def test_mobilenet_v2_fp16_channels_last(batch, image):
     np.testing.assert_array_equal(res[0], out16[0])
 
 
+def test_bert_fp16():
+    """A two-layer BERT-base encoder with fp16 weights and activations: the products on the generic fp16 kernel
+    (batched, bias + residual + GELU fused with `fuse_matmul_bias`), soft-max, LayerNorm, GELU, gathers and
+    transposes in their fp16 forms; against the fp32 oracle on the same fp16-representable weights (LayerNorm
+    outputs are O(1): rtol 2e-2, atol 3e-2), unfused and with the fused paths, the fused attention call among
+    them."""
+    build16 = lambda: models.bert_encoder(layers=2, dtype=np.float16)  # noqa: E731
+    ref, _ = run(lambda: models.bert_encoder(layers=2, dtype=np.float16), ORACLE_PATH)
+    ref32 = None
+    g16, in16 = build16()
+    g32 = compiler.Graph()
+    for name, (shape, dt) in g16.input_shapes.items():
+        g32.input(name, shape, dt if np.dtype(dt).kind == "i" else np.float32)
+    for name, arr in g16.constants.items():
+        g32.constant(arr if arr.dtype.kind == "i" else arr.astype(np.float32), name)
+    for op, ins, out, at in g16.nodes:
+        g32.node(op, ins, out, **at)
+    for o in g16.outputs:
+        g32.output(o)
+    s32 = g32.compile().session(runtime_library=ORACLE_PATH)
+    ref32 = s32.run(*in16)[0]
+    s32.close()
+    for flags in (dict(), dict(recompose=True, fusion=True, fuse_matmul_bias=True, alias_copies=True, compact_pool=True),
+                  dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True, alias_copies=True)):
+        out, info = run(build16, **flags)
+        got = out[0].astype(np.float32)
+        assert np.isfinite(got).all()
+        np.testing.assert_allclose(got, ref32, rtol=2e-2, atol=3e-2)
+        np.testing.assert_allclose(got, ref[0].astype(np.float32), rtol=2e-2, atol=3e-2)
+        res, _ = run(build16, mode=compiler.MODE_RESIDENT, **flags)
+        np.testing.assert_array_equal(res[0], out[0])
+
+
 def test_compact_pool_on_the_gpu():
     """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
     inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured

@@ -296,6 +296,13 @@ def test_matmul_nd(gpu, cpu):
         ref = oc.matmul_nd(cpu, a, b)
         close(oc.matmul_nd(gpu, a, b), ref)
         close(oc.matmul_nd(gpu, a, b), ref)   # again: the split-reduction counters must be back at zero
+    # fp16 tensors (fp32 accumulation, one rounding): the transformer shapes, broadcast batches, ragged tiles
+    for sa, sb in [((1, 128, 768), (768, 768)), ((1, 12, 128, 64), (1, 12, 64, 128)), ((1, 12, 128, 128), (1, 12, 128, 64)),
+                   ((4, 6), (6, 3)), ((2, 4, 6), (6, 3)), ((2, 3, 4, 6), (2, 3, 6, 5)), ((2, 4, 6), (2, 6, 3)), ((4, 6), (3, 6, 2)),
+                   ((2, 77, 130), (130, 70))]:
+        a = r.standard_normal(sa).astype(np.float16)
+        b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float16)
+        np.testing.assert_allclose(oc.matmul_nd(gpu, a, b).astype(np.float32), oc.matmul_nd(cpu, a, b).astype(np.float32), rtol=2e-3, atol=2e-3)
 
 
 def test_split_reduction_hand_over_is_deterministic(gpu, cpu):
@@ -349,8 +356,16 @@ def test_matmul_nd_bias(gpu, cpu):
         z = r.standard_normal(np.broadcast_shapes(sa[:-2], sb[:-2]) + (sa[-2], sb[-1])).astype(np.float32)
         close(oc.matmul_nd_bias(gpu, a, b, bias, z=z), oc.matmul_nd_bias(cpu, a, b, bias, z=z))
         close(oc.matmul_nd_bias(gpu, a, b, bias, gelu=True), oc.matmul_nd_bias(cpu, a, b, bias, gelu=True))
-    with pytest.raises(RuntimeError):
-        oc.matmul_nd_bias(gpu, a.astype(np.float16), b.astype(np.float16), bias.astype(np.float16))  # not built: loud
+    # fp16 tensors: the generic fp16 product (fp32 accumulation, bias, residual and GELU before the one rounding;
+    # the oracle rounds to fp16 after the product and after each of the three)
+    for sa, sb in [((1, 128, 768), (768, 768)), ((5, 7), (7, 3)), ((3, 6, 5), (3, 5, 4)), ((2, 12, 40, 64), (2, 12, 64, 40)), ((1, 3, 33), (33, 130))]:
+        a = r.standard_normal(sa).astype(np.float16)
+        b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float16)
+        bias = r.standard_normal(sb[-1]).astype(np.float16)
+        z = r.standard_normal(np.broadcast_shapes(sa[:-2], sb[:-2]) + (sa[-2], sb[-1])).astype(np.float16)
+        for kw in (dict(), dict(z=z), dict(gelu=True), dict(z=z, gelu=True)):
+            np.testing.assert_allclose(oc.matmul_nd_bias(gpu, a, b, bias, **kw).astype(np.float32),
+                                       oc.matmul_nd_bias(cpu, a, b, bias, **kw).astype(np.float32), rtol=1e-2, atol=1e-2)
 
 
 def test_attention(gpu, cpu):
@@ -365,6 +380,14 @@ def test_attention(gpu, cpu):
     close(oc.attention_packed(gpu, qkv, 4, 0.125), oc.attention_packed(cpu, qkv, 4, 0.125), 1e-4, 1e-5)
     with pytest.raises(RuntimeError):
         oc.attention(gpu, q[:, :, :96], k[:, :, :96], v[:, :, :96], 2, 1.0)   # head size 48
+    # fp16 tensors: widened on the way in, fp32 in between, one rounding on the way out (the oracle does the same)
+    for B, Sq, Sk, H, D in [(1, 128, 128, 12, 64), (2, 50, 77, 3, 32), (1, 33, 129, 4, 64), (1, 40, 300, 2, 128)]:
+        q, k, v = (r.standard_normal((B, S, H * D)).astype(np.float16) for S in (Sq, Sk, Sk))
+        np.testing.assert_allclose(oc.attention(gpu, q, k, v, H, 1.0 / np.sqrt(D)).astype(np.float32),
+                                   oc.attention(cpu, q, k, v, H, 1.0 / np.sqrt(D)).astype(np.float32), rtol=2e-3, atol=2e-3)
+    qkv = r.standard_normal((2, 130, 3 * 256)).astype(np.float16)
+    np.testing.assert_allclose(oc.attention_packed(gpu, qkv, 4, 0.125).astype(np.float32),
+                               oc.attention_packed(cpu, qkv, 4, 0.125).astype(np.float32), rtol=2e-3, atol=2e-3)
 
 
 # ---- data movement -------------------------------------------------------------------------
@@ -1063,7 +1086,18 @@ def test_matmul2d_f16(gpu, cpu):
         row = r.standard_normal(N).astype(np.float16)
         np.testing.assert_allclose(oc.matmul2d_row(gpu, a, b, row, transB=1).astype(np.float32),
                                    oc.matmul2d_row(cpu, a, b, row, transB=1).astype(np.float32), rtol=2e-3, atol=4e-3)
-    with pytest.raises(RuntimeError):
-        oc.matmul2d(gpu, np.zeros((4, 8), np.float16), np.zeros((8, 4), np.float16))  # layout not built: loud
-    with pytest.raises(RuntimeError):
-        oc.matmul2d_row(gpu, a, b, row, beta=0.5, transB=1)                           # only beta = 1 is built
+    # every other form on the generic fp16 kernel: the four operand layouts, alpha and beta with a row or a matrix C
+    # (the matrix updated in place), ragged tiles
+    for M, K, N in [(130, 96, 72), (5, 7, 3), (64, 200, 65)]:
+        for tA in (0, 1):
+            for tB in (0, 1):
+                a = r.standard_normal((K, M) if tA else (M, K)).astype(np.float16)
+                b = (r.standard_normal((N, K) if tB else (K, N)) / np.sqrt(K)).astype(np.float16)
+                c = r.standard_normal((M, N)).astype(np.float16)
+                row = r.standard_normal(N).astype(np.float16)
+                for kw in (dict(), dict(alpha=0.5), dict(c=c, alpha=1.5, beta=0.5), dict(c=c, beta=1.0)):
+                    np.testing.assert_allclose(oc.matmul2d(gpu, a, b, transA=tA, transB=tB, **kw).astype(np.float32),
+                                               oc.matmul2d(cpu, a, b, transA=tA, transB=tB, **kw).astype(np.float32), rtol=4e-3, atol=6e-3)
+                if not tA:
+                    np.testing.assert_allclose(oc.matmul2d_row(gpu, a, b, row, beta=0.5, transB=tB).astype(np.float32),
+                                               oc.matmul2d_row(cpu, a, b, row, beta=0.5, transB=tB).astype(np.float32), rtol=4e-3, atol=6e-3)
