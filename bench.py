@@ -13,7 +13,7 @@ headline record (value, roofline, cpu_baseline ...) is ResNet-50 fp16 batch 64
 and the key "fp32_bs1" holds the same record for ResNet-50 fp32 batch 1.
 Other workloads: resnet50_fp32_bs1, resnet50_fp16_bs64, mobilenet_v2_fp32_bs1,
 bert_base_fp32_seq128, single_conv_fp32, alexnet_fp32_bs1, yolo_v1_fp32_bs2,
-srgan_fp32_96x96.  --layers writes a per-operation table (algorithmic FLOP and
+srgan_fp32_96x96, ssd_resnet50_fp32_bs3.  --layers writes a per-operation table (algorithmic FLOP and
 bytes, the roofline bound, measured time) of the headline workload to FILE.
 """
 import argparse
@@ -56,6 +56,9 @@ def build_workload(name, batch=None):
         return models.alexnet(1, np.float32), dict(fusion=True, fuse_matmul_bias=True), 1, "img/s", "f32"
     if name == "yolo_v1_fp32_bs2":
         return models.yolo_v1(2, np.float32), dict(fusion=True, fuse_activations=True, fuse_matmul_bias=True), 2, "img/s", "f32"
+    if name == "ssd_resnet50_fp32_bs3":  # the reference's test runs three images
+        return (models.ssd_resnet50(3, np.float32),
+                dict(fusion=True, fuse_residual=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True, inplace_residual=True, compact_pool=True), 3, "img/s", "f32")
     if name == "srgan_fp32_96x96":
         return models.srgan_generator(1, np.float32, height=96, width=96), dict(fusion=True, fuse_residual=True, fuse_activations=True), 1, "img/s", "f32"
     raise SystemExit(f"unknown workload {name}")

@@ -89,6 +89,58 @@ def resnet50(batch=1, dtype=np.float32, seed=2, image=224, classes=1000):
     return g, [x_np]
 
 
+def ssd_resnet50(batch=1, dtype=np.float32, seed=8, image=300, labels=81):
+    """SSD300 on a ResNet-50 backbone as the reference's test exports it
+    (test/models/ssd-resnet50/run.py: NVIDIA's `nvidia_ssd`, whose forward pass ends at the box and class
+    tensors; decoding and non-maximum suppression happen in Python afterwards and are not part of the
+    network): ResNet-50 up to its third stage with that stage's stride removed (1024 channels at 38 x 38 for
+    a 300 x 300 image), five extra blocks of 1x1 -> 3x3 convolutions (BatchNorm folded, ReLU) down to 1 x 1,
+    a 3x3 location head and a 3x3 class head on each of the six feature maps (4, 6, 6, 6, 4, 4 boxes per
+    cell), every head's result viewed as [N, 4 or labels, boxes] and concatenated: two results,
+    [N, 4, 8732] and [N, labels, 8732]."""
+    init = _Init(seed, dtype)
+    g = Graph()
+    x_np = rng.normal(seed, 0, (batch, 3, image, image)).astype(dtype)
+    g.input("input", x_np.shape, dtype)
+    x = g.node("Relu", [_conv(g, init, "input", 3, 64, 7, 2, 3)])
+    x = g.node("MaxPool", [x], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
+    size = ((image + 6 - 7) // 2 + 1 + 2 - 3) // 2 + 1
+    cin = 64
+    for planes, blocks, stride in [(64, 3, 1), (128, 4, 2), (256, 6, 1)]:  # the third stage keeps its input's size
+        for b in range(blocks):
+            s = stride if b == 0 else 1
+            identity = x
+            o = g.node("Relu", [_conv(g, init, x, cin, planes, 1, 1, 0)])
+            o = g.node("Relu", [_conv(g, init, o, planes, planes, 3, s, 1)])
+            o = _conv(g, init, o, planes, planes * 4, 1, 1, 0)
+            if b == 0:
+                identity = _conv(g, init, x, cin, planes * 4, 1, s, 0)
+            x = g.node("Relu", [g.node("Add", [o, identity])])
+            cin = planes * 4
+        size = (size - 1) // stride + 1
+    feeds = [(x, cin, size)]
+    for i, (cout, mid) in enumerate(zip([512, 512, 256, 256, 256], [256, 256, 128, 128, 128])):
+        o = g.node("Relu", [_conv(g, init, x, cin, mid, 1, 1, 0)])
+        if i < 3:
+            x = g.node("Relu", [_conv(g, init, o, mid, cout, 3, 2, 1)])
+            size = (size + 2 - 3) // 2 + 1
+        else:
+            x = g.node("Relu", [_conv(g, init, o, mid, cout, 3, 1, 0)])
+            size = size - 2
+        cin = cout
+        feeds.append((x, cin, size))
+    locs, confs = [], []
+    for (f, c, sz), boxes in zip(feeds, [4, 6, 6, 6, 4, 4]):
+        n = boxes * sz * sz
+        loc = _conv(g, init, f, c, boxes * 4, 3, 1, 1)
+        conf = _conv(g, init, f, c, boxes * labels, 3, 1, 1)
+        locs.append(g.node("Reshape", [loc, g.constant(np.array([batch, 4, n], np.int64))]))
+        confs.append(g.node("Reshape", [conf, g.constant(np.array([batch, labels, n], np.int64))]))
+    g.output(g.node("Concat", locs, "locs", axis=2))
+    g.output(g.node("Concat", confs, "confs", axis=2))
+    return g, [x_np]
+
+
 def mobilenet_v2(batch=1, dtype=np.float32, seed=3, image=224, classes=1000):
     """MobileNetV2 width 1.0; ReLU6 is Clip(0, 6) with constant bounds."""
     init = _Init(seed, dtype)

@@ -314,6 +314,25 @@ def test_bert_fp16_fused_paths_on_the_oracle():
     np.testing.assert_allclose(fused[0].astype(np.float32), want, rtol=2e-2, atol=3e-2)
 
 
+def test_ssd_resnet50_program():
+    """SSD300 on ResNet-50 as the reference's test exports it (the network only: decoding and non-maximum
+    suppression are Python in test/models/ssd-resnet50/run.py): 8732 boxes at 300 x 300, two results; the fused
+    program (residual blocks, shortcut pairs, first layer with its pooling, in-place sums) gives the oracle's
+    unfused result to the fp32 tolerance."""
+    build = lambda: models.ssd_resnet50(1, labels=7)  # noqa: E731
+    g, inputs = build()
+    plain = g.compile()
+    assert [shape for shape, _ in plain.output_info()] == [(1, 4, 8732), (1, 7, 8732)]
+    flags = dict(fusion=True, fuse_residual=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True, inplace_residual=True, compact_pool=True)
+    fused = build()[0].compile(**flags)
+    assert fused.num_ops(compute_only=True) < plain.num_ops(compute_only=True) // 2
+    assert fused.text.count("add-conv") == 3 and "maxpoolfwd" in fused.text
+    a = plain.session(runtime_library=ORACLE_PATH).run(*inputs)
+    b = fused.session(runtime_library=ORACLE_PATH).run(*inputs)
+    for x, y in zip(a, b):
+        np.testing.assert_allclose(y, x, rtol=1e-4, atol=1e-4 * float(np.abs(x).max()))
+
+
 def test_compact_pool_changes_nothing():
     """Offsets from the planner that knows every lifetime: the same bits from the oracle, per inference with a
     poisoned pool and resident, for ResNet-50 with every fusion, MobileNetV2, BERT and YOLOv1."""

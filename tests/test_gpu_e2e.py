@@ -322,6 +322,25 @@ def test_bert_fp16():
         np.testing.assert_array_equal(res[0], out[0])
 
 
+@pytest.mark.parametrize("batch", [1, 3])
+def test_ssd_resnet50(batch):
+    """SSD300 on ResNet-50 (the reference's test/models/ssd-resnet50 network: 300 x 300 images, 8732 boxes, box and
+    class tensors; three images there) against the oracle running the unfused program, with the reference's flags
+    and with every fusion, per inference and resident."""
+    build = lambda: models.ssd_resnet50(batch, labels=21)  # noqa: E731
+    ref, _ = run(build, ORACLE_PATH)
+    for flags in (dict(), dict(fusion=True, fuse_residual=True, fuse_first_layer_maxpool=True, fuse_projection_shortcut=True,
+                               inplace_residual=True, compact_pool=True)):
+        out, info = run(build, **flags)
+        assert info["requested"] == info["pool"]
+        assert [o.shape for o in out] == [(batch, 4, 8732), (batch, 21, 8732)]
+        for a, b in zip(out, ref):
+            close(a, b, 1e-4, 1e-4)
+        res, _ = run(build, mode=compiler.MODE_RESIDENT, **flags)
+        for a, b in zip(res, out):
+            np.testing.assert_array_equal(a, b)
+
+
 def test_compact_pool_on_the_gpu():
     """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
     inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured
