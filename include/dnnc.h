@@ -122,8 +122,11 @@ dnncSession *dnncSessionCreate(dnncProgram *p, const char *runtime_library, int3
 void dnncSessionDestroy(dnncSession *s);
 /* host buffers in, host buffers out; returns when the results are in `outputs` */
 int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *outputs);
-/* resident mode only.  on_device: inputs/outputs are device buffers and the call does not
- * wait (dnncSessionSync does); use_graph: replay the kernels from a captured graph */
+/* resident mode only.  on_device != 0: inputs/outputs are device buffers and the call does not
+ * wait (dnncSessionSync does); on_device == 2: the kernels read the input buffers where they
+ * are instead of copying them into the pool first -- the caller leaves them unchanged until
+ * the run is over, and passing other addresses than last time records the graph again;
+ * use_graph: replay the kernels from a captured graph */
 int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
 int32_t dnncSessionSync(dnncSession *s);
 /* Tuning and tests: dnnrtSetConvTile on the session's handle (0 = automatic choice); a captured

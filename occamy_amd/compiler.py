@@ -296,11 +296,12 @@ class Session:
             raise RuntimeError("run: " + _err())
         return outs
 
-    def run_device(self, in_ptrs, out_ptrs, use_graph=True):
-        """Resident mode: device addresses in and out; returns without waiting."""
+    def run_device(self, in_ptrs, out_ptrs, use_graph=True, in_place=False):
+        """Resident mode: device addresses in and out; returns without waiting.  in_place: the kernels read the
+        input buffers where they are (no copy into the pool); they must stay unchanged until the run is over."""
         ip = (C.c_void_p * max(len(in_ptrs), 1))(*in_ptrs)
         op = (C.c_void_p * max(len(out_ptrs), 1))(*out_ptrs)
-        if lib().dnncSessionRunResident(self._s, ip, op, 1, int(use_graph)):
+        if lib().dnncSessionRunResident(self._s, ip, op, 2 if in_place else 1, int(use_graph)):
             raise RuntimeError("run_device: " + _err())
 
     def profile(self, in_ptrs_or_arrays, on_device=False, by_class=False):

@@ -477,9 +477,11 @@ bool Session::issue_all_compute(std::string &err) {
 // Resident inference.  `on_device` != 0: inputs/outputs are device pointers and
 // the call returns without waiting (sync() does).
 bool Session::run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err) {
+  const bool borrow = on_device == 2 && !host_backend;
   // The pool reuses the inputs' slots for later tensors, so every pass over
   // the kernels must be preceded by a fresh copy of the inputs.
   auto copy_inputs = [&]() -> bool {
+    if (borrow) return true;
     for (const Op *op : prog->ops) {
       if (op->kind != OP_MEMCPY || op->mode != 1) continue;
       const Value *src = op->operands[1];
@@ -493,6 +495,20 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
     }
     return true;
   };
+  // on_device == 2: the kernels read the caller's input buffers where they are (no copy into the pool slots).  The
+  // argument slots' values point at those buffers for as long as the caller keeps passing the same addresses; a
+  // recorded graph holds them, so a change of address drops it.
+  {
+    bool moved = false;
+    for (const Op *op : prog->ops) {
+      if (op->kind != OP_MEMCPY || op->mode != 1 || op->operands[1]->arg_index < 0) continue;
+      const size_t slot = (size_t)op->operands[0]->id;
+      if (!arg_home.count(slot)) arg_home[slot] = ptr[slot];
+      void *want = borrow ? const_cast<void *>(inputs[(size_t)op->operands[1]->arg_index]) : arg_home[slot];
+      if (ptr[slot] != want) { ptr[slot] = want; moved = true; }
+    }
+    if (moved && graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
+  }
   const bool graphed = use_graph && !host_backend;
   if (graphed && !graph) {
     // One eager pass on real data first: it validates every call outside of
@@ -535,6 +551,12 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
 
 bool Session::profile_resident(const void *const *inputs, int on_device, bool by_class, std::vector<float> &ms, std::string &err) {
   if (mode != MODE_RESIDENT) { err = "profiling needs a resident session"; return false; }
+  // profiling copies the inputs into their pool slots: argument values that point at a caller's buffers go home
+  for (const auto &h : arg_home)
+    if (ptr[h.first] != h.second) {
+      ptr[h.first] = h.second;
+      if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
+    }
   // the operations that launch something, in program order (an aliased copy only hands its input's address on;
   // a first eager pass has set those)
   std::vector<const Op *> compute;

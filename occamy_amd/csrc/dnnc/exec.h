@@ -115,6 +115,7 @@ class Session {
   std::vector<char> filter_crsk;           // value id -> its device copy is C,R,S,K
   void *pool = nullptr, *weights = nullptr, *graph = nullptr;
   std::vector<void *> ptr;  // value id -> address (host or device)
+  std::map<size_t, void *> arg_home;  // resident mode: value id of a function argument's pool slot -> its address in the pool
   std::map<std::string, void *> host_const;
   std::vector<void *> host_out, host_in;
   // resident mode: results produced mid-program, whose pool bytes a later

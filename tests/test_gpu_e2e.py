@@ -341,6 +341,48 @@ def test_ssd_resnet50(batch):
             np.testing.assert_array_equal(a, b)
 
 
+def test_resident_run_reads_device_inputs_in_place():
+    """run_device(in_place=True): the kernels read the caller's input buffer instead of a copy in the pool; the
+    same bits as with the copy, eager and replayed; the input buffer is left as it was; another input address
+    (the graph is recorded again), then the copying mode and the profiler on the same session."""
+    import torch
+    for builder, flags in ((lambda: models.resnet50(4, np.float16, seed=5, image=64),
+                            dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
+                                 fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True, compact_pool=True)),
+                           (lambda: models.resnet50(2, seed=6, image=64, classes=100), dict(fusion=True, fuse_residual=True, fuse_first_layer_maxpool=True)),
+                           (lambda: models.bert_encoder(layers=2), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True))):
+        want, _ = run(builder, **flags)
+        g, inputs = builder()
+        p = g.compile(**flags)
+        s = p.session(compiler.MODE_RESIDENT)
+        (shape, dt), = p.output_info()[:1]
+        out = torch.empty(shape, dtype=torch.from_numpy(np.empty(0, dt)).dtype, device="cuda")
+        a = [torch.from_numpy(x).cuda() for x in inputs]
+        b = [torch.from_numpy(x).cuda() for x in inputs]   # the same values at other addresses
+        for dev, graph in ((a, False), (a, True), (a, True), (b, True), (b, False)):
+            out.zero_()
+            torch.cuda.synchronize()
+            s.run_device([t.data_ptr() for t in dev], [out.data_ptr()], use_graph=graph, in_place=True)
+            s.sync()
+            np.testing.assert_array_equal(out.cpu().numpy(), want[0])
+            for t, x in zip(dev, inputs):
+                np.testing.assert_array_equal(t.cpu().numpy(), x)
+        out.zero_()
+        torch.cuda.synchronize()
+        s.run_device([t.data_ptr() for t in a], [out.data_ptr()], use_graph=True)   # copying again
+        s.sync()
+        np.testing.assert_array_equal(out.cpu().numpy(), want[0])
+        s.run_device([t.data_ptr() for t in a], [out.data_ptr()], use_graph=True, in_place=True)
+        s.sync()
+        assert len(s.profile(inputs)) == p.num_ops(compute_only=True)
+        out.zero_()
+        torch.cuda.synchronize()
+        s.run_device([t.data_ptr() for t in b], [out.data_ptr()], use_graph=True, in_place=True)
+        s.sync()
+        np.testing.assert_array_equal(out.cpu().numpy(), want[0])
+        s.close()
+
+
 def test_compact_pool_on_the_gpu():
     """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
     inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured
