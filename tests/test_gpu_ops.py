@@ -96,6 +96,78 @@ def test_conv_f32(gpu, cpu, case):
     np.testing.assert_array_equal(oc.conv(cpu, x, w, b, *args, _abi.ACT_RELU, z=z, inplace=True), oc.conv(cpu, x, w, b, *args, _abi.ACT_RELU, z=z))
 
 
+def random_conv_cases(seed, count, f16):
+    """Seeded shapes around the kernels' boundaries: channel counts on both sides of the multiples of 8, 32 and
+    64 the fast paths ask for, filter sizes 1 / 2 / 3 / 5 / 7, strides 1-3 (different along the two axes now and
+    then), padding up to the filter's half and beyond, a few hundred to a few thousand output pixels."""
+    r = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        R, S = (int(v) for v in r.choice([1, 1, 2, 3, 3, 3, 5, 7], 2)) if r.random() < 0.3 else (int(r.choice([1, 3, 3, 5])),) * 2
+        grp = int(r.choice([1, 1, 1, 1, 2, 4])) if not f16 or r.random() < 0.3 else 1
+        cg = int(r.choice([1, 3, 8, 16, 31, 32, 33, 64, 96, 128, 160, 192, 256])) if f16 else int(r.choice([1, 2, 3, 5, 8, 16, 24, 33, 64, 100]))
+        kg = int(r.choice([1, 2, 8, 24, 40, 64, 72, 128, 136, 200, 256])) if f16 else int(r.choice([1, 2, 3, 4, 7, 16, 33, 64, 130]))
+        if grp > 1:
+            cg, kg = min(cg, 32), min(kg, 40)
+        N, H, W = int(r.integers(1, 5)), int(r.integers(1, 30)), int(r.integers(1, 30))
+        sh, sw = (int(r.integers(1, 4)),) * 2 if r.random() < 0.8 else (int(r.integers(1, 4)), int(r.integers(1, 4)))
+        ph, pw = int(r.integers(0, R // 2 + 2)), int(r.integers(0, S // 2 + 2))
+        P, Q = (H + 2 * ph - R) // sh + 1, (W + 2 * pw - S) // sw + 1
+        if P < 1 or Q < 1 or H + 2 * ph < R or W + 2 * pw < S or N * cg * grp * H * W > 2_000_000 or N * kg * grp * P * Q > 2_000_000:
+            continue
+        cases.append((N, cg * grp, H, W, kg * grp, R, S, sh, sw, ph, pw, grp))
+    return cases
+
+
+def test_conv_f32_random_shapes(gpu, cpu):
+    """120 seeded shapes through dnnrtConvBiasActiv / dnnrtConvBiasAddActiv on fp32 N,C,H,W tensors against the
+    oracle (rtol 1e-4, atol 1e-5), with both filter layouts, each activation mode once in a while, and the residual
+    form also written over its residual operand."""
+    for i, (N, C, H, W, K, R, S, sh, sw, ph, pw, grp) in enumerate(random_conv_cases(2024, 120, False)):
+        r = rng(1000 + i)
+        x = r.standard_normal((N, C, H, W)).astype(np.float32)
+        w = (r.standard_normal((K, C // grp, R, S)) * np.sqrt(2.0 / (C // grp * R * S))).astype(np.float32)
+        b = r.uniform(-0.3, 0.3, K).astype(np.float32)
+        activ, coef = [(_abi.ACT_RELU, None), (_abi.ACT_IDENTITY, None), (_abi.ACT_CLIPPED_RELU, 0.7), (_abi.ACT_LEAKY_RELU, 0.1)][i % 4]
+        what = f"case {i}: x {x.shape} w {w.shape} strides {(sh, sw)} pads {(ph, pw)} group {grp} act {activ}"
+        ref = oc.conv(cpu, x, w, b, (ph, pw), (sh, sw), grp, activ, coef=coef)
+        for crsk in (False, True):
+            got = oc.conv(gpu, x, w, b, (ph, pw), (sh, sw), grp, activ, crsk=crsk, coef=coef)
+            np.testing.assert_allclose(got, ref, rtol=RTOL, atol=ATOL, err_msg=what)
+        z = r.standard_normal(ref.shape).astype(np.float32)
+        refz = oc.conv(cpu, x, w, b, (ph, pw), (sh, sw), grp, activ, z=z, coef=coef)
+        gotz = oc.conv(gpu, x, w, b, (ph, pw), (sh, sw), grp, activ, z=z, coef=coef)
+        np.testing.assert_allclose(gotz, refz, rtol=RTOL, atol=ATOL, err_msg=what + " + z")
+        np.testing.assert_array_equal(oc.conv(gpu, x, w, b, (ph, pw), (sh, sw), grp, activ, z=z, coef=coef, inplace=True), gotz, err_msg=what + " in place")
+
+
+def test_conv_f16_random_shapes(gpu, cpu):
+    """120 seeded shapes through the fp16 convolution, channels-last (every fast path's boundary: channel counts
+    around the multiples of 8 / 32 / 64, a few steps or many, padded or not, grouped and depthwise) and, every
+    third case, N,C,H,W; against the oracle to one fp16 rounding (rtol 2e-3, atol 2e-3; 4e-3 with a residual),
+    the residual form also in place."""
+    for i, (N, C, H, W, K, R, S, sh, sw, ph, pw, grp) in enumerate(random_conv_cases(4048, 120, True)):
+        if R != S or sh != sw or ph != pw:  # the fp16 helper takes square geometry
+            S, sw, pw = R, sh, ph
+            if (W + 2 * pw - S) // sw + 1 < 1 or W + 2 * pw < S:
+                continue
+        r = rng(3000 + i)
+        x = r.standard_normal((N, C, H, W)).astype(np.float16)
+        w = (r.standard_normal((K, C // grp, R, R)) * np.sqrt(2.0 / (C // grp * R * R))).astype(np.float16)
+        b = r.uniform(-0.3, 0.3, K).astype(np.float16)
+        fmt = _abi.NCHW if i % 3 == 2 else _abi.NHWC
+        what = f"case {i}: x {x.shape} w {w.shape} stride {sh} pad {ph} group {grp} format {fmt}"
+        ref = oc.conv(cpu, x, w, b, (ph, ph), (sh, sh), grp, _abi.ACT_RELU)
+        got = conv_f16(gpu, x, w, b, (ph, ph), (sh, sh), grp, _abi.ACT_RELU, fmt)
+        np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3, err_msg=what)
+        z = r.standard_normal(ref.shape).astype(np.float16)
+        refz = oc.conv(cpu, x, w, b, (ph, ph), (sh, sh), grp, _abi.ACT_RELU, z=z)
+        gotz = conv_f16(gpu, x, w, b, (ph, ph), (sh, sh), grp, _abi.ACT_RELU, fmt, z=z)
+        np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3, err_msg=what + " + z")
+        np.testing.assert_array_equal(conv_f16(gpu, x, w, b, (ph, ph), (sh, sh), grp, _abi.ACT_RELU, fmt, z=z, inplace=True), gotz,
+                                      err_msg=what + " in place")
+
+
 def test_conv_closed_forms(gpu):
     x = rng(1).standard_normal((1, 3, 8, 8)).astype(np.float32)
     w = np.zeros((3, 3, 3, 3), np.float32)
