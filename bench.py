@@ -13,7 +13,7 @@ headline record (value, roofline, cpu_baseline ...) is ResNet-50 fp16 batch 64
 and the key "fp32_bs1" holds the same record for ResNet-50 fp32 batch 1.
 Other workloads: resnet50_fp32_bs1, resnet50_fp16_bs64, mobilenet_v2_fp32_bs1,
 bert_base_fp32_seq128, single_conv_fp32, alexnet_fp32_bs1, yolo_v1_fp32_bs2,
-srgan_fp32_96x96, ssd_resnet50_fp32_bs3.  --layers writes a per-operation table (algorithmic FLOP and
+srgan_fp32_96x96, ssd_resnet50_fp32_bs3, mobilenet_v2_fp16_bs64, bert_base_fp16_seq128.  --layers writes a per-operation table (algorithmic FLOP and
 bytes, the roofline bound, measured time) of the headline workload to FILE.
 """
 import argparse
@@ -50,6 +50,13 @@ def build_workload(name, batch=None):
         return models.mobilenet_v2(1, np.float32), dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True, alias_copies=True), 1, "img/s", "f32"
     if name == "bert_base_fp32_seq128":
         return models.bert_encoder(), dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True, alias_copies=True), 1, "seq/s", "f32"
+    if name == "mobilenet_v2_fp16_bs64":
+        return (models.mobilenet_v2(64, np.float16),
+                dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True, channels_last=True, alias_copies=True,
+                     inplace_residual=True, compact_pool=True), 64, "img/s", "f16")
+    if name == "bert_base_fp16_seq128":
+        return (models.bert_encoder(dtype=np.float16),
+                dict(recompose=True, fusion=True, fuse_matmul_bias=True, fuse_attention=True, alias_copies=True, compact_pool=True), 1, "seq/s", "f16")
     if name == "single_conv_fp32":
         return models.single_conv(), dict(fusion=True), 1, "img/s", "f32"
     if name == "alexnet_fp32_bs1":

@@ -260,7 +260,7 @@ static bool match_layernorm(const Matcher &m, const GNode &root, GNode &fused, s
   two_name = pow_->inputs[1];
   if (sub->inputs.size() != 2 || !(mean1 = m.def(sub->inputs[1], "ReduceMean")) || mean1->inputs[0] != sub->inputs[0]) return false;
   double eps, two;
-  if (!m.scalar(eps_name, eps) || !m.scalar(two_name, two) || two != 2.0 || !(eps > 0.0)) return false;
+  if (!m.scalar(eps_name, eps) || !m.scalar(two_name, two) || two != 2.0 || !(eps >= 0.0)) return false;  // (1e-12 stored as fp16 is 0)
   if (!m.last_axis_mean(*mean1) || !m.last_axis_mean(*mean2)) return false;
   const GTensor &x = m.g.tensors.at(sub->inputs[0]);
   auto vec_const = [&](const std::string &n) {

@@ -392,7 +392,7 @@ void fuse_matmul_bias(Program &p) {
   for (Op *op : p.ops)
     if (op->kind == OP_MATMULND) mms.push_back(op);
   for (Op *mm : mms) {
-    if (mm->result->dtype != F32 || mm->result->uses.size() != 1) continue;
+    if ((mm->result->dtype != F32 && mm->result->dtype != F16) || mm->result->uses.size() != 1) continue;
     Op *add = mm->result->uses.front().first;
     if (add->kind != OP_ADD || add->coef != 1.f || add->operands[0] != mm->result) continue;
     bool row = !add->dimB.empty() && add->dimB.back() == mm->dimOut.back();

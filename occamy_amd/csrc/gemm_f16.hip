@@ -4,7 +4,8 @@
 // other form -- B stored K x N, transposed A, batches, alpha / beta, a bias
 // row with a residual matrix and an activation behind it -- goes to one
 // generic kernel: a 64 x 64 tile of Out per workgroup, operands gathered
-// element by element into LDS (strides are runtime values), 32x32x16 MFMA,
+// into LDS in runs of eight along their contiguous direction (strides are
+// runtime values; one 16-byte load per run where alignment allows), 32x32x16 MFMA,
 // fp32 accumulation, one rounding to fp16 at the end.
 #include "gemm_f16.h"
 
@@ -25,9 +26,10 @@ struct GemmF16Args {
   float alpha, beta;
   int act;
   float act_coef;
+  bool a_vec, b_vec;                // the contiguous direction of A / B may be read eight elements (16 bytes) at a time
 };
 
-constexpr int G_BK = 32, G_ROW = 40;  // k per step; halfs per LDS row (32 + 8 of padding)
+constexpr int G_BK = 64, G_ROW = 72;  // k per step; halfs per LDS row (64 + 8 of padding)
 
 // Tile: 64 columns n x 64 rows m; the MFMA's row operand is the B side (n), its column operand the A side (m), so
 // that a lane ends up with four consecutive n of one m: an 8-byte store.
@@ -48,17 +50,55 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
   g_floatx16 acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  // A step is 64 rows x 64 k per operand = 512 runs of eight elements along the operand's contiguous direction;
+  // a thread takes two runs of each operand.  Run r along k: row r / 8, k 8 (r % 8); along the row index: k r / 8,
+  // rows 8 (r % 8) ...  A run is one 16-byte load where the operand allows it, eight 2-byte loads otherwise.
   for (int k0 = 0; k0 < a.K; k0 += G_BK) {
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-      // A side -> Ms[m][k]
-      const int am = a_k_fast ? tid >> 2 : ((tid & 7) << 3) + e, ak = a_k_fast ? ((tid & 3) << 3) + e : tid >> 3;
-      const int gm = m0 + am, gk = k0 + ak;
-      Ms[am * G_ROW + ak] = (gm < a.M && gk < a.K) ? Ag[(int64_t)gm * a.a_sm + (int64_t)gk * a.a_sk] : (_Float16)0.f;
-      // B side -> Ns[n][k]
-      const int bn = b_k_fast ? tid >> 2 : ((tid & 7) << 3) + e, bk = b_k_fast ? ((tid & 3) << 3) + e : tid >> 3;
-      const int gn = n0 + bn, gk2 = k0 + bk;
-      Ns[bn * G_ROW + bk] = (gn < a.N && gk2 < a.K) ? Bg[(int64_t)gk2 * a.b_sk + (int64_t)gn * a.b_sn] : (_Float16)0.f;
+    for (int h = 0; h < 2; h++) {
+      const int r = tid + 256 * h;
+      {  // A side -> Ms[m][k]
+        const int row0 = a_k_fast ? r >> 3 : (r & 7) << 3, kk0 = a_k_fast ? (r & 7) << 3 : r >> 3;
+        const int64_t at = (int64_t)(m0 + row0) * a.a_sm + (int64_t)(k0 + kk0) * a.a_sk;
+        g_half8 v;
+        const bool whole = a_k_fast ? (m0 + row0 < a.M && k0 + kk0 + 8 <= a.K) : (m0 + row0 + 8 <= a.M && k0 + kk0 < a.K);
+        if (a.a_vec && whole) {
+          v = *reinterpret_cast<const g_half8 *>(Ag + at);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const int gm = m0 + row0 + (a_k_fast ? 0 : e), gk = k0 + kk0 + (a_k_fast ? e : 0);
+            v[e] = (gm < a.M && gk < a.K) ? Ag[(int64_t)gm * a.a_sm + (int64_t)gk * a.a_sk] : (_Float16)0.f;
+          }
+        }
+        if (a_k_fast) {
+          *reinterpret_cast<g_half8 *>(Ms + row0 * G_ROW + kk0) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) Ms[(row0 + e) * G_ROW + kk0] = v[e];
+        }
+      }
+      {  // B side -> Ns[n][k]
+        const int row0 = b_k_fast ? r >> 3 : (r & 7) << 3, kk0 = b_k_fast ? (r & 7) << 3 : r >> 3;
+        const int64_t at = (int64_t)(k0 + kk0) * a.b_sk + (int64_t)(n0 + row0) * a.b_sn;
+        g_half8 v;
+        const bool whole = b_k_fast ? (n0 + row0 < a.N && k0 + kk0 + 8 <= a.K) : (n0 + row0 + 8 <= a.N && k0 + kk0 < a.K);
+        if (a.b_vec && whole) {
+          v = *reinterpret_cast<const g_half8 *>(Bg + at);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const int gn = n0 + row0 + (b_k_fast ? 0 : e), gk = k0 + kk0 + (b_k_fast ? e : 0);
+            v[e] = (gn < a.N && gk < a.K) ? Bg[(int64_t)gk * a.b_sk + (int64_t)gn * a.b_sn] : (_Float16)0.f;
+          }
+        }
+        if (b_k_fast) {
+          *reinterpret_cast<g_half8 *>(Ns + row0 * G_ROW + kk0) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) Ns[(row0 + e) * G_ROW + kk0] = v[e];
+        }
+      }
     }
     __syncthreads();
 #pragma unroll
@@ -112,6 +152,11 @@ bool gemm_f16(const dnnrtContext *ctx, const __half *A, const __half *B, const _
   g.az = az; g.bz = bz; g.yz = yz;
   g.c_sm = c_is_row ? 0 : N; g.cz = c_is_row ? 0 : yz;
   g.alpha = alpha; g.beta = beta; g.act = act; g.act_coef = ctx->act_coef;
+  // a run of eight along the contiguous direction is one aligned 16-byte load when every run starts on a multiple
+  // of eight elements: base, batch stride and the other direction's stride
+  const int64_t a_other = transA ? g.a_sk : g.a_sm, b_other = transB ? g.b_sn : g.b_sk;
+  g.a_vec = aligned16(A) && a_other % 8 == 0 && az % 8 == 0;
+  g.b_vec = aligned16(B) && b_other % 8 == 0 && bz % 8 == 0;
   hipLaunchKernelGGL(gemm_f16_generic_kernel, dim3((unsigned)tiles, 1, (unsigned)Z), dim3(256), 0, ctx->stream, g);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("matmul(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
