@@ -168,6 +168,76 @@ def test_conv_f16_random_shapes(gpu, cpu):
                                       err_msg=what + " in place")
 
 
+def test_rowwise_ops_random_shapes(gpu, cpu):
+    """Seeded sweeps of soft-max, LayerNorm, ReduceMean and the poolings over shapes around their kernels'
+    boundaries (row lengths on both sides of 4-element groups, of the in-register limit and of a wavefront;
+    reductions over an inner, a middle and an outer run), fp32 and fp16, against the oracle."""
+    r = np.random.default_rng(77)
+    for i in range(60):
+        rows = int(r.choice([1, 2, 3, 7, 64, 130]))
+        L = int(r.choice([1, 2, 3, 4, 5, 31, 32, 33, 63, 64, 65, 127, 128, 255, 256, 257, 768, 1000, 1024, 2047, 2048, 2049, 2052, 3000, 4100]))
+        for dtype, tol in ((np.float32, 1e-4), (np.float16, 4e-3)):
+            x = (r.standard_normal((rows, L)) * 2 + 0.5).astype(dtype)
+            close(oc.softmax(gpu, x, 1), oc.softmax(cpu, x, 1), tol, tol * 1e-2 if dtype == np.float32 else tol)
+            if L > 1:
+                g, b = r.standard_normal(L).astype(dtype), r.standard_normal(L).astype(dtype)
+                close(oc.layernorm(gpu, x, g, b, 1e-5), oc.layernorm(cpu, x, g, b, 1e-5), max(tol, 2e-4), max(tol, 2e-4) * 4)
+    for i in range(40):
+        outer, red, inner = (int(v) for v in (r.integers(1, 9), r.choice([1, 2, 5, 7, 49, 64, 100, 257]), r.choice([1, 2, 3, 4, 8, 16, 48, 130])))
+        for dtype, tol in ((np.float32, 1e-5), (np.float16, 2e-3)):
+            x = r.standard_normal((outer, red, inner)).astype(dtype)
+            close(oc.reduce_mean(gpu, x, (outer, 1, inner)), oc.reduce_mean(cpu, x, (outer, 1, inner)), tol, tol)
+    for i in range(40):
+        N, C, H, W = (int(v) for v in (r.integers(1, 4), r.choice([1, 3, 8, 16, 24, 33]), r.integers(2, 24), r.integers(2, 24)))
+        k = (int(r.integers(1, 4)), int(r.integers(1, 4)))
+        st = (int(r.integers(1, 4)), int(r.integers(1, 4)))
+        pd = (int(r.integers(0, (k[0] + 1) // 2 + (k[0] > 1) - (k[0] == 2))), int(r.integers(0, (k[1] + 1) // 2 + (k[1] > 1) - (k[1] == 2))))
+        pd = (min(pd[0], k[0] // 2), min(pd[1], k[1] // 2))
+        if H + 2 * pd[0] < k[0] or W + 2 * pd[1] < k[1]:
+            continue
+        for dtype in (np.float32, np.float16):
+            x = r.standard_normal((N, C, H, W)).astype(dtype)
+            if i % 5 == 0:
+                x[0, 0, H // 2, W // 2] = np.nan
+            got, ref = oc.pool(gpu, "max", x, k, pd, st), oc.pool(cpu, "max", x, k, pd, st)
+            np.testing.assert_array_equal(got, ref, err_msg=f"max pool {x.shape} k {k} pads {pd} strides {st} {dtype.__name__}")
+            if i % 5:
+                tol = 1e-5 if dtype == np.float32 else 2e-3
+                close(oc.pool(gpu, "avg", x, k, pd, st), oc.pool(cpu, "avg", x, k, pd, st), tol, tol)
+
+
+def test_products_random_shapes(gpu, cpu):
+    """Seeded sweeps of the 2-D product (every layout, alpha / beta, row and matrix C) and the batched product with
+    bias, residual and GELU over ragged shapes, fp32 and fp16, against the oracle."""
+    r = np.random.default_rng(78)
+    dims = [1, 2, 3, 5, 8, 17, 31, 32, 33, 64, 65, 100, 128, 130, 257]
+    for i in range(50):
+        M, K, N = (int(r.choice(dims)) for _ in range(3))
+        tA, tB = int(r.integers(0, 2)), int(r.integers(0, 2))
+        for dtype, tol in ((np.float32, (1e-4, 1e-4)), (np.float16, (4e-3, 8e-3))):
+            a = r.standard_normal((K, M) if tA else (M, K)).astype(dtype)
+            b = (r.standard_normal((N, K) if tB else (K, N)) / np.sqrt(K)).astype(dtype)
+            kw = [dict(), dict(alpha=0.5), dict(c=r.standard_normal((M, N)).astype(dtype), alpha=1.5, beta=0.5)][i % 3]
+            got, ref = oc.matmul2d(gpu, a, b, transA=tA, transB=tB, **kw), oc.matmul2d(cpu, a, b, transA=tA, transB=tB, **kw)
+            np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=tol[0], atol=tol[1],
+                                       err_msg=f"[{M},{K}]x[{K},{N}] transA {tA} transB {tB} {kw.keys()} {dtype.__name__}")
+    for i in range(40):
+        M, K, N = (int(r.choice(dims)) for _ in range(3))
+        batch = [(), (2,), (3, 2)][i % 3]
+        shared_b = i % 2 == 0
+        for dtype, tol in ((np.float32, (1e-4, 1e-4)), (np.float16, (1e-2, 1e-2))):
+            a = r.standard_normal(batch + (M, K)).astype(dtype)
+            b = (r.standard_normal((() if shared_b else batch) + (K, N)) / np.sqrt(K)).astype(dtype)
+            bias = r.standard_normal(N).astype(dtype)
+            z = r.standard_normal(batch + (M, N)).astype(dtype)
+            kw = [dict(), dict(z=z), dict(gelu=True), dict(z=z, gelu=True)][i % 4]
+            got, ref = oc.matmul_nd_bias(gpu, a, b, bias, **kw), oc.matmul_nd_bias(cpu, a, b, bias, **kw)
+            np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=tol[0], atol=tol[1],
+                                       err_msg=f"{a.shape} x {b.shape} {list(kw)} {dtype.__name__}")
+            got, ref = oc.matmul_nd(gpu, a, b), oc.matmul_nd(cpu, a, b)
+            np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=tol[0], atol=tol[1], err_msg=f"{a.shape} x {b.shape}")
+
+
 def test_conv_closed_forms(gpu):
     x = rng(1).standard_normal((1, 3, 8, 8)).astype(np.float32)
     w = np.zeros((3, 3, 3, 3), np.float32)
