@@ -6,7 +6,8 @@
 // generic kernel: a 64 x 64 tile of Out per workgroup, operands gathered
 // into LDS in runs of eight along their contiguous direction (strides are
 // runtime values; one 16-byte load per run where alignment allows), 32x32x16 MFMA,
-// fp32 accumulation, one rounding to fp16 at the end.
+// fp32 accumulation, one rounding to fp16 at the end; with few tiles and a
+// long reduction the reduction is split over workgroups.
 #include "gemm_f16.h"
 
 #include "conv_f16.h"
@@ -27,6 +28,9 @@ struct GemmF16Args {
   int act;
   float act_coef;
   bool a_vec, b_vec;                // the contiguous direction of A / B may be read eight elements (16 bytes) at a time
+  int steps_per_split;              // 64-k steps per workgroup along gridDim.y (the reduction split over workgroups)
+  float *partials;                  // the handle's scratch: one 64 x 64 fp32 tile per (tile, split)
+  unsigned *counters;               // ... and one arrival counter per tile, zero between kernels
 };
 
 constexpr int G_BK = 64, G_ROW = 72;  // k per step; halfs per LDS row (64 + 8 of padding)
@@ -36,6 +40,7 @@ constexpr int G_BK = 64, G_ROW = 72;  // k per step; halfs per LDS row (64 + 8 o
 __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args a) {
   __shared__ __attribute__((aligned(16))) _Float16 Ns[64 * G_ROW];  // [n][k]
   __shared__ __attribute__((aligned(16))) _Float16 Ms[64 * G_ROW];  // [m][k]
+  __shared__ unsigned arrived_before;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, half = lane >> 5;
   const int wn0 = (wave >> 1) * 32, wm0 = (wave & 1) * 32;
@@ -53,7 +58,8 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
   // A step is 64 rows x 64 k per operand = 512 runs of eight elements along the operand's contiguous direction;
   // a thread takes two runs of each operand.  Run r along k: row r / 8, k 8 (r % 8); along the row index: k r / 8,
   // rows 8 (r % 8) ...  A run is one 16-byte load where the operand allows it, eight 2-byte loads otherwise.
-  for (int k0 = 0; k0 < a.K; k0 += G_BK) {
+  const int k_begin = (int)blockIdx.y * a.steps_per_split * G_BK, k_end = min(a.K, k_begin + a.steps_per_split * G_BK);
+  for (int k0 = k_begin; k0 < k_end; k0 += G_BK) {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       const int r = tid + 256 * h;
@@ -109,6 +115,38 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
     }
     __syncthreads();
   }
+  // The reduction split over gridDim.y workgroups: each leaves its partial tile in the scratch and bumps the tile's
+  // arrival counter; whoever arrives last adds the partial tiles up in split order (the same bits whatever the order
+  // of arrival) and finishes the tile; nobody waits for anybody.  The hand-over is the one of the fp32 small-problem
+  // kernels (igemm_f32_small.hip): device-scope atomic stores of the partial tile, a wait until every one of the
+  // wavefront's stores is acknowledged, a barrier (all four wavefronts are there), then one device-scope atomic
+  // increment; the last arriver reads with device-scope atomic loads and puts the counter back to zero.
+  const int splits = (int)gridDim.y;
+  if (splits > 1) {
+    const unsigned tile = (unsigned)z * gridDim.x + blockIdx.x;
+    float *mine = a.partials + ((size_t)tile * splits + blockIdx.y) * 4096;
+#pragma unroll
+    for (int r = 0; r < 16; r++) __hip_atomic_store(&mine[r * 256 + tid], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __builtin_amdgcn_s_waitcnt(0);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    __syncthreads();
+    if (tid == 0) arrived_before = __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrived_before != (unsigned)splits - 1) return;
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    const float *all = a.partials + (size_t)tile * splits * 4096 + tid;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    for (int y = 0; y < splits; y++) {
+      float p[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) p[r] = __hip_atomic_load(all + (size_t)y * 4096 + r * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] += p[r];
+    }
+    if (tid == 0) __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   // register r of a lane: n = n0 + wn0 + 8 (r >> 2) + 4 half + (r & 3), m = m0 + wm0 + l32
   const int m = m0 + wm0 + l32;
   if (m >= a.M) return;
@@ -157,7 +195,18 @@ bool gemm_f16(const dnnrtContext *ctx, const __half *A, const __half *B, const _
   const int64_t a_other = transA ? g.a_sk : g.a_sm, b_other = transB ? g.b_sn : g.b_sk;
   g.a_vec = aligned16(A) && a_other % 8 == 0 && az % 8 == 0;
   g.b_vec = aligned16(B) && b_other % 8 == 0 && bz % 8 == 0;
-  hipLaunchKernelGGL(gemm_f16_generic_kernel, dim3((unsigned)tiles, 1, (unsigned)Z), dim3(256), 0, ctx->stream, g);
+  // Few tiles and a long reduction (a transformer's Linear layers at batch 1: 128 rows): the reduction is split over
+  // workgroups until the chip has one per CU, as far as the handle's scratch holds the partial tiles.
+  const int steps = (int)ceil_div(K, G_BK);
+  int splits = 1;
+  while (!ctx->splitk_shared && splits < 16 && tiles * Z * splits < ctx->num_cu && steps / (splits * 2) >= 2 &&
+         tiles * Z * splits * 2 * 16384 <= ctx->splitk_partial_bytes && tiles * Z <= ctx->splitk_max_tiles)
+    splits *= 2;
+  g.steps_per_split = (int)ceil_div(steps, splits);
+  splits = (int)ceil_div(steps, g.steps_per_split);
+  g.partials = ctx->splitk_partials;
+  g.counters = ctx->splitk_counters;
+  hipLaunchKernelGGL(gemm_f16_generic_kernel, dim3((unsigned)tiles, (unsigned)splits, (unsigned)Z), dim3(256), 0, ctx->stream, g);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { set_error("matmul(fp16): launch failed: %s", hipGetErrorString(e)); return false; }
   return true;

@@ -441,10 +441,16 @@ def test_matmul_nd(gpu, cpu):
     # fp16 tensors (fp32 accumulation, one rounding): the transformer shapes, broadcast batches, ragged tiles
     for sa, sb in [((1, 128, 768), (768, 768)), ((1, 12, 128, 64), (1, 12, 64, 128)), ((1, 12, 128, 128), (1, 12, 128, 64)),
                    ((4, 6), (6, 3)), ((2, 4, 6), (6, 3)), ((2, 3, 4, 6), (2, 3, 6, 5)), ((2, 4, 6), (2, 6, 3)), ((4, 6), (3, 6, 2)),
-                   ((2, 77, 130), (130, 70))]:
+                   ((2, 77, 130), (130, 70)),
+                   # few tiles and long reductions: split over 2 to 16 workgroups (odd step counts too), twice each
+                   # (the arrival counters must be back at zero)
+                   ((1, 128, 768), (768, 3072)), ((1, 128, 3072), (3072, 768)), ((1, 33, 1100), (1100, 100)), ((3, 64, 4000), (4000, 64))]:
         a = r.standard_normal(sa).astype(np.float16)
         b = (r.standard_normal(sb) / np.sqrt(sb[-2])).astype(np.float16)
-        np.testing.assert_allclose(oc.matmul_nd(gpu, a, b).astype(np.float32), oc.matmul_nd(cpu, a, b).astype(np.float32), rtol=2e-3, atol=2e-3)
+        ref = oc.matmul_nd(cpu, a, b).astype(np.float32)
+        first = oc.matmul_nd(gpu, a, b)
+        np.testing.assert_allclose(first.astype(np.float32), ref, rtol=2e-3, atol=2e-3)
+        np.testing.assert_array_equal(oc.matmul_nd(gpu, a, b), first)
 
 
 def test_split_reduction_hand_over_is_deterministic(gpu, cpu):
