@@ -735,28 +735,35 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       const bool dma_ok = dma_conv_applies(am);
       const int patch_cap = patch_conv_applies(am) ? patch_conv_capacity(am, 128) : 0;
       const bool one_per_cu = 5 * t128 >= 3 * cus && 4 * t128 < 5 * cus, fewer = 5 * t128 < 3 * cus;
-      // 3x3 stride-1 layers with at most about one 128x128 tile per CU (14x14 and 7x7 images at batch 64): the
+      // 3x3 stride-1 layers with up to two 128x128 tiles per CU (28x28, 14x14 and 7x7 images at batch 64): the
       // input patch stays in LDS (inside the network 33 -> 24 us on 256 -> 256 at 14x14, 41 -> 27 us on 512 -> 512
-      // at 7x7, where 64-row tiles give twice the workgroups); with more tiles per CU the im2col tiles are as fast
+      // at 7x7, where 64-row tiles give twice the workgroups); with more tiles per CU the im2col tiles are as fast.
       // Inside a network the filters come from HBM (activations pass through the caches in between), so the
-      // variants that keep three (128-row tiles) or six (64-row tiles) filter steps in flight are the ones
-      // chosen: 27 -> 25 us and 36 -> 26 us against two steps in flight.
+      // variants that keep four (128-row tiles) or six (64-row tiles) filter steps in flight are the ones
+      // chosen: 27 -> 25 us and 36 -> 26 us against two steps in flight.  With 128-row tiles the eight wavefronts
+      // split the tile (two rows by four columns of 64 x 32 blocks) rather than the reduction: no partial sums to
+      // hand over at the end (25 -> 22 us on 256 -> 256 at 14x14, 28.3 -> 26.5 us on 128 -> 128 at 28x28).
       // 64 -> 64 channels, 3x3, on images wide enough to fill the persistent kernel's two-row tiles and with several
       // tiles per workgroup: its filter stays in registers (inside the network 36 -> 27.5 us at 56x56, batch 64)
       const int64_t c64_tiles = (int64_t)a.N * ((a.H + 1) / 2) * ceil_div(a.K, 64);
       if (c64_conv_applies(am) && 2 * a.W >= 96 && c64_tiles >= 4 * cus) sel = 70;
-      else if (patch_cap && one_per_cu) sel = patch_cap == 256 ? 48 : 52;
+      else if (patch_cap && 5 * t128 >= 3 * cus && t128 < 2 * cus) sel = patch_cap == 256 ? 54 : 57;
       else if (patch_cap && fewer) sel = patch_cap == 256 ? 47 : 49;
       else if (nk <= 4) sel = 18;  // up to four steps (1x1 over up to 256 channels): the single-stage 64x64 variant
                               // (27 vs 34 us on 64 -> 256 at 56x56, 22.6 vs 26.6 on 128 -> 512 at 28x28, 18.3 vs 21.7 on 256 -> 1024 at 14x14)
       else if (a.K <= 64) sel = 4;
+      // From about one 128x128 tile per CU to two (14x14 layers and the long reductions of the 28x28 layers at
+      // batch 64): operands straight into a four-stage LDS ring, two steps in flight, on eight wavefronts: with
+      // two wavefronts per SIMD one computes while the other waits for its operands (inside the network, against
+      // the same ring on four wavefronts: 17.5 -> 14.8 us on 1x1 1024 -> 256 at 14x14, 29 -> 24 us on the strided
+      // 3x3 256 -> 256, 26 -> 24.5 us on 1x1 1024 -> 512; against the register-staged 128x128 tiles 29.5 -> 28.3 us
+      // on the 3x3 layers over 128 channels at 28x28).
+      else if (dma_ok && 5 * t128 >= 3 * cus && t128 < 2 * cus && (one_per_cu || nk >= 16)) sel = 64;
       else if (4 * t128 >= 5 * cus) sel = 3;
-      else if (one_per_cu) sel = dma_ok ? 33 : 12;  // operands straight into a four-stage LDS ring, two steps in flight
-                                                    // (inside the network 37 -> 30 us on the strided 3x3 256 -> 256,
-                                                    // 20 -> 18 us on 1x1 1024 -> 256 at 14x14)
-      else sel = dma_ok && nk >= 8 ? 62 : 4;  // fewer 128x128 tiles than that (7x7 layers at batch 64): 64-row tiles with a six-stage
-                     // ring, four steps of the filter in flight (strided 3x3 512 -> 512: 37.5 -> 32 us inside the
-                     // network, 1x1 2048 -> 512: 21 -> 18.7 us); short reductions keep the 64x64 tiles
+      else if (one_per_cu) sel = 12;
+      // Fewer 128x128 tiles than that (7x7 layers at batch 64): 64-row tiles on eight wavefronts (1x1 2048 -> 512:
+      // 20.5 -> 17 us inside the network, strided 3x3 512 -> 512: 35 -> 30 us); short reductions keep the 64x64 tiles.
+      else sel = dma_ok && nk >= 8 ? 66 : 4;
     }
     if ((sel >= 31 && sel <= 40) || (sel >= 60 && sel <= 69)) {
       if (!dma_conv_applies(am)) { set_error("conv(fp16): tile %d needs tensors below 2 GiB", sel); return false; }

@@ -456,6 +456,8 @@ static bool patch_variant(const dnnrtContext *ctx, const ConvF16Args &a, int var
     case 49: return launch_patch<64, 128, 1, 2, 4, 320, 8>(ctx, a, only_ask);
     case 51: return launch_patch<128, 128, 2, 2, 2, 256, 6>(ctx, a, only_ask);  // four (all of the LDS)
     case 52: return launch_patch<128, 128, 2, 2, 2, 320, 5>(ctx, a, only_ask);
+    case 54: return launch_patch<128, 128, 2, 4, 1, 256, 6>(ctx, a, only_ask);  // eight wavefronts over the tile, none over the reduction
+    case 57: return launch_patch<128, 128, 2, 4, 1, 320, 5>(ctx, a, only_ask);
     default: if (!only_ask) set_error("conv(fp16): no patch variant %d", variant); return false;
   }
 }

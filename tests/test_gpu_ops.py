@@ -1105,6 +1105,8 @@ F16_BATCH64_CASES = [
     (61, 128, 28, 28, 136, 3, 1, 1),   # ragged in pixels (47824 = 373.6 x 128) and in filters
     (64, 512, 7, 7, 512, 3, 1, 1),     # 7 x 7: few, deep tiles
     (64, 1024, 14, 14, 256, 1, 1, 0),  # sixteen steps
+    (64, 2048, 7, 7, 512, 1, 1, 0),    # 7 x 7, 1x1: 64-row tiles on eight wavefronts
+    (64, 512, 14, 14, 512, 3, 2, 1),   # the same, strided 3x3
 ]
 
 
