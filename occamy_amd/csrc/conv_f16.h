@@ -34,6 +34,11 @@ bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &l
 // Yp the pooled tensor N x PP x QQ x 64.  Fails with an error on any other shape.
 bool launch_conv_f16_stem_pool(const dnnrtContext *ctx, const ConvF16Args &a, __half *Yp, int PP, int QQ);
 
+// Channels-last 1x1 stride-1 layers over a multiple of 8 channels up to 256 (conv_f16_pointwise.hip): one wavefront
+// per 32 pixels, operands read from global memory in the MFMA's shape.
+bool pointwise_conv_applies(const ConvF16Args &a);
+bool launch_conv_f16_pointwise(const dnnrtContext *ctx, const ConvF16Args &a);
+
 // Channels-last convolutions whose operands are loaded straight into LDS (conv_f16_dma.hip): `variant` is one of
 // that file's tile ids, `a` must satisfy dma_conv_applies and carry the division constants.
 bool dma_conv_applies(const ConvF16Args &a);

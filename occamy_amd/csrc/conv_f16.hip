@@ -627,6 +627,78 @@ __global__ __launch_bounds__(256) void dwconv_f16_nhwc_kernel(const ConvF16Args 
   *reinterpret_cast<half8 *>(reinterpret_cast<_Float16 *>(a.Y) + off) = out;
 }
 
+// The 3x3 depthwise layers (stride 1 or 2) again, without LDS and without a barrier: the thread's 72 filter values
+// are nine 16-byte loads from the K x 3 x 3 filter as it lies in memory (eight filters are contiguous), the loops
+// over the taps are unrolled, and the thread index is taken apart with multiply-high divisions (the 64-bit
+// divisions of the kernel above cost more instructions than its arithmetic).  PIX neighbouring pixels of an output
+// row per thread share their input vectors; one pixel is what is compiled: with two and four the registers (153,
+// 177) leave too few wavefronts to hide the loads (MobileNetV2 at batch 64, 144 channels at 56 x 56: 71, 73 and
+// 89 us).  Taps are summed in the order of the kernel above; taps in the padding multiply a zero.
+template <int STRIDE, int PIX>
+__global__ __launch_bounds__(256) void dwconv3x3_f16_nhwc_kernel(const ConvF16Args a, const int total, const int qstrips, const unsigned magic_k8,
+                                                                 const unsigned magic_qs, const unsigned magic_p) {
+  const int i = (int)(blockIdx.x * 256 + threadIdx.x);
+  if (i >= total) return;
+  constexpr int COLS = 3 + (PIX - 1) * STRIDE;
+  const int K8 = a.K >> 3;
+  int t = div_magic(i, K8, magic_k8);
+  const int c8 = i - t * K8;
+  const int row = div_magic(t, qstrips, magic_qs);
+  const int q0 = PIX * (t - row * qstrips);
+  const int n = div_magic(row, a.P, magic_p), p = row - n * a.P;
+  const _Float16 *__restrict__ Wg = reinterpret_cast<const _Float16 *>(a.Wt) + (int64_t)c8 * 72;
+  half8 wraw[9];  // filter 8 c8 + e, tap t: element 9 e + t
+#pragma unroll
+  for (int j = 0; j < 9; j++) wraw[j] = *reinterpret_cast<const half8 *>(Wg + 8 * j);
+  const _Float16 *__restrict__ Xg = reinterpret_cast<const _Float16 *>(a.X) + (int64_t)n * a.H * a.W * a.C + 8 * c8;
+  const int ih0 = p * STRIDE - a.ph, iw0 = q0 * STRIDE - a.pw;
+  half8 zero8;
+#pragma unroll
+  for (int e = 0; e < 8; e++) zero8[e] = (_Float16)0.f;
+  float acc[PIX][8];
+#pragma unroll
+  for (int j = 0; j < PIX; j++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[j][e] = 0.f;
+#pragma unroll
+  for (int r = 0; r < 3; r++) {
+    const int ih = ih0 + r;
+    const bool row_ok = (unsigned)ih < (unsigned)a.H;
+    half8 xv[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; c++) {
+      const int iw = iw0 + c;
+      const bool ok = row_ok && (unsigned)iw < (unsigned)a.W;
+      xv[c] = ok ? *reinterpret_cast<const half8 *>(Xg + ((int64_t)ih * a.W + iw) * a.C) : zero8;
+    }
+#pragma unroll
+    for (int j = 0; j < PIX; j++)
+#pragma unroll
+      for (int s = 0; s < 3; s++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const int at = 9 * e + 3 * r + s;
+          acc[j][e] = fmaf((float)xv[j * STRIDE + s][e], (float)wraw[at >> 3][at & 7], acc[j][e]);
+        }
+  }
+  const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
+  const _Float16 *Zg = reinterpret_cast<const _Float16 *>(a.Z);  // may be Y itself: a thread reads an element, then writes it
+#pragma unroll
+  for (int j = 0; j < PIX; j++) {
+    if (q0 + j >= a.Q) break;
+    const int64_t off = ((((int64_t)n * a.P + p) * a.Q) + q0 + j) * a.K + 8 * c8;
+    half8 out;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      float v = acc[j][e];
+      if (biasg) v += (float)biasg[8 * c8 + e];
+      if (Zg) v = (float)(_Float16)v + (float)Zg[off + e];
+      out[e] = (_Float16)apply_act(v, a.act, a.act_coef);
+    }
+    *reinterpret_cast<half8 *>(reinterpret_cast<_Float16 *>(a.Y) + off) = out;
+  }
+}
+
 static bool dwconv_f16_applies(const ConvF16Args &a) {
   return a.format == DNNRT_NHWC && a.group > 1 && a.group == a.C && a.K == a.C && a.Cg == 1 && a.C % 8 == 0 &&
          (int64_t)a.K * a.R * a.S * 2 <= 48 * 1024 && aligned16(a.X) && aligned16(a.Y) && aligned16(a.Z);
@@ -811,9 +883,19 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
       default: LAUNCH_FAST(64, 64, 2, 2, 2, 2, 1, 0); break;
     }
 #undef LAUNCH_FAST
+  } else if (pointwise_conv_applies(a)) {
+    return launch_conv_f16_pointwise(ctx, a);
   } else if (dwconv_f16_applies(a)) {
     const int64_t total = NPQ * (a.K / 8), blocks = ceil_div(total, 256);
     if (blocks > INT32_MAX) { set_error("conv(fp16): depthwise output too large"); return false; }
+    if (a.R == 3 && a.S == 3 && a.sh == a.sw && (a.sh == 1 || a.sh == 2) && aligned16(a.Wt) && total + 256 < (1ll << 31)) {
+      const int qstrips = a.Q;  // one pixel per thread
+      const int64_t threads = (int64_t)a.N * a.P * qstrips * (a.K / 8);
+      const unsigned grid = (unsigned)ceil_div(threads, 256);
+      const unsigned m_k8 = magic_of(a.K / 8), m_qs = magic_of(qstrips), m_p = magic_of(a.P);
+      if (a.sh == 1) hipLaunchKernelGGL((dwconv3x3_f16_nhwc_kernel<1, 1>), dim3(grid), dim3(256), 0, ctx->stream, a, (int)threads, qstrips, m_k8, m_qs, m_p);
+      else hipLaunchKernelGGL((dwconv3x3_f16_nhwc_kernel<2, 1>), dim3(grid), dim3(256), 0, ctx->stream, a, (int)threads, qstrips, m_k8, m_qs, m_p);
+    } else
     hipLaunchKernelGGL(dwconv_f16_nhwc_kernel, dim3((unsigned)blocks), dim3(256), (size_t)a.K * a.R * a.S * 2, ctx->stream, a, total);
   } else {
     const int Kg = a.K / a.group;

@@ -59,61 +59,87 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
   // a thread takes two runs of each operand.  Run r along k: row r / 8, k 8 (r % 8); along the row index: k r / 8,
   // rows 8 (r % 8) ...  A run is one 16-byte load where the operand allows it, eight 2-byte loads otherwise.
   const int k_begin = (int)blockIdx.y * a.steps_per_split * G_BK, k_end = min(a.K, k_begin + a.steps_per_split * G_BK);
-  for (int k0 = k_begin; k0 < k_end; k0 += G_BK) {
+  // Four steps of operands are requested ahead, in registers: a workgroup of a split reduction has a handful of
+  // steps, so all of its loads are in flight before the first one is used.
+  constexpr int AHEAD = 4;
+  g_half8 ra[AHEAD][2], rb[AHEAD][2];
+  auto request = [&](g_half8 (&va)[2], g_half8 (&vb)[2], const int k0) {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       const int r = tid + 256 * h;
-      {  // A side -> Ms[m][k]
+      {  // A side
         const int row0 = a_k_fast ? r >> 3 : (r & 7) << 3, kk0 = a_k_fast ? (r & 7) << 3 : r >> 3;
         const int64_t at = (int64_t)(m0 + row0) * a.a_sm + (int64_t)(k0 + kk0) * a.a_sk;
-        g_half8 v;
         const bool whole = a_k_fast ? (m0 + row0 < a.M && k0 + kk0 + 8 <= a.K) : (m0 + row0 + 8 <= a.M && k0 + kk0 < a.K);
         if (a.a_vec && whole) {
-          v = *reinterpret_cast<const g_half8 *>(Ag + at);
+          va[h] = *reinterpret_cast<const g_half8 *>(Ag + at);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; e++) {
             const int gm = m0 + row0 + (a_k_fast ? 0 : e), gk = k0 + kk0 + (a_k_fast ? e : 0);
-            v[e] = (gm < a.M && gk < a.K) ? Ag[(int64_t)gm * a.a_sm + (int64_t)gk * a.a_sk] : (_Float16)0.f;
+            va[h][e] = (gm < a.M && gk < a.K) ? Ag[(int64_t)gm * a.a_sm + (int64_t)gk * a.a_sk] : (_Float16)0.f;
           }
         }
-        if (a_k_fast) {
-          *reinterpret_cast<g_half8 *>(Ms + row0 * G_ROW + kk0) = v;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; e++) Ms[(row0 + e) * G_ROW + kk0] = v[e];
-        }
       }
-      {  // B side -> Ns[n][k]
+      {  // B side
         const int row0 = b_k_fast ? r >> 3 : (r & 7) << 3, kk0 = b_k_fast ? (r & 7) << 3 : r >> 3;
         const int64_t at = (int64_t)(k0 + kk0) * a.b_sk + (int64_t)(n0 + row0) * a.b_sn;
-        g_half8 v;
         const bool whole = b_k_fast ? (n0 + row0 < a.N && k0 + kk0 + 8 <= a.K) : (n0 + row0 + 8 <= a.N && k0 + kk0 < a.K);
         if (a.b_vec && whole) {
-          v = *reinterpret_cast<const g_half8 *>(Bg + at);
+          vb[h] = *reinterpret_cast<const g_half8 *>(Bg + at);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; e++) {
             const int gn = n0 + row0 + (b_k_fast ? 0 : e), gk = k0 + kk0 + (b_k_fast ? e : 0);
-            v[e] = (gn < a.N && gk < a.K) ? Bg[(int64_t)gk * a.b_sk + (int64_t)gn * a.b_sn] : (_Float16)0.f;
+            vb[h][e] = (gn < a.N && gk < a.K) ? Bg[(int64_t)gk * a.b_sk + (int64_t)gn * a.b_sn] : (_Float16)0.f;
           }
-        }
-        if (b_k_fast) {
-          *reinterpret_cast<g_half8 *>(Ns + row0 * G_ROW + kk0) = v;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; e++) Ns[(row0 + e) * G_ROW + kk0] = v[e];
         }
       }
     }
-    __syncthreads();
+  };
+  auto to_lds = [&](const g_half8 (&va)[2], const g_half8 (&vb)[2]) {
 #pragma unroll
-    for (int ks = 0; ks < G_BK; ks += 16) {
-      const g_half8 nv = *reinterpret_cast<const g_half8 *>(Ns + (wn0 + l32) * G_ROW + ks + half * 8);
-      const g_half8 mv = *reinterpret_cast<const g_half8 *>(Ms + (wm0 + l32) * G_ROW + ks + half * 8);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(nv, mv, acc, 0, 0, 0);
+    for (int h = 0; h < 2; h++) {
+      const int r = tid + 256 * h;
+      {  // -> Ms[m][k]
+        const int row0 = a_k_fast ? r >> 3 : (r & 7) << 3, kk0 = a_k_fast ? (r & 7) << 3 : r >> 3;
+        if (a_k_fast) {
+          *reinterpret_cast<g_half8 *>(Ms + row0 * G_ROW + kk0) = va[h];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) Ms[(row0 + e) * G_ROW + kk0] = va[h][e];
+        }
+      }
+      {  // -> Ns[n][k]
+        const int row0 = b_k_fast ? r >> 3 : (r & 7) << 3, kk0 = b_k_fast ? (r & 7) << 3 : r >> 3;
+        if (b_k_fast) {
+          *reinterpret_cast<g_half8 *>(Ns + row0 * G_ROW + kk0) = vb[h];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; e++) Ns[(row0 + e) * G_ROW + kk0] = vb[h][e];
+        }
+      }
     }
-    __syncthreads();
+  };
+#pragma unroll
+  for (int s = 0; s < AHEAD; s++)
+    if (k_begin + s * G_BK < k_end) request(ra[s], rb[s], k_begin + s * G_BK);
+  for (int k0 = k_begin; k0 < k_end; k0 += AHEAD * G_BK) {
+#pragma unroll
+    for (int s = 0; s < AHEAD; s++) {
+      const int ks0 = k0 + s * G_BK;
+      if (ks0 >= k_end) break;  // the same for every thread
+      to_lds(ra[s], rb[s]);
+      __syncthreads();
+      if (ks0 + AHEAD * G_BK < k_end) request(ra[s], rb[s], ks0 + AHEAD * G_BK);
+#pragma unroll
+      for (int ks = 0; ks < G_BK; ks += 16) {
+        const g_half8 nv = *reinterpret_cast<const g_half8 *>(Ns + (wn0 + l32) * G_ROW + ks + half * 8);
+        const g_half8 mv = *reinterpret_cast<const g_half8 *>(Ms + (wm0 + l32) * G_ROW + ks + half * 8);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(nv, mv, acc, 0, 0, 0);
+      }
+      __syncthreads();
+    }
   }
   // The reduction split over gridDim.y workgroups: each leaves its partial tile in the scratch and bumps the tile's
   // arrival counter; whoever arrives last adds the partial tiles up in split order (the same bits whatever the order
@@ -138,12 +164,21 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
     const float *all = a.partials + (size_t)tile * splits * 4096 + tid;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    for (int y = 0; y < splits; y++) {
-      float p[16];
+    for (int y0 = 0; y0 < splits; y0 += 4) {  // four partial tiles requested at a time, added in split order
+      float p[4][16];
 #pragma unroll
-      for (int r = 0; r < 16; r++) p[r] = __hip_atomic_load(all + (size_t)y * 4096 + r * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int j = 0; j < 4; j++)
+        if (y0 + j < splits) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[r] += p[r];
+          for (int r = 0; r < 16; r++)
+            p[j][r] = __hip_atomic_load(all + (size_t)(y0 + j) * 4096 + r * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (y0 + j < splits) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[r] += p[j][r];
+        }
     }
     if (tid == 0) __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -196,14 +231,19 @@ bool gemm_f16(const dnnrtContext *ctx, const __half *A, const __half *B, const _
   g.a_vec = aligned16(A) && a_other % 8 == 0 && az % 8 == 0;
   g.b_vec = aligned16(B) && b_other % 8 == 0 && bz % 8 == 0;
   // Few tiles and a long reduction (a transformer's Linear layers at batch 1: 128 rows): the reduction is split over
-  // workgroups until the chip has one per CU, as far as the handle's scratch holds the partial tiles.
+  // workgroups up to about 1.75 workgroups per CU (two on a CU run out of step and fill each other's waits), as
+  // far as the handle's scratch holds the partial tiles.
   const int steps = (int)ceil_div(K, G_BK);
-  int splits = 1;
-  while (!ctx->splitk_shared && splits < 16 && tiles * Z * splits < ctx->num_cu && steps / (splits * 2) >= 2 &&
-         tiles * Z * splits * 2 * 16384 <= ctx->splitk_partial_bytes && tiles * Z <= ctx->splitk_max_tiles)
-    splits *= 2;
+  int64_t splits = 1;
+  const int64_t want = 7 * (int64_t)ctx->num_cu / 4, have = tiles * Z;
+  if (!ctx->splitk_shared && have < want && have <= ctx->splitk_max_tiles) {
+    splits = (want + have / 2) / have;
+    splits = splits > 16 ? 16 : splits;
+    splits = splits > steps ? steps : splits;
+    while (splits > 1 && have * splits * 16384 > (int64_t)ctx->splitk_partial_bytes) splits--;  // 64 x 64 fp32 per tile and split
+  }
   g.steps_per_split = (int)ceil_div(steps, splits);
-  splits = (int)ceil_div(steps, g.steps_per_split);
+  splits = ceil_div(steps, g.steps_per_split);  // no empty split: every arrival carries a partial tile
   g.partials = ctx->splitk_partials;
   g.counters = ctx->splitk_counters;
   hipLaunchKernelGGL(gemm_f16_generic_kernel, dim3((unsigned)tiles, (unsigned)splits, (unsigned)Z), dim3(256), 0, ctx->stream, g);

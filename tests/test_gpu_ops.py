@@ -767,6 +767,15 @@ F16_CASES = [
     (2, 3, 45, 37, 64, 7, 2, 3),       # first-layer kernel, ragged tiles (23 x 19 output pixels)
     (1, 3, 224, 224, 64, 7, 2, 3),     # the ResNet first layer at full size
     (1, 20, 9, 9, 24, 3, 1, 1),        # generic path: C % 32 != 0
+    # channels-last 1x1 layers over a multiple of 8 channels that is not one of 64: one wavefront per 32 pixels
+    (2, 16, 20, 20, 96, 1, 1, 0),      # one 16-channel step
+    (3, 24, 9, 11, 144, 1, 1, 0),      # half of the second step is past the channels; 297 pixels: a ragged last wavefront
+    (2, 144, 7, 9, 24, 1, 1, 0),       # nine steps, fewer filters than a block
+    (1, 160, 7, 7, 960, 1, 1, 0),      # 49 pixels: the filter blocks are dealt over the grid
+    (5, 8, 3, 3, 8, 1, 1, 0),          # the smallest
+    (1, 248, 6, 5, 40, 1, 1, 0),       # sixteen steps, the last one half empty
+    (1, 200, 9, 9, 72, 1, 1, 0),
+    (8, 24, 56, 56, 144, 1, 1, 0),     # a MobileNetV2 expansion layer
 ]
 
 
