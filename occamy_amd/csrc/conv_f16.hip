@@ -669,7 +669,10 @@ __global__ __launch_bounds__(256) void dwconv3x3_f16_nhwc_kernel(const ConvF16Ar
     for (int c = 0; c < COLS; c++) {
       const int iw = iw0 + c;
       const bool ok = row_ok && (unsigned)iw < (unsigned)a.W;
-      xv[c] = ok ? *reinterpret_cast<const half8 *>(Xg + ((int64_t)ih * a.W + iw) * a.C) : zero8;
+      // unconditional, from a clamped address: a load under a branch is waited for before the next one is issued
+      const int ihc = min(max(ih, 0), a.H - 1), iwc = min(max(iw, 0), a.W - 1);
+      const half8 v = *reinterpret_cast<const half8 *>(Xg + ((int64_t)ihc * a.W + iwc) * a.C);
+      xv[c] = ok ? v : zero8;
     }
 #pragma unroll
     for (int j = 0; j < PIX; j++)

@@ -49,15 +49,19 @@ __global__ __launch_bounds__(256) void conv1x1_f16_pointwise_kernel(const ConvF1
   pw_half8 xf[STEPS];
 #pragma unroll
   for (int s = 0; s < STEPS; s++) {
+    // loads are unconditional, from clamped addresses (a load under a branch is waited for before the next one
+    // is issued); what must not contribute is replaced by zeros afterwards
     const int ch = (2 * s + half) * 8;
-    xf[s] = (pix_ok && ch < a.C) ? *reinterpret_cast<const pw_half8 *>(Xg + pix * a.C + ch) : zero8;
+    const pw_half8 v = *reinterpret_cast<const pw_half8 *>(Xg + (pix_ok ? pix : (int64_t)npq - 1) * a.C + (ch < a.C ? ch : 0));
+    xf[s] = (pix_ok && ch < a.C) ? v : zero8;
   }
   auto filter_block = [&](pw_half8 (&wf)[STEPS], const int kb) {
     const int krow = kb * 32 + l32;
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
       const int ch = (2 * s + half) * 8;
-      wf[s] = (krow < a.K && ch < a.C) ? *reinterpret_cast<const pw_half8 *>(Wg + (int64_t)krow * a.C + ch) : zero8;
+      const pw_half8 v = *reinterpret_cast<const pw_half8 *>(Wg + (int64_t)min(krow, a.K - 1) * a.C + (ch < a.C ? ch : 0));
+      wf[s] = (krow < a.K && ch < a.C) ? v : zero8;
     }
   };
   // Results leave through a staging tile of the wavefront's own (32 pixels x up to four filter blocks, fp16): the
