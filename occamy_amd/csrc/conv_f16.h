@@ -2,7 +2,22 @@
 #pragma once
 #include "common.h"
 
+#include <type_traits>
+
 namespace dnnrt {
+
+// f(std::integral_constant<int, mode>{}) for the activation mode `act` names: a kernel's epilogue loop is compiled
+// once per mode and picked once, instead of asking for the mode per value.
+template <typename F>
+__device__ __forceinline__ void by_act_mode(int act, F &&f) {
+  switch (act) {
+    case DNNRT_ACT_RELU: f(std::integral_constant<int, DNNRT_ACT_RELU>{}); break;
+    case DNNRT_ACT_CLIPPED_RELU: f(std::integral_constant<int, DNNRT_ACT_CLIPPED_RELU>{}); break;
+    case DNNRT_ACT_LEAKY_RELU: f(std::integral_constant<int, DNNRT_ACT_LEAKY_RELU>{}); break;
+    case ACT_GELU: f(std::integral_constant<int, ACT_GELU>{}); break;
+    default: f(std::integral_constant<int, DNNRT_ACT_IDENTITY>{}); break;
+  }
+}
 
 struct ConvF16Args {
   const __half *X, *Wt, *bias;

@@ -633,9 +633,10 @@ __global__ __launch_bounds__(256) void dwconv_f16_nhwc_kernel(const ConvF16Args 
 // divisions of the kernel above cost more instructions than its arithmetic).  PIX neighbouring pixels of an output
 // row per thread share their input vectors; one pixel is what is compiled: with two and four the registers (153,
 // 177) leave too few wavefronts to hide the loads (MobileNetV2 at batch 64, 144 channels at 56 x 56: 71, 73 and
-// 89 us).  Taps are summed in the order of the kernel above; taps in the padding multiply a zero.
+// 89 us).  Compiled for six wavefronts per SIMD (80 registers): 68 us against 72 with five, 90 with eight, which
+// spills.  Taps are summed in the order of the kernel above; taps in the padding multiply a zero.
 template <int STRIDE, int PIX>
-__global__ __launch_bounds__(256) void dwconv3x3_f16_nhwc_kernel(const ConvF16Args a, const int total, const int qstrips, const unsigned magic_k8,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void dwconv3x3_f16_nhwc_kernel(const ConvF16Args a, const int total, const int qstrips, const unsigned magic_k8,
                                                                  const unsigned magic_qs, const unsigned magic_p) {
   const int i = (int)(blockIdx.x * 256 + threadIdx.x);
   if (i >= total) return;
@@ -686,20 +687,27 @@ __global__ __launch_bounds__(256) void dwconv3x3_f16_nhwc_kernel(const ConvF16Ar
   }
   const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
   const _Float16 *Zg = reinterpret_cast<const _Float16 *>(a.Z);  // may be Y itself: a thread reads an element, then writes it
+  auto finish = [&](auto mode_c) {  // one copy per activation mode, picked once
+    constexpr int MODE = decltype(mode_c)::value;
+    float bias8[8];
 #pragma unroll
-  for (int j = 0; j < PIX; j++) {
-    if (q0 + j >= a.Q) break;
-    const int64_t off = ((((int64_t)n * a.P + p) * a.Q) + q0 + j) * a.K + 8 * c8;
-    half8 out;
+    for (int e = 0; e < 8; e++) bias8[e] = biasg ? (float)biasg[8 * c8 + e] : 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-      float v = acc[j][e];
-      if (biasg) v += (float)biasg[8 * c8 + e];
-      if (Zg) v = (float)(_Float16)v + (float)Zg[off + e];
-      out[e] = (_Float16)apply_act(v, a.act, a.act_coef);
+    for (int j = 0; j < PIX; j++) {
+      if (q0 + j >= a.Q) break;
+      const int64_t off = ((((int64_t)n * a.P + p) * a.Q) + q0 + j) * a.K + 8 * c8;
+      half8 z8, out;
+      if (Zg) z8 = *reinterpret_cast<const half8 *>(Zg + off);
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float v = acc[j][e] + bias8[e];
+        if (Zg) v = (float)(_Float16)v + (float)z8[e];
+        out[e] = (_Float16)apply_act(v, MODE, a.act_coef);
+      }
+      *reinterpret_cast<half8 *>(reinterpret_cast<_Float16 *>(a.Y) + off) = out;
     }
-    *reinterpret_cast<half8 *>(reinterpret_cast<_Float16 *>(a.Y) + off) = out;
-  }
+  };
+  by_act_mode(a.act, finish);
 }
 
 static bool dwconv_f16_applies(const ConvF16Args &a) {

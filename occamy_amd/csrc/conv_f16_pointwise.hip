@@ -87,24 +87,29 @@ __global__ __launch_bounds__(256) void conv1x1_f16_pointwise_kernel(const ConvF1
       for (int s = 0; s < STEPS; s++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[s], xf[s], acc, 0, 0, 0);
       // acc[4 g + i]: filter 32 kb + 8 g + 4 half + i of pixel l32.  With a residual the tile holds the rounded
       // sum of product and bias, the rest follows when the tile is read back; without, the finished value.
+      // one copy of the loop per activation mode, picked once: the mode is the same for every lane
+      auto finish_block = [&](auto mode_c) {
+        constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int kk = kb * 32 + 8 * g + 4 * half;
-        pw_half4 b4, z4, o4;
-        const bool k_ok = kk < a.K;  // K is a multiple of four: a run of four is inside or outside as a whole
-        const int64_t at = pix * a.K + kk;
-        if (biasg && k_ok) b4 = *reinterpret_cast<const pw_half4 *>(biasg + kk);
-        if (!STAGED && Zg && k_ok && pix_ok) z4 = *reinterpret_cast<const pw_half4 *>(Zg + at);
+        for (int g = 0; g < 4; g++) {
+          const int kk = kb * 32 + 8 * g + 4 * half;
+          pw_half4 b4, z4, o4;
+          const bool k_ok = kk < a.K;  // K is a multiple of four: a run of four is inside or outside as a whole
+          const int64_t at = pix * a.K + kk;
+          if (biasg && k_ok) b4 = *reinterpret_cast<const pw_half4 *>(biasg + kk);
+          if (!STAGED && Zg && k_ok && pix_ok) z4 = *reinterpret_cast<const pw_half4 *>(Zg + at);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          float v = acc[4 * g + i];
-          if (biasg && k_ok) v += (float)b4[i];
-          if (!STAGED && Zg && k_ok && pix_ok) v = (float)(_Float16)v + (float)z4[i];
-          o4[i] = (_Float16)((STAGED && Zg) ? v : apply_act(v, a.act, a.act_coef));
+          for (int i = 0; i < 4; i++) {
+            float v = acc[4 * g + i];
+            if (biasg && k_ok) v += (float)b4[i];
+            if (!STAGED && Zg && k_ok && pix_ok) v = (float)(_Float16)v + (float)z4[i];
+            o4[i] = (_Float16)((STAGED && Zg) ? v : apply_act(v, MODE, a.act_coef));
+          }
+          if (STAGED) *reinterpret_cast<pw_half4 *>(stage + l32 * PW_STAGE_ROW + j * 32 + 8 * g + 4 * half) = o4;
+          else if (k_ok && pix_ok) *reinterpret_cast<pw_half4 *>(Yg + at) = o4;
         }
-        if (STAGED) *reinterpret_cast<pw_half4 *>(stage + l32 * PW_STAGE_ROW + j * 32 + 8 * g + 4 * half) = o4;
-        else if (k_ok && pix_ok) *reinterpret_cast<pw_half4 *>(Yg + at) = o4;
-      }
+      };
+      by_act_mode(a.act, finish_block);
 #pragma unroll
       for (int s = 0; s < STEPS; s++) wf[s] = wn[s];
     }
@@ -115,20 +120,25 @@ __global__ __launch_bounds__(256) void conv1x1_f16_pointwise_kernel(const ConvF1
     __builtin_amdgcn_wave_barrier();
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
     const int parts = 4 * nb;  // 16-byte parts of a pixel's row in the tile
-    for (int i = lane; i < 32 * parts; i += 64) {
-      const int prow = i / parts, part = i - prow * parts;
-      const int kk = kc * 32 + 8 * part;
-      if (p0 + prow < npq && kk < a.K) {  // K is a multiple of eight
-        const int64_t at = (p0 + prow) * a.K + kk;
-        pw_half8 v8 = *reinterpret_cast<const pw_half8 *>(stage + prow * PW_STAGE_ROW + 8 * part);
-        if (Zg) {
-          const pw_half8 z8 = *reinterpret_cast<const pw_half8 *>(Zg + at);
+    const unsigned by_parts = nb == 1 ? 16384u : nb == 2 ? 8192u : nb == 3 ? 5462u : 4096u;  // ceil(2^16 / parts): i / parts for i < 512
+    auto finish_tile = [&](auto mode_c) {
+      constexpr int MODE = decltype(mode_c)::value;
+      for (int i = lane; i < 32 * parts; i += 64) {
+        const int prow = (int)(((unsigned)i * by_parts) >> 16), part = i - prow * parts;
+        const int kk = kc * 32 + 8 * part;
+        if (p0 + prow < npq && kk < a.K) {  // K is a multiple of eight
+          const int64_t at = (p0 + prow) * a.K + kk;
+          pw_half8 v8 = *reinterpret_cast<const pw_half8 *>(stage + prow * PW_STAGE_ROW + 8 * part);
+          if (Zg) {
+            const pw_half8 z8 = *reinterpret_cast<const pw_half8 *>(Zg + at);
 #pragma unroll
-          for (int e = 0; e < 8; e++) v8[e] = (_Float16)apply_act((float)v8[e] + (float)z8[e], a.act, a.act_coef);
+            for (int e = 0; e < 8; e++) v8[e] = (_Float16)apply_act((float)v8[e] + (float)z8[e], MODE, a.act_coef);
+          }
+          *reinterpret_cast<pw_half8 *>(Yg + at) = v8;
         }
-        *reinterpret_cast<pw_half8 *>(Yg + at) = v8;
       }
-    }
+    };
+    by_act_mode(a.act, finish_tile);
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_wave_barrier();
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
