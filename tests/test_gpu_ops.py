@@ -168,6 +168,47 @@ def test_conv_f16_random_shapes(gpu, cpu):
                                       err_msg=what + " in place")
 
 
+def test_conv_f16_pointwise_and_depthwise_random_shapes(gpu, cpu):
+    """Seeded channels-last fp16 shapes aimed at the two kernels without a workgroup tile: 1x1 stride-1 layers over
+    a multiple of 8 channels up to 256 that is not a multiple of 64 (one to sixteen 16-channel steps, the last one
+    half empty every other time; few and many filters, so that results leave both through the staging tile and
+    straight from the accumulators; ragged last wavefronts; few pixels, so that the filter blocks are dealt over the
+    grid) and 3x3 depthwise layers with stride 1 and 2 and padding 0 to 2; each activation mode in turn, with and
+    without a residual, which is also written in place.  Against the oracle to one fp16 rounding."""
+    r = np.random.default_rng(909)
+    acts = [(_abi.ACT_RELU, None), (_abi.ACT_IDENTITY, None), (_abi.ACT_CLIPPED_RELU, 0.7), (_abi.ACT_LEAKY_RELU, 0.1)]
+    for i in range(60):
+        N, H, W = int(r.integers(1, 5)), int(r.integers(1, 25)), int(r.integers(1, 25))
+        if i % 2 == 0:  # pointwise
+            C = 8 * int(r.integers(1, 33))
+            if C % 64 == 0:
+                C += 8
+            K = 8 * int(r.choice([1, 2, 3, 4, 5, 8, 9, 12, 18, 40]))
+            R, st, pd, grp = 1, 1, 0, 1
+        else:           # depthwise
+            C = K = 8 * int(r.integers(1, 40))
+            R, st, pd, grp = 3, int(r.integers(1, 3)), int(r.integers(0, 3)), C
+            if H + 2 * pd < 3 or W + 2 * pd < 3:
+                H, W = H + 3, W + 3
+        activ, coef = acts[(i // 2) % 4]
+        q = rng(5000 + i)
+        x = q.standard_normal((N, C, H, W)).astype(np.float16)
+        w = (q.standard_normal((K, C // grp, R, R)) * np.sqrt(2.0 / (C // grp * R * R))).astype(np.float16)
+        b = q.uniform(-0.3, 0.3, K).astype(np.float16)
+        what = f"case {i}: x {x.shape} w {w.shape} stride {st} pad {pd} group {grp} act {activ}"
+        if coef is not None:
+            gpu.ops.set_activation_coef(coef)
+        ref = oc.conv(cpu, x, w, b, (pd, pd), (st, st), grp, activ, coef=coef)
+        got = conv_f16(gpu, x, w, b, (pd, pd), (st, st), grp, activ, _abi.NHWC)
+        np.testing.assert_allclose(got.astype(np.float32), ref.astype(np.float32), rtol=2e-3, atol=2e-3, err_msg=what)
+        z = q.standard_normal(ref.shape).astype(np.float16)
+        refz = oc.conv(cpu, x, w, b, (pd, pd), (st, st), grp, activ, z=z, coef=coef)
+        gotz = conv_f16(gpu, x, w, b, (pd, pd), (st, st), grp, activ, _abi.NHWC, z=z)
+        np.testing.assert_allclose(gotz.astype(np.float32), refz.astype(np.float32), rtol=4e-3, atol=4e-3, err_msg=what + " + z")
+        np.testing.assert_array_equal(conv_f16(gpu, x, w, b, (pd, pd), (st, st), grp, activ, _abi.NHWC, z=z, inplace=True), gotz,
+                                      err_msg=what + " in place")
+
+
 def test_rowwise_ops_random_shapes(gpu, cpu):
     """Seeded sweeps of soft-max, LayerNorm, ReduceMean and the poolings over shapes around their kernels'
     boundaries (row lengths on both sides of 4-element groups, of the in-register limit and of a wavefront;
