@@ -45,6 +45,9 @@ constexpr int FEWPIX_MAX_PIXELS = 64;
 bool launch_conv_f16_fewpix(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 // The 3-channel 7x7 stride-2 first layer (NCHW in, NHWC out); `launched` says whether it took the problem.
 bool launch_conv_f16_stem(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
+// Other first layers (conv_f16_first.hip): N,C,H,W input of at most four channels, a filter of at most 3x3, 16 to 64
+// filters, channels-last output; `launched` says whether it took the problem.
+bool launch_conv_f16_first(const dnnrtContext *ctx, const ConvF16Args &a, bool &launched);
 // The same layer with the 3x3 stride-2 pad-1 max-pool behind it in one kernel: `a` is the convolution (a.Y unused),
 // Yp the pooled tensor N x PP x QQ x 64.  Fails with an error on any other shape.
 bool launch_conv_f16_stem_pool(const dnnrtContext *ctx, const ConvF16Args &a, __half *Yp, int PP, int QQ);

@@ -763,6 +763,9 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
   bool stem_launched = false;
   if (!launch_conv_f16_stem(ctx, a, stem_launched)) return false;
   if (stem_launched) return true;
+  bool first_launched = false;
+  if (!launch_conv_f16_first(ctx, a, first_launched)) return false;
+  if (first_launched) return true;
   bool few_launched = false;
   if (!launch_conv_f16_fewpix(ctx, a, few_launched)) return false;
   if (few_launched) return true;

@@ -817,6 +817,13 @@ F16_CASES = [
     (1, 248, 6, 5, 40, 1, 1, 0),       # sixteen steps, the last one half empty
     (1, 200, 9, 9, 72, 1, 1, 0),
     (8, 24, 56, 56, 144, 1, 1, 0),     # a MobileNetV2 expansion layer
+    # first layers other than the 7x7 one (N,C,H,W in, channels-last out): a thread per output pixel
+    (2, 3, 33, 30, 32, 3, 2, 1),       # MobileNetV2's, on a ragged image
+    (1, 3, 224, 224, 32, 3, 2, 1),     # ... at full size
+    (2, 3, 20, 17, 64, 3, 1, 1),       # a VGG's
+    (3, 1, 12, 12, 16, 3, 1, 0),       # one channel, no padding
+    (2, 4, 9, 9, 24, 1, 1, 0),         # four channels, 1x1
+    (1, 2, 10, 11, 48, 2, 2, 1),       # 2x2 filter
 ]
 
 
