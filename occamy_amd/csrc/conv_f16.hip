@@ -629,14 +629,18 @@ __global__ __launch_bounds__(256) void dwconv_f16_nhwc_kernel(const ConvF16Args 
 
 // The 3x3 depthwise layers (stride 1 or 2) again, without LDS and without a barrier: the thread's 72 filter values
 // are nine 16-byte loads from the K x 3 x 3 filter as it lies in memory (eight filters are contiguous), the loops
-// over the taps are unrolled, and the thread index is taken apart with multiply-high divisions (the 64-bit
-// divisions of the kernel above cost more instructions than its arithmetic).  PIX neighbouring pixels of an output
-// row per thread share their input vectors; one pixel is what is compiled: with two and four the registers (153,
-// 177) leave too few wavefronts to hide the loads (MobileNetV2 at batch 64, 144 channels at 56 x 56: 71, 73 and
-// 89 us).  Compiled for six wavefronts per SIMD (80 registers): 68 us against 72 with five, 90 with eight, which
-// spills.  Taps are summed in the order of the kernel above; taps in the padding multiply a zero.
-template <int STRIDE, int PIX>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void dwconv3x3_f16_nhwc_kernel(const ConvF16Args a, const int total, const int qstrips, const unsigned magic_k8,
+// over the taps are unrolled, and the thread index is taken apart with multiply-high divisions.  A thread computes
+// PIX neighbouring pixels of an output row, which share their input vectors: 3 x (PIX - 1) x STRIDE + 9 loads
+// instead of 9 PIX (the kernel is bound by the requests it sends to L2, not by its arithmetic: without the FMAs
+// it runs 13 % faster, no more).  Every load is unconditional, from a clamped address, and a tap in the padding
+// has its value replaced by zero: a load under a divergent branch is waited for before the next one is issued,
+// which with more than one pixel per thread costs more than the shared loads give.  WAVES: the wavefronts per
+// SIMD the register allocation aims at.  MobileNetV2 at batch 64, 144 channels at 56 x 56, stride 1: 65 us with
+// one pixel per thread (six wavefronts), 54 with two (five), 49 with three (four), 45.5 with four (four; 47.8 at
+// three); the stride-2 layers gain less and run with two pixels (four wavefronts).  Taps are summed in the order
+// of the kernel above.
+template <int STRIDE, int PIX, int WAVES>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WAVES, WAVES))) void dwconv3x3_f16_nhwc_kernel(const ConvF16Args a, const int total, const int qstrips, const unsigned magic_k8,
                                                                  const unsigned magic_qs, const unsigned magic_p) {
   const int i = (int)(blockIdx.x * 256 + threadIdx.x);
   if (i >= total) return;
@@ -903,12 +907,15 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     const int64_t total = NPQ * (a.K / 8), blocks = ceil_div(total, 256);
     if (blocks > INT32_MAX) { set_error("conv(fp16): depthwise output too large"); return false; }
     if (a.R == 3 && a.S == 3 && a.sh == a.sw && (a.sh == 1 || a.sh == 2) && aligned16(a.Wt) && total + 256 < (1ll << 31)) {
-      const int qstrips = a.Q;  // one pixel per thread
+      const int pix = a.sh == 1 ? 4 : 2;  // pixels of an output row per thread
+      const int qstrips = (a.Q + pix - 1) / pix;
       const int64_t threads = (int64_t)a.N * a.P * qstrips * (a.K / 8);
       const unsigned grid = (unsigned)ceil_div(threads, 256);
       const unsigned m_k8 = magic_of(a.K / 8), m_qs = magic_of(qstrips), m_p = magic_of(a.P);
-      if (a.sh == 1) hipLaunchKernelGGL((dwconv3x3_f16_nhwc_kernel<1, 1>), dim3(grid), dim3(256), 0, ctx->stream, a, (int)threads, qstrips, m_k8, m_qs, m_p);
-      else hipLaunchKernelGGL((dwconv3x3_f16_nhwc_kernel<2, 1>), dim3(grid), dim3(256), 0, ctx->stream, a, (int)threads, qstrips, m_k8, m_qs, m_p);
+#define DW_LAUNCH(ST, PX, WV) hipLaunchKernelGGL((dwconv3x3_f16_nhwc_kernel<ST, PX, WV>), dim3(grid), dim3(256), 0, ctx->stream, a, (int)threads, qstrips, m_k8, m_qs, m_p)
+      if (a.sh == 1) DW_LAUNCH(1, 4, 4);
+      else DW_LAUNCH(2, 2, 4);
+#undef DW_LAUNCH
     } else
     hipLaunchKernelGGL(dwconv_f16_nhwc_kernel, dim3((unsigned)blocks), dim3(256), (size_t)a.K * a.R * a.S * 2, ctx->stream, a, total);
   } else {
