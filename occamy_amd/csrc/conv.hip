@@ -55,6 +55,46 @@ __global__ __launch_bounds__(256) void dwconv_f32_nchw_kernel(
   Y[i] = acc;
 }
 
+// The 3x3 case on outputs of fewer than 2^31 elements (every depthwise layer of a MobileNetV2).  At batch 1 such a
+// layer is one short wave of threads and what it costs is its chain of dependent steps: here the nine input and
+// nine filter values are requested together, from clamped addresses (a load under a divergent branch is waited
+// for before the next one is issued: nine memory round trips one after the other), a tap in the padding has its
+// value replaced by zero, and the index is taken apart with multiply-high divisions instead of 64-bit ones.
+// Taps are summed in the order of the kernel above.
+__global__ __launch_bounds__(256) void dwconv3x3_f32_nchw_kernel(
+    const float *__restrict__ X, const float *__restrict__ Wt, const float *__restrict__ bias, const float *Zr, float *Y, int C,
+    int H, int W, int K, int Kg, int P, int Q, int ph, int pw, int sh, int sw, int act, float act_coef, int total, int w_k_stride,
+    int w_tap_stride, unsigned magic_q, unsigned magic_p, unsigned magic_k, unsigned magic_kg) {
+  const int i = (int)(blockIdx.x * 256 + threadIdx.x);
+  if (i >= total) return;
+  int t = div_magic(i, Q, magic_q);
+  const int q = i - t * Q;
+  const int t2 = div_magic(t, P, magic_p), p = t - t2 * P;
+  const int n = div_magic(t2, K, magic_k), k = t2 - n * K;
+  const int c = div_magic(k, Kg, magic_kg);
+  const float *__restrict__ x = X + ((int64_t)n * C + c) * H * W;
+  const float *__restrict__ w = Wt + (int64_t)k * w_k_stride;
+  const int ih0 = p * sh - ph, iw0 = q * sw - pw;
+  float xv[9], wv[9];
+#pragma unroll
+  for (int r = 0; r < 3; r++)
+#pragma unroll
+    for (int s = 0; s < 3; s++) {
+      const int ih = ih0 + r, iw = iw0 + s;
+      const bool ok = (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+      const float v = x[min(max(ih, 0), H - 1) * W + min(max(iw, 0), W - 1)];
+      xv[3 * r + s] = ok ? v : 0.f;
+      wv[3 * r + s] = w[(3 * r + s) * w_tap_stride];
+    }
+  const float b = bias ? bias[k] : 0.f, z = Zr ? Zr[i] : 0.f;
+  float acc = 0.f;
+#pragma unroll
+  for (int j = 0; j < 9; j++) acc = fmaf(xv[j], wv[j], acc);
+  if (bias) acc += b;
+  if (Zr) acc += z;
+  Y[i] = apply_act(acc, act, act_coef);
+}
+
 struct ConvShape {
   int N, C, H, W, K, Cg, R, S, P, Q, ph, pw, sh, sw, group;
 };
@@ -205,7 +245,11 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
     dim3 grid((unsigned)ceil_div(total, 256)), block(256);
     if (ceil_div(total, 256) > INT32_MAX) DNNRT_FAIL("conv: depthwise output too large");
     const int w_k = crsk ? 1 : s.R * s.S, w_tap = crsk ? s.K : 1;
-    if (s.R == 3 && s.S == 3)
+    if (s.R == 3 && s.S == 3 && total + 256 < (1ll << 31) && (int64_t)s.H * s.W < (1ll << 31))
+      hipLaunchKernelGGL(dwconv3x3_f32_nchw_kernel, grid, block, 0, ctx->stream, X, Wt, bias, Z, Y, s.C, s.H, s.W, s.K, Kg, s.P,
+                         s.Q, s.ph, s.pw, s.sh, s.sw, act, ctx->act_coef, (int)total, w_k, w_tap, magic_of(s.Q), magic_of(s.P),
+                         magic_of(s.K), magic_of(Kg));
+    else if (s.R == 3 && s.S == 3)
       hipLaunchKernelGGL((dwconv_f32_nchw_kernel<3, 3>), grid, block, 0, ctx->stream, X, Wt, bias, Z, Y,
                          s.C, s.H, s.W, s.K, Kg, s.P, s.Q, s.ph, s.pw, s.sh, s.sw, 3, 3, act, ctx->act_coef, total, w_k, w_tap);
     else
