@@ -35,6 +35,11 @@ struct IgemmArgs {
   int64_t a_z_stride, x_z_stride, y_z_stride, bias_z_stride;
   unsigned magic_rs, magic_s;  // filled in by launch_igemm_f32: magic_of(R * S), magic_of(S), for the generic filter sizes
   int xcd_m;          // (small kernels, set by their launcher) the XCDs form an xcd_m x (8 / xcd_m) grid over the tile plane
+  // ... and what the kernels would otherwise divide for at their start, before any load can be issued (a
+  // division is some twenty dependent instructions): log2(8 / xcd_m), tiles per XCD along m and n, and the
+  // multiply-high constants of tn_per, P * Q and Q
+  int xcd_n_log2, tm_per, tn_per;
+  unsigned magic_tn_per, magic_pq, magic_q;
   // (conv1x1_f32_small_kernel) a second 1x1 convolution onto the same result, its reduction appended to the first's:
   // filter A2 ([M][Kdim2] or, a_mcontig, [Kdim2][a_ld]), input X2 of H2 x W2 pixels per channel read with strides sh2, sw2,
   // bias2 per row or null.  A2 == nullptr: none.

@@ -199,11 +199,11 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   // filter and xcd_m / 8 of the activations, where a run of consecutive tiles per XCD fetches all of one operand
   // into all eight L2s.  The launcher picks xcd_m from the two operands' sizes.
   const int tiles_m = (a.M + 31) / 32, tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * tiles_m;
-  const int xcd_n = 8 / a.xcd_m;
-  const int tm_per = (tiles_m + a.xcd_m - 1) / a.xcd_m, tn_per = (tiles_n + xcd_n - 1) / xcd_n;
+  const int tm_per = a.tm_per, tn_per = a.tn_per;
   const int xcd = (int)(blockIdx.x & 7), in_xcd = (int)(blockIdx.x >> 3);
-  const int tm_local = in_xcd / tn_per;
-  const int tile_m = (xcd / xcd_n) * tm_per + tm_local, tile_n = (xcd % xcd_n) * tn_per + (in_xcd - tm_local * tn_per);
+  const int tm_local = div_magic(in_xcd, tn_per, a.magic_tn_per);
+  const int tile_m = (xcd >> a.xcd_n_log2) * tm_per + tm_local;
+  const int tile_n = (xcd & ((1 << a.xcd_n_log2) - 1)) * tn_per + (in_xcd - tm_local * tn_per);
   if (tm_local >= tm_per || tile_m >= tiles_m || tile_n >= tiles_n) return;
   const int tile_id = tile_m * tiles_n + tile_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
@@ -217,8 +217,8 @@ __global__ __launch_bounds__(64 * KS) void conv3x3_f32_small_kernel(const IgemmA
   float bias_r[16];
   prefetch_bias(a, z, m0, half, bias_r);
   const float bias_c = 0.f;  // a per-column bias belongs to matrix products, which are never 3x3
-  const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
-  const int p = pq / a.Q, q = pq - p * a.Q;
+  const int img = col_ok ? div_magic(col, PQ, a.magic_pq) : 0, pq = col_ok ? col - img * PQ : 0;
+  const int p = div_magic(pq, a.Q, a.magic_q), q = pq - p * a.Q;
   const int ih0 = p * a.sh - a.ph, iw0 = q * a.sw - a.pw;
   unsigned tap_off[9], tap_mask[9];
 #pragma unroll
@@ -305,11 +305,11 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
   // filter and xcd_m / 8 of the activations, where a run of consecutive tiles per XCD fetches all of one operand
   // into all eight L2s.  The launcher picks xcd_m from the two operands' sizes.
   const int tiles_m = (a.M + 31) / 32, tiles_n = (a.Ncols + 31) / 32, tiles = tiles_n * tiles_m;
-  const int xcd_n = 8 / a.xcd_m;
-  const int tm_per = (tiles_m + a.xcd_m - 1) / a.xcd_m, tn_per = (tiles_n + xcd_n - 1) / xcd_n;
+  const int tm_per = a.tm_per, tn_per = a.tn_per;
   const int xcd = (int)(blockIdx.x & 7), in_xcd = (int)(blockIdx.x >> 3);
-  const int tm_local = in_xcd / tn_per;
-  const int tile_m = (xcd / xcd_n) * tm_per + tm_local, tile_n = (xcd % xcd_n) * tn_per + (in_xcd - tm_local * tn_per);
+  const int tm_local = div_magic(in_xcd, tn_per, a.magic_tn_per);
+  const int tile_m = (xcd >> a.xcd_n_log2) * tm_per + tm_local;
+  const int tile_n = (xcd & ((1 << a.xcd_n_log2) - 1)) * tn_per + (in_xcd - tm_local * tn_per);
   if (tm_local >= tm_per || tile_m >= tiles_m || tile_n >= tiles_n) return;
   const int tile_id = tile_m * tiles_n + tile_n;
   const int m0 = tile_m * 32, n0 = tile_n * 32, z = blockIdx.z;
@@ -332,8 +332,8 @@ __global__ __launch_bounds__(64 * KS) void conv1x1_f32_small_kernel(const IgemmA
     for (int r = 0; r < 16; r++) bias_r[r] += a.bias2[min(acc_row(m0, half, r), a.M - 1)];
   }
   const float bias_c = load_bias_col(a, col_ok ? col : 0);  // requested up front as well
-  const int img = col_ok ? col / PQ : 0, pq = col_ok ? col - img * PQ : 0;
-  const int p = pq / a.Q, q = pq - p * a.Q;
+  const int img = col_ok ? div_magic(col, PQ, a.magic_pq) : 0, pq = col_ok ? col - img * PQ : 0;
+  const int p = div_magic(pq, a.Q, a.magic_q), q = pq - p * a.Q;
   const unsigned x_pix = second ? (unsigned)((int64_t)img * a.x2_img_stride + (int64_t)(p * a.sh2) * a.W2 + q * a.sw2)
                                 : (unsigned)((int64_t)img * a.x_img_stride + (int64_t)(p * a.sh) * a.W + q * a.sw);
   const unsigned a_row = (unsigned)mrow * (unsigned)Kd, lda = (unsigned)a.a_ld;
@@ -475,6 +475,15 @@ bool launch_igemm_f32_small(const dnnrtContext *ctx, const IgemmArgs &a, int rsm
     if (slots == 0) { am.xcd_m = 1; slots = 8 * ceil_div(tiles_m, 1) * ceil_div(tiles_n, 8); }  // a single tile either way
   }
   if (slots > INT32_MAX) return true;
+  {
+    const int xn = 8 / am.xcd_m;
+    am.xcd_n_log2 = xn == 8 ? 3 : xn == 4 ? 2 : xn == 2 ? 1 : 0;
+    am.tm_per = (int)ceil_div(tiles_m, am.xcd_m);
+    am.tn_per = (int)ceil_div(tiles_n, xn);
+    am.magic_tn_per = magic_of(am.tn_per);
+    am.magic_pq = magic_of(a.P * a.Q);
+    am.magic_q = magic_of(a.Q);
+  }
   dim3 grid((unsigned)slots, splits, a.Z);
   if (ctx->splitk_shared && splits > 1) clear_split_counters(ctx, tiles * a.Z);
 #define LAUNCH_KS2(KERNEL, AMC_, ARG)                                                                  \
