@@ -54,9 +54,23 @@ __global__ __launch_bounds__(256) void attention_kernel(const T *__restrict__ Q,
   const T *Vg = V + (int64_t)b * Sk * ld_in + head * DH;
 
   // the query tile (rows past the end repeat the last query; they are not stored)
-  for (int i = tid; i < ATT_QB * (DH / 4); i += 256) {
-    const int r = i / (DH / 4), c4 = i - r * (DH / 4);
-    *reinterpret_cast<float4 *>(Qs + r * ROW + c4 * 4) = load4(Qg + (int64_t)min(q0 + r, Sq - 1) * ld_in + c4 * 4);
+  // All of a tile's loads are requested before the first value goes to LDS (as a load-then-store loop the
+  // compiler keeps one round trip to memory per turn: two for the queries, eight per block of keys and values,
+  // most of the kernel's time at sequence length 128).
+  constexpr int Q_TURNS = ATT_QB * (DH / 4) / 256, KV_TURNS = ATT_KB * (DH / 4) / 256, KV_CHUNK = KV_TURNS < 8 ? KV_TURNS : 8;
+  static_assert(ATT_QB * (DH / 4) % 256 == 0 && ATT_KB * (DH / 4) % 256 == 0, "tile loads divide over the threads");
+  {
+    float4 qv[Q_TURNS];
+#pragma unroll
+    for (int u = 0; u < Q_TURNS; u++) {
+      const int i = tid + 256 * u, r = i / (DH / 4), c4 = i - r * (DH / 4);
+      qv[u] = load4(Qg + (int64_t)min(q0 + r, Sq - 1) * ld_in + c4 * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < Q_TURNS; u++) {
+      const int i = tid + 256 * u, r = i / (DH / 4), c4 = i - r * (DH / 4);
+      *reinterpret_cast<float4 *>(Qs + r * ROW + c4 * 4) = qv[u];
+    }
   }
 
   floatx16 o[TD];
@@ -68,11 +82,22 @@ __global__ __launch_bounds__(256) void attention_kernel(const T *__restrict__ Q,
 
   for (int kb = 0; kb < Sk; kb += ATT_KB) {
     __syncthreads();  // everyone is done with the previous block's K and V
-    for (int i = tid; i < ATT_KB * (DH / 4); i += 256) {
-      const int r = i / (DH / 4), c4 = i - r * (DH / 4);
-      const int64_t row = (int64_t)min(kb + r, Sk - 1) * ld_in + c4 * 4;
-      *reinterpret_cast<float4 *>(Ks + r * ROW + c4 * 4) = load4(Kg + row);
-      *reinterpret_cast<float4 *>(Vs + r * ROW + c4 * 4) = load4(Vg + row);
+#pragma unroll
+    for (int u0 = 0; u0 < KV_TURNS; u0 += KV_CHUNK) {  // at most eight turns (64 registers) in flight
+      float4 kv[KV_CHUNK], vv[KV_CHUNK];
+#pragma unroll
+      for (int u = 0; u < KV_CHUNK; u++) {
+        const int i = tid + 256 * (u0 + u), r = i / (DH / 4), c4 = i - r * (DH / 4);
+        const int64_t row = (int64_t)min(kb + r, Sk - 1) * ld_in + c4 * 4;
+        kv[u] = load4(Kg + row);
+        vv[u] = load4(Vg + row);
+      }
+#pragma unroll
+      for (int u = 0; u < KV_CHUNK; u++) {
+        const int i = tid + 256 * (u0 + u), r = i / (DH / 4), c4 = i - r * (DH / 4);
+        *reinterpret_cast<float4 *>(Ks + r * ROW + c4 * 4) = kv[u];
+        *reinterpret_cast<float4 *>(Vs + r * ROW + c4 * 4) = vv[u];
+      }
     }
     __syncthreads();
 
