@@ -28,9 +28,19 @@ __global__ __launch_bounds__(256) void conv_f16_first_kernel(const ConvF16Args a
   __shared__ __attribute__((aligned(16))) _Float16 wt[FIRST_MAX_TAPS * K];  // [tap][filter], tap = (r S + s) C + c
   const int taps = a.R * a.S * a.C;
   const _Float16 *__restrict__ Wg = reinterpret_cast<const _Float16 *>(a.Wt);  // K x R x S x C
-  for (int e = threadIdx.x; e < K * taps; e += 256) {
-    const int k = e / taps, t = e - k * taps;
-    wt[t * K + k] = Wg[e];
+  {  // every value requested before the first one is stored: a load-then-store loop pays a memory round trip per turn
+    constexpr int TURNS = (FIRST_MAX_TAPS * K + 255) / 256;
+    _Float16 wv[TURNS];
+#pragma unroll
+    for (int u = 0; u < TURNS; u++) wv[u] = Wg[min((int)threadIdx.x + 256 * u, K * taps - 1)];
+#pragma unroll
+    for (int u = 0; u < TURNS; u++) {
+      const int e = (int)threadIdx.x + 256 * u;
+      if (e < K * taps) {
+        const int k = e / taps, t = e - k * taps;
+        wt[t * K + k] = wv[u];
+      }
+    }
   }
   __syncthreads();
   const int i = (int)(blockIdx.x * 256 + threadIdx.x);
