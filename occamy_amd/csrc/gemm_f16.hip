@@ -81,8 +81,8 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
           }
         }
       }
-      {  // B side
-        const int row0 = b_k_fast ? r >> 3 : (r & 7) << 3, kk0 = b_k_fast ? (r & 7) << 3 : r >> 3;
+      {  // B side (n contiguous: the thread's two runs are rows k = 2 (tid / 8) and the next one, which go to LDS as pairs)
+        const int row0 = b_k_fast ? r >> 3 : (tid & 7) << 3, kk0 = b_k_fast ? (r & 7) << 3 : 2 * (tid >> 3) + h;
         const int64_t at = (int64_t)(k0 + kk0) * a.b_sk + (int64_t)(n0 + row0) * a.b_sn;
         const bool whole = b_k_fast ? (n0 + row0 < a.N && k0 + kk0 + 8 <= a.K) : (n0 + row0 + 8 <= a.N && k0 + kk0 < a.K);
         if (a.b_vec && whole) {
@@ -110,15 +110,30 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
           for (int e = 0; e < 8; e++) Ms[(row0 + e) * G_ROW + kk0] = va[h][e];
         }
       }
-      {  // -> Ns[n][k]
-        const int row0 = b_k_fast ? r >> 3 : (r & 7) << 3, kk0 = b_k_fast ? (r & 7) << 3 : r >> 3;
-        if (b_k_fast) {
-          *reinterpret_cast<g_half8 *>(Ns + row0 * G_ROW + kk0) = vb[h];
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; e++) Ns[(row0 + e) * G_ROW + kk0] = vb[h][e];
-        }
+      if (b_k_fast) {  // -> Ns[n][k]
+        const int row0 = r >> 3, kk0 = (r & 7) << 3;
+        *reinterpret_cast<g_half8 *>(Ns + row0 * G_ROW + kk0) = vb[h];
       }
+    }
+    if (!b_k_fast) {
+      // n contiguous in memory: -> Nd[k / 2][n], one 32-bit word per pair of consecutive k of a column n, so that the
+      // thread's two runs (rows k, k + 1 of eight columns) are eight consecutive words, two 16-byte stores, and an
+      // MFMA operand (eight consecutive k of one n) is four words 72 words apart.  (Element by element into
+      // Ns[n][k] this was sixteen 2-byte stores a thread and step, most of them on the same banks.)
+      typedef unsigned g_uintx4 __attribute__((ext_vector_type(4)));
+      unsigned *Nd = reinterpret_cast<unsigned *>(Ns);
+      const g_uintx4 d0 = __builtin_bit_cast(g_uintx4, vb[0]), d1 = __builtin_bit_cast(g_uintx4, vb[1]);  // word j: columns 2j, 2j + 1
+      g_uintx4 lo, hi;  // columns 0..3 and 4..7, each word (row k, row k + 1)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        lo[2 * j] = (d0[j] & 0xffffu) | (d1[j] << 16);
+        lo[2 * j + 1] = (d0[j] >> 16) | (d1[j] & 0xffff0000u);
+        hi[2 * j] = (d0[2 + j] & 0xffffu) | (d1[2 + j] << 16);
+        hi[2 * j + 1] = (d0[2 + j] >> 16) | (d1[2 + j] & 0xffff0000u);
+      }
+      unsigned *dst = Nd + (tid >> 3) * G_ROW + ((tid & 7) << 3);
+      *reinterpret_cast<g_uintx4 *>(dst) = lo;
+      *reinterpret_cast<g_uintx4 *>(dst + 4) = hi;
     }
   };
 #pragma unroll
@@ -134,7 +149,15 @@ __global__ __launch_bounds__(256) void gemm_f16_generic_kernel(const GemmF16Args
       if (ks0 + AHEAD * G_BK < k_end) request(ra[s], rb[s], ks0 + AHEAD * G_BK);
 #pragma unroll
       for (int ks = 0; ks < G_BK; ks += 16) {
-        const g_half8 nv = *reinterpret_cast<const g_half8 *>(Ns + (wn0 + l32) * G_ROW + ks + half * 8);
+        g_half8 nv;
+        if (b_k_fast) {
+          nv = *reinterpret_cast<const g_half8 *>(Ns + (wn0 + l32) * G_ROW + ks + half * 8);
+        } else {
+          const unsigned *Nd = reinterpret_cast<const unsigned *>(Ns) + ((ks >> 1) + half * 4) * G_ROW + wn0 + l32;
+          typedef unsigned g_uintx4 __attribute__((ext_vector_type(4)));
+          const g_uintx4 w4 = {Nd[0], Nd[G_ROW], Nd[2 * G_ROW], Nd[3 * G_ROW]};
+          nv = __builtin_bit_cast(g_half8, w4);
+        }
         const g_half8 mv = *reinterpret_cast<const g_half8 *>(Ms + (wm0 + l32) * G_ROW + ks + half * 8);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(nv, mv, acc, 0, 0, 0);
       }
