@@ -124,9 +124,11 @@ void dnncSessionDestroy(dnncSession *s);
 int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *outputs);
 /* resident mode only.  on_device != 0: inputs/outputs are device buffers and the call does not
  * wait (dnncSessionSync does); on_device == 2: the kernels read the input buffers where they
- * are instead of copying them into the pool first -- the caller leaves them unchanged until
- * the run is over, and passing other addresses than last time records the graph again;
- * use_graph: replay the kernels from a captured graph */
+ * are instead of copying them into the pool first, and the operations that produce the
+ * results write them into `outputs` instead of a pool tensor that is copied there afterwards
+ * -- the caller leaves the inputs unchanged and the result buffers alone until the run is
+ * over, no buffer overlaps another, and passing other addresses than last time records the
+ * graph again; use_graph: replay the kernels from a captured graph */
 int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
 int32_t dnncSessionSync(dnncSession *s);
 /* Tuning and tests: dnnrtSetConvTile on the session's handle (0 = automatic choice); a captured

@@ -298,7 +298,9 @@ class Session:
 
     def run_device(self, in_ptrs, out_ptrs, use_graph=True, in_place=False):
         """Resident mode: device addresses in and out; returns without waiting.  in_place: the kernels read the
-        input buffers where they are (no copy into the pool); they must stay unchanged until the run is over."""
+        input buffers where they are (no copy into the pool) and the operations that produce the results write them
+        into the result buffers (no copy out of the pool): the inputs must stay unchanged and the result buffers
+        untouched until the run is over, and neither may overlap the other."""
         ip = (C.c_void_p * max(len(in_ptrs), 1))(*in_ptrs)
         op = (C.c_void_p * max(len(out_ptrs), 1))(*out_ptrs)
         if lib().dnncSessionRunResident(self._s, ip, op, 2 if in_place else 1, int(use_graph)):

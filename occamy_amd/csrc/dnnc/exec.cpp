@@ -478,6 +478,11 @@ bool Session::issue_all_compute(std::string &err) {
 // the call returns without waiting (sync() does).
 bool Session::run_resident(const void *const *inputs, void *const *outputs, int on_device, int use_graph, std::string &err) {
   const bool borrow = on_device == 2 && !host_backend;
+  auto other_slot = [&](const Op *op) -> size_t {  // the pool tensor behind a result copy (see below)
+    const Value *v = op->operands[1];
+    if (v->def && v->def->kind == OP_MEM_OFFSET) return (size_t)v->id;
+    return (size_t)v->def->operands.back()->id;
+  };
   // The pool reuses the inputs' slots for later tensors, so every pass over
   // the kernels must be preceded by a fresh copy of the inputs.
   auto copy_inputs = [&]() -> bool {
@@ -507,6 +512,30 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
       void *want = borrow ? const_cast<void *>(inputs[(size_t)op->operands[1]->arg_index]) : arg_home[slot];
       if (ptr[slot] != want) { ptr[slot] = want; moved = true; }
     }
+    // The same for the results: the pool tensor a result is computed into (the output operand of the operation
+    // that produces it) points at the caller's result buffer, so the last kernel writes there and no copy
+    // follows.  Only that one tensor value moves: whatever else the planner put at the same pool offset at other
+    // times stays in the pool, and a copy-type operation that would have aliased it copies instead.
+    direct_out.clear();
+    for (const Op *op : prog->ops) {
+      if (op->kind != OP_MEMCPY || op->mode != 2 || staged_out.count(op)) continue;
+      const Value *v = op->operands[1], *bv = nullptr;
+      if (v->def && v->def->kind == OP_MEM_OFFSET) bv = v;
+      else if (v->def && is_compute(v->def->kind) && !v->def->operands.empty()) {
+        const Value *o = v->def->operands.back();
+        if (o->def && o->def->kind == OP_MEM_OFFSET) bv = o;
+      }
+      if (!bv) continue;
+      const size_t slot = (size_t)bv->id;
+      if (!out_home.count(slot)) out_home[slot] = ptr[slot];
+      void *dst = outputs[(size_t)op->operands[0]->def->out_index];
+      bool shared = false;  // two results out of one tensor, or a tensor that is also an argument's slot: copy as before
+      for (const Op *other : direct_out) shared = shared || other_slot(other) == slot;
+      shared = shared || arg_home.count(slot) != 0;
+      void *want = (borrow && !shared) ? dst : out_home[slot];
+      if (ptr[slot] != want) { ptr[slot] = want; moved = true; }
+      if (borrow && !shared) direct_out.push_back(op);
+    }
     if (moved && graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
   }
   const bool graphed = use_graph && !host_backend;
@@ -532,6 +561,7 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
   // 3. outputs
   for (const Op *op : prog->ops) {
     if (op->kind != OP_MEMCPY || op->mode != 2) continue;
+    if (std::find(direct_out.begin(), direct_out.end(), op) != direct_out.end()) continue;  // written in place
     const Op *ha = op->operands[0]->def;
     const size_t oi = (size_t)ha->out_index;
     void *dst = on_device ? outputs[oi] : host_out[oi];
@@ -557,6 +587,12 @@ bool Session::profile_resident(const void *const *inputs, int on_device, bool by
       ptr[h.first] = h.second;
       if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
     }
+  for (const auto &h : out_home)
+    if (ptr[h.first] != h.second) {
+      ptr[h.first] = h.second;
+      if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
+    }
+  direct_out.clear();
   // the operations that launch something, in program order (an aliased copy only hands its input's address on;
   // a first eager pass has set those)
   std::vector<const Op *> compute;

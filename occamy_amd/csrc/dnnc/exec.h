@@ -116,6 +116,8 @@ class Session {
   void *pool = nullptr, *weights = nullptr, *graph = nullptr;
   std::vector<void *> ptr;  // value id -> address (host or device)
   std::map<size_t, void *> arg_home;  // resident mode: value id of a function argument's pool slot -> its address in the pool
+  std::vector<const Op *> direct_out;  // the result copies of the current run that are not needed for that reason
+  std::map<size_t, void *> out_home;  // ... and of a result's pool tensor, when results are written where the caller wants them
   std::map<std::string, void *> host_const;
   std::vector<void *> host_out, host_in;
   // resident mode: results produced mid-program, whose pool bytes a later

@@ -342,9 +342,10 @@ def test_ssd_resnet50(batch):
 
 
 def test_resident_run_reads_device_inputs_in_place():
-    """run_device(in_place=True): the kernels read the caller's input buffer instead of a copy in the pool; the
-    same bits as with the copy, eager and replayed; the input buffer is left as it was; another input address
-    (the graph is recorded again), then the copying mode and the profiler on the same session."""
+    """run_device(in_place=True): the kernels read the caller's input buffer instead of a copy in the pool and write
+    the result into the caller's result buffer instead of copying it there; the same bits as with the copies, eager
+    and replayed; the input buffer is left as it was; another input address and another result address (the graph is
+    recorded again), then the copying mode and the profiler on the same session."""
     import torch
     for builder, flags in ((lambda: models.resnet50(4, np.float16, seed=5, image=64),
                             dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
@@ -380,6 +381,16 @@ def test_resident_run_reads_device_inputs_in_place():
         s.run_device([t.data_ptr() for t in b], [out.data_ptr()], use_graph=True, in_place=True)
         s.sync()
         np.testing.assert_array_equal(out.cpu().numpy(), want[0])
+        # the result is written where the caller wants it as well: another result address (the graph is recorded
+        # again), and the first one is left alone by that run
+        out2 = torch.zeros_like(out)
+        out.fill_(7)
+        torch.cuda.synchronize()
+        s.run_device([t.data_ptr() for t in b], [out2.data_ptr()], use_graph=True, in_place=True)
+        s.run_device([t.data_ptr() for t in b], [out2.data_ptr()], use_graph=True, in_place=True)
+        s.sync()
+        np.testing.assert_array_equal(out2.cpu().numpy(), want[0])
+        assert bool((out == 7).all())
         s.close()
 
 
