@@ -394,6 +394,49 @@ def test_resident_run_reads_device_inputs_in_place():
         s.close()
 
 
+def test_resident_run_in_place_with_two_results():
+    """Two results, the first of them produced before the last operation and read again by it: with
+    run_device(in_place=True) both land in the caller's buffers with the bits of the copying mode, eager and
+    replayed, also after the result addresses change."""
+    import torch
+    from occamy_amd.compiler import Graph
+
+    def builder():
+        r = np.random.default_rng(12)
+        g = Graph()
+        x = r.standard_normal((2, 16, 12, 12)).astype(np.float32)
+        g.input("X", x.shape, np.float32)
+        w1 = g.constant((r.standard_normal((24, 16, 3, 3)) * 0.1).astype(np.float32))
+        b1 = g.constant(r.uniform(-0.1, 0.1, 24).astype(np.float32))
+        a = g.node("Relu", [g.node("Conv", ["X", w1, b1], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1], group=1)])
+        w2 = g.constant((r.standard_normal((8, 24, 1, 1)) * 0.1).astype(np.float32))
+        b2 = g.constant(r.uniform(-0.1, 0.1, 8).astype(np.float32))
+        c = g.node("Conv", [a, w2, b2], kernel_shape=[1, 1], pads=[0, 0, 0, 0], strides=[1, 1], group=1)
+        g.output(a)
+        g.output(c)
+        return g, [x]
+
+    want, _ = run(builder, fusion=True)
+    g, inputs = builder()
+    p = g.compile(fusion=True)
+    s = p.session(compiler.MODE_RESIDENT)
+    x = torch.from_numpy(inputs[0]).cuda()
+    outs = [[torch.zeros(tuple(w.shape), device="cuda") for w in want] for _ in range(2)]
+    for o, graph in ((outs[0], False), (outs[0], True), (outs[0], True), (outs[1], True), (outs[0], True)):
+        for t in o:
+            t.zero_()
+        torch.cuda.synchronize()
+        s.run_device([x.data_ptr()], [t.data_ptr() for t in o], use_graph=graph, in_place=True)
+        s.sync()
+        for t, w in zip(o, want):
+            np.testing.assert_array_equal(t.cpu().numpy(), w)
+    s.run_device([x.data_ptr()], [t.data_ptr() for t in outs[1]], use_graph=True)   # the copying mode again
+    s.sync()
+    for t, w in zip(outs[1], want):
+        np.testing.assert_array_equal(t.cpu().numpy(), w)
+    s.close()
+
+
 def test_compact_pool_on_the_gpu():
     """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
     inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured
