@@ -531,6 +531,21 @@ def test_split_reduction_hand_over_is_deterministic(gpu, cpu):
         gpu.sync()
         return Y
     repeat(mm_call, ref)
+    # the fp16 product splits its reduction the same way (3072 -> 768: eleven workgroups per tile, 768 -> 3072: none)
+    for K, N in ((3072, 768), (768, 768)):
+        a16 = r.standard_normal((1, 128, K)).astype(np.float16)
+        b16 = (r.standard_normal((K, N)) / np.sqrt(K)).astype(np.float16)
+        ref16 = oc.matmul_nd(cpu, a16, b16).astype(np.float32)
+        A16, B16, Y16 = gpu.put(a16), gpu.put(b16), gpu.empty((1, 128, N), np.float16)
+        def mm16_call():
+            gpu.ops.matmul_nd(gpu.ptr(A16), a16.shape, gpu.ptr(B16), b16.shape, gpu.ptr(Y16), (1, 128, N), _abi.F16)
+            gpu.sync()
+            return Y16
+        first = mm16_call()
+        np.testing.assert_allclose(gpu.get(first).astype(np.float32), ref16, rtol=4e-3, atol=8e-3)
+        first = first.clone()
+        for i in range(200):
+            assert gpu.torch.equal(mm16_call(), first), f"fp16 product {K} -> {N}: repetition {i} differs"
 
 
 def test_matmul_nd_bias(gpu, cpu):
