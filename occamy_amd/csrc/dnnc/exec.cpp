@@ -49,9 +49,16 @@ bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
 
 static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+void Session::drop_graphs() {
+  if (graph) rt.dnnrtGraphDestroy(graph);
+  graph = nullptr;
+  for (auto &g : parked_graphs) rt.dnnrtGraphDestroy(g.second);
+  parked_graphs.clear();
+}
+
 Session::~Session() {
   if (!rt.dl) return;
-  if (graph) rt.dnnrtGraphDestroy(graph);
+  drop_graphs();
   if (handle) rt.dnnrtSync(handle);
   if (pool) rt.dnnrtDealloc(pool);
   if (weights) rt.dnnrtDealloc(weights);
@@ -536,7 +543,20 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
       if (ptr[slot] != want) { ptr[slot] = want; moved = true; }
       if (borrow && !shared) direct_out.push_back(op);
     }
-    if (moved && graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
+    // the addresses this run's kernels see: the key of its graph
+    std::vector<void *> key;
+    for (const auto &h : arg_home) key.push_back(ptr[h.first]);
+    for (const auto &h : out_home) key.push_back(ptr[h.first]);
+    if (moved || key != graph_key) {
+      if (graph) {  // park the current one, take back the one recorded with these addresses if there is one
+        parked_graphs.emplace_back(graph_key, graph);
+        graph = nullptr;
+        if (parked_graphs.size() > 4) { rt.dnnrtGraphDestroy(parked_graphs.front().second); parked_graphs.erase(parked_graphs.begin()); }
+      }
+      for (size_t i = 0; i < parked_graphs.size(); i++)
+        if (parked_graphs[i].first == key) { graph = parked_graphs[i].second; parked_graphs.erase(parked_graphs.begin() + (long)i); break; }
+      graph_key = key;
+    }
   }
   const bool graphed = use_graph && !host_backend;
   if (graphed && !graph) {
@@ -582,16 +602,8 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
 bool Session::profile_resident(const void *const *inputs, int on_device, bool by_class, std::vector<float> &ms, std::string &err) {
   if (mode != MODE_RESIDENT) { err = "profiling needs a resident session"; return false; }
   // profiling copies the inputs into their pool slots: argument values that point at a caller's buffers go home
-  for (const auto &h : arg_home)
-    if (ptr[h.first] != h.second) {
-      ptr[h.first] = h.second;
-      if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
-    }
-  for (const auto &h : out_home)
-    if (ptr[h.first] != h.second) {
-      ptr[h.first] = h.second;
-      if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
-    }
+  for (const auto &h : arg_home) ptr[h.first] = h.second;
+  for (const auto &h : out_home) ptr[h.first] = h.second;
   direct_out.clear();
   // the operations that launch something, in program order (an aliased copy only hands its input's address on;
   // a first eager pass has set those)
@@ -686,7 +698,7 @@ bool Session::profile_classes(const void *const *inputs, int on_device, const st
 
 bool Session::set_conv_tile(int tile, std::string &err) {
   if (rt.dnnrtSetConvTile(handle, tile)) { err = rt_error("dnnrtSetConvTile"); return false; }
-  if (graph) { rt.dnnrtGraphDestroy(graph); graph = nullptr; }
+  drop_graphs();
   return true;
 }
 

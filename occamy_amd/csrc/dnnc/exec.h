@@ -114,6 +114,12 @@ class Session {
   std::map<std::string, bool> crsk_const;  // constants re-laid C,R,S,K on the host
   std::vector<char> filter_crsk;           // value id -> its device copy is C,R,S,K
   void *pool = nullptr, *weights = nullptr, *graph = nullptr;
+  // Recorded graphs of other argument / result addresses than the current ones (runs in place hold the caller's
+  // addresses in the graph): a caller that alternates between a few sets of buffers gets its graph back instead
+  // of a new recording each time.  At most four; the oldest goes first.
+  std::vector<std::pair<std::vector<void *>, void *>> parked_graphs;
+  std::vector<void *> graph_key;  // the addresses `graph` was recorded with
+  void drop_graphs();
   std::vector<void *> ptr;  // value id -> address (host or device)
   std::map<size_t, void *> arg_home;  // resident mode: value id of a function argument's pool slot -> its address in the pool
   std::vector<const Op *> direct_out;  // the result copies of the current run that are not needed for that reason
