@@ -233,7 +233,8 @@ def record(res, steps, warmup, cpu_seconds):
         "latency_ms": res["latency_ms"], "dtype": res["dtype"], "data": "synthetic",
         "config": {"workload": res["name"], "batch": res["batch"],
                    "fusion": ", ".join(k for k, v in res["flags"].items() if v and (k.startswith("fus") or k in ("recompose", "alias_copies", "channels_last", "inplace_residual", "compact_pool"))),
-                   "mode": "weights and input resident in HBM (the first layer reads the input buffer in place, the last one writes the result buffer), kernels replayed from a captured graph",
+                   "mode": "weights and input resident in HBM (the first layer reads the input buffer in place, the last one writes the result buffer), "
+                           + ("kernels replayed from a captured graph" if res["kernels_per_step"] > 3 else "kernels launched one by one (up to three: a graph launch costs the host more)"),
                    "kernels_per_step": res["kernels_per_step"]},
         "roofline": roofline_of(res),
         "cpu_baseline": cpu_baseline(res, cpu_seconds) if cpu_seconds > 0 else None,

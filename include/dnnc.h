@@ -129,7 +129,8 @@ int32_t dnncSessionRun(dnncSession *s, const void *const *inputs, void *const *o
  * -- the caller leaves the inputs unchanged and the result buffers alone until the run is
  * over, no buffer overlaps another, and passing other addresses than last time records the
  * graph again (the graphs of the last four other sets of addresses are kept and come back
- * when those addresses do); use_graph: replay the kernels from a captured graph */
+ * when those addresses do); use_graph: replay the kernels from a captured graph (programs
+ * of up to three kernels are issued directly all the same: a graph launch costs more) */
 int32_t dnncSessionRunResident(dnncSession *s, const void *const *inputs, void *const *outputs, int32_t on_device, int32_t use_graph);
 int32_t dnncSessionSync(dnncSession *s);
 /* Tuning and tests: dnnrtSetConvTile on the session's handle (0 = automatic choice); a captured
