@@ -155,7 +155,6 @@ int32_t dnnrtIsHostBackend(void);
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes);
 /* DNNAPISpecs.inc:47 "wrapDNNMemOffset" (wrapDNNMemOffset.cpp:19-34). */
 int32_t dnnrtMemOffset(void **ptr, void *base, int64_t offset, int64_t bytes);
-/* DNNAPISpecs.inc:45 "wrapDNNMemcpy" (wrapDNNMemcpy.cpp:17-61). */
 /* New, for debugging.  Fills bytes [ptr, ptr + bytes) with `byte` on `stream` (a
  * kernel, so it can be captured into a graph).  The reference clears every
  * tensor's slot as it carves it out of the pool
@@ -164,6 +163,7 @@ int32_t dnnrtMemOffset(void **ptr, void *base, int64_t offset, int64_t bytes);
  * wants to see that claim tested fills each slot with 0xFF (a NaN in fp16 and
  * fp32) before its producer runs and looks for NaNs in the results. */
 int32_t dnnrtMemFill(void *ptr, int32_t byte, int64_t bytes, dnnrtStream_t stream);
+/* DNNAPISpecs.inc:45 "wrapDNNMemcpy" (wrapDNNMemcpy.cpp:17-61). */
 int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind,
                     dnnrtStream_t stream);
 /* DNNAPISpecs.inc:40 "wrapDNNMalloc" (wrapDNNMalloc.cpp). */

@@ -110,6 +110,7 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
   // re-laid once, in the pinned host copy: K,R,S,C for a channels-last (fp16)
   // program, C,R,S,K for fp32 programs on the GPU runtime.
   std::map<std::string, bool> is_filter;
+  std::map<const Value *, std::string> device_copy_of;  // device tensor -> the constant uploaded into it
   for (const Op *op : prog->ops) {
     if (op->kind != OP_MEMCPY || op->mode != 1) continue;
     const Value *src = op->operands[1];
@@ -128,6 +129,19 @@ bool Session::init(const Program *p,const std::string &runtime_path, int mode_, 
     auto it = is_filter.find(name);
     if (it == is_filter.end()) is_filter[name] = f;
     else it->second = it->second && f;
+    device_copy_of[op->operands[0]] = name;
+  }
+  // The two filters of a fused shortcut pair go to one kernel, which takes one layout: if one of them has to
+  // stay as it is (another operator reads the same constant), so does the other.
+  for (bool changed = true; changed;) {
+    changed = false;
+    for (const Op *op : prog->ops) {
+      if (op->kind != OP_CONV_ADD_CONV_ACTIV) continue;
+      const auto a = device_copy_of.find(op->operands[1]), b = device_copy_of.find(op->operands[5]);
+      if (a == device_copy_of.end() || b == device_copy_of.end()) continue;
+      bool &fa = is_filter[a->second], &fb = is_filter[b->second];
+      if (fa != fb) { fa = fb = false; changed = true; }
+    }
   }
 
   // Constants: one pinned host copy each (the reference keeps them as globals
@@ -534,14 +548,15 @@ bool Session::run_resident(const void *const *inputs, void *const *outputs, int 
       }
       if (!bv) continue;
       const size_t slot = (size_t)bv->id;
-      if (!out_home.count(slot)) out_home[slot] = ptr[slot];
-      void *dst = outputs[(size_t)op->operands[0]->def->out_index];
-      bool shared = false;  // two results out of one tensor, or a tensor that is also an argument's slot: copy as before
+      // A second result out of one tensor, or a tensor that is also an argument's slot, is copied after the
+      // kernels as before, from wherever the first result or the argument put the tensor for this run.
+      bool shared = arg_home.count(slot) != 0;
       for (const Op *other : direct_out) shared = shared || other_slot(other) == slot;
-      shared = shared || arg_home.count(slot) != 0;
-      void *want = (borrow && !shared) ? dst : out_home[slot];
+      if (shared) continue;
+      if (!out_home.count(slot)) out_home[slot] = ptr[slot];
+      void *want = borrow ? outputs[(size_t)op->operands[0]->def->out_index] : out_home[slot];
       if (ptr[slot] != want) { ptr[slot] = want; moved = true; }
-      if (borrow && !shared) direct_out.push_back(op);
+      if (borrow) direct_out.push_back(op);
     }
     // the addresses this run's kernels see: the key of its graph
     std::vector<void *> key;

@@ -252,11 +252,16 @@ void alias_copies(Program &p) {
           u.first->operands.back() == buf)
         other_writer = true;
     if (other_writer) continue;
-    p.set_operands(op, {x, buf});
+    // Something besides the copy and the deallocs names the copy's own buffer (the copy to the host of a returned
+    // tensor reads the buffer, not the result): the copy stays a copy.
     std::vector<Op *> deallocs;
-    for (const auto &u : old_out->uses)
+    bool other_user = false;
+    for (const auto &u : old_out->uses) {
       if (u.first->kind == OP_DEALLOC) deallocs.push_back(u.first);
-    if (old_out->uses.size() != deallocs.size()) continue;  // something else uses the old buffer: leave it allocated
+      else if (u.first != op) other_user = true;
+    }
+    if (other_user) continue;
+    p.set_operands(op, {x, buf});
     for (Op *d : deallocs) p.erase(d);
     if (old_out->def && old_out->def->kind == OP_MALLOC) p.erase(old_out->def);
   }
@@ -514,6 +519,8 @@ void fuse_matmul_bias(Program &p) {
 // producer's result is still read afterwards; with the pool pass a later
 // tensor can then land on it.  Here the readers of every writer's result
 // count as uses, which gives the reference's placement in every other case.
+// The same rule keeps a buffer alive that an aliasing copy (alias_copies)
+// writes a second time while the first writer's result still has readers.
 void dealloc_opt(Program &p) {
   std::vector<Op *> deallocs;
   for (Op *op : p.ops)
@@ -528,16 +535,15 @@ void dealloc_opt(Program &p) {
     // dnn.memcpy carries its byte count as last operand in the reference, so
     // it never counts as "writes its last operand"
     auto writes = [&](const Op *u) { return u->kind != OP_MEMCPY && u->kind != OP_DEALLOC && !u->operands.empty() && u->operands.back() == buf; };
+    // The latest reader of ANY writer's result: with one writer, or a chain of in-place writers each read only
+    // by the next (convolution, then the bias added in place), that is the reader of the last writer's result,
+    // the reference's placement.  A copy that shares its input's buffer (alias_copies) is a second writer whose
+    // result can have its last reader before the first writer's has.
     Op *last = ldu;
-    if (writes(ldu) && ldu->result) {
-      Op *r = p.last_user(ldu->result);
-      if (r) last = r;
-    } else {
-      for (const auto &u : buf->uses) {
-        if (!writes(u.first) || !u.first->result) continue;
-        Op *r = p.last_user(u.first->result);
-        if (r && p.order(r) > p.order(last)) last = r;
-      }
+    for (const auto &u : buf->uses) {
+      if (!writes(u.first) || !u.first->result) continue;
+      Op *r = p.last_user(u.first->result);
+      if (r && p.order(r) > p.order(last)) last = r;
     }
     p.move_after(d, last);
   }

@@ -59,8 +59,11 @@ def _conv(g, init, x, cin, cout, k, stride, pad, group=1, bias=True):
     return g.node("Conv", ins, kernel_shape=[k, k], pads=[pad] * 4, strides=[stride, stride], group=group)
 
 
-def resnet50(batch=1, dtype=np.float32, seed=2, image=224, classes=1000):
-    """ResNet-50 v1.5: bottlenecks [3,4,6,3], stride on the 3x3, folded BN."""
+def resnet50(batch=1, dtype=np.float32, seed=2, image=224, classes=1000, stage_means=False):
+    """ResNet-50 v1.5: bottlenecks [3,4,6,3], stride on the 3x3, folded BN.
+    stage_means: the per-channel spatial mean of each of the four stages' results is returned after the logits
+    ([batch, 256], [batch, 512], [batch, 1024], [batch, 2048]), so that a comparison sees every stage at its own
+    magnitude and not only through the classifier."""
     init = _Init(seed, dtype)
     g = Graph()
     x_np = rng.normal(seed, 0, (batch, 3, image, image)).astype(dtype)
@@ -69,6 +72,7 @@ def resnet50(batch=1, dtype=np.float32, seed=2, image=224, classes=1000):
     x = g.node("Relu", [x])
     x = g.node("MaxPool", [x], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
     cin = 64
+    taps = []
     for planes, blocks, stride in [(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)]:
         for b in range(blocks):
             s = stride if b == 0 else 1
@@ -80,12 +84,16 @@ def resnet50(batch=1, dtype=np.float32, seed=2, image=224, classes=1000):
                 identity = _conv(g, init, x, cin, planes * 4, 1, s, 0)
             x = g.node("Relu", [g.node("Add", [o, identity])])
             cin = planes * 4
+        if stage_means and planes != 512:
+            taps.append(g.node("Flatten", [g.node("GlobalAveragePool", [x])], axis=1))
     x = g.node("GlobalAveragePool", [x])
     x = g.node("Flatten", [x], axis=1)
     w = g.constant(init.he_normal((classes, cin)))
     bias = g.constant(np.zeros((classes,), dtype))
     y = g.node("Gemm", [x, w, bias], "logits", alpha=1.0, beta=1.0, transB=1)
     g.output(y)
+    for t in taps + ([x] if stage_means else []):
+        g.output(t)
     return g, [x_np]
 
 

@@ -390,6 +390,54 @@ def test_aliased_copies_change_nothing(builder, copies):
     s.close()
 
 
+def test_aliased_copy_that_is_returned():
+    """A Flatten whose result the function returns: the copy to the host reads the copy's own buffer, so the copy
+    cannot share its input's (it stays a copy); one that also feeds the classifier among them."""
+    small = lambda: models.resnet50(2, image=32, classes=10, stage_means=True)  # noqa: E731
+    want = check(small)
+    assert len(want) == 5
+    for flags in (dict(alias_copies=True), dict(fusion=True, alias_copies=True, dealloc_opt=False)):
+        for mode in (compiler.MODE_OCCAMY, compiler.MODE_RESIDENT):
+            _, _, got = run_oracle(small, mode=mode, **flags)
+            for a, b in zip(got, want):
+                if flags.get("fusion"):
+                    np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-3)
+                else:
+                    np.testing.assert_array_equal(a, b)
+
+
+def _residual_around_a_reshape():
+    # t = Relu(x); y = Reshape(t); a chain of unary operators on y; out = Add(t, Reshape(chain)): t is read again
+    # after the copy of it has had its last reader, the shape of a residual branch around a reshape
+    g = compiler.Graph()
+    x = g.input("x", (2, 8, 16))
+    t = g.node("Relu", [x])
+    y = g.node("Reshape", [t, g.constant(np.array([16, 16], np.int64))])
+    for op in ("Sigmoid", "Tanh", "Sigmoid", "Tanh"):
+        y = g.node(op, [y])
+    back = g.node("Reshape", [y, g.constant(np.array([2, 8, 16], np.int64))])
+    g.output(g.node("Add", [t, back]))
+    rng = np.random.default_rng(11)
+    return g, [rng.standard_normal((2, 8, 16)).astype(np.float32)]
+
+
+def test_aliased_copy_whose_input_is_read_again_later():
+    """A copy that shares its input's buffer is a second writer of that buffer; the buffer must outlive the readers
+    of every writer's result, not only those of the last one."""
+    check(_residual_around_a_reshape)
+    _, _, a = run_oracle(_residual_around_a_reshape)
+    for mode in (compiler.MODE_OCCAMY, compiler.MODE_RESIDENT):
+        _, _, b = run_oracle(_residual_around_a_reshape, mode=mode, alias_copies=True)
+        np.testing.assert_array_equal(a[0], b[0])
+    g, inputs = _residual_around_a_reshape()
+    p = g.compile(alias_copies=True)
+    assert p.num_ops(compute_only=True) == _residual_around_a_reshape()[0].compile().num_ops(compute_only=True) - 2
+    s = p.session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+    s.set_debug_fill(0xFF)
+    np.testing.assert_array_equal(a[0], s.run(*inputs)[0])
+    s.close()
+
+
 @pytest.mark.parametrize("builder", [lambda: models.resnet50(image=32, classes=10), ALEX,
                                      lambda: models.mobilenet_v2(image=32, classes=10)],
                          ids=["resnet50", "alexnet", "mobilenet_v2"])

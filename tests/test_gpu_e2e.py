@@ -1,7 +1,7 @@
 """Whole programs on the MI355X: the same compiled DNN program is executed
 through the C ABI against the gfx950 library and against the CPU oracle, on
 the same seeded inputs.  Tolerances: rtol 1e-4 / atol 1e-5 (scaled by the
-output's magnitude) for fp32; rtol 2e-2 for fp16."""
+output's magnitude) for fp32; rtol 2e-2 with an absolute floor of 4e-3 of the largest reference value for fp16."""
 import numpy as np
 import pytest
 
@@ -144,10 +144,39 @@ def as_fp32_graph(g16, inputs):
     return g, [a.astype(np.float32) for a in inputs]
 
 
+def close16(got, want):
+    """fp16 storage against the fp32 oracle on the same fp16-representable weights and input: rtol 2e-2 with an
+    absolute floor of 4e-3 of the largest reference value (the networks measure 4e-4 .. 7e-4 of it: every
+    activation is rounded to fp16 between layers), and the same arg-max along the last axis nearly everywhere."""
+    got, want = got.astype(np.float32), want.astype(np.float32)
+    assert np.isfinite(got).all()
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=4e-3 * float(np.abs(want).max()))
+
+
+def test_resnet50_fp16_batch_64_every_stage():
+    """Batch 64 with the benchmark's flags, and the per-channel spatial mean of every residual stage's result
+    returned beside the logits: each stage is compared at its own magnitude (rtol 2e-2 of values that are means
+    of non-negative activations), so a wrong late layer cannot hide behind the size of the logits."""
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
+                 fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True, compact_pool=True)
+    build16 = lambda: models.resnet50(64, np.float16, seed=5, stage_means=True)  # noqa: E731
+    out16, info = run(build16, **flags)
+    assert info["requested"] == info["pool"]
+    ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
+    assert [o.shape for o in out16] == [(64, 1000), (64, 256), (64, 512), (64, 1024), (64, 2048)]
+    for got, want in zip(out16, ref):
+        close16(got, want)
+    for got, want in zip(out16[1:], ref[1:]):  # means of ReLU outputs: compare where the mean is not nearly zero
+        got, want = got.astype(np.float32), want
+        big = want > 0.05 * want.max()
+        assert big.mean() > 0.5
+        np.testing.assert_allclose(got[big], want[big], rtol=2e-2)
+
+
 def test_resnet50_fp16_batch_64_as_benchmarked():
     """The throughput configuration at its own size and with the benchmark's own flags (64 x 3 x 224 x 224,
     fp16 storage, fp32 accumulation, channels-last, every fusion bench.py switches on), against the fp32
-    oracle on the same fp16-representable weights and input: rtol 2e-2, atol 2e-2 of the largest logit."""
+    oracle on the same fp16-representable weights and input: rtol 2e-2, atol 4e-3 of the largest logit."""
     flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
                  fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True, compact_pool=True)
     build16 = lambda: models.resnet50(64, np.float16, seed=5)  # noqa: E731
@@ -156,7 +185,7 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
     got, want = out16[0].astype(np.float32), ref[0]
     assert got.shape == (64, 1000) and np.isfinite(got).all()
-    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    close16(got, want)
     assert (got.argmax(1) == want.argmax(1)).mean() > 0.9
     # resident mode, replayed from a captured graph (what bench.py times): the same bits
     import torch
@@ -197,10 +226,10 @@ def test_resnet50_fp16_channels_last(batch, image):
     ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
     got, want = out16[0].astype(np.float32), ref[0]
     assert np.isfinite(got).all()
-    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    close16(got, want)
     # the classifier's bias folded into the product: one launch fewer, same tolerance
     fused, _ = run(build16, fusion=True, channels_last=True, fuse_residual=True, fuse_matmul_bias=True)
-    np.testing.assert_allclose(fused[0].astype(np.float32), want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    close16(fused[0], want)
     assert "dimC=[1," in build16()[0].compile(fusion=True, channels_last=True, fuse_matmul_bias=True).text
     # resident + graph replay gives the same bits as the per-inference mode
     g, inputs = build16()
@@ -225,7 +254,7 @@ def test_first_layer_maxpool_fusion_fp16_channels_last(batch, image):
     res, _ = run(build16, mode=compiler.MODE_RESIDENT, fuse_first_layer_maxpool=True, **flags)
     np.testing.assert_array_equal(res[0], one[0])
     ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
-    np.testing.assert_allclose(one[0].astype(np.float32), ref[0], rtol=2e-2, atol=2e-2 * float(np.abs(ref[0]).max()))
+    close16(one[0], ref[0])
 
 
 @pytest.mark.parametrize("batch,image", [(1, 224), (2, 75)])
@@ -274,7 +303,7 @@ def test_inplace_residual_on_the_gpu(dtype, batch, image):
 def test_mobilenet_v2_fp16_channels_last(batch, image):
     """MobileNetV2 with fp16 weights and activations, channels-last on the device: its depthwise layers on the
     channels-last depthwise kernel, ReLU6 fused as a clipped ReLU, inverted-residual sums written in place; against
-    the fp32 oracle on the same fp16-representable weights and input (rtol 2e-2, atol 2e-2 of the largest logit),
+    the fp32 oracle on the same fp16-representable weights and input (rtol 2e-2, atol 4e-3 of the largest logit),
     per inference and replayed from a captured graph."""
     build16 = lambda: models.mobilenet_v2(batch, np.float16, seed=4, image=image, classes=100)  # noqa: E731
     flags = dict(fusion=True, fuse_residual=True, fuse_activations=True, fuse_matmul_bias=True, channels_last=True, alias_copies=True,
@@ -284,7 +313,7 @@ def test_mobilenet_v2_fp16_channels_last(batch, image):
     ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
     got, want = out16[0].astype(np.float32), ref[0]
     assert np.isfinite(got).all()
-    np.testing.assert_allclose(got, want, rtol=2e-2, atol=2e-2 * float(np.abs(want).max()))
+    close16(got, want)
     res, _ = run(build16, mode=compiler.MODE_RESIDENT, **flags)
     np.testing.assert_array_equal(res[0], out16[0])
 
@@ -437,6 +466,43 @@ def test_resident_run_in_place_with_two_results():
     s.close()
 
 
+def test_resident_run_in_place_with_one_tensor_returned_twice():
+    """The same tensor listed as a result twice (two device-to-host copies of one pool tensor behind the last
+    operation): in place, the first lands in the caller's buffer directly and the second is copied from there;
+    eager, replayed, and after the result addresses change."""
+    import torch
+    from occamy_amd.compiler import Graph
+
+    def builder():
+        r = np.random.default_rng(13)
+        g = Graph()
+        x = r.standard_normal((2, 16, 12, 12)).astype(np.float32)
+        g.input("X", x.shape, np.float32)
+        w1 = g.constant((r.standard_normal((24, 16, 3, 3)) * 0.1).astype(np.float32))
+        b1 = g.constant(r.uniform(-0.1, 0.1, 24).astype(np.float32))
+        a = g.node("Relu", [g.node("Conv", ["X", w1, b1], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1], group=1)])
+        g.output(a)
+        g.output(a)
+        return g, [x]
+
+    want, _ = run(builder, fusion=True)
+    assert len(want) == 2
+    np.testing.assert_array_equal(want[0], want[1])
+    g, inputs = builder()
+    s = g.compile(fusion=True).session(compiler.MODE_RESIDENT)
+    x = torch.from_numpy(inputs[0]).cuda()
+    outs = [[torch.zeros(tuple(w.shape), device="cuda") for w in want] for _ in range(2)]
+    for o, graph in ((outs[0], False), (outs[0], True), (outs[1], True), (outs[0], True)):
+        for t in o:
+            t.zero_()
+        torch.cuda.synchronize()
+        s.run_device([x.data_ptr()], [t.data_ptr() for t in o], use_graph=graph, in_place=True)
+        s.sync()
+        for t, w in zip(o, want):
+            np.testing.assert_array_equal(t.cpu().numpy(), w)
+    s.close()
+
+
 def test_compact_pool_on_the_gpu():
     """Offsets from the planner that knows every lifetime: the same bits as with the reference's first fit, per
     inference with a poisoned pool (what a tensor placed over a live one would show) and replayed from a captured
@@ -520,6 +586,38 @@ def test_projection_shortcut_fusion_fp32(oracle_outputs):
     np.testing.assert_array_equal(res[0], out[0])
 
 
+def test_projection_shortcut_pair_whose_filters_cannot_share_a_layout():
+    """A fused shortcut pair takes both filters in one layout.  Here the shortcut's filter constant is also read by
+    an operator that is no convolution, so it stays K,C,R,S on the device, and the closing filter has to stay with
+    it: the pair runs and gives the oracle's result, per inference and resident."""
+    from occamy_amd.compiler import Graph
+
+    def builder():
+        r = np.random.default_rng(14)
+        g = Graph()
+        x = r.standard_normal((1, 32, 14, 14)).astype(np.float32)
+        g.input("X", x.shape, np.float32)
+        conv = lambda src, w, b, **kw: g.node("Conv", [src, w, b], kernel_shape=[1, 1], pads=[0, 0, 0, 0], strides=[1, 1], group=1, **kw)  # noqa: E731
+        w1 = g.constant((r.standard_normal((16, 32, 1, 1)) * 0.2).astype(np.float32))
+        b1 = g.constant(r.uniform(-0.1, 0.1, 16).astype(np.float32))
+        w2 = g.constant((r.standard_normal((64, 16, 1, 1)) * 0.2).astype(np.float32))
+        b2 = g.constant(r.uniform(-0.1, 0.1, 64).astype(np.float32))
+        wsc = g.constant((r.standard_normal((64, 32, 1, 1)) * 0.2).astype(np.float32))
+        bsc = g.constant(r.uniform(-0.1, 0.1, 64).astype(np.float32))
+        main = conv(g.node("Relu", [conv("X", w1, b1)]), w2, b2)
+        g.output(g.node("Relu", [g.node("Add", [main, conv("X", wsc, bsc)])]))
+        g.output(g.node("Relu", [wsc]))  # the second reader of the shortcut's filter
+        return g, [x]
+
+    flags = dict(fusion=True, fuse_residual=True, fuse_projection_shortcut=True)
+    assert "add-conv" in builder()[0].compile(**flags).text
+    want, _ = run(builder, ORACLE_PATH)
+    for mode in (compiler.MODE_OCCAMY, compiler.MODE_RESIDENT):
+        got, _ = run(builder, mode=mode, **flags)
+        for a, b in zip(got, want):
+            close(a, b)
+
+
 @pytest.mark.parametrize("name", ["resnet50", "mobilenet_v2"])
 def test_residual_fusion_fp32(name, oracle_outputs):
     """conv+bias -> add -> relu as one call: against the oracle, and bit for
@@ -539,8 +637,7 @@ def test_residual_fusion_fp16_channels_last():
     # the fused closer rounds conv+bias to fp16 exactly where the chain stores
     # it, so only the final fp32->fp16 rounding of the sum can differ (the chain
     # adds in fp16 arithmetic): a few fp16 ulps after 16 blocks
-    np.testing.assert_allclose(fused[0].astype(np.float32), chain[0].astype(np.float32), rtol=2e-2,
-                               atol=2e-2 * float(np.abs(chain[0].astype(np.float32)).max()))
+    close16(fused[0], chain[0])
 
 
 @pytest.mark.parametrize("name", ["mobilenet_v2", "yolo_v1", "srgan"])
