@@ -136,6 +136,22 @@ int32_t dnncSessionSync(dnncSession *s);
 /* Tuning and tests: dnnrtSetConvTile on the session's handle (0 = automatic choice); a captured
  * graph is dropped and recorded again by the next replayed run. */
 int32_t dnncSessionSetConvTile(dnncSession *s, int32_t tile);
+/* The measured choice of convolution variant: the reference times cuDNN's algorithms on the build machine's GPU
+ * when it compiles a model and passes the winner as each convolution's `algo` operand
+ * (src/Conversion/ONNXToDNN/ONNXToDNNCommonCUDA.cu:57-111 calculateConvAlgo, Ops/cudnn/Conv.cpp:82-83).  Here a
+ * resident session on the GPU runtime times every variant dnnrtListConvTiles names on every fp16 channels-last
+ * convolution of its program, in place (inside whole passes over the program, `reps` passes per variant, on the
+ * given inputs; on_device: they are device buffers), and an operation gets a variant as its `algo` operand
+ * (DNNRT_CONV_ALGO_BASE + id) when that is faster than the runtime's own choice by more than 3 % in the median.
+ * Returns how many operations got one (0 for programs with nothing to tune and on the host build of the ABI),
+ * -1 on error.  Every variant computes the same sums in the same order per output element or to the kernels'
+ * common tolerance; recorded graphs are dropped.
+ * dnncSessionGetAlgos / SetAlgos: the choices as two variant ids per operation that launches
+ * (dnncProgramComputeOp order; the second is for the second convolution of a fused shortcut pair; 0 = the
+ * runtime's own choice), so that a tuning can be kept beside the model and applied to a later session. */
+int64_t dnncSessionTune(dnncSession *s, const void *const *inputs, int32_t on_device, int32_t reps);
+int64_t dnncSessionGetAlgos(const dnncSession *s, int64_t *algos, int64_t cap);
+int32_t dnncSessionSetAlgos(dnncSession *s, const int64_t *algos, int64_t n);
 /* Debugging, per-inference (occamy) mode: fill the pool when it is allocated, and every tensor's slot when it
  * is carved out of the pool, with `byte` (0..255; -1 switches it off).  With 0xFF a byte that a kernel leaves
  * unwritten, or that is read before its producer ran, shows up as NaN in the results. */
@@ -150,6 +166,12 @@ int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on
 int64_t dnncSessionWeightsBytes(const dnncSession *s);
 /* bytes the last occamy-mode run requested from dnnrtMemPoolInit (-1 before any run) */
 int64_t dnncSessionLastPoolBytes(const dnncSession *s);
+/* The runtime library's device-memory accounting (dnnrtDeviceMemoryStats of the library the session is bound
+ * to): bytes it holds from the device allocator now, the peak of that sum (reset_peak != 0: the peak restarts from
+ * the current value after the read), and the size of the library's static device arrays.  Per process, over all
+ * sessions bound to that library. */
+int32_t dnncSessionDeviceBytes(const dnncSession *s, int64_t *allocated_now, int64_t *allocated_peak,
+                               int64_t *static_bytes, int32_t reset_peak);
 
 #ifdef __cplusplus
 }

@@ -84,11 +84,27 @@ enum { DNNRT_REDUCE_AVG = 5 };
 /* memcpy kinds (src/Dialect/DNN/DNN.td:61-83). */
 enum { DNNRT_H2D = 1, DNNRT_D2H = 2, DNNRT_D2D = 3 };
 
+/* `algo` operand of the convolution calls: BASE + a variant id of dnnrtListConvTiles */
+enum { DNNRT_CONV_ALGO_BASE = 1000 };
+
 /* ---- handle / stream ------------------------------------------------- */
 
 /* DNNAPISpecs.inc:92 "cudnnCreate" (emitted at function entry,
  * src/Conversion/DNNToLLVM/DNNToLLVMCommon.cpp:172-177). */
 int32_t dnnrtCreate(dnnrtHandle_t *handle);
+/* New, for accounting; no counterpart in the reference.  Every byte the
+ * library has taken from the device allocator and not yet returned
+ * (`allocated_now`: pools, dnnrtMalloc, and a handle's reduction scratch when
+ * it could not have the static one), the largest value that sum has had
+ * (`allocated_peak`; reset_peak != 0 makes it `allocated_now` after the read),
+ * and the size of the library's static device arrays (`static_bytes`: the
+ * reduction scratch that the first live handle of a device uses, 8 MiB +
+ * 64 KiB, and that of dnnrtConvBiasActivNoAlloc, 1 MiB + 4 KiB; they are part
+ * of the loaded code object and taken from no allocator).  A program that
+ * runs on the only handle of its device therefore holds its pool and nothing
+ * else.  Counted per process, over all handles; any pointer may be null. */
+int32_t dnnrtDeviceMemoryStats(int64_t *allocated_now, int64_t *allocated_peak,
+                               int64_t *static_bytes, int32_t reset_peak);
 /* DNNAPISpecs.inc:93 "cudnnDestroy". */
 int32_t dnnrtDestroy(dnnrtHandle_t handle);
 /* DNNAPISpecs.inc:94 "cudaStreamCreate" (DNNToLLVMCommon.cpp:208-213). */
@@ -180,7 +196,15 @@ int32_t dnnrtHostFree(void *ptr);
  * (src/Tools/dnn-wrapper/cudnn/CUDNNConvFunc.cpp:9-105).
  * Y = conv2d(X[N,C,H,W], W[K,C/group,R,S]); cross-correlation, dilation 1,
  * pads = {pad_h, pad_w} (symmetric), strides = {stride_h, stride_w}.
- * `workspace`, `workspaceBytes` and `algo` are accepted and ignored. */
+ * `workspace` and `workspaceBytes` are accepted and ignored (no kernel here
+ * needs one).  `algo`: the reference times cuDNN's algorithms when it compiles
+ * a model and passes the winner's number
+ * (src/Conversion/ONNXToDNN/ONNXToDNNCommonCUDA.cu:57-111, Ops/cudnn/Conv.cpp:82-83).
+ * Here DNNRT_CONV_ALGO_BASE + id names the fp16 channels-last variant `id` of
+ * dnnrtListConvTiles: the call uses it where it can run the problem, and the
+ * automatic choice otherwise, as for every other value of `algo` (cuDNN's
+ * numbers name nothing here).  Every variant gives results to the same
+ * tolerance; a handle's dnnrtSetConvTile goes first. */
 void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX,
                 const void *W, const int64_t *dimW, void *workspace,
                 int64_t workspaceBytes, int64_t algo, int64_t group,
@@ -255,17 +279,19 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X,
  * batch-1 kernels (the two reductions are then one sum, rounded once: within
  * an fp32 ulp or two of the chain).  Everywhere else the call runs the two
  * convolutions one after the other with the shortcut's result passing through
- * Y, which gives the chain's bits. */
+ * Y, which gives the chain's bits; `algo` and `algo2` are then the `algo`
+ * operands of the first (closing) and the second (shortcut) convolution. */
 void *dnnrtConvBiasAddConvBiasActiv(
     dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
     const int64_t *dimW, const void *B, const int64_t *pads,
     const int64_t *strides, const void *X2, const int64_t *dimX2,
     const void *W2, const int64_t *dimW2, const void *B2, const int64_t *pads2,
-    const int64_t *strides2, int64_t activMode, void *Y, int32_t dtype);
+    const int64_t *strides2, int64_t activMode, int64_t algo, int64_t algo2,
+    void *Y, int32_t dtype);
 /* No counterpart in the reference.  dnnrtConvBiasActiv for callers that cannot
  * allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  It takes the stream where the other calls
- * take a handle (dnnrtCreate allocates the handle's reduction scratch) and
+ * take a handle (dnnrtCreate may allocate the handle's reduction scratch) and
  * calls no hipMalloc, hipFree or allocating library routine; the scratch its
  * split-reduction kernels need (partial tiles and arrival counters) is a static
  * device array of 1 MiB + 4 KiB that every GPU the library runs on holds until

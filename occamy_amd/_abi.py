@@ -18,6 +18,7 @@ i64, i32, f32 = C.c_int64, C.c_int32, C.c_float
 SIGNATURES = {
     "dnnrtCreate": (i32, [C.POINTER(P)]),
     "dnnrtDestroy": (i32, [P]),
+    "dnnrtDeviceMemoryStats": (i32, [I64P, I64P, I64P, i32]),
     "dnnrtStreamCreate": (i32, [C.POINTER(P)]),
     "dnnrtStreamDestroy": (i32, [P]),
     "dnnrtSetStream": (i32, [P, P]),
@@ -49,7 +50,7 @@ SIGNATURES = {
     "dnnrtConvBiasActiv": (P, [P, P, I64P, P, I64P, P, I64P, P, i64, i64, i64, I64P, I64P, i64, P, i32]),
     "dnnrtConvBiasAddActiv": (P, [P, P, I64P, P, I64P, P, I64P, P, P, i64, i64, i64, I64P, I64P, i64, P, i32]),
     "dnnrtConvBiasActivMaxPool": (P, [P, P, I64P, P, I64P, P, I64P, i64, I64P, I64P, i64, I64P, I64P, I64P, P, I64P, i32]),
-    "dnnrtConvBiasAddConvBiasActiv": (P, [P, P, I64P, P, I64P, P, I64P, I64P, P, I64P, P, I64P, P, I64P, I64P, i64, P, i32]),
+    "dnnrtConvBiasAddConvBiasActiv": (P, [P, P, I64P, P, I64P, P, I64P, I64P, P, I64P, P, I64P, P, I64P, I64P, i64, i64, i64, P, i32]),
     "dnnrtConvBiasActivNoAlloc": (P, [P, P, I64P, P, I64P, P, I64P, i64, I64P, I64P, i64, P, i32]),
     "dnnrtActive": (P, [P, P, I64P, i32, P, i32]),
     "dnnrtTensorOp": (P, [P, i64, P, I64P, i32, P, I64P, i32, P, I64P, i32, f32, i32]),
@@ -89,6 +90,7 @@ ACT_SIGMOID, ACT_RELU, ACT_TANH, ACT_CLIPPED_RELU, ACT_IDENTITY, ACT_LEAKY_RELU 
 OP_ADD, OP_MUL, OP_SQRT = 0, 1, 4
 REDUCE_AVG = 5
 H2D, D2H, D2D = 1, 2, 3
+CONV_ALGO_BASE = 1000
 
 
 def bind(cdll):

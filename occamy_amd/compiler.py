@@ -78,9 +78,13 @@ def lib():
         "dnncSessionRunResident": (C.c_int32, [P, C.POINTER(P), C.POINTER(P), C.c_int32, C.c_int32]),
         "dnncSessionSync": (C.c_int32, [P]),
         "dnncSessionSetConvTile": (C.c_int32, [P, C.c_int32]),
+        "dnncSessionTune": (C.c_int64, [P, C.POINTER(P), C.c_int32, C.c_int32]),
+        "dnncSessionGetAlgos": (C.c_int64, [P, I64P, C.c_int64]),
+        "dnncSessionSetAlgos": (C.c_int32, [P, I64P, C.c_int64]),
         "dnncSessionSetDebugFill": (C.c_int32, [P, C.c_int32]),
         "dnncSessionWeightsBytes": (C.c_int64, [P]),
         "dnncSessionLastPoolBytes": (C.c_int64, [P]),
+        "dnncSessionDeviceBytes": (C.c_int32, [P, I64P, I64P, I64P, C.c_int32]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -329,6 +333,33 @@ class Session:
         if lib().dnncSessionSetConvTile(self._s, tile):
             raise RuntimeError("set_conv_tile: " + _err())
 
+    def tune(self, in_ptrs_or_arrays, on_device=False, reps=7):
+        """Resident mode: time every convolution variant on every fp16 channels-last convolution of the program, in
+        place, and keep the winners as the calls' `algo` operands; returns how many operations got a variant."""
+        if on_device:
+            ip = (C.c_void_p * max(len(in_ptrs_or_arrays), 1))(*in_ptrs_or_arrays)
+        else:
+            keep = [np.ascontiguousarray(a) for a in in_ptrs_or_arrays]
+            ip = (C.c_void_p * max(len(keep), 1))(*[a.ctypes.data for a in keep])
+        n = lib().dnncSessionTune(self._s, ip, int(on_device), reps)
+        if n < 0:
+            raise RuntimeError("tune: " + _err())
+        return n
+
+    def algos(self):
+        """[(variant of the convolution, variant of a fused pair's second convolution)] per operation that launches;
+        0 = the runtime's own choice."""
+        n = lib().dnncSessionGetAlgos(self._s, None, 0)
+        buf = (C.c_int64 * max(n, 1))()
+        lib().dnncSessionGetAlgos(self._s, buf, n)
+        return [(buf[i], buf[i + 1]) for i in range(0, n, 2)]
+
+    def set_algos(self, pairs):
+        flat = [int(v) for p in pairs for v in p]
+        buf = (C.c_int64 * max(len(flat), 1))(*flat)
+        if lib().dnncSessionSetAlgos(self._s, buf, len(flat)):
+            raise RuntimeError("set_algos: " + _err())
+
     def sync(self):
         if lib().dnncSessionSync(self._s):
             raise RuntimeError("sync: " + _err())
@@ -340,3 +371,11 @@ class Session:
     @property
     def last_pool_bytes(self):
         return lib().dnncSessionLastPoolBytes(self._s)
+
+    def device_bytes(self, reset_peak=False):
+        """(bytes the runtime library holds from the device allocator now, the peak of that sum, the size of the
+        library's static device arrays); counted per process over every session bound to the same library."""
+        now, peak, static = C.c_int64(), C.c_int64(), C.c_int64()
+        if lib().dnncSessionDeviceBytes(self._s, C.byref(now), C.byref(peak), C.byref(static), int(reset_peak)):
+            raise RuntimeError("device_bytes: " + _err())
+        return now.value, peak.value, static.value

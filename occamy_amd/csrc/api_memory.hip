@@ -6,6 +6,9 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
+#include <unordered_map>
+
 namespace dnnrt {
 static thread_local char g_err[512] = "";
 void set_error(const char *fmt, ...) {
@@ -30,6 +33,44 @@ __global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *p, unsig
     for (int64_t i = at; i < n && i < at + 16; i++) p[i] = byte;
   }
 }
+}  // namespace dnnrt
+
+namespace dnnrt {
+// Every byte this library takes from the device allocator, counted: the pool, dnnrtMalloc, and a handle's
+// reduction scratch when it cannot have the static one.
+static std::mutex g_mem_mutex;
+static std::unordered_map<void *, int64_t> g_mem_sizes;
+static int64_t g_mem_now = 0, g_mem_peak = 0;
+
+static hipError_t counted_malloc(void **ptr, int64_t bytes) {
+  const int64_t n = bytes > 0 ? bytes : 1;
+  hipError_t e = hipMalloc(ptr, (size_t)n);
+  if (e != hipSuccess) return e;
+  std::lock_guard<std::mutex> lock(g_mem_mutex);
+  g_mem_sizes[*ptr] = n;
+  g_mem_now += n;
+  if (g_mem_now > g_mem_peak) g_mem_peak = g_mem_now;
+  return e;
+}
+static hipError_t counted_free(void *ptr) {
+  if (ptr) {
+    std::lock_guard<std::mutex> lock(g_mem_mutex);
+    auto it = g_mem_sizes.find(ptr);
+    if (it != g_mem_sizes.end()) { g_mem_now -= it->second; g_mem_sizes.erase(it); }
+  }
+  return hipFree(ptr);
+}
+
+// The reduction scratch of a handle (partial tiles, then arrival counters) is a static array of the library: part
+// of the loaded code object, so creating a handle takes nothing from the device allocator and a program's device
+// memory is its pool.  One handle per device holds it at a time; a handle created while another one has it gets
+// buffers of its own from the allocator (and those are counted).
+constexpr int64_t HANDLE_SCRATCH_BYTES = SPLITK_PARTIAL_BYTES + (int64_t)SPLITK_MAX_TILES * sizeof(unsigned);
+static __device__ __align__(256) unsigned char handle_scratch[HANDLE_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+static unsigned char *g_scratch_at[MAX_DEVICES];      // this device's copy of handle_scratch
+static const dnnrtContext *g_scratch_holder[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
 }  // namespace dnnrt
 
 #define HIP_RET(call, what)                                                    \
@@ -65,13 +106,32 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
   c->num_cu = prop.multiProcessorCount;
   c->splitk_partials = nullptr;
   c->splitk_counters = nullptr;
-  if (hipMalloc((void **)&c->splitk_partials, dnnrt::SPLITK_PARTIAL_BYTES) != hipSuccess ||
-      hipMalloc((void **)&c->splitk_counters, dnnrt::SPLITK_MAX_TILES * sizeof(unsigned)) != hipSuccess ||
+  c->scratch_is_static = false;
+  if (dev >= 0 && dev < dnnrt::MAX_DEVICES) {
+    std::lock_guard<std::mutex> lock(dnnrt::g_scratch_mutex);
+    if (!dnnrt::g_scratch_holder[dev]) {
+      if (!dnnrt::g_scratch_at[dev]) {
+        void *at = nullptr;
+        hipError_t e = hipGetSymbolAddress(&at, HIP_SYMBOL(dnnrt::handle_scratch));
+        if (e != hipSuccess || !at) {
+          set_error("dnnrtCreate: hipGetSymbolAddress: %s", hipGetErrorString(e));
+          delete c;
+          return 1;
+        }
+        dnnrt::g_scratch_at[dev] = static_cast<unsigned char *>(at);
+      }
+      c->splitk_partials = reinterpret_cast<float *>(dnnrt::g_scratch_at[dev]);
+      c->splitk_counters = reinterpret_cast<unsigned *>(dnnrt::g_scratch_at[dev] + dnnrt::SPLITK_PARTIAL_BYTES);
+      c->scratch_is_static = true;
+      dnnrt::g_scratch_holder[dev] = c;
+    }
+  }
+  if ((!c->scratch_is_static &&
+       (dnnrt::counted_malloc((void **)&c->splitk_partials, dnnrt::SPLITK_PARTIAL_BYTES) != hipSuccess ||
+        dnnrt::counted_malloc((void **)&c->splitk_counters, dnnrt::SPLITK_MAX_TILES * sizeof(unsigned)) != hipSuccess)) ||
       hipMemset(c->splitk_counters, 0, dnnrt::SPLITK_MAX_TILES * sizeof(unsigned)) != hipSuccess) {
-    set_error("dnnrtCreate: cannot allocate the handle's reduction scratch");
-    (void)hipFree(c->splitk_partials);
-    (void)hipFree(c->splitk_counters);
-    delete c;
+    set_error("dnnrtCreate: cannot set up the handle's reduction scratch");
+    dnnrtDestroy(c);
     return 1;
   }
   c->splitk_partial_bytes = dnnrt::SPLITK_PARTIAL_BYTES;
@@ -84,10 +144,26 @@ int32_t dnnrtCreate(dnnrtHandle_t *handle) {
 
 int32_t dnnrtDestroy(dnnrtHandle_t handle) {
   if (handle) {
-    (void)hipFree(handle->splitk_partials);
-    (void)hipFree(handle->splitk_counters);
+    if (handle->scratch_is_static) {
+      (void)hipDeviceSynchronize();  // the next holder must not meet this handle's kernels (hipFree waits likewise)
+      std::lock_guard<std::mutex> lock(dnnrt::g_scratch_mutex);
+      if (handle->device >= 0 && handle->device < dnnrt::MAX_DEVICES && dnnrt::g_scratch_holder[handle->device] == handle)
+        dnnrt::g_scratch_holder[handle->device] = nullptr;
+    } else {
+      (void)dnnrt::counted_free(handle->splitk_partials);
+      (void)dnnrt::counted_free(handle->splitk_counters);
+    }
   }
   delete handle;
+  return 0;
+}
+
+int32_t dnnrtDeviceMemoryStats(int64_t *allocated_now, int64_t *allocated_peak, int64_t *static_bytes, int32_t reset_peak) {
+  std::lock_guard<std::mutex> lock(dnnrt::g_mem_mutex);
+  if (allocated_now) *allocated_now = dnnrt::g_mem_now;
+  if (allocated_peak) *allocated_peak = dnnrt::g_mem_peak;
+  if (static_bytes) *static_bytes = dnnrt::HANDLE_SCRATCH_BYTES + dnnrt::NOALLOC_PARTIAL_BYTES + (int64_t)dnnrt::NOALLOC_MAX_TILES * (int64_t)sizeof(unsigned);
+  if (reset_peak) dnnrt::g_mem_peak = dnnrt::g_mem_now;
   return 0;
 }
 
@@ -214,7 +290,7 @@ int32_t dnnrtEventDestroy(void *event) {
 
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
   if (!pool || bytes < 0) { set_error("dnnrtMemPoolInit: bad arguments"); return 1; }
-  HIP_RET(hipMalloc(pool, (size_t)(bytes > 0 ? bytes : 1)), "dnnrtMemPoolInit: hipMalloc");
+  HIP_RET(dnnrt::counted_malloc(pool, bytes), "dnnrtMemPoolInit: hipMalloc");
   return 0;
 }
 
@@ -251,12 +327,12 @@ int32_t dnnrtMemcpy(void *dst, void *src, int64_t bytes, int32_t kind, dnnrtStre
 
 int32_t dnnrtMalloc(void **ptr, int64_t bytes) {
   if (!ptr || bytes < 0) { set_error("dnnrtMalloc: bad arguments"); return 1; }
-  HIP_RET(hipMalloc(ptr, (size_t)(bytes > 0 ? bytes : 1)), "dnnrtMalloc: hipMalloc");
+  HIP_RET(dnnrt::counted_malloc(ptr, bytes), "dnnrtMalloc: hipMalloc");
   return 0;
 }
 
 int32_t dnnrtDealloc(void *ptr) {
-  HIP_RET(hipFree(ptr), "dnnrtDealloc");
+  HIP_RET(dnnrt::counted_free(ptr), "dnnrtDealloc");
   return 0;
 }
 

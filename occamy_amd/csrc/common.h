@@ -18,8 +18,9 @@ struct dnnrtContext {
   int device;
   int num_cu;
   // Scratch for reductions split over workgroups: partial tiles and one
-  // arrival counter per output tile (all zero between kernels).  Allocated with
-  // the handle; kernels of one handle run in stream order, so they share it.
+  // arrival counter per output tile (all zero between kernels).  The library's
+  // static array for the first live handle of a device, allocated for any
+  // further one; kernels of one handle run in stream order, so they share it.
   float *splitk_partials;
   unsigned *splitk_counters;
   int64_t splitk_partial_bytes;  // what the two buffers hold
@@ -28,6 +29,7 @@ struct dnnrtContext {
   // dnnrtConvBiasActivNoAlloc): clear the counters a launch uses before it, and refuse a problem whose
   // split would have to shrink to fit instead of shrinking it.
   bool splitk_shared;
+  bool scratch_is_static;  // the two buffers are the library's static array (held by one handle per device), not allocations
   int f16_tile;        // dnnrtSetConvTile: 0 = pick the fp16 convolution variant by problem size, otherwise one of F16_TILE_IDS
 };
 

@@ -305,10 +305,21 @@ static void *conv_f32_nchw(const dnnrtContext *ctx, const ConvShape &s, const fl
   return Y;
 }
 
+// The `algo` operand of the convolution calls: DNNRT_CONV_ALGO_BASE + id asks for the fp16 channels-last variant
+// `id` of dnnrtListConvTiles where that variant can run the problem (else, and for every other value, the
+// automatic choice).  Values below the base are cuDNN's algorithm numbers, which name nothing here.
+static int variant_of_algo(int64_t algo) {
+  if (algo <= DNNRT_CONV_ALGO_BASE || algo >= DNNRT_CONV_ALGO_BASE + 1000) return 0;
+  const int id = (int)(algo - DNNRT_CONV_ALGO_BASE);
+  for (const int *t = F16_TILE_IDS; *t; t++)
+    if (*t == id) return id;
+  return 0;
+}
+
 static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, const int64_t *dX,
                            const void *W, const int64_t *dW, const void *B, const void *Z, int64_t group,
                            const int64_t *pads, const int64_t *strides, int act, void *Y,
-                           int32_t dtype) {
+                           int32_t dtype, int64_t algo = 0) {
   if (!h) DNNRT_FAIL("%s: null handle", who);
   if (!X || !W || !Y) DNNRT_FAIL("%s: null tensor", who);
   // an empty batch is no work: nothing is launched and Y is left as it is
@@ -325,6 +336,7 @@ static void *conv_dispatch(const char *who, dnnrtHandle_t h, const void *X, cons
     a.N = s.N; a.C = s.C; a.H = s.H; a.W = s.W; a.K = s.K; a.Cg = s.Cg; a.R = s.R; a.S = s.S;
     a.P = s.P; a.Q = s.Q; a.ph = s.ph; a.pw = s.pw; a.sh = s.sh; a.sw = s.sw; a.group = s.group;
     a.act = act; a.act_coef = h->act_coef; a.format = h->format;
+    a.variant = variant_of_algo(algo);
     if (!launch_conv_f16(h, a)) return nullptr;
     return Y;
   }
@@ -411,22 +423,22 @@ void *dnnrtConvBiasActivNoAlloc(dnnrtStream_t stream, const void *X, const int64
 void *dnnrtConv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
                 const int64_t *dimW, void *workspace, int64_t workspaceBytes, int64_t algo,
                 int64_t group, const int64_t *pads, const int64_t *strides, void *Y, int32_t dtype) {
-  (void)workspace; (void)workspaceBytes; (void)algo;
+  (void)workspace; (void)workspaceBytes;
   return dnnrt::conv_dispatch("dnnrtConv", handle, X, dimX, W, dimW, nullptr, nullptr, group, pads, strides,
-                              DNNRT_ACT_IDENTITY, Y, dtype);
+                              DNNRT_ACT_IDENTITY, Y, dtype, algo);
 }
 
 void *dnnrtConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
                          const int64_t *dimW, const void *B, const int64_t *dimB, void *workspace,
                          int64_t workspaceBytes, int64_t algo, int64_t group, const int64_t *pads,
                          const int64_t *strides, int64_t activMode, void *Y, int32_t dtype) {
-  (void)workspace; (void)workspaceBytes; (void)algo;
+  (void)workspace; (void)workspaceBytes;
   if (!dnnrt::fusable_act(activMode))
     DNNRT_FAIL("dnnrtConvBiasActiv: activMode %ld (1 ReLU, 3 clipped ReLU, 5 identity, 6 leaky ReLU)", (long)activMode);
   if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
     DNNRT_FAIL("dnnrtConvBiasActiv: bias must hold K values");
   return dnnrt::conv_dispatch("dnnrtConvBiasActiv", handle, X, dimX, W, dimW, B, nullptr, group, pads,
-                              strides, (int)activMode, Y, dtype);
+                              strides, (int)activMode, Y, dtype, algo);
 }
 
 void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
@@ -469,7 +481,8 @@ void *dnnrtConvBiasActivMaxPool(dnnrtHandle_t handle, const void *X, const int64
 void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W, const int64_t *dimW,
                                     const void *B, const int64_t *pads, const int64_t *strides, const void *X2,
                                     const int64_t *dimX2, const void *W2, const int64_t *dimW2, const void *B2,
-                                    const int64_t *pads2, const int64_t *strides2, int64_t activMode, void *Y, int32_t dtype) {
+                                    const int64_t *pads2, const int64_t *strides2, int64_t activMode, int64_t algo,
+                                    int64_t algo2, void *Y, int32_t dtype) {
   const char *who = "dnnrtConvBiasAddConvBiasActiv";
   if (!handle) DNNRT_FAIL("%s: null handle", who);
   if (!X || !W || !X2 || !W2 || !Y) DNNRT_FAIL("%s: null tensor", who);
@@ -524,8 +537,8 @@ void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t handle, const void *X, const i
   }
   // ... and everywhere else the two calls it stands for, the shortcut's result passing through Y itself: the closing
   // call reads its residual operand and writes its result element by element, each by the thread that read it
-  if (!dnnrt::conv_dispatch(who, handle, X2, dimX2, W2, dimW2, B2, nullptr, 1, pads2, strides2, DNNRT_ACT_IDENTITY, Y, dtype)) return nullptr;
-  return dnnrt::conv_dispatch(who, handle, X, dimX, W, dimW, B, Y, 1, pads, strides, (int)activMode, Y, dtype);
+  if (!dnnrt::conv_dispatch(who, handle, X2, dimX2, W2, dimW2, B2, nullptr, 1, pads2, strides2, DNNRT_ACT_IDENTITY, Y, dtype, algo2)) return nullptr;
+  return dnnrt::conv_dispatch(who, handle, X, dimX, W, dimW, B, Y, 1, pads, strides, (int)activMode, Y, dtype, algo);
 }
 
 void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X, const int64_t *dimX, const void *W,
@@ -533,14 +546,14 @@ void *dnnrtConvBiasAddActiv(dnnrtHandle_t handle, const void *X, const int64_t *
                             void *workspace, int64_t workspaceBytes, int64_t algo, int64_t group,
                             const int64_t *pads, const int64_t *strides, int64_t activMode, void *Y,
                             int32_t dtype) {
-  (void)workspace; (void)workspaceBytes; (void)algo;
+  (void)workspace; (void)workspaceBytes;
   if (!dnnrt::fusable_act(activMode))
     DNNRT_FAIL("dnnrtConvBiasAddActiv: activMode %ld (1 ReLU, 3 clipped ReLU, 5 identity, 6 leaky ReLU)", (long)activMode);
   if (!B || !dimB || !dimW || dnnrt::numel(dimB, 4) != dimW[0])
     DNNRT_FAIL("dnnrtConvBiasAddActiv: bias must hold K values");
   if (!Z) DNNRT_FAIL("dnnrtConvBiasAddActiv: null residual tensor");
   return dnnrt::conv_dispatch("dnnrtConvBiasAddActiv", handle, X, dimX, W, dimW, B, Z, group, pads,
-                              strides, (int)activMode, Y, dtype);
+                              strides, (int)activMode, Y, dtype, algo);
 }
 
 }  // extern "C"

@@ -27,6 +27,7 @@ struct ConvF16Args {
   int act;     // DNNRT_ACT_{IDENTITY, RELU, CLIPPED_RELU, LEAKY_RELU}
   float act_coef;  // ceiling / slope of the last two
   int format;  // physical layout of X and Y (DNNRT_NCHW / NHWC / NCHW_TO_NHWC)
+  int variant;  // the call's own choice of channels-last variant (its `algo` operand), used where it can run the problem; 0: none
   unsigned magic_pq, magic_q;  // filled in by the launcher: ceil(2^32 / (P*Q)), ceil(2^32 / Q)
   unsigned magic_pw, magic_hp;  // (conv_f16_patch.hip) ceil(2^32 / (W + 2)), ceil(2^32 / (H + 2))
   // a second 1x1 convolution onto the same result (launch_conv_f16_dual): input N x H2 x W2 x C2 read with strides

@@ -807,7 +807,8 @@ bool launch_conv_f16(const dnnrtContext *ctx, const ConvF16Args &a) {
     // first, so that an XCD touches a slice of a large filter only, changed
     // nothing on the 7x7 layers).
     // 0 = automatic; > 0 forced (tuning and tests); < 0: that variant where it can run the problem, else automatic
-    const int tile_sel = ctx->f16_tile;
+    // the handle's forced variant (tests, sweeps) goes before the call's own (its `algo` operand, a tuned program)
+    const int tile_sel = ctx->f16_tile ? ctx->f16_tile : -a.variant;
     int sel = tile_sel;
     if (sel < 0) {
       const int want = -sel, steps = a.R * a.S * (a.C / BKF);

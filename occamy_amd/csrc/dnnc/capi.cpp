@@ -334,6 +334,27 @@ int32_t dnncSessionSetConvTile(dnncSession *s, int32_t tile) {
   return s->s.set_conv_tile(tile, err) ? 0 : fail(err);
 }
 
+int64_t dnncSessionTune(dnncSession *s, const void *const *inputs, int32_t on_device, int32_t reps) {
+  if (!s || !inputs) { fail("dnncSessionTune: bad arguments"); return -1; }
+  std::string err;
+  int64_t changed = 0;
+  if (!s->s.tune(inputs, on_device, reps, changed, err)) { fail(err); return -1; }
+  return changed;
+}
+
+int64_t dnncSessionGetAlgos(const dnncSession *s, int64_t *algos, int64_t cap) {
+  if (!s) { fail("dnncSessionGetAlgos: null session"); return -1; }
+  const std::vector<int64_t> a = s->s.algos();
+  for (size_t i = 0; algos && i < a.size() && (int64_t)i < cap; i++) algos[i] = a[i];
+  return (int64_t)a.size();
+}
+
+int32_t dnncSessionSetAlgos(dnncSession *s, const int64_t *algos, int64_t n) {
+  if (!s) return fail("dnncSessionSetAlgos: null session");
+  std::string err;
+  return s->s.set_algos(algos, n, err) ? 0 : fail(err);
+}
+
 int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on_device, float *ms, int64_t cap) {
   if (!s || !inputs) { fail("dnncSessionProfile: bad arguments"); return -1; }
   std::vector<float> t;
@@ -345,5 +366,9 @@ int64_t dnncSessionProfile(dnncSession *s, const void *const *inputs, int32_t on
 
 int64_t dnncSessionWeightsBytes(const dnncSession *s) { return s ? s->s.weights_bytes : -1; }
 int64_t dnncSessionLastPoolBytes(const dnncSession *s) { return s ? s->s.last_pool_bytes : -1; }
+int32_t dnncSessionDeviceBytes(const dnncSession *s, int64_t *allocated_now, int64_t *allocated_peak, int64_t *static_bytes, int32_t reset_peak) {
+  if (!s) { g_err = "dnncSessionDeviceBytes: no session"; return 1; }
+  return s->s.device_bytes(allocated_now, allocated_peak, static_bytes, reset_peak);
+}
 
 }  // extern "C"

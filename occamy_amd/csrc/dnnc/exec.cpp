@@ -31,8 +31,8 @@ namespace dnnc {
 bool load_runtime(const std::string &path, RuntimeApi &rt, std::string &err) {
   rt.dl = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
   if (!rt.dl) { err = std::string("cannot load runtime library: ") + dlerror(); return false; }
-  LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
-  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtSetConvTile); LOAD(dnnrtMemFill); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
+  LOAD(dnnrtCreate); LOAD(dnnrtDestroy); LOAD(dnnrtDeviceMemoryStats); LOAD(dnnrtStreamCreate); LOAD(dnnrtStreamDestroy);
+  LOAD(dnnrtSetStream); LOAD(dnnrtSetTensorFormat); LOAD(dnnrtSetFilterLayout); LOAD(dnnrtSetActivationCoef); LOAD(dnnrtSetConvTile); LOAD(dnnrtListConvTiles); LOAD(dnnrtMemFill); LOAD(dnnrtMatmulNdBias); LOAD(dnnrtAttention); LOAD(dnnrtSync); LOAD(dnnrtLastError);
   LOAD(dnnrtIsHostBackend); LOAD(dnnrtGraphBegin); LOAD(dnnrtGraphEnd); LOAD(dnnrtGraphLaunch);
   LOAD(dnnrtGraphDestroy); LOAD(dnnrtEventCreate); LOAD(dnnrtEventRecord); LOAD(dnnrtEventElapsedMs);
   LOAD(dnnrtEventDestroy); LOAD(dnnrtMemPoolInit); LOAD(dnnrtMemOffset); LOAD(dnnrtMemcpy);
@@ -272,18 +272,18 @@ bool Session::issue(const Op *op, std::string &err) {
   auto pad4 =[](const Shape &s) { Shape o = s; while (o.size() < 4) o.push_back(1); return o; };
   switch (op->kind) {
     case OP_CONVFWD:
-      r = rt.dnnrtConv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), 0, op->algo, op->group,
+      r = rt.dnnrtConv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), 0, algo_operand(op, 0, op->algo), op->group,
                        op->pads.data(), op->strides.data(), out, dt);
       break;
     case OP_CONV_BIAS_ACTIV: {
       const int64_t dimB[4] = {1, op->dimB[0], 1, 1};
-      r = rt.dnnrtConvBiasActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, P(3), 0, 1,
+      r = rt.dnnrtConvBiasActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, P(3), 0, algo_operand(op, 0, 1),
                                 op->group, op->pads.data(), op->strides.data(), op->mode, out, dt);
       break;
     }
     case OP_CONV_BIAS_ADD_ACTIV: {  // operands: x, w, bias, workspace, z, out
       const int64_t dimB[4] = {1, op->dimB[0], 1, 1};
-      r = rt.dnnrtConvBiasAddActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, P(4), P(3), 0, 1,
+      r = rt.dnnrtConvBiasAddActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), dimB, P(4), P(3), 0, algo_operand(op, 0, 1),
                                    op->group, op->pads.data(), op->strides.data(), op->mode, out, dt);
       break;
     }
@@ -297,7 +297,7 @@ bool Session::issue(const Op *op, std::string &err) {
     case OP_CONV_ADD_CONV_ACTIV:  // operands: x, w, bias, workspace, x2, w2, bias2, workspace2, out
       r = rt.dnnrtConvBiasAddConvBiasActiv(handle, P(0), op->dimA.data(), P(1), op->dimB.data(), P(2), op->pads.data(), op->strides.data(),
                                            P(4), op->dimA2.data(), P(5), op->dimB2.data(), P(6), op->pads2.data(), op->strides2.data(),
-                                           op->mode, out, dt);
+                                           op->mode, algo_operand(op, 0, 1), algo_operand(op, 1, 1), out, dt);
       break;
     case OP_ACTIVATION: {
       const Shape d = pad4(op->dimA);  // the lowering pads the dims to 4 with trailing ones
@@ -713,6 +713,115 @@ bool Session::profile_classes(const void *const *inputs, int on_device, const st
   rt.dnnrtEventDestroy(e0);
   rt.dnnrtEventDestroy(e1);
   return ok;
+}
+
+int64_t Session::algo_operand(const Op *op, int which, int64_t reference_value) const {
+  const auto it = tuned.find(op);
+  const int64_t id = it == tuned.end() ? 0 : (which ? it->second.second : it->second.first);
+  return id > 0 ? DNNRT_CONV_ALGO_BASE + id : reference_value;
+}
+
+static bool tunable(const Op *op) {
+  return (op->kind == OP_CONVFWD || op->kind == OP_CONV_BIAS_ACTIV || op->kind == OP_CONV_BIAS_ADD_ACTIV || op->kind == OP_CONV_ADD_CONV_ACTIV) &&
+         !op->operands.empty() && op->operands.back()->dtype == F16;
+}
+
+std::vector<int64_t> Session::algos() const {
+  std::vector<int64_t> out;
+  for (const Op *op : prog->ops) {
+    if (!launches(op)) continue;
+    const auto it = tuned.find(op);
+    out.push_back(it == tuned.end() ? 0 : it->second.first);
+    out.push_back(it == tuned.end() ? 0 : it->second.second);
+  }
+  return out;
+}
+
+bool Session::set_algos(const int64_t *a, int64_t n, std::string &err) {
+  std::vector<const Op *> compute;
+  for (const Op *op : prog->ops)
+    if (launches(op)) compute.push_back(op);
+  if (!a || n != 2 * (int64_t)compute.size()) { err = "set_algos: two values per operation that launches are expected"; return false; }
+  tuned.clear();
+  for (size_t i = 0; i < compute.size(); i++) {
+    if (a[2 * i] < 0 || a[2 * i + 1] < 0 || a[2 * i] >= 1000 || a[2 * i + 1] >= 1000) { err = "set_algos: a variant id is 0 .. 999"; return false; }
+    if ((a[2 * i] || a[2 * i + 1]) && tunable(compute[i])) tuned[compute[i]] = {a[2 * i], a[2 * i + 1]};
+  }
+  drop_graphs();
+  return true;
+}
+
+bool Session::tune(const void *const *inputs, int on_device, int reps, int64_t &changed, std::string &err) {
+  changed = 0;
+  if (mode != MODE_RESIDENT) { err = "tuning needs a resident session"; return false; }
+  std::vector<const Op *> compute;
+  for (const Op *op : prog->ops)
+    if (launches(op)) compute.push_back(op);
+  bool any = false;
+  for (const Op *op : compute) any = any || tunable(op);
+  if (host_backend || !prog->channels_last || !any) return true;
+  std::vector<int32_t> ids((size_t)std::max(rt.dnnrtListConvTiles(nullptr, 0), 0));
+  rt.dnnrtListConvTiles(ids.data(), (int32_t)ids.size());
+  reps = std::max(reps, 3);
+  const std::map<const Op *, std::pair<int64_t, int64_t>> before = tuned;
+  // median per operation over `reps` profiled passes with the current choices
+  auto measure = [&](std::vector<float> &med) -> bool {
+    std::vector<std::vector<float>> runs;
+    std::vector<float> ms;
+    if (!profile_resident(inputs, on_device, false, ms, err)) return false;  // one pass to settle (code, caches)
+    for (int r = 0; r < reps; r++) {
+      if (!profile_resident(inputs, on_device, false, ms, err)) return false;
+      runs.push_back(ms);
+    }
+    med.assign(compute.size(), 0.f);
+    for (size_t i = 0; i < compute.size(); i++) {
+      std::vector<float> v;
+      for (const auto &r : runs) v.push_back(r[i]);
+      std::sort(v.begin(), v.end());
+      med[i] = v[v.size() / 2];
+    }
+    return true;
+  };
+  bool ok = true;
+  for (int which = 0; which < 2 && ok; which++) {  // 0: every operation's (first) convolution; 1: the second one of the pairs
+    std::vector<const Op *> targets;
+    for (const Op *op : compute)
+      if (tunable(op) && (which == 0 || op->kind == OP_CONV_ADD_CONV_ACTIV)) targets.push_back(op);
+    if (targets.empty()) break;
+    const auto chosen = tuned;  // what this round starts from
+    auto with = [&](int64_t id) {
+      tuned = chosen;
+      for (const Op *op : targets) {
+        auto &t = tuned[op];
+        (which ? t.second : t.first) = id;
+      }
+    };
+    std::vector<float> base;
+    with(0);
+    ok = measure(base);
+    std::vector<float> best = base;
+    std::vector<int64_t> best_id(compute.size(), 0);
+    for (size_t c = 0; ok && c < ids.size(); c++) {
+      std::vector<float> t;
+      with(ids[c]);
+      ok = measure(t);
+      for (size_t i = 0; ok && i < compute.size(); i++)
+        if (t[i] < best[i]) { best[i] = t[i]; best_id[i] = ids[c]; }
+    }
+    tuned = chosen;
+    for (size_t i = 0; ok && i < compute.size(); i++) {
+      if (std::find(targets.begin(), targets.end(), compute[i]) == targets.end()) continue;
+      auto &t = tuned[compute[i]];
+      (which ? t.second : t.first) = best[i] < 0.97f * base[i] ? best_id[i] : 0;
+    }
+  }
+  if (!ok) { tuned = before; drop_graphs(); return false; }
+  for (auto it = tuned.begin(); it != tuned.end();) {
+    if (!it->second.first && !it->second.second) it = tuned.erase(it);
+    else { changed++; ++it; }
+  }
+  drop_graphs();
+  return true;
 }
 
 bool Session::set_conv_tile(int tile, std::string &err) {

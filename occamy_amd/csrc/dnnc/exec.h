@@ -13,6 +13,7 @@ struct RuntimeApi {
   void *dl = nullptr;
   decltype(&::dnnrtCreate) dnnrtCreate = nullptr;
   decltype(&::dnnrtDestroy) dnnrtDestroy = nullptr;
+  decltype(&::dnnrtDeviceMemoryStats) dnnrtDeviceMemoryStats = nullptr;
   decltype(&::dnnrtStreamCreate) dnnrtStreamCreate = nullptr;
   decltype(&::dnnrtStreamDestroy) dnnrtStreamDestroy = nullptr;
   decltype(&::dnnrtSetStream) dnnrtSetStream = nullptr;
@@ -63,6 +64,7 @@ struct RuntimeApi {
   decltype(&::dnnrtGather) dnnrtGather = nullptr;
   decltype(&::dnnrtSetActivationCoef) dnnrtSetActivationCoef = nullptr;
   decltype(&::dnnrtSetConvTile) dnnrtSetConvTile = nullptr;
+  decltype(&::dnnrtListConvTiles) dnnrtListConvTiles = nullptr;
   decltype(&::dnnrtMemFill) dnnrtMemFill = nullptr;
   decltype(&::dnnrtMatmulNdBias) dnnrtMatmulNdBias = nullptr;
   decltype(&::dnnrtAttention) dnnrtAttention = nullptr;
@@ -95,6 +97,20 @@ class Session {
   bool profile_classes(const void *const *inputs, int on_device, const std::vector<const Op *> &compute,
                        std::vector<float> &ms, std::string &err);
 
+  // The measured choice of convolution variant, where the reference times cuDNN's algorithms at compile time
+  // and passes the winner as the call's `algo` operand (src/Conversion/ONNXToDNN/ONNXToDNNCommonCUDA.cu:57-111).
+  // Resident sessions on the GPU runtime: every variant the runtime lists is tried on every convolution of the
+  // program in place, i.e. timed inside whole passes over the program (a layer's operands are then where the
+  // layers before it leave them: in HBM or in a cache); a variant replaces the runtime's own choice for an
+  // operation when it is faster by more than 3 % in the median of `reps` passes.  `changed`: how many operations
+  // got a variant.  A session on the host build of the ABI, or a program without fp16 channels-last convolutions,
+  // has nothing to tune (changed = 0).
+  bool tune(const void *const *inputs, int on_device, int reps, int64_t &changed, std::string &err);
+  // The choices, two per operation that launches (dnncProgramComputeOp order): the `algo` operand and, for a
+  // fused shortcut pair, that of its second convolution; 0 = the runtime's own choice.
+  std::vector<int64_t> algos() const;
+  bool set_algos(const int64_t *a, int64_t n, std::string &err);
+
   const Program *prog = nullptr;
   int mode = MODE_OCCAMY;
   int64_t weights_bytes = 0;     // bytes of the constants arena (resident mode)
@@ -103,6 +119,10 @@ class Session {
   // producer ran, a NaN in the results.
   int debug_fill = -1;
   int64_t last_pool_bytes = -1;  // bytes the last occamy-mode run asked the runtime for
+  // the bound runtime library's device-memory accounting (dnnrtDeviceMemoryStats)
+  int device_bytes(int64_t *now, int64_t *peak, int64_t *static_bytes, int reset_peak) const {
+    return rt.dnnrtDeviceMemoryStats ? rt.dnnrtDeviceMemoryStats(now, peak, static_bytes, reset_peak) : 1;
+  }
 
  private:
   RuntimeApi rt;
@@ -121,6 +141,8 @@ class Session {
   std::vector<void *> graph_key;  // the addresses `graph` was recorded with
   void drop_graphs();
   std::vector<void *> ptr;  // value id -> address (host or device)
+  std::map<const Op *, std::pair<int64_t, int64_t>> tuned;  // operation -> variant ids of its one or two convolutions (0: automatic)
+  int64_t algo_operand(const Op *op, int which, int64_t reference_value) const;
   std::map<size_t, void *> arg_home;  // resident mode: value id of a function argument's pool slot -> its address in the pool
   std::vector<const Op *> direct_out;  // the result copies of the current run that are not needed for that reason
   std::map<size_t, void *> out_home;  // ... and of a result's pool tensor, when results are written where the caller wants them

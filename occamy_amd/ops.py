@@ -92,14 +92,14 @@ class Ops:
         self._check(self.lib.dnnrtDealloc(p), "dnnrtDealloc")
 
     # -- compute ---------------------------------------------------------------
-    def conv(self, X, dimX, W, dimW, pads, strides, Y, group=1, dtype=_abi.F32):
-        return self._ret(self.lib.dnnrtConv(self.handle, X, dims(dimX), W, dims(dimW), None, 0, 0,
+    def conv(self, X, dimX, W, dimW, pads, strides, Y, group=1, dtype=_abi.F32, algo=0):
+        return self._ret(self.lib.dnnrtConv(self.handle, X, dims(dimX), W, dims(dimW), None, 0, algo,
                                             group, dims(pads), dims(strides), Y, dtype), "dnnrtConv")
 
-    def conv_bias_activ(self, X, dimX, W, dimW, B, pads, strides, activ, Y, group=1, dtype=_abi.F32):
+    def conv_bias_activ(self, X, dimX, W, dimW, B, pads, strides, activ, Y, group=1, dtype=_abi.F32, algo=1):
         dimB = [1, dimW[0], 1, 1]
         return self._ret(self.lib.dnnrtConvBiasActiv(self.handle, X, dims(dimX), W, dims(dimW), B,
-                                                     dims(dimB), None, 0, 1, group, dims(pads),
+                                                     dims(dimB), None, 0, algo, group, dims(pads),
                                                      dims(strides), activ, Y, dtype),
                          "dnnrtConvBiasActiv")
 
@@ -110,10 +110,10 @@ class Ops:
                                                             dims(pads), dims(strides), activ, Y, dtype),
                          "dnnrtConvBiasActivNoAlloc")
 
-    def conv_bias_add_activ(self, X, dimX, W, dimW, B, Z, pads, strides, activ, Y, group=1, dtype=_abi.F32):
+    def conv_bias_add_activ(self, X, dimX, W, dimW, B, Z, pads, strides, activ, Y, group=1, dtype=_abi.F32, algo=1):
         dimB = [1, dimW[0], 1, 1]
         return self._ret(self.lib.dnnrtConvBiasAddActiv(self.handle, X, dims(dimX), W, dims(dimW), B,
-                                                        dims(dimB), Z, None, 0, 1, group, dims(pads),
+                                                        dims(dimB), Z, None, 0, algo, group, dims(pads),
                                                         dims(strides), activ, Y, dtype),
                          "dnnrtConvBiasAddActiv")
 
@@ -126,10 +126,10 @@ class Ops:
                          "dnnrtConvBiasActivMaxPool")
 
     def conv_bias_add_conv_bias_activ(self, X, dimX, W, dimW, B, pads, strides, X2, dimX2, W2, dimW2, B2, pads2, strides2, activ, Y,
-                                      dtype=_abi.F16):
+                                      dtype=_abi.F16, algo=0, algo2=0):
         return self._ret(self.lib.dnnrtConvBiasAddConvBiasActiv(self.handle, X, dims(dimX), W, dims(dimW), B, dims(pads), dims(strides),
                                                                 X2, dims(dimX2), W2, dims(dimW2), B2, dims(pads2), dims(strides2),
-                                                                activ, Y, dtype),
+                                                                activ, algo, algo2, Y, dtype),
                          "dnnrtConvBiasAddConvBiasActiv")
 
     def active(self, X, dimX, mode, Y, dtype=_abi.F32):

@@ -188,13 +188,42 @@ int32_t dnnrtEventElapsedMs(void *a, void *b, float *ms) { *ms = (float)(*(doubl
 int32_t dnnrtEventDestroy(void *e) { free(e); return 0; }
 
 /* wrapDNNMemPoolInit.cpp:19-29 / wrapDNNMalloc.cpp: one allocation. */
+/* "Device" memory of the host build is heap memory behind a 64-byte header that holds the block's size, so that
+ * the same accounting call exists here (dnnrtDeviceMemoryStats): bytes taken and not yet returned, and their peak. */
+static int64_t g_mem_now = 0, g_mem_peak = 0;
 int32_t dnnrtMemPoolInit(void **pool, int64_t bytes) {
-  *pool = malloc((size_t)(bytes > 0 ? bytes : 1));
-  return *pool ? 0 : 1;
+  const int64_t n = bytes > 0 ? bytes : 1;
+  void *base = NULL;
+  if (posix_memalign(&base, 64, (size_t)n + 64)) { *pool = NULL; return 1; }
+  *(int64_t *)base = n;
+  *pool = (char *)base + 64;
+#pragma omp critical(dnnrt_mem)
+  {
+    g_mem_now += n;
+    if (g_mem_now > g_mem_peak) g_mem_peak = g_mem_now;
+  }
+  return 0;
 }
 int32_t dnnrtMalloc(void **p, int64_t bytes) { return dnnrtMemPoolInit(p, bytes); }
-int32_t dnnrtDealloc(void *p) { free(p); return 0; }
-int32_t dnnrtHostAlloc(void **p, int64_t bytes) { return dnnrtMemPoolInit(p, bytes); }
+int32_t dnnrtDealloc(void *p) {
+  if (!p) return 0;
+  void *base = (char *)p - 64;
+#pragma omp critical(dnnrt_mem)
+  g_mem_now -= *(int64_t *)base;
+  free(base);
+  return 0;
+}
+int32_t dnnrtDeviceMemoryStats(int64_t *allocated_now, int64_t *allocated_peak, int64_t *static_bytes, int32_t reset_peak) {
+  if (allocated_now) *allocated_now = g_mem_now;
+  if (allocated_peak) *allocated_peak = g_mem_peak;
+  if (static_bytes) *static_bytes = 0;
+  if (reset_peak) g_mem_peak = g_mem_now;
+  return 0;
+}
+int32_t dnnrtHostAlloc(void **p, int64_t bytes) {
+  *p = malloc((size_t)(bytes > 0 ? bytes : 1));
+  return *p ? 0 : 1;
+}
 int32_t dnnrtHostFree(void *p) { free(p); return 0; }
 /* wrapDNNMemOffset.cpp:26: *p = base + offset. */
 int32_t dnnrtMemOffset(void **p, void *base, int64_t off, int64_t bytes) {
@@ -721,7 +750,8 @@ void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t h, const void *X, const int64_
                                     const int64_t *strides, const void *X2, const int64_t *dX2,
                                     const void *W2, const int64_t *dW2, const void *B2,
                                     const int64_t *pads2, const int64_t *strides2, int64_t act,
-                                    void *Y, int32_t dtype) {
+                                    int64_t algo, int64_t algo2, void *Y, int32_t dtype) {
+  (void)algo; (void)algo2;
   if (bad_dtype(dtype)) FAIL("convBiasAddConvBiasActiv: bad dtype");
   const int64_t P = (dX2[2] + 2 * pads2[0] - dW2[2]) / strides2[0] + 1,
                 Q = (dX2[3] + 2 * pads2[1] - dW2[3]) / strides2[1] + 1;

@@ -96,7 +96,7 @@ for rank in (2, 3, 4, 6):
         MAP[f"CUDATranspose{rank}D{ty}Func"] = ("dnnrtTranspose", handle_first_dtype_last)
 
 # entry points with no row in the reference's table (include/dnnrt.h says "New" on each)
-NEW = {"dnnrtLastError", "dnnrtIsHostBackend", "dnnrtSetStream", "dnnrtSetTensorFormat", "dnnrtSetFilterLayout",
+NEW = {"dnnrtLastError", "dnnrtIsHostBackend", "dnnrtDeviceMemoryStats", "dnnrtSetStream", "dnnrtSetTensorFormat", "dnnrtSetFilterLayout",
        "dnnrtSetActivationCoef", "dnnrtListConvTiles", "dnnrtSetConvTile", "dnnrtSync", "dnnrtGraphBegin", "dnnrtGraphEnd",
        "dnnrtGraphLaunch", "dnnrtGraphDestroy", "dnnrtEventCreate", "dnnrtEventRecord", "dnnrtEventElapsedMs",
        "dnnrtEventDestroy", "dnnrtHostAlloc", "dnnrtHostFree", "dnnrtMemFill", "dnnrtConvBiasAddActiv", "dnnrtConvBiasActivNoAlloc", "dnnrtConvBiasActivMaxPool", "dnnrtConvBiasAddConvBiasActiv",

@@ -40,6 +40,20 @@ def test_single_conv():
     assert a[0].shape == (1, 64, 56, 56) and (a[0] >= 0).all()
 
 
+def test_device_memory_accounting_of_the_executor():
+    # what the executor takes from the runtime's allocator per inference is the planned pool and nothing else
+    # (the host build of the ABI counts its heap blocks the way the GPU build counts hipMalloc)
+    g, inputs = models.resnet50(image=32, classes=10)
+    p = g.compile()
+    s = p.session(compiler.MODE_OCCAMY, runtime_library=ORACLE_PATH)
+    base, _, static = s.device_bytes(reset_peak=True)
+    assert static == 0
+    s.run(*inputs)
+    now, peak, _ = s.device_bytes()
+    assert now == base and peak - base == p.pool_bytes
+    s.close()
+
+
 def test_modes_and_flags_agree():
     small = lambda: models.resnet50(image=32, classes=10)  # noqa: E731
     base = check(small)

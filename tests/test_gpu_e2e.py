@@ -53,6 +53,29 @@ def test_occamy_mode_matches_oracle(name, oracle_outputs):
         close(o, r)
 
 
+@pytest.mark.parametrize("name", ["single_conv", "resnet50", "mobilenet_v2", "bert_2_layers"])
+def test_device_memory_is_the_planned_pool(name):
+    """Every byte the runtime library takes from the device allocator is counted (dnnrtDeviceMemoryStats).  Per
+    inference (the reference's semantics) the peak of a run is the planned pool, to the byte, and nothing is held
+    before or after it: the handle's reduction scratch is the library's static array (8 MiB + 64 KiB, plus the
+    1 MiB + 4 KiB of the entry point that allocates nothing), not an allocation.  Resident: pool + the constants'
+    arena, held for the session's life."""
+    g, inputs = CONFIGS[name]()
+    p = g.compile()
+    s = p.session(compiler.MODE_OCCAMY)
+    base, _, static = s.device_bytes(reset_peak=True)
+    assert static == (8 << 20) + (64 << 10) + (1 << 20) + (4 << 10)
+    s.run(*inputs)
+    now, peak, _ = s.device_bytes()
+    assert now == base and peak - base == p.pool_bytes == s.last_pool_bytes
+    s.close()
+    s = p.session(compiler.MODE_RESIDENT)
+    s.run(*inputs)
+    now, peak, _ = s.device_bytes()
+    assert now - base == peak - base == p.pool_bytes + s.weights_bytes
+    s.close()
+
+
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_fused_program_matches_oracle(name, oracle_outputs):
     out, _ = run(CONFIGS[name], fusion=True)
