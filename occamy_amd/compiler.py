@@ -16,7 +16,8 @@ import numpy as np
 from . import _abi
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-DNNC_PATH = os.path.join(_HERE, "lib", "libdnnc.so")
+# DNNC_PATH in the environment names another build of the same library (the sanitizer build, `make asan`)
+DNNC_PATH = os.environ.get("DNNC_PATH") or os.path.join(_HERE, "lib", "libdnnc.so")
 
 F32, F16, I64 = 0, 1, 2
 _NP = {F32: np.float32, F16: np.float16, I64: np.int64}

@@ -226,6 +226,50 @@ def test_resnet50_fp16_batch_64_as_benchmarked():
     s.close()
 
 
+def test_measured_choice_of_convolution_variants():
+    """Session.tune times the runtime's fp16 channels-last convolution variants on the program's own layers and
+    keeps the winners as the calls' `algo` operands: the results stay within the fp16 tolerance of the fp32 oracle
+    (variants may split a reduction differently), a second session given the same choices gives the first one's
+    bits, eager and replayed from a graph, and an fp32 program has nothing to tune."""
+    import torch
+    flags = dict(fusion=True, fuse_residual=True, fuse_matmul_bias=True, channels_last=True, fuse_first_layer_maxpool=True,
+                 fuse_projection_shortcut=True, alias_copies=True, inplace_residual=True, compact_pool=True)
+    build16 = lambda: models.resnet50(8, np.float16, seed=5, image=96)  # noqa: E731
+    ref, _ = run(lambda: as_fp32_graph(*build16()), ORACLE_PATH, fusion=True)
+    g, inputs = build16()
+    p = g.compile(**flags)
+    s = p.session(compiler.MODE_RESIDENT)
+    plain = s.run(*inputs)[0]
+    close16(plain, ref[0])
+    assert all(a == (0, 0) for a in s.algos()) and len(s.algos()) == p.num_ops(compute_only=True)
+    changed = s.tune(inputs, reps=3)
+    chosen = s.algos()
+    assert changed == sum(1 for a in chosen if a != (0, 0))
+    tuned = s.run(*inputs)[0]
+    close16(tuned, ref[0])
+    s.close()
+    # every variant id on every convolution that can take it, through the algo operand: still the oracle's result
+    s2 = p.session(compiler.MODE_RESIDENT)
+    s2.set_algos(chosen)
+    np.testing.assert_array_equal(s2.run(*inputs)[0], tuned)
+    dev_in = [torch.from_numpy(a).cuda() for a in inputs]
+    dev_out = torch.empty(tuned.shape, dtype=torch.float16, device="cuda")
+    for _ in range(2):
+        s2.run_device([t.data_ptr() for t in dev_in], [dev_out.data_ptr()], use_graph=True)
+        s2.sync()
+        np.testing.assert_array_equal(dev_out.cpu().numpy(), tuned)
+    for vid in (3, 4, 12, 64, 66, 54):
+        s2.set_algos([(vid, vid)] * len(chosen))
+        close16(s2.run(*inputs)[0], ref[0])
+    with pytest.raises(RuntimeError):
+        s2.set_algos([(0, 0)])
+    s2.close()
+    g32, in32 = models.resnet50(image=64, classes=10)
+    s32 = g32.compile(fusion=True).session(compiler.MODE_RESIDENT)
+    assert s32.tune(in32, reps=3) == 0
+    s32.close()
+
+
 def test_bert_base_12_layers_as_benchmarked():
     """BERT-base at its full depth with the benchmark's flags, against the oracle running the unfused
     program (tolerance: rtol 1e-4, atol 1e-4 on outputs of order one after the final LayerNorm)."""
