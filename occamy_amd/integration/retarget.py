@@ -21,12 +21,24 @@ edit is computed from the checkout's own files):
 * ``src/Conversion/DNNToLLVM/Ops/cudnn/fusedOps/ConvBiasActiv.cpp`` -- the call
   passes ``group`` after the algorithm and the element type last.
 
-The remaining call sites (one ``callApi`` per file under ``Ops/cuda`` and
-``Ops/cublas``) each gain the handle as first operand and the element type as
-last; the script lists them instead of rewriting them, since they differ in how
-they name their operands.  The compiler cannot be built in this repository's
-environment (no MLIR); ``tests/test_boundary_vs_reference.py`` checks that the
-table this script writes declares exactly the prototypes of ``include/dnnrt.h``.
+* ``src/Conversion/DNNToLLVM/DNNRuntimeAPI.hpp`` -- the ``API`` enum gains
+  ``SET_STREAM`` and ``SYNC``.
+* ``src/Conversion/DNNToLLVM/DNNToLLVMCommon.{hpp,cpp}`` -- four small helpers are
+  added (the handle loaded from the slot ``generateDNNHandle`` creates, and the
+  element-type code, rank and host dims array of a tensor value);
+  ``generateDNNHandle`` keeps the slot and calls ``dnnrtSync`` in front of
+  ``dnnrtDestroy``; ``generateCUDAStream`` calls ``dnnrtSetStream`` once the stream
+  exists.
+* every ``callApi`` site under ``src/Conversion/DNNToLLVM/Ops`` -- its operand list
+  is transformed exactly as its row of the table: the handle first where the row
+  took none, the element type last, and for PRelu / Squeeze / Unsqueeze / Expand /
+  NonZero the operand shapes ``include/dnnrt.h`` declares.  The operands keep the
+  names each file gives them; what is added comes from the helpers.
+
+The compiler cannot be built in this repository's environment (no MLIR);
+``tests/test_boundary_vs_reference.py`` checks that the table this script writes
+declares exactly the prototypes of ``include/dnnrt.h`` and that every rewritten
+call site passes as many operands as its rewritten row declares.
 """
 import argparse
 import difflib
@@ -38,6 +50,10 @@ SPECS = "src/Conversion/DNNToLLVM/DNNAPISpecs.inc"
 DIALECT = "src/Dialect/DNN/DNN.td"
 FUSION = "src/Transform/DNN/opFusing/fuseConvBiasRelu.cpp"
 FUSED_LOWERING = "src/Conversion/DNNToLLVM/Ops/cudnn/fusedOps/ConvBiasActiv.cpp"
+API_HPP = "src/Conversion/DNNToLLVM/DNNRuntimeAPI.hpp"
+COMMON_HPP = "src/Conversion/DNNToLLVM/DNNToLLVMCommon.hpp"
+COMMON_CPP = "src/Conversion/DNNToLLVM/DNNToLLVMCommon.cpp"
+OPS_DIR = "src/Conversion/DNNToLLVM/Ops"
 
 H, DT, I64, P = "handlePtrTy", "int32Ty", "int64Ty", "int64PtrTy"
 
@@ -168,20 +184,229 @@ def pass_group_and_dtype_when_lowering(text):
     return text[:anchor] + consts + text[anchor:]
 
 
-EDITS = [(SPECS, retarget_table), (DIALECT, add_group_attribute), (FUSION, pass_group_when_fusing),
-         (FUSED_LOWERING, pass_group_and_dtype_when_lowering)]
+def add_api_enumerators(text):
+    m = re.search(r"STREAM_DESTROY,\s*\n", text)
+    if not m:
+        raise SystemExit(f"{API_HPP}: STREAM_DESTROY not found in the API enum")
+    indent = re.match(r"\s*", text[text.rfind("\n", 0, m.start()) + 1:m.start()]).group(0)
+    return text[:m.end()] + f"{indent}SET_STREAM,\n{indent}SYNC,\n" + text[m.end():]
 
 
-def remaining_call_sites(root):
-    """Files under Ops/ whose callApi still needs the handle first and the element type last."""
+HELPER_DECLS = """// ---- libdnnrt: what every call site passes besides its own operands ----
+extern mlir::Value dnnrtHandleSlot;  // the alloca generateDNNHandle creates
+mlir::Value dnnrtHandle(mlir::OpBuilder &builder, mlir::Location loc);
+mlir::Value dnnrtElementType(mlir::OpBuilder &builder, mlir::Location loc, mlir::Value tensor);
+mlir::Value dnnrtRank(mlir::OpBuilder &builder, mlir::Location loc, mlir::Value tensor);
+mlir::Value dnnrtDims(mlir::OpBuilder &builder, mlir::Location loc, mlir::Value tensor);
+
+"""
+
+HELPER_DEFS = """// ---- libdnnrt: what every call site passes besides its own operands ----
+mlir::Value dnnrtHandleSlot;
+
+// the runtime handle, loaded from the slot generateDNNHandle creates
+mlir::Value dnnrtHandle(mlir::OpBuilder &builder, mlir::Location loc) {
+  auto *context = builder.getContext();
+  auto handlePtrTy = LLVM::LLVMPointerType::get(LLVM::LLVMStructType::getOpaque("cudnnContext", context));
+  return builder.create<LLVM::LoadOp>(loc, handlePtrTy, dnnrtHandleSlot);
+}
+
+// include/dnnrt.h: DNNRT_F32 = 0, DNNRT_F16 = 1, DNNRT_I64 = 2
+mlir::Value dnnrtElementType(mlir::OpBuilder &builder, mlir::Location loc, mlir::Value tensor) {
+  auto elem = tensor.getType().cast<mlir::ShapedType>().getElementType();
+  int32_t code = elem.isF16() ? 1 : (elem.isa<mlir::IntegerType>() ? 2 : 0);
+  return builder.create<LLVM::ConstantOp>(loc, builder.getI32Type(), builder.getI32IntegerAttr(code));
+}
+
+mlir::Value dnnrtRank(mlir::OpBuilder &builder, mlir::Location loc, mlir::Value tensor) {
+  int64_t rank = tensor.getType().cast<mlir::ShapedType>().getRank();
+  return builder.create<LLVM::ConstantOp>(loc, builder.getI64Type(), builder.getI64IntegerAttr(rank));
+}
+
+// a host int64 array holding the tensor's static shape
+mlir::Value dnnrtDims(mlir::OpBuilder &builder, mlir::Location loc, mlir::Value tensor) {
+  auto shape = tensor.getType().cast<mlir::ShapedType>().getShape();
+  auto int64Ty = builder.getI64Type();
+  auto int64PtrTy = LLVM::LLVMPointerType::get(int64Ty);
+  auto count = builder.create<LLVM::ConstantOp>(loc, int64Ty, builder.getI64IntegerAttr(std::max<int64_t>(shape.size(), 1)));
+  auto dims = builder.create<LLVM::AllocaOp>(loc, int64PtrTy, count, 0);
+  for (size_t i = 0; i < shape.size(); i++) {
+    auto at = builder.create<LLVM::ConstantOp>(loc, builder.getI32Type(), builder.getI32IntegerAttr((int32_t)i));
+    auto value = builder.create<LLVM::ConstantOp>(loc, int64Ty, builder.getI64IntegerAttr(shape[i]));
+    auto slot = builder.create<LLVM::GEPOp>(loc, int64PtrTy, dims, ArrayRef<Value>({at}));
+    builder.create<LLVM::StoreOp>(loc, value, slot);
+  }
+  return dims;
+}
+
+"""
+
+
+def declare_helpers(text):
+    at = text.find("void generateDNNHandle(")
+    if at < 0:
+        raise SystemExit(f"{COMMON_HPP}: generateDNNHandle is not declared here")
+    return text[:at] + HELPER_DECLS + text[at:]
+
+
+def define_helpers_and_calls(text):
+    """generateDNNHandle keeps the slot and waits for the stream before the handle goes; generateCUDAStream hands the
+    stream to the handle; the helpers' definitions go in front of generateDNNHandle."""
+    at = text.find("void generateDNNHandle(")
+    if at < 0:
+        raise SystemExit(f"{COMMON_CPP}: generateDNNHandle not found")
+    text = text[:at] + HELPER_DEFS + text[at:]
+    m = re.search(r"(\n(\s*))auto handleDestroy = DNNRuntimeAPI::callApi\(", text)
+    if not m:
+        raise SystemExit(f"{COMMON_CPP}: the dnnrtDestroy call of generateDNNHandle is not the one this script knows")
+    ind = m.group(2)
+    sync = (f"{m.group(1)}auto handleSync = DNNRuntimeAPI::callApi(builder, loc, apiRegistry,"
+            f"\n{ind}    DNNRuntimeAPI::API::SYNC, {{handleLoad}});")
+    text = text[:m.start()] + sync + text[m.start():]
+    m = re.search(r"(\n(\s*))handleDestroy\.getDefiningOp\(\)->moveBefore\(&parentBlock\.back\(\)\);", text)
+    if not m:
+        raise SystemExit(f"{COMMON_CPP}: generateDNNHandle does not move its destroy call the way this script knows")
+    text = text[:m.start()] + f"{m.group(1)}handleSync.getDefiningOp()->moveBefore(&parentBlock.back());" + text[m.start():]
+    m = re.search(r"(\n(\s*))cudnnHandle = handleAlloca;", text)
+    if not m:
+        raise SystemExit(f"{COMMON_CPP}: generateDNNHandle does not hand out its slot the way this script knows")
+    text = text[:m.end()] + f"{m.group(1)}dnnrtHandleSlot = handleAlloca;" + text[m.end():]
+    # the stream: once it exists, and before the load that belongs to its destruction, give it to the handle
+    m = re.search(r"(\n(\s*))auto streamLoad = builder\.create<LLVM::LoadOp>\(", text)
+    if not m:
+        raise SystemExit(f"{COMMON_CPP}: generateCUDAStream is not the one this script knows")
+    ind = m.group(2)
+    set_stream = (f"{m.group(1)}auto streamForHandle = builder.create<LLVM::LoadOp>(loc, streamPtrTy, streamAlloca);"
+                  f"{m.group(1)}DNNRuntimeAPI::callApi(builder, loc, apiRegistry, DNNRuntimeAPI::API::SET_STREAM,"
+                  f"\n{ind}    {{dnnrtHandle(builder, loc), streamForHandle}});")
+    return text[:m.start()] + set_stream + text[m.start():]
+
+
+# ---- the call sites -----------------------------------------------------------------------------------------------
+HANDLE_X = "dnnrtHandle(rewriter, loc)"
+DTYPE_X = "dnnrtElementType(rewriter, loc, op->getResult(0))"
+RANK_IN_X = "dnnrtRank(rewriter, loc, op->getOperand(0))"
+RANK_OUT_X = "dnnrtRank(rewriter, loc, op->getResult(0))"
+
+CALL_RE = re.compile(r"callApi\(\s*rewriter,\s*loc,\s*apiRegistry,\s*(?:core_dnn::)?DNNRuntimeAPI::\s*API::(\w+),\s*\{", re.S)
+
+
+def split_operands(body):
+    """Top-level comma split of a braced operand list (comments are no operands)."""
+    body = re.sub(r"/\*.*?\*/", " ", body, flags=re.S)
+    body = re.sub(r"//[^\n]*", " ", body)
+    out, depth, cur = [], 0, ""
+    for ch in body:
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+        if ch == "," and depth == 0:
+            out.append(" ".join(cur.split()))
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        out.append(" ".join(cur.split()))
+    return out
+
+
+def call_sites(text):
+    """[(API enumerator, index of the operand list's '{', index behind its '}', operands)] of a source file."""
     out = []
-    base = os.path.join(root, "src/Conversion/DNNToLLVM/Ops")
-    for d, _, files in sorted(os.walk(base)):
+    for m in CALL_RE.finditer(text):
+        depth, i = 1, m.end()
+        while depth and i < len(text):
+            depth += text[i] == "{"
+            depth -= text[i] == "}"
+            i += 1
+        out.append((m.group(1), m.end() - 1, i, split_operands(text[m.end():i - 1])))
+    return out
+
+
+def site_operands(api, name, ops, rel):
+    """The operand expressions of a call site after the transformation its table row gets."""
+    change = ROWS[name][1]
+    if change is same:
+        return ops
+    if change is dtype_last:
+        return ops + [DTYPE_X]
+    if change is handle_first_dtype_last:
+        return [HANDLE_X] + ops + [DTYPE_X]
+    if change is prelu:       # (X, Y, dimY, slope, rank) -> (handle, X, Y, dimY, slope, dimSlope, rank, dtype)
+        if len(ops) != 5:
+            raise SystemExit(f"{rel}: the PRelu call is not the one this script knows")
+        return [HANDLE_X] + ops[:4] + ["dnnrtDims(rewriter, loc, slope)"] + ops[4:] + [DTYPE_X]
+    # the (handle, X, dimX, rankX, Y, dimY, rankY, dtype) rows
+    if api.startswith("CUDA_SQUEEZE") or api.startswith("CUDA_UNSQUEEZE"):   # (X, dimX, Y, dimY, axes, rank)
+        if len(ops) != 6:
+            raise SystemExit(f"{rel}: the Squeeze / Unsqueeze call is not the one this script knows")
+        return [HANDLE_X, ops[0], ops[1], RANK_IN_X, ops[2], ops[3], RANK_OUT_X, DTYPE_X]
+    if api == "CUDA_EXPAND":                                               # (X, dimX, rankX, Y, dimY, shape, dimShape)
+        if len(ops) != 7:
+            raise SystemExit(f"{rel}: the Expand call is not the one this script knows")
+        return [HANDLE_X] + ops[:5] + [RANK_OUT_X, DTYPE_X]
+    if api.startswith("CUDA_NONZERO"):                                      # (X, dimX, Y, dimY, rank)
+        if len(ops) != 5:
+            raise SystemExit(f"{rel}: the NonZero call is not the one this script knows")
+        return [HANDLE_X, ops[0], ops[1], ops[4], ops[2], ops[3], RANK_OUT_X, DTYPE_X]
+    raise SystemExit(f"{rel}: no operand rule for {api}")
+
+
+def api_names(specs_text):
+    """API enumerator -> the reference's symbol, from the table."""
+    return {m.group(1): m.group(2) for m in ROW_RE.finditer(specs_text)}
+
+
+def retarget_call_sites(text, rel, names):
+    """Every callApi of one Ops/ file with its operand list transformed as its row is (the fused convolution's file
+    has an edit of its own)."""
+    out, pos = "", 0
+    for api, lo, hi, ops in call_sites(text):
+        if api not in names:
+            raise SystemExit(f"{rel}: API::{api} has no row in the table")
+        new_ops = site_operands(api, names[api], ops, rel)
+        if new_ops == ops:
+            continue
+        indent = re.match(r"\s*", text[text.rfind("\n", 0, lo) + 1:lo]).group(0)
+        lines, cur = [], "{"
+        for i, o in enumerate(new_ops):
+            piece = o + (", " if i + 1 < len(new_ops) else "")
+            if len(cur) + len(piece) + len(indent) > 100 and cur.strip("{ "):
+                lines.append(cur.rstrip())
+                cur = ""
+            cur += piece
+        lines.append(cur + "}")
+        out += text[pos:lo] + ("\n" + indent).join(lines)
+        pos = hi
+    return out + text[pos:]
+
+
+def ops_files(root):
+    out = []
+    for d, _, files in sorted(os.walk(os.path.join(root, OPS_DIR))):
         for f in sorted(files):
             path = os.path.join(d, f)
-            if f.endswith(".cpp") and os.path.relpath(path, root) != FUSED_LOWERING and "callApi" in open(path).read():
+            if f.endswith(".cpp") and "callApi" in open(path).read():
                 out.append(os.path.relpath(path, root))
     return out
+
+
+def all_edits(root):
+    """[(relative path, old text, new text)] of everything the script changes."""
+    read = lambda rel: open(os.path.join(root, rel)).read()  # noqa: E731
+    names = api_names(read(SPECS))
+    edits = []
+    for rel, edit in [(SPECS, retarget_table), (DIALECT, add_group_attribute), (FUSION, pass_group_when_fusing),
+                      (API_HPP, add_api_enumerators), (COMMON_HPP, declare_helpers), (COMMON_CPP, define_helpers_and_calls)]:
+        old = read(rel)
+        edits.append((rel, old, edit(old)))
+    for rel in ops_files(root):
+        old = read(rel)
+        new = pass_group_and_dtype_when_lowering(old) if rel == FUSED_LOWERING else retarget_call_sites(old, rel, names)
+        if new != old:
+            edits.append((rel, old, new))
+    return edits
 
 
 def main(argv=None):
@@ -189,17 +414,11 @@ def main(argv=None):
     ap.add_argument("checkout")
     ap.add_argument("--write", action="store_true", help="edit the checkout in place instead of printing the diff")
     args = ap.parse_args(argv)
-    for rel, edit in EDITS:
-        path = os.path.join(args.checkout, rel)
-        old = open(path).read()
-        new = edit(old)
+    for rel, old, new in all_edits(args.checkout):
         if args.write:
-            open(path, "w").write(new)
+            open(os.path.join(args.checkout, rel), "w").write(new)
         else:
             sys.stdout.writelines(difflib.unified_diff(old.splitlines(True), new.splitlines(True), "a/" + rel, "b/" + rel))
-    print("# call sites that still take the handle as first and the element type as last operand by hand:", file=sys.stderr)
-    for rel in remaining_call_sites(args.checkout):
-        print("#   " + rel, file=sys.stderr)
 
 
 if __name__ == "__main__":
