@@ -494,7 +494,7 @@ void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t handle, const void *X, const i
     DNNRT_FAIL("%s: the two convolutions give [%d,%d,%d,%d] and [%d,%d,%d,%d]", who, s1.N, s1.K, s1.P, s1.Q, s2.N, s2.K, s2.P, s2.Q);
   const bool both_1x1 = s1.R == 1 && s1.S == 1 && s2.R == 1 && s2.S == 1 && !s1.ph && !s1.pw && !s2.ph && !s2.pw && s1.sh == 1 && s1.sw == 1;
   // one kernel where that is the faster way ...
-  if (dtype == DNNRT_F16 && both_1x1 && ((s1.C == 64 && s2.C == 64) || (s1.C == 128 && s2.C == 256))) {
+  if (dtype == DNNRT_F16 && both_1x1) {
     dnnrt::ConvF16Args a{};
     a.X = (const __half *)X; a.Wt = (const __half *)W; a.bias = (const __half *)B; a.Z = nullptr; a.Y = (__half *)Y;
     a.N = s1.N; a.C = s1.C; a.H = s1.H; a.W = s1.W; a.K = s1.K; a.Cg = s1.Cg; a.R = 1; a.S = 1;
@@ -502,7 +502,25 @@ void *dnnrtConvBiasAddConvBiasActiv(dnnrtHandle_t handle, const void *X, const i
     a.act = (int)activMode; a.act_coef = handle->act_coef; a.format = handle->format;
     a.X2 = (const __half *)X2; a.Wt2 = (const __half *)W2; a.bias2 = (const __half *)B2;
     a.C2 = s2.C; a.H2 = s2.H; a.W2 = s2.W; a.sh2 = s2.sh; a.sw2 = s2.sw;
-    if (dnnrt::dual_conv_applies(a)) {
+    // Short reductions (64 + 64 or 128 + 256 channels), where the pair is bound by the bytes of the result: the
+    // kernel that gives the two calls' bits.  Longer ones, and the short ones when the call's `algo` names a variant
+    // of it: one reduction over both convolutions' channels, rounded once (closer to the exact sum than the
+    // chain, not its bits).
+    const int asked = dnnrt::variant_of_algo(algo);
+    const bool short_pair = (s1.C == 64 && s2.C == 64) || (s1.C == 128 && s2.C == 256);
+    if (short_pair && !dnnrt::dma_dual_variant(asked) && dnnrt::dual_conv_applies(a)) {
+      if (!dnnrt::launch_conv_f16_dual(handle, a)) return nullptr;
+      return Y;
+    }
+    if (handle->f16_tile == 0 && dnnrt::dma_dual_applies(a)) {
+      a.magic_pq = dnnrt::magic_of(a.P * a.Q);
+      a.magic_q = dnnrt::magic_of(a.Q);
+      if (!dnnrt::launch_conv_f16_dma_dual(handle, a, asked)) return nullptr;
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) DNNRT_FAIL("%s: launch failed: %s", who, hipGetErrorString(e));
+      return Y;
+    }
+    if (short_pair && dnnrt::dual_conv_applies(a)) {
       if (!dnnrt::launch_conv_f16_dual(handle, a)) return nullptr;
       return Y;
     }

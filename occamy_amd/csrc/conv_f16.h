@@ -62,6 +62,12 @@ bool launch_conv_f16_pointwise(const dnnrtContext *ctx, const ConvF16Args &a);
 // that file's tile ids, `a` must satisfy dma_conv_applies and carry the division constants.
 bool dma_conv_applies(const ConvF16Args &a);
 bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int variant);
+// Y = act(conv(X, W) + bias + conv(X2, W2) + bias2) as one reduction over both convolutions' channels (both 1x1, no
+// padding; the sum is formed in fp32 and rounded once); variant: one of the ids dma_dual_variant accepts, else the
+// launcher picks.
+bool dma_dual_applies(const ConvF16Args &a);
+bool dma_dual_variant(int variant);
+bool launch_conv_f16_dma_dual(const dnnrtContext *ctx, const ConvF16Args &a, int variant);
 
 // 3x3 stride-1 pad-1 channels-last convolutions over at least 128 channels with the input patch kept in LDS
 // (conv_f16_patch.hip): `variant` is one of that file's tile ids, `a` must satisfy patch_conv_applies and carry the

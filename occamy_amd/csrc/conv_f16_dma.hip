@@ -58,7 +58,11 @@ __device__ __forceinline__ void ring_barrier() {
 // (BM / WM) x (BN / WN) of it as 32x32 MFMA blocks, NS LDS stages.
 // MASKED: some lane of some step may have to read zeros in place of an
 // activation (padding, or pixel rows past the end of the tensor).
-template <int BM, int BN, int WM, int WN, int NS, bool MASKED>
+// DUAL: two 1x1 convolutions without padding onto the same result as ONE reduction (a residual block's projection
+// shortcut and its last convolution): the steps over the second convolution's channels (X2, Wt2) come first, then
+// those over the first one's; a step differs from another only in which tensors and per-lane offsets its loads
+// use.  The sum of both reductions and both biases is formed in fp32 and rounded once.
+template <int BM, int BN, int WM, int WN, int NS, bool MASKED, bool DUAL = false>
 __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF16Args a, const int tiles_total) {
   // The buffer-resource type exists for the device target only: the host pass, which needs just the launch stub,
   // would silently drop a kernel whose body it cannot type-check.
@@ -131,15 +135,58 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
     b_out[i] = ~in;
   }
 
-  const int steps_c = a.C >> 6, nk = a.R * a.S * steps_c;
+  // DUAL: the same for the second convolution (1x1, no padding: one tap, always inside; a pixel past the end of the
+  // tensor is an out-of-range offset, and so it is for the first convolution in this form)
+  [[maybe_unused]] unsigned a2_off[DUAL ? A_L : 1], b2_base[DUAL ? B_L : 1];
+  [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc_w2 = rsrc_w, rsrc_x2 = rsrc_x;
+  if constexpr (DUAL) {
+    rsrc_w2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(a.Wt2), 0, 2 * a.K * a.C2, 0x00020000);
+    rsrc_x2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(a.X2), 0, 2 * a.N * a.H2 * a.W2 * a.C2, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < A_L; i++) {
+      const int row = 8 * (wave + i * NW) + (lane >> 3), ch = (lane & 7) ^ ((row >> 1) & 7);
+      const int k_out = m0 + row;
+      a2_off[i] = k_out < a.K ? 2u * (unsigned)(k_out * a.C2 + ch * 8) : DMA_OUT_OF_RANGE;
+    }
+#pragma unroll
+    for (int i = 0; i < B_L; i++) {
+      const int row = 8 * (wave + i * NW) + (lane >> 3), ch = (lane & 7) ^ ((row >> 1) & 7);
+      const int pix = n0 + row;
+      const bool ok = pix < NPQ;
+      const int n = ok ? div_magic(pix, PQ, a.magic_pq) : 0;
+      const int pq = ok ? pix - n * PQ : 0;
+      const int p = div_magic(pq, a.Q, a.magic_q), q = pq - p * a.Q;
+      b2_base[i] = ok ? 2u * (unsigned)(((n * a.H2 + p * a.sh2) * a.W2 + q * a.sw2) * a.C2 + ch * 8) : DMA_OUT_OF_RANGE;
+      if (!ok) b_base[i] = (int)DMA_OUT_OF_RANGE;
+    }
+  }
+
+  const int steps_c = a.C >> 6, steps_2 = DUAL ? a.C2 >> 6 : 0, nk = a.R * a.S * steps_c + steps_2;
   // cursor of the next step to load (all scalar)
   int l_r = 0, l_s = 0, l_c0 = 0, l_stage = 0, l_k = 0;
+  [[maybe_unused]] int l_it = 0;
 
   // The loads of one step, in three parts so that they can be issued between the MFMA groups of another step
   // (a wavefront that issues them all at once sits in the memory pipeline's queue while its MFMA queue drains).
   auto issue_loads = [&](auto lo_c, auto hi_c) {
     constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
     char *As = smem + l_stage * STAGE, *Bs = As + BM * 128;
+    if constexpr (DUAL) {
+      if (l_it < steps_2) {
+#pragma unroll
+        for (int n = LO; n < HI; n++) {
+          if (n < A_L) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w2, (lds_ptr)(As + 1024 * (wave + n * NW)), 16, a2_off[n], 2 * l_c0, 0, 0);
+          else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x2, (lds_ptr)(Bs + 1024 * (wave + (n - A_L) * NW)), 16, b2_base[n - A_L], 2 * l_c0, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int n = LO; n < HI; n++) {
+          if (n < A_L) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_ptr)(As + 1024 * (wave + n * NW)), 16, a_off[n], 2 * l_c0, 0, 0);
+          else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (lds_ptr)(Bs + 1024 * (wave + (n - A_L) * NW)), 16, (unsigned)b_base[n - A_L], 2 * l_c0, 0, 0);
+        }
+      }
+      return;
+    }
     const int tap = l_r * a.S + l_s;
     const int x_tap = 2 * ((l_r * a.W + l_s) * a.C);  // bytes from tap (0, 0) to this tap
 #pragma unroll
@@ -161,8 +208,13 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
     }
   };
   auto advance_loader = [&]() {
-    l_k += 64;
     l_stage = l_stage + 1 == NS ? 0 : l_stage + 1;
+    if constexpr (DUAL) {  // channel offset inside the convolution the step belongs to
+      l_it++;
+      l_c0 = l_it == steps_2 ? 0 : l_c0 + 64;
+      return;
+    }
+    l_k += 64;
     const int c0n = l_c0 + 64, sn = l_s + 1;
     const bool wrap_c = c0n == a.C, wrap_s = wrap_c && sn == a.S;
     l_c0 = wrap_c ? 0 : c0n;
@@ -193,6 +245,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
   // before the ring starts (older loads complete first, so the ring's counted
   // waits cover them).
   half4 bias4[TM][4];
+  [[maybe_unused]] half4 bias4b[DUAL ? TM : 1][4];  // DUAL: the second convolution's
   {
     const _Float16 *__restrict__ biasg = reinterpret_cast<const _Float16 *>(a.bias);
 #pragma unroll
@@ -203,6 +256,17 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
         const half4 zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
         bias4[i][g] = biasg ? *reinterpret_cast<const half4 *>(biasg + (k_out < a.K ? k_out : 0)) : zero;
       }
+    if constexpr (DUAL) {
+      const _Float16 *__restrict__ bias2g = reinterpret_cast<const _Float16 *>(a.bias2);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const int k_out = m0 + wm0 + i * 32 + 8 * g + 4 * half;
+          const half4 zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+          bias4b[i][g] = bias2g ? *reinterpret_cast<const half4 *>(bias2g + (k_out < a.K ? k_out : 0)) : zero;
+        }
+    }
     // The counted waits below assume these loads are older than every ring load: nothing may move across here.
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -325,7 +389,11 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
           const int kl = wm0 + i * 32 + 8 * g + 4 * half;
           half4 o;
 #pragma unroll
-          for (int e = 0; e < 4; e++) o[e] = (_Float16)apply_act(acc[i][j][4 * g + e] + (float)bias4[i][g][e], MODE, a.act_coef);
+          for (int e = 0; e < 4; e++) {
+            float v = acc[i][j][4 * g + e] + (float)bias4[i][g][e];
+            if constexpr (DUAL) v += (float)bias4b[i][g][e];
+            o[e] = (_Float16)apply_act(v, MODE, a.act_coef);
+          }
           *reinterpret_cast<half4 *>(Cs + (wn0 + j * 32 + l32) * CROW + kl) = o;
         }
   });
@@ -355,21 +423,29 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_f16_dma_kernel(const ConvF1
 }
 
 // More than 64 KiB of LDS per workgroup has to be asked for, once per kernel and device.
-template <int BM, int BN, int WM, int WN, int NS, bool MASKED>
+template <int BM, int BN, int WM, int WN, int NS, bool MASKED, bool DUAL = false>
 static bool launch_dma_masked(const dnnrtContext *ctx, const ConvF16Args &a, unsigned grid, int tiles) {
   constexpr int SMEM = NS * (BM + BN) * 128;
   static bool raised[16] = {};
   if (ctx->device < 0 || ctx->device >= 16) { set_error("conv(fp16): device ordinal %d", ctx->device); return false; }
   if (!raised[ctx->device]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_f16_dma_kernel<BM, BN, WM, WN, NS, MASKED>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_f16_dma_kernel<BM, BN, WM, WN, NS, MASKED, DUAL>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess) {
       set_error("conv(fp16): cannot reserve %d bytes of LDS", SMEM);
       return false;
     }
     raised[ctx->device] = true;
   }
-  hipLaunchKernelGGL((conv_f16_dma_kernel<BM, BN, WM, WN, NS, MASKED>), dim3(grid), dim3(64 * WM * WN), SMEM, ctx->stream, a, tiles);
+  hipLaunchKernelGGL((conv_f16_dma_kernel<BM, BN, WM, WN, NS, MASKED, DUAL>), dim3(grid), dim3(64 * WM * WN), SMEM, ctx->stream, a, tiles);
   return true;
+}
+
+template <int BM, int BN, int WM, int WN, int NS>
+static bool launch_dma_dual(const dnnrtContext *ctx, const ConvF16Args &a) {
+  const int64_t NPQ = (int64_t)a.N * a.P * a.Q;
+  const int64_t tiles = ceil_div(a.K, BM) * ceil_div(NPQ, BN);
+  if (tiles + 8 > INT32_MAX) { set_error("conv(fp16): too many tiles"); return false; }
+  return launch_dma_masked<BM, BN, WM, WN, NS, false, true>(ctx, a, (unsigned)(ceil_div(tiles, 8) * 8), (int)tiles);
 }
 
 template <int BM, int BN, int WM, int WN, int NS>
@@ -404,6 +480,34 @@ bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int vari
     case 66: return launch_dma<64, 128, 2, 4, 4>(ctx, a);   // the same on 64-row tiles
     default: set_error("conv(fp16): no direct-to-LDS variant %d", variant); return false;
   }
+}
+
+// The two-convolution form (one reduction over both, one rounding): `a` must satisfy dma_dual_applies and carry the
+// division constants; variant 0 picks by the number of tiles.
+bool dma_dual_variant(int variant) { return variant == 33 || variant == 39 || variant == 61 || variant == 64 || variant == 66 || variant == 37; }
+bool launch_conv_f16_dma_dual(const dnnrtContext *ctx, const ConvF16Args &a, int variant) {
+  if (!dma_dual_variant(variant)) {
+    const int64_t t128 = ceil_div(a.K, 128) * ceil_div((int64_t)a.N * a.P * a.Q, 128);
+    variant = 2 * t128 >= 3 * ctx->num_cu ? 64 : 66;
+  }
+  switch (variant) {
+    case 33: return launch_dma_dual<128, 128, 2, 2, 4>(ctx, a);
+    case 37: return launch_dma_dual<64, 128, 1, 4, 4>(ctx, a);
+    case 39: return launch_dma_dual<256, 128, 2, 2, 3>(ctx, a);
+    case 61: return launch_dma_dual<128, 128, 2, 2, 5>(ctx, a);
+    case 64: return launch_dma_dual<128, 128, 4, 2, 4>(ctx, a);
+    default: return launch_dma_dual<64, 128, 2, 4, 4>(ctx, a);
+  }
+}
+
+bool dma_dual_applies(const ConvF16Args &a) {
+  return a.format == DNNRT_NHWC && a.group == 1 && a.R == 1 && a.S == 1 && a.ph == 0 && a.pw == 0 && a.Z == nullptr && a.X2 && a.Wt2 &&
+         a.C % 64 == 0 && a.C2 % 64 == 0 && a.K % 8 == 0 && (a.H - 1) / a.sh + 1 == a.P && (a.W - 1) / a.sw + 1 == a.Q &&
+         (a.H2 - 1) / a.sh2 + 1 == a.P && (a.W2 - 1) / a.sw2 + 1 == a.Q &&
+         (int64_t)a.N * a.H * a.W * a.C < (1ll << 30) && (int64_t)a.N * a.H2 * a.W2 * a.C2 < (1ll << 30) &&
+         (int64_t)a.K * a.C < (1ll << 30) && (int64_t)a.K * a.C2 < (1ll << 30) && aligned16(a.X) && aligned16(a.Wt) && aligned16(a.Y) &&
+         aligned16(a.X2) && aligned16(a.Wt2) && (reinterpret_cast<uintptr_t>(a.bias) & 7u) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.bias2) & 7u) == 0;
 }
 
 bool dma_conv_applies(const ConvF16Args &a) {

@@ -21,10 +21,20 @@
 // with an out-of-range offset: they arrive as zeros.
 //
 // LDS layout: a slab is [patch pixel][128 bytes], the 16-byte chunk c of patch
-// pixel p kept at position c ^ ((p >> 1) & 7), which makes the MFMA operand
-// reads (32 consecutive pixels, one chunk) and the direct-to-LDS writes
-// conflict-free; two slabs (the one being read, the next one landing); filter
-// stages [k_out][128 bytes] with the same swizzle.
+// pixel p kept at position c ^ ((u >> 1) & 7) with u = p - 2 * (p / (W + 2)),
+// the pixel's index with the two frame columns of every patch row before it
+// taken out.  An MFMA operand read takes one chunk of 32 consecutive output
+// pixels at one tap; their patch indices jump by two wherever the run goes
+// on to the next image row, but their u are consecutive (the pixel behind a
+// row's last one has the next row's column `s`, which is W further in u), so
+// 16 lanes always land in 16 different 16-byte bank groups: u mod 16 picks
+// the group, its lowest bit through the address (p and u have the same
+// parity) and the next three through the position.  With p in place of u
+// every row change inside a run of 16 lanes put two lanes on one group, and
+// on 14 x 14 images every such run has one.  The direct-to-LDS writes are
+// linear, so conflict-free either way.  Two slabs (the one being read, the
+// next one landing); filter stages [k_out][128 bytes], chunk c of row k at
+// c ^ ((k >> 1) & 7).
 //
 // Reduction order: slab-major, tap-minor (the filter row of k_out holds, for
 // tap t, its C channels contiguously: step (slab, t) reads 128 bytes at
@@ -131,8 +141,9 @@ __global__ __launch_bounds__(64 * WM * WN * KG) void conv3x3_f16_patch_kernel(co
   unsigned p_off[P_L];
 #pragma unroll
   for (int i = 0; i < P_L; i++) {
-    const int pp = 8 * (wave + i * NW) + (lane >> 3), ch = (lane & 7) ^ ((pp >> 1) & 7);
+    const int pp = 8 * (wave + i * NW) + (lane >> 3);
     const int prow_rel = div_magic(pp, PW, a.magic_pw), col = pp - prow_rel * PW;
+    const int ch = (lane & 7) ^ (((pp - 2 * prow_rel) >> 1) & 7);
     const int prow = prow0 + prow_rel;
     const int n = div_magic(prow, Hp, a.magic_hp), hr = prow - n * Hp;
     const bool ok = pp < pp_needed && n < a.N && hr >= 1 && hr <= a.H && col >= 1 && col <= a.W;
@@ -147,13 +158,15 @@ __global__ __launch_bounds__(64 * WM * WN * KG) void conv3x3_f16_patch_kernel(co
     a_off[i] = k_out < a.K ? 2u * (unsigned)(k_out * CRS + ch * 8) : PATCH_OUT_OF_RANGE;
   }
   // operand fetch: patch index of tap (0, 0) of the pixel whose column of D this lane holds, per 32-pixel block
-  int pp00[TN];
+  // ... and the same index with the frame columns of the patch rows before it taken out (what the swizzle goes by)
+  int pp00[TN], uu00[TN];
 #pragma unroll
   for (int j = 0; j < TN; j++) {
     const int pix = min(n0 + wn0 + j * 32 + l32, NPQ - 1);  // a column past the end computes a copy that is never stored
     const int n = div_magic(pix, PQ, a.magic_pq), pq = pix - n * PQ;
     const int p = div_magic(pq, a.Q, a.magic_q), q = pq - p * a.Q;
     pp00[j] = (n * Hp + p - prow0) * PW + q;
+    uu00[j] = pp00[j] - 2 * (n * Hp + p - prow0);
   }
   const unsigned ld_a0 = (unsigned)((wm0 + l32) * 128 + ((half ^ ((l32 >> 1) & 7)) * 16));
 
@@ -208,11 +221,11 @@ __global__ __launch_bounds__(64 * WM * WN * KG) void conv3x3_f16_patch_kernel(co
   // ---- operand fetch -----------------------------------------------------------
   half8 fa[2][TM], fb[2][TN];
   unsigned bad[TN];  // this lane's patch addresses of the current tap (chunk of sub-step 0)
-  auto tap_addresses = [&](int tap_off) {
+  auto tap_addresses = [&](int tap_r, int tap_s) {  // tap (r, s): r patch rows down, s columns right
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const int pp = pp00[j] + tap_off;
-      bad[j] = (unsigned)(pp * 128 + (((half ^ (pp >> 1)) & 7) << 4));
+      const int pp = pp00[j] + tap_r * PW + tap_s, u = uu00[j] + tap_r * a.W + tap_s;
+      bad[j] = (unsigned)(pp * 128 + (((half ^ (u >> 1)) & 7) << 4));
     }
   };
   auto read_frags = [&](const char *stage, const char *slab, half8 (&qa)[TM], half8 (&qb)[TN], int sub) {
@@ -263,7 +276,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG) void conv3x3_f16_patch_kernel(co
     const char *nstage = ring + c_stage * A_STAGE;
     const char *nslab_ptr = NEXT == 0 ? patch + ((slab + 1) & 1) * SLAB : cur;
     if constexpr (SUBS == 1) { mfma_frags(fa[0], fb[0]); PIN(); }  // before its operand registers are fetched into again
-    tap_addresses((NEXT / 3) * PW + NEXT % 3);
+    tap_addresses(NEXT / 3, NEXT % 3);
     read_frags(nstage, nslab_ptr, fa[0], fb[0], kg); PIN();
     if constexpr (SUBS > 1) { mfma_frags(fa[1], fb[1]); PIN(); }
   };
@@ -274,7 +287,7 @@ __global__ __launch_bounds__(64 * WM * WN * KG) void conv3x3_f16_patch_kernel(co
   for (int q = 0; q < P; q++) issue_filter();
   patch_wait_vmcnt<(P - 1) * A_L>();
   patch_barrier();
-  tap_addresses(0);
+  tap_addresses(0, 0);
   read_frags(ring, patch, fa[0], fb[0], kg); PIN();
   for (int slab = 0; slab < nslab; slab++) {
     step(slab, std::integral_constant<int, 0>{});
