@@ -44,7 +44,7 @@ constexpr int NOALLOC_MAX_TILES = 1024;
 
 // The fp16 channels-last convolution variants dnnrtSetConvTile can force
 // (zero-terminated; what each one is: launch_conv_f16 in conv_f16.hip).
-constexpr int F16_TILE_IDS[] = {3, 4, 11, 12, 15, 17, 18, 31, 32, 33, 34, 35, 36, 37, 38, 39, 40, 60, 61, 62, 64, 66,
+constexpr int F16_TILE_IDS[] = {3, 4, 11, 12, 15, 17, 18, 31, 32, 33, 34, 35, 36, 37, 38, 39, 40, 60, 61, 62, 63, 64, 65, 66, 67, 69,
                                   41, 42, 43, 44, 45, 46, 47, 48, 49, 51, 52, 54, 57, 70, 0};
 
 void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));

@@ -476,6 +476,12 @@ bool launch_conv_f16_dma(const dnnrtContext *ctx, const ConvF16Args &a, int vari
     case 60: return launch_dma<128, 64, 2, 2, 6>(ctx, a);
     case 61: return launch_dma<128, 128, 2, 2, 5>(ctx, a);
     case 62: return launch_dma<64, 128, 1, 4, 6>(ctx, a);
+    // three stages only: 72 KiB (48 KiB) of LDS, so that two (three) workgroups share a compute unit and one's epilogue
+    // runs under another's reduction
+    case 63: return launch_dma<128, 64, 2, 2, 3>(ctx, a);
+    case 65: return launch_dma<64, 128, 2, 2, 3>(ctx, a);
+    case 67: return launch_dma<64, 128, 1, 4, 3>(ctx, a);
+    case 69: return launch_dma<64, 64, 2, 2, 3>(ctx, a);
     case 64: return launch_dma<128, 128, 4, 2, 4>(ctx, a);  // eight wavefronts: two per SIMD, one fills the other's waits
     case 66: return launch_dma<64, 128, 2, 4, 4>(ctx, a);   // the same on 64-row tiles
     default: set_error("conv(fp16): no direct-to-LDS variant %d", variant); return false;
