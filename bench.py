@@ -153,7 +153,11 @@ def measure(name, steps, warmup, profile_only=False, tune=True, reference_leg=Tr
     res["tuning"] = None
     if tune and dtype == "f16":
         t0 = time.perf_counter()
-        changed = sess.tune(ip, on_device=True, reps=5)
+        try:
+            changed = sess.tune(ip, on_device=True, reps=5)
+        except RuntimeError as e:  # the runtime's own choices stay in force; say what happened
+            changed = 0
+            res["tuning_error"] = str(e)
         tune_s = time.perf_counter() - t0
         res["tuning"] = dict(operations_with_a_measured_variant=changed, seconds=round(tune_s, 2),
                              ms_per_step_runtime_choice=1e3 * dt / steps)
@@ -327,7 +331,7 @@ def compact_record(res, steps, warmup):
     return {"value": res["value"], "unit": res["unit"], "steps": steps, "warmup": warmup, "ms_per_step": res["ms_per_step"],
             "latency_ms": res["latency_ms"], "dtype": res["dtype"],
             "config": {"workload": res["name"], "batch": res["batch"], "kernels_per_step": res["kernels_per_step"]},
-            "roofline": roofline_of(res), "by_class": class_figures(res),
+            "roofline": roofline_of(res), "by_class": class_figures(res), "tuning": res.get("tuning"),
             "pool_bytes": res["pool_bytes"], "pool_bytes_reference_flags": res["pool_bytes_reference_flags"],
             "weights_bytes": res["weights_bytes"], "device_bytes_total": res["device_bytes"]["total"],
             "occamy_semantics_value": res["occamy_semantics_value"]}
