@@ -4,6 +4,7 @@ flags and time it, the way the reference's test scripts do
 --dnn-malloc-pool-opt=true model.onnx``, run N times discarding the first,
 report mean / P90 / P95 / P99 in milliseconds)."""
 import argparse
+import json
 import time
 
 import numpy as np
@@ -32,6 +33,9 @@ def main():
     ap.add_argument("--fuse-first-layer-maxpool", action="store_true",
                     help="with --dnn-kernel-fusion and --channels-last: a ResNet's first convolution and its max-pool in one call")
     ap.add_argument("--resident", action="store_true", help="keep pool and weights on the device between runs")
+    ap.add_argument("--tune", metavar="FILE", help="with --resident: time the runtime's convolution variants on this model's layers, in place, "
+                    "keep the winners as the calls' algo operands (the reference picks cuDNN's algorithm the same way when it compiles a model) and write them to FILE")
+    ap.add_argument("--algos", metavar="FILE", help="with --resident: apply the choices an earlier --tune wrote to FILE")
     ap.add_argument("--runtime", default=None, help="shared object exporting include/dnnrt.h (default: the gfx950 library)")
     ap.add_argument("--iterations", type=int, default=100)
     ap.add_argument("--seed", type=int, default=0)
@@ -53,6 +57,20 @@ def main():
     for name, (shape, dt) in graph.input_shapes.items():
         inputs.append(rng.integers(0, 100, shape).astype(dt) if dt == np.int64 else rng.standard_normal(shape).astype(dt))
     sess = prog.session(compiler.MODE_RESIDENT if args.resident else compiler.MODE_OCCAMY, runtime_library=args.runtime)
+    if (args.tune or args.algos) and not args.resident:
+        raise SystemExit("--tune and --algos need --resident")
+    if args.algos:
+        with open(args.algos) as f:
+            saved = json.load(f)
+        if saved.get("program_ops") != prog.num_ops(compute_only=True):
+            raise SystemExit(f"{args.algos} was written for another program")
+        sess.set_algos([tuple(a) for a in saved["algos"]])
+    if args.tune:
+        sess.run(*inputs)
+        changed = sess.tune(inputs)
+        with open(args.tune, "w") as f:
+            json.dump({"program_ops": prog.num_ops(compute_only=True), "algos": sess.algos()}, f)
+        print(f"tuned: {changed} operation(s) got a measured variant; written to {args.tune}")
     times = []
     for i in range(args.iterations + 1):
         t0 = time.perf_counter()

@@ -5,6 +5,8 @@ tests/onnx_writer.py, written from the same published onnx.proto3 as the reader
 but independently of it (Python, emitting; the reader is C++, parsing), plus one
 model assembled by hand below.  A graph that went through a file must compile to
 the very same DNN program (text, pool layout) as the graph built in memory."""
+import os
+
 import numpy as np
 import pytest
 
@@ -223,3 +225,23 @@ def test_unknown_fields_are_skipped():
         ow.tag(31, 1) + b"\1\2\3\4\5\6\7\x08"
     p = compiler.load_onnx(junk + data).compile()
     assert p.pool_bytes == 1753344
+
+
+def test_command_line_tune_and_algos(tmp_path):
+    """python -m occamy_amd model.onnx --resident --tune FILE / --algos FILE: on the host build of the ABI there is
+    nothing to tune (no variant is chosen), the file holds two entries per runtime call, and it is accepted back."""
+    import json
+    import subprocess
+    import sys
+    g0, _ = models.single_conv()
+    model, saved = tmp_path / "m.onnx", tmp_path / "algos.json"
+    model.write_bytes(ow.model_bytes(g0))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    base = [sys.executable, "-m", "occamy_amd", str(model), "--runtime", ORACLE_PATH, "--iterations", "1"]
+    r = subprocess.run(base + ["--resident", "--tune", str(saved)], capture_output=True, text=True, cwd=root)
+    assert r.returncode == 0 and "tuned: 0 operation(s)" in r.stdout, r.stderr
+    assert json.loads(saved.read_text()) == {"program_ops": 3, "algos": [[0, 0]] * 3}
+    r = subprocess.run(base + ["--resident", "--algos", str(saved)], capture_output=True, text=True, cwd=root)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run(base + ["--tune", str(saved)], capture_output=True, text=True, cwd=root)
+    assert r.returncode != 0 and "--resident" in r.stderr
